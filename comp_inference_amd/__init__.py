@@ -1,0 +1,32 @@
+"""comp_inference_amd: the compressed-weight hot path of comp_inference for MI355X (gfx950).
+
+The public names follow the reference package (comp_inference/__init__.py:13-59); the
+implementation is a C-ABI HIP library (libcomp_inference_hip.so) driven through ctypes.
+"""
+from . import ccore
+from .comp_inference import (
+    compressed_nbytes,
+    extract_exp_and_mantissa,
+    get_rans_lut,
+    interleave_mantissas,
+    rans_compress_gate_up_fused,
+    rans_compress_module_weight,
+    rans_compress_qkv_fused,
+    rans_decompress_module_weight,
+    reconstruct_from_exp_and_mantissa,
+    uninterleave_mantissas,
+)
+from .linear_hip import (
+    fused_rans_linear,
+    fused_rans_linear_triton,
+    fused_rans_linear_triton_uncoalesced,
+    fused_rans_linear_uncoalesced,
+    splitk_reduce,
+)
+from .rans_hip import (
+    rans_decomp_flat,
+    rans_decomp_tiled,
+    rans_decomp_tiled_uncoalesced,
+    rans_decomp_triton,
+    rans_decomp_triton_tiled,
+)

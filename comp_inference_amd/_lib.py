@@ -1,0 +1,77 @@
+"""Loader of libcomp_inference_hip.so and the small amount of glue every op needs.
+
+There is no CPU or eager fallback: if the shared library is missing, or the current device
+is not a gfx950, the ops raise.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+import torch
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG, "libcomp_inference_hip.so")
+_lib = None
+_device_ok: set[int] = set()
+
+
+class Tiling(C.Structure):
+    _fields_ = [(n, C.c_uint32) for n in (
+        "K", "N", "tile_height", "tile_width", "num_tiles_k", "num_tiles_n", "num_tiles",
+        "streams_per_tile", "num_streams", "capacity")]
+
+
+def lib() -> C.CDLL:
+    """The shared library; raises RuntimeError when it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `python -m comp_inference_amd.build` "
+                "(hipcc, gfx950). The HIP extension is the only implementation of these ops.")
+        _lib = C.CDLL(LIB_PATH)
+        _lib.ci_last_error.restype = C.c_char_p
+        _lib.ci_encode_scratch_bytes.restype = C.c_size_t
+        _lib.ci_fused_linear_workspace_bytes.restype = C.c_size_t
+    return _lib
+
+
+def check(rc: int) -> None:
+    """0 -> return; anything else -> RuntimeError carrying the library's message (the reference
+    surfaces the same conditions as RuntimeError through pybind11)."""
+    if rc != 0:
+        raise RuntimeError(lib().ci_last_error().decode() or f"comp_inference_hip error {rc}")
+
+
+def require_device(t: torch.Tensor) -> None:
+    """Ops run on gfx950 tensors only."""
+    if not t.is_cuda:
+        raise RuntimeError("tensor must be on the GPU")  # src/python_bindings.cpp:68-69
+    idx = t.device.index if t.device.index is not None else torch.cuda.current_device()
+    if idx not in _device_ok:
+        with torch.cuda.device(idx):
+            check(lib().ci_check_device())
+        _device_ok.add(idx)
+
+
+def ptr(t: torch.Tensor | None) -> C.c_void_p:
+    return C.c_void_p(t.data_ptr()) if t is not None and t.numel() else C.c_void_p(0)
+
+
+def stream_handle(device: torch.device) -> C.c_void_p:
+    return C.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def as_u32(t: torch.Tensor, device) -> torch.Tensor:
+    """uint32/int32 metadata tensors are accepted interchangeably (the reference's callers pass
+    both, comp_inference/comp_inference.py:636-642 vs comp_inference/rans_saving.py:396-404)."""
+    if t.dtype not in (torch.uint32, torch.int32):
+        t = t.to(torch.int64).to(torch.uint32) if t.dtype != torch.uint32 else t
+    return t.to(device).contiguous()
+
+
+def as_u8(t: torch.Tensor, device) -> torch.Tensor:
+    if t.dtype != torch.uint8:
+        t = t.to(torch.uint8)
+    return t.to(device).contiguous()

@@ -1,0 +1,213 @@
+// Stand-alone rANS decode of the tiled two-streams-per-column format (gfx950).
+//
+// Work decomposition for the default 32-column tile: one wavefront per tile.  Lanes 0..31
+// own the top-half streams of columns 0..31, lanes 32..63 the bottom-half streams, so one
+// stored byte row (64 bytes) is one byte per lane.  Eight waves (eight neighbouring column
+// tiles) form a workgroup and share one LDS slot table; each wave stages its whole tile body
+// in LDS with 16-byte coalesced loads and then runs the sequential decode out of LDS.
+#include "ci_common.h"
+#include "rans_device.h"
+
+namespace ci {
+
+constexpr int kDecWaves = 8;
+
+struct DecodeArgs {
+    const uint8_t *stream;
+    uint64_t stream_len;
+    const uint32_t *states;
+    const uint32_t *tables;
+    const uint8_t *slot_map;
+    const uint32_t *tile_offsets;
+    const uint32_t *tile_max_lens;
+    uint32_t K, N, th, tw, tiles_n, num_tiles;
+    uint8_t *out_exp;
+    const uint8_t *man_tiled;
+    uint16_t *out_bf16;
+    uint32_t stage_bytes;  // LDS bytes per wave for the tile body
+};
+
+// The decode loop of one lane.  kFull: every lane takes all `half` steps (no row or column
+// masking).  kMerge: emit bf16 instead of the exponent byte.
+template <bool kFull, bool kMerge, typename Bytes>
+__device__ __forceinline__ void decode_lane(Bytes &src, uint32_t x, const uint2 *tab, uint32_t half,
+                                            uint32_t my_steps, uint8_t *out_row0, uint32_t lane_off,
+                                            uint32_t N, const uint8_t *man_row0, uint32_t man_off,
+                                            uint16_t *out16_row0) {
+    for (uint32_t i = 0; i < half; ++i) {
+        if (kFull || i < my_steps) {
+            uint32_t w = decode_symbol(x, tab);
+            uint32_t sym = w >> 24;
+            src.renorm(x);
+            src.renorm(x);
+            if (kMerge) {
+                uint32_t man = man_row0[(size_t)i * 32 + man_off];
+                out16_row0[(size_t)i * N + lane_off] = (uint16_t)assemble_bf16(sym, man);
+            } else {
+                out_row0[(size_t)i * N + lane_off] = (uint8_t)sym;
+            }
+        }
+    }
+}
+
+template <bool kMerge>
+__global__ __launch_bounds__(kDecWaves *kWave) void decode_tiled32_kernel(DecodeArgs a) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    uint2 *tab = reinterpret_cast<uint2 *>(lds);
+    const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
+    uint8_t *stage = lds + kSlotTableBytes + (size_t)wave * a.stage_bytes;
+
+    build_slot_table(tab, a.tables, a.slot_map, tid, kDecWaves * kWave);
+
+    const uint32_t tile = blockIdx.x * kDecWaves + wave;
+    const bool have_tile = tile < a.num_tiles;
+    uint32_t depth = 0;
+    uint64_t base = 0;
+    bool in_lds = false;
+    if (have_tile) {
+        base = a.tile_offsets[tile];
+        depth = a.tile_max_lens[tile];
+        // A body that would run past the stream is treated as empty rather than read.
+        if (base + (uint64_t)depth * 64 > a.stream_len) depth = 0;
+        in_lds = depth * 64u <= a.stage_bytes;
+        if (in_lds) stage_to_lds(stage, a.stream + base, depth * 64u, lane);
+    }
+    __syncthreads();
+    if (!have_tile) return;
+
+    const uint32_t tk = tile / a.tiles_n, tn = tile % a.tiles_n;
+    const uint32_t half = a.th / 2, hsel = lane / 32, c = lane % 32;
+    const uint32_t row0 = tk * a.th, col0 = tn * 32;
+    const uint32_t my_row0 = row0 + hsel * half;
+    uint32_t my_steps = 0;
+    if (col0 + c < a.N && my_row0 < a.K) my_steps = min(half, a.K - my_row0);
+    const bool full = __builtin_amdgcn_ballot_w64(my_steps != half) == 0;
+
+    uint32_t x = a.states[(size_t)tile * 64 + lane];
+    // wave-uniform row base + 32-bit per-lane offset keeps the address math scalar
+    uint8_t *out_row0 = kMerge ? nullptr : a.out_exp + (size_t)row0 * a.N + col0;
+    uint16_t *out16_row0 = kMerge ? a.out_bf16 + (size_t)row0 * a.N + col0 : nullptr;
+    const uint32_t lane_off = hsel * half * a.N + c;
+    const uint8_t *man_row0 = kMerge ? a.man_tiled + (size_t)tile * a.th * 32 : nullptr;
+    const uint32_t man_off = hsel * half * 32 + c;
+
+    if (in_lds) {
+        LdsBytes src;
+        src.init(stage, depth, 64, lane);
+        if (full)
+            decode_lane<true, kMerge>(src, x, tab, half, my_steps, out_row0, lane_off, a.N, man_row0,
+                                      man_off, out16_row0);
+        else
+            decode_lane<false, kMerge>(src, x, tab, half, my_steps, out_row0, lane_off, a.N, man_row0,
+                                       man_off, out16_row0);
+    } else {
+        GlobalBytes src;
+        src.init(a.stream + base, depth, 64, lane);
+        decode_lane<false, kMerge>(src, x, tab, half, my_steps, out_row0, lane_off, a.N, man_row0,
+                                   man_off, out16_row0);
+    }
+}
+
+// Any tile width: one thread per stream, bytes read where they lie.  Used for widths other
+// than 32 (the reference's tests sweep 16..128, tests/test_mat_mul.py:263-264).
+template <bool kMerge>
+__global__ __launch_bounds__(256) void decode_tiled_generic_kernel(DecodeArgs a) {
+    __shared__ uint2 tab[kProbScale];
+    build_slot_table(tab, a.tables, a.slot_map, threadIdx.x, 256);
+    __syncthreads();
+    const uint32_t spt = 2 * a.tw;
+    const uint64_t sid = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (sid >= (uint64_t)a.num_tiles * spt) return;
+    const uint32_t tile = (uint32_t)(sid / spt), q = (uint32_t)(sid % spt);
+    const uint32_t tk = tile / a.tiles_n, tn = tile % a.tiles_n;
+    const uint32_t half = a.th / 2, hsel = q / a.tw, c = q % a.tw;
+    const uint32_t col = tn * a.tw + c, my_row0 = tk * a.th + hsel * half;
+    if (col >= a.N || my_row0 >= a.K) return;
+    const uint32_t my_steps = min(half, a.K - my_row0);
+    uint64_t base = a.tile_offsets[tile];
+    uint32_t depth = a.tile_max_lens[tile];
+    if (base + (uint64_t)depth * spt > a.stream_len) depth = 0;
+    GlobalBytes src;
+    src.init(a.stream + base, depth, spt, q);
+    uint32_t x = a.states[sid];
+    const uint8_t *man = kMerge ? a.man_tiled + (size_t)tile * a.th * a.tw + (size_t)hsel * half * a.tw + c
+                                : nullptr;
+    for (uint32_t i = 0; i < my_steps; ++i) {
+        uint32_t sym = decode_symbol(x, tab) >> 24;
+        src.renorm(x);
+        src.renorm(x);
+        size_t o = (size_t)(my_row0 + i) * a.N + col;
+        if (kMerge)
+            a.out_bf16[o] = (uint16_t)assemble_bf16(sym, man[(size_t)i * a.tw]);
+        else
+            a.out_exp[o] = (uint8_t)sym;
+    }
+}
+
+}  // namespace ci
+
+using namespace ci;
+
+extern "C" int ci_decode_tiled_ilp2(const uint8_t *d_stream, uint64_t stream_len,
+                                    const uint32_t *d_states, const uint32_t *d_tables,
+                                    const uint8_t *d_slot_map, const uint32_t *d_tile_offsets,
+                                    const uint32_t *d_tile_max_lens, uint32_t K, uint32_t N,
+                                    uint32_t tile_height, uint32_t tile_width, uint8_t *d_out_exp,
+                                    const uint8_t *d_man_tiled, uint16_t *d_out_bf16,
+                                    ci_stream_t stream) {
+    if (K == 0 || N == 0) return CI_OK;
+    if (!d_states || !d_tables || !d_slot_map || !d_tile_offsets || !d_tile_max_lens)
+        return fail(CI_ERR_ARG, "ci_decode_tiled_ilp2: null table or metadata pointer");
+    if (stream_len && !d_stream) return fail(CI_ERR_ARG, "ci_decode_tiled_ilp2: null stream");
+    if (tile_height == 0 || tile_width == 0 || (tile_height & 1))
+        return fail(CI_ERR_ARG, "ci_decode_tiled_ilp2: tile_height must be even and non-zero");
+    const bool merge = d_man_tiled != nullptr;
+    if (merge && !d_out_bf16) return fail(CI_ERR_ARG, "ci_decode_tiled_ilp2: merge asked without bf16 output");
+    if (!merge && !d_out_exp) return fail(CI_ERR_ARG, "ci_decode_tiled_ilp2: null output");
+    if (!aligned(d_slot_map, 4)) return fail(CI_ERR_ARG, "ci_decode_tiled_ilp2: slot_map must be 4-byte aligned");
+
+    DecodeArgs a;
+    a.stream = d_stream;
+    a.stream_len = stream_len;
+    a.states = d_states;
+    a.tables = d_tables;
+    a.slot_map = d_slot_map;
+    a.tile_offsets = d_tile_offsets;
+    a.tile_max_lens = d_tile_max_lens;
+    a.K = K;
+    a.N = N;
+    a.th = tile_height;
+    a.tw = tile_width;
+    a.tiles_n = ceil_div(N, tile_width);
+    a.num_tiles = ceil_div(K, tile_height) * a.tiles_n;
+    a.out_exp = d_out_exp;
+    a.man_tiled = d_man_tiled;
+    a.out_bf16 = d_out_bf16;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+
+    if (tile_width == 32 && aligned(d_stream, 16)) {
+        a.stage_bytes = 14336;  // 224 byte rows per tile; deeper tiles read from global memory
+        const uint32_t lds_bytes = kSlotTableBytes + kDecWaves * a.stage_bytes;
+        const dim3 grid(ceil_div(a.num_tiles, kDecWaves)), block(kDecWaves * kWave);
+        if (merge) {
+            CI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(decode_tiled32_kernel<true>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes));
+            hipLaunchKernelGGL(decode_tiled32_kernel<true>, grid, block, lds_bytes, s, a);
+        } else {
+            CI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(decode_tiled32_kernel<false>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes));
+            hipLaunchKernelGGL(decode_tiled32_kernel<false>, grid, block, lds_bytes, s, a);
+        }
+        CI_LAUNCH_CHECK("decode_tiled32_kernel");
+    } else {
+        a.stage_bytes = 0;
+        const uint64_t streams = (uint64_t)a.num_tiles * 2 * tile_width;
+        const dim3 grid((uint32_t)((streams + 255) / 256)), block(256);
+        if (merge)
+            hipLaunchKernelGGL(decode_tiled_generic_kernel<true>, grid, block, 0, s, a);
+        else
+            hipLaunchKernelGGL(decode_tiled_generic_kernel<false>, grid, block, 0, s, a);
+        CI_LAUNCH_CHECK("decode_tiled_generic_kernel");
+    }
+    return CI_OK;
+}

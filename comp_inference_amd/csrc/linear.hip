@@ -1,0 +1,479 @@
+// Fused decompress + GEMV/GEMM and the split-K reduction (gfx950).
+//
+// out[M,N] = x[M,K] * W[K,N] (+ bias), W stored as rANS-coded exponent plane + raw
+// sign|mantissa plane; W is never materialised.  Replaces fused_rans_linear_triton and its
+// kernel fused_rans_matmul_kernel_ilp2_splitk (comp_inference/linear_triton.py:229-552) and
+// the torch.sum split-K reduction (comp_inference/linear_triton.py:303-314).
+//
+// Mapping for the default 32-column tile: one wavefront per tile; lanes 0..31 decode the
+// top-half streams of the tile's 32 columns, lanes 32..63 the bottom-half streams.  After 8
+// decode steps lane l holds 8 consecutive-k bf16 weights of column l%32 -- which is exactly
+// the A-operand fragment of v_mfma_f32_32x32x16_bf16 (A = W^T tile, 32 columns x 16 k, where
+// k 0..7 are the 8 top-half rows and k 8..15 the 8 bottom-half rows).  The B operand is the
+// matching slice of x for up to 32 rows of M, loaded straight from global memory.  One MFMA per
+// 8 decode steps does the whole contraction for any M <= 32, so the VALU only decodes.
+//
+// A workgroup is kw x nw waves: kw k-tiles of nw neighbouring column tiles.  The kw partial
+// accumulators are summed through LDS in a fixed order (deterministic); if one workgroup spans
+// all of K the result is written as bf16 directly, otherwise fp32 partials go to a workspace and
+// splitk_reduce_kernel sums them in index order.
+#include "ci_common.h"
+#include "rans_device.h"
+
+namespace ci {
+
+constexpr int kLinMaxWaves = 8;
+constexpr uint32_t kLinStageBytes = 14336;  // 224 byte rows per tile in LDS
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+struct LinearArgs {
+    const uint16_t *x;
+    uint32_t M, K, N, x_stride;
+    const uint8_t *stream;
+    uint64_t stream_len;
+    const uint32_t *states;
+    const uint32_t *tables;
+    const uint8_t *slot_map;
+    const uint32_t *tile_offsets;
+    const uint32_t *tile_max_lens;
+    const uint32_t *stream_offsets;  // dense layout
+    const uint32_t *stream_sizes;    // dense layout
+    const uint8_t *man_tiled;
+    const uint16_t *bias;
+    float *partial;   // [P][M][N] when P > 1
+    uint16_t *out;    // [M][N]
+    uint32_t out_stride;
+    uint32_t th, tw, tiles_n, tiles_k, kw, nw, P;
+    uint32_t stage_bytes;
+    int x_vec_ok;  // x rows may be read with 16-byte loads
+};
+
+__device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x40u);
+    u += 0x7FFFu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+__device__ __forceinline__ float bf16_to_f32(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
+
+// torch semantics of `out_bf16 += bias_bf16`: add in fp32, round once.
+__device__ __forceinline__ uint16_t finish_bf16(float acc, const uint16_t *bias, uint32_t n) {
+    uint16_t r = f32_to_bf16_rne(acc);
+    if (bias) r = f32_to_bf16_rne(bf16_to_f32(r) + bf16_to_f32(bias[n]));
+    return r;
+}
+
+// Two decoded symbols (top bytes of w0, w1) + two sign|mantissa bytes -> two bf16 in one dword
+// (row of w0 in the low half).
+__device__ __forceinline__ uint32_t pack_bf16_pair(uint32_t w0, uint32_t w1, uint32_t m0, uint32_t m1) {
+    const uint32_t e = __builtin_amdgcn_perm(w1, w0, 0x070C030Cu) >> 1;  // s1 << 23 | s0 << 7
+    const uint32_t mm = __builtin_amdgcn_perm(m1, m0, 0x04040000u);       // [m1 m1 m0 m0]
+    return (e & 0x7F807F80u) | (mm & 0x807F807Fu);
+}
+
+// Eight decode steps + operand assembly + MFMA for one block of 8 rows per half tile.
+// kFull: the whole tile lies inside [K,N] and the lane takes every step.
+template <int MB, bool kFull, typename Bytes>
+__device__ __forceinline__ void linear_tile(Bytes &src, uint32_t x, const uint2 *tab, const LinearArgs &a,
+                                            uint32_t half, uint32_t my_steps, const uint8_t *man,
+                                            const uint16_t *xrow[MB], bool m_ok[MB], uint32_t k0,
+                                            f32x16 acc[MB]) {
+    for (uint32_t i = 0; i < half; i += 8) {
+        // x fragment: 8 consecutive k of row m for this lane's half tile
+        u32x4 xv[MB];
+#pragma unroll
+        for (int b = 0; b < MB; ++b) {
+            xv[b] = (u32x4){0, 0, 0, 0};
+            if (m_ok[b]) {
+                if (kFull && a.x_vec_ok) {
+                    xv[b] = *reinterpret_cast<const u32x4 *>(xrow[b] + k0 + i);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        const uint32_t k = k0 + i + j;
+                        const uint32_t v = k < a.K ? xrow[b][k] : 0u;
+                        xv[b][j / 2] |= v << (16 * (j & 1));
+                    }
+                }
+            }
+        }
+        uint32_t mb[8], w[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) mb[j] = (kFull || i + j < my_steps) ? man[(size_t)(i + j) * 32] : 0u;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            if (kFull || i + j < my_steps) {
+                w[j] = decode_symbol(x, tab);
+                src.renorm(x);
+                src.renorm(x);
+            } else {
+                w[j] = 0;
+            }
+        }
+        u32x4 wv;
+#pragma unroll
+        for (int p = 0; p < 4; ++p) wv[p] = pack_bf16_pair(w[2 * p], w[2 * p + 1], mb[2 * p], mb[2 * p + 1]);
+#pragma unroll
+        for (int b = 0; b < MB; ++b)
+            acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, wv),
+                                                             __builtin_bit_cast(bf16x8, xv[b]), acc[b], 0, 0, 0);
+    }
+}
+
+// grid: (ceil(tiles_n / nw), P, ceil(M / (32 * MB)))   block: kw * nw waves
+template <int MB>
+__global__ __launch_bounds__(kLinMaxWaves *kWave) void fused_linear32_kernel(LinearArgs a) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    uint2 *tab = reinterpret_cast<uint2 *>(lds);
+    const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
+    const int nthreads = blockDim.x;
+    uint8_t *stage = lds + kSlotTableBytes + (size_t)wave * a.stage_bytes;
+
+    build_slot_table(tab, a.tables, a.slot_map, tid, nthreads);
+
+    const uint32_t kidx = wave % a.kw, nidx = wave / a.kw;
+    const uint32_t tk = blockIdx.y * a.kw + kidx, tn = blockIdx.x * a.nw + nidx;
+    const bool have_tile = tk < a.tiles_k && tn < a.tiles_n;
+    const uint32_t tile = tk * a.tiles_n + tn;
+    uint32_t depth = 0;
+    uint64_t base = 0;
+    bool in_lds = false;
+    if (have_tile) {
+        base = a.tile_offsets[tile];
+        depth = a.tile_max_lens[tile];
+        if (base + (uint64_t)depth * 64 > a.stream_len) depth = 0;
+        in_lds = depth * 64u <= a.stage_bytes;
+        if (in_lds) stage_to_lds(stage, a.stream + base, depth * 64u, lane);
+    }
+    __syncthreads();
+
+    const uint32_t half = a.th / 2, hsel = lane / 32, c = lane % 32;
+    const uint32_t m_base = blockIdx.z * 32 * MB;
+    f32x16 acc[MB];
+#pragma unroll
+    for (int b = 0; b < MB; ++b)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[b][v] = 0.f;
+
+    if (have_tile) {
+        const uint32_t col0 = tn * 32, k0 = tk * a.th + hsel * half;
+        uint32_t my_steps = 0;
+        if (col0 + c < a.N && k0 < a.K) my_steps = min(half, a.K - k0);
+        const bool full = __builtin_amdgcn_ballot_w64(my_steps != half) == 0;
+        const uint16_t *xrow[MB];
+        bool m_ok[MB];
+#pragma unroll
+        for (int b = 0; b < MB; ++b) {
+            const uint32_t m = m_base + b * 32 + c;
+            m_ok[b] = m < a.M;
+            xrow[b] = a.x + (size_t)(m_ok[b] ? m : 0) * a.x_stride;
+        }
+        const uint8_t *man = a.man_tiled + (size_t)tile * a.th * 32 + (size_t)hsel * half * 32 + c;
+        uint32_t x = a.states[(size_t)tile * 64 + lane];
+        if (in_lds) {
+            LdsBytes src;
+            src.init(stage, depth, 64, lane);
+            if (full)
+                linear_tile<MB, true>(src, x, tab, a, half, my_steps, man, xrow, m_ok, k0, acc);
+            else
+                linear_tile<MB, false>(src, x, tab, a, half, my_steps, man, xrow, m_ok, k0, acc);
+        } else {
+            GlobalBytes src;
+            src.init(a.stream + base, depth, 64, lane);
+            linear_tile<MB, false>(src, x, tab, a, half, my_steps, man, xrow, m_ok, k0, acc);
+        }
+    }
+
+    // Sum the kw accumulators of each column tile in k order.  The staging area is free now;
+    // every wave stores its fragment as [v][lane] floats (4 KB per m-block).
+    __syncthreads();
+    float *red = reinterpret_cast<float *>(lds + kSlotTableBytes);
+    const uint32_t frag = 16 * kWave;  // floats per wave per m-block
+#pragma unroll
+    for (int b = 0; b < MB; ++b) {
+        if (b > 0) __syncthreads();
+#pragma unroll
+        for (int v = 0; v < 16; ++v) red[(size_t)wave * frag + v * kWave + lane] = acc[b][v];
+        __syncthreads();
+        if (kidx == 0 && tn < a.tiles_n) {
+            const uint32_t m = m_base + b * 32 + c;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                float s = 0.f;
+                for (uint32_t kk = 0; kk < a.kw; ++kk) s += red[(size_t)(nidx * a.kw + kk) * frag + v * kWave + lane];
+                // MFMA 32x32 result layout: register v of lane l is row (v/4)*8 + (l/32)*4 + v%4
+                // (= column of the tile), column l%32 (= row m of x)
+                const uint32_t n = tn * 32 + (v / 4) * 8 + hsel * 4 + (v % 4);
+                if (m < a.M && n < a.N) {
+                    if (a.P == 1)
+                        a.out[(size_t)m * a.out_stride + n] = finish_bf16(s, a.bias, n);
+                    else
+                        a.partial[((size_t)blockIdx.y * a.M + m) * a.N + n] = s;
+                }
+            }
+        }
+    }
+}
+
+// Any tile width, either tiled layout: one thread per stream, eight rows of x per pass.
+// Partial sums (one per stream, i.e. per (k-tile[, half])) go to the fp32 workspace.
+// grid: (ceil(streams / 256), ceil(M / 8))
+template <bool kDense>
+__global__ __launch_bounds__(256) void fused_linear_generic_kernel(LinearArgs a) {
+    __shared__ uint2 tab[kProbScale];
+    build_slot_table(tab, a.tables, a.slot_map, threadIdx.x, 256);
+    __syncthreads();
+    const uint32_t spt = (kDense ? 1 : 2) * a.tw;
+    const uint64_t sid = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (sid >= (uint64_t)a.tiles_k * a.tiles_n * spt) return;
+    const uint32_t tile = (uint32_t)(sid / spt), q = (uint32_t)(sid % spt);
+    const uint32_t tk = tile / a.tiles_n, tn = tile % a.tiles_n;
+    const uint32_t span = kDense ? a.th : a.th / 2, hsel = kDense ? 0 : q / a.tw, c = q % a.tw;
+    const uint32_t col = tn * a.tw + c, k0 = tk * a.th + hsel * span;
+    if (col >= a.N) return;
+    const uint32_t my_steps = k0 < a.K ? min(span, a.K - k0) : 0;
+    const uint32_t m0 = blockIdx.y * 8;
+    float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    uint32_t x = a.states[sid];
+    const uint8_t *man = a.man_tiled + (size_t)tile * a.th * a.tw + (size_t)hsel * span * a.tw + c;
+
+    auto run = [&](auto &src) {
+        for (uint32_t i = 0; i < my_steps; ++i) {
+            const uint32_t sym = decode_symbol(x, tab) >> 24;
+            src.renorm(x);
+            src.renorm(x);
+            const float w = bf16_to_f32((uint16_t)assemble_bf16(sym, man[(size_t)i * a.tw]));
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                if (m0 + j < a.M) acc[j] += bf16_to_f32(a.x[(size_t)(m0 + j) * a.x_stride + k0 + i]) * w;
+        }
+    };
+    if (kDense) {
+        const uint64_t off = a.stream_offsets[sid];
+        uint32_t size = a.stream_sizes[sid];
+        if (off + size > a.stream_len) size = 0;
+        DenseBytes src;
+        src.init(a.stream + off, size);
+        run(src);
+    } else {
+        uint64_t base = a.tile_offsets[tile];
+        uint32_t depth = a.tile_max_lens[tile];
+        if (base + (uint64_t)depth * spt > a.stream_len) depth = 0;
+        GlobalBytes src;
+        src.init(a.stream + base, depth, spt, q);
+        run(src);
+    }
+    const uint32_t p = kDense ? tk : tk * 2 + hsel;
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+        if (m0 + j < a.M) a.partial[((size_t)p * a.M + m0 + j) * a.N + col] = acc[j];
+}
+
+// Clears the workspace.  A kernel rather than hipMemsetAsync so that the launch sequence can be
+// captured into a HIP graph.
+__global__ __launch_bounds__(256) void zero_f32_kernel(float *p, uint64_t n) {
+    const uint64_t e = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (e < n) p[e] = 0.f;
+}
+
+// out[m][n] = bf16(sum_p partial[p][m][n]) (+ bias), p in index order.
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *partial, uint32_t P, uint32_t M,
+                                                            uint32_t N, const uint16_t *bias, uint16_t *out,
+                                                            uint32_t out_stride) {
+    const uint64_t e = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (e >= (uint64_t)M * N) return;
+    const uint32_t m = (uint32_t)(e / N), n = (uint32_t)(e % N);
+    float s = 0.f;
+    for (uint32_t p = 0; p < P; ++p) s += partial[(size_t)p * M * N + e];
+    out[(size_t)m * out_stride + n] = finish_bf16(s, bias, n);
+}
+
+// Same reduction over a bf16 workspace [P][M][N], the layout the reference's own kernels leave
+// behind (comp_inference/linear_triton.py:257-264, :303-314).
+__global__ __launch_bounds__(256) void splitk_reduce_bf16_kernel(const uint16_t *partial, uint32_t P,
+                                                                 uint32_t M, uint32_t N, const uint16_t *bias,
+                                                                 uint16_t *out, uint32_t out_stride) {
+    const uint64_t e = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (e >= (uint64_t)M * N) return;
+    const uint32_t m = (uint32_t)(e / N), n = (uint32_t)(e % N);
+    float s = 0.f;
+    for (uint32_t p = 0; p < P; ++p) s += bf16_to_f32(partial[(size_t)p * M * N + e]);
+    out[(size_t)m * out_stride + n] = finish_bf16(s, bias, n);
+}
+
+struct LinearPlan {
+    bool fast;
+    uint32_t kw, nw, P;
+};
+
+static LinearPlan plan_linear(uint32_t K, uint32_t th, uint32_t tw, uint32_t tiles_n, bool dense,
+                              bool stream_aligned) {
+    LinearPlan p;
+    const uint32_t tiles_k = ceil_div(K, th);
+    p.fast = !dense && tw == 32 && th % 16 == 0 && stream_aligned;
+    if (p.fast) {
+        p.P = ceil_div(tiles_k, kLinMaxWaves);
+        p.kw = ceil_div(tiles_k, p.P);
+        p.nw = kLinMaxWaves / p.kw;
+        if (p.nw > tiles_n) p.nw = tiles_n;
+        if (p.nw == 0) p.nw = 1;
+    } else {
+        p.kw = p.nw = 1;
+        p.P = dense ? tiles_k : tiles_k * 2;
+    }
+    return p;
+}
+
+}  // namespace ci
+
+using namespace ci;
+
+extern "C" size_t ci_fused_linear_workspace_bytes(uint32_t M, uint32_t K, uint32_t N, uint32_t tile_height,
+                                                  uint32_t tile_width, int dense) {
+    if (tile_height == 0 || tile_width == 0) return 0;
+    // sized for the slower plan so that the answer does not depend on pointer alignment
+    const LinearPlan fast = plan_linear(K, tile_height, tile_width, ceil_div(N, tile_width), dense != 0, true);
+    const LinearPlan slow = plan_linear(K, tile_height, tile_width, ceil_div(N, tile_width), dense != 0, false);
+    const uint32_t P = fast.P > slow.P ? fast.P : slow.P;
+    return P > 1 ? (size_t)P * M * N * sizeof(float) : 0;
+}
+
+static int fused_linear_impl(const uint16_t *d_x, uint32_t M, uint32_t K, uint32_t N, uint32_t x_stride,
+                             const uint8_t *d_stream, uint64_t stream_len, const uint32_t *d_states,
+                             const uint32_t *d_tables, const uint8_t *d_slot_map, const uint32_t *d_meta0,
+                             const uint32_t *d_meta1, const uint8_t *d_man_tiled, uint32_t th, uint32_t tw,
+                             const uint16_t *d_bias, uint16_t *d_out, uint32_t out_stride, void *d_workspace,
+                             size_t workspace_bytes, bool dense, hipStream_t s) {
+    if (M == 0 || N == 0) return CI_OK;
+    if (K == 0) return fail(CI_ERR_ARG, "fused linear: K is 0");
+    if (!d_x || !d_states || !d_tables || !d_slot_map || !d_meta0 || !d_meta1 || !d_man_tiled || !d_out)
+        return fail(CI_ERR_ARG, "fused linear: null pointer");
+    if (stream_len && !d_stream) return fail(CI_ERR_ARG, "fused linear: null stream");
+    if (th == 0 || tw == 0 || (!dense && (th & 1))) return fail(CI_ERR_ARG, "fused linear: bad tile shape");
+    if (x_stride < K || out_stride < N) return fail(CI_ERR_ARG, "fused linear: row stride shorter than the row");
+    if (!aligned(d_slot_map, 4)) return fail(CI_ERR_ARG, "fused linear: slot_map must be 4-byte aligned");
+
+    LinearArgs a;
+    a.x = d_x;
+    a.M = M;
+    a.K = K;
+    a.N = N;
+    a.x_stride = x_stride;
+    a.stream = d_stream;
+    a.stream_len = stream_len;
+    a.states = d_states;
+    a.tables = d_tables;
+    a.slot_map = d_slot_map;
+    a.tile_offsets = dense ? nullptr : d_meta0;
+    a.tile_max_lens = dense ? nullptr : d_meta1;
+    a.stream_offsets = dense ? d_meta0 : nullptr;
+    a.stream_sizes = dense ? d_meta1 : nullptr;
+    a.man_tiled = d_man_tiled;
+    a.bias = d_bias;
+    a.out = d_out;
+    a.out_stride = out_stride;
+    a.th = th;
+    a.tw = tw;
+    a.tiles_n = ceil_div(N, tw);
+    a.tiles_k = ceil_div(K, th);
+    a.stage_bytes = kLinStageBytes;
+    a.x_vec_ok = aligned(d_x, 16) && x_stride % 8 == 0 && th % 16 == 0;
+    const LinearPlan p = plan_linear(K, th, tw, a.tiles_n, dense, aligned(d_stream, 16));
+    a.kw = p.kw;
+    a.nw = p.nw;
+    a.P = p.P;
+    a.partial = static_cast<float *>(d_workspace);
+    if (p.P > 1) {
+        const size_t need = (size_t)p.P * M * N * sizeof(float);
+        if (!d_workspace || workspace_bytes < need)
+            return fail(CI_ERR_CAPACITY, "fused linear: workspace needs %zu bytes, got %zu", need, workspace_bytes);
+        if (!aligned(d_workspace, 4)) return fail(CI_ERR_ARG, "fused linear: workspace must be 4-byte aligned");
+    }
+
+    if (p.fast) {
+        const uint32_t waves = p.kw * p.nw;
+        const uint32_t lds_bytes = kSlotTableBytes + waves * a.stage_bytes;
+        static bool attr_set = false;
+        if (!attr_set) {
+            CI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(fused_linear32_kernel<1>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit));
+            CI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(fused_linear32_kernel<2>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit));
+            attr_set = true;
+        }
+        const dim3 block(waves * kWave);
+        if (M <= 32) {
+            hipLaunchKernelGGL(fused_linear32_kernel<1>, dim3(ceil_div(a.tiles_n, p.nw), p.P, 1), block, lds_bytes,
+                               s, a);
+        } else {
+            hipLaunchKernelGGL(fused_linear32_kernel<2>, dim3(ceil_div(a.tiles_n, p.nw), p.P, ceil_div(M, 64)),
+                               block, lds_bytes, s, a);
+        }
+        CI_LAUNCH_CHECK("fused_linear32_kernel");
+    } else {
+        const uint64_t streams = (uint64_t)a.tiles_k * a.tiles_n * (dense ? 1 : 2) * tw;
+        const dim3 grid((uint32_t)((streams + 255) / 256), ceil_div(M, 8)), block(256);
+        // columns >= N and empty half tiles leave their slots untouched: start from zero
+        const uint64_t nz = (uint64_t)p.P * M * N;
+        hipLaunchKernelGGL(zero_f32_kernel, dim3((uint32_t)((nz + 255) / 256)), dim3(256), 0, s, a.partial, nz);
+        CI_LAUNCH_CHECK("zero_f32_kernel");
+        if (dense)
+            hipLaunchKernelGGL(fused_linear_generic_kernel<true>, grid, block, 0, s, a);
+        else
+            hipLaunchKernelGGL(fused_linear_generic_kernel<false>, grid, block, 0, s, a);
+        CI_LAUNCH_CHECK("fused_linear_generic_kernel");
+    }
+    if (p.P > 1) {
+        const uint64_t n = (uint64_t)M * N;
+        hipLaunchKernelGGL(splitk_reduce_kernel, dim3((uint32_t)((n + 255) / 256)), dim3(256), 0, s, a.partial, p.P,
+                           M, N, d_bias, d_out, out_stride);
+        CI_LAUNCH_CHECK("splitk_reduce_kernel");
+    }
+    return CI_OK;
+}
+
+extern "C" int ci_fused_linear_ilp2(const uint16_t *d_x, uint32_t M, uint32_t K, uint32_t N, uint32_t x_stride,
+                                    const uint8_t *d_stream, uint64_t stream_len, const uint32_t *d_states,
+                                    const uint32_t *d_tables, const uint8_t *d_slot_map,
+                                    const uint32_t *d_tile_offsets, const uint32_t *d_tile_max_lens,
+                                    const uint8_t *d_man_tiled, uint32_t tile_height, uint32_t tile_width,
+                                    const uint16_t *d_bias, uint16_t *d_out, uint32_t out_stride,
+                                    void *d_workspace, size_t workspace_bytes, ci_stream_t stream) {
+    return fused_linear_impl(d_x, M, K, N, x_stride, d_stream, stream_len, d_states, d_tables, d_slot_map,
+                             d_tile_offsets, d_tile_max_lens, d_man_tiled, tile_height, tile_width, d_bias, d_out,
+                             out_stride, d_workspace, workspace_bytes, false, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int ci_fused_linear_dense(const uint16_t *d_x, uint32_t M, uint32_t K, uint32_t N, uint32_t x_stride,
+                                     const uint8_t *d_stream, uint64_t stream_len, const uint32_t *d_states,
+                                     const uint32_t *d_tables, const uint8_t *d_slot_map,
+                                     const uint32_t *d_stream_offsets, const uint32_t *d_stream_sizes,
+                                     const uint8_t *d_man_tiled, uint32_t tile_height, uint32_t tile_width,
+                                     const uint16_t *d_bias, uint16_t *d_out, uint32_t out_stride,
+                                     void *d_workspace, size_t workspace_bytes, ci_stream_t stream) {
+    return fused_linear_impl(d_x, M, K, N, x_stride, d_stream, stream_len, d_states, d_tables, d_slot_map,
+                             d_stream_offsets, d_stream_sizes, d_man_tiled, tile_height, tile_width, d_bias, d_out,
+                             out_stride, d_workspace, workspace_bytes, true, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int ci_splitk_reduce(const void *d_partial, int partial_is_bf16, uint32_t P, uint32_t M, uint32_t N,
+                                const uint16_t *d_bias, uint16_t *d_out, uint32_t out_stride,
+                                ci_stream_t stream) {
+    if (M == 0 || N == 0) return CI_OK;
+    if (!d_partial || !d_out || P == 0) return fail(CI_ERR_ARG, "ci_splitk_reduce: null pointer or P == 0");
+    if (out_stride < N) return fail(CI_ERR_ARG, "ci_splitk_reduce: row stride shorter than the row");
+    const uint64_t n = (uint64_t)M * N;
+    const dim3 grid((uint32_t)((n + 255) / 256)), block(256);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (partial_is_bf16)
+        hipLaunchKernelGGL(splitk_reduce_bf16_kernel, grid, block, 0, s, static_cast<const uint16_t *>(d_partial), P,
+                           M, N, d_bias, d_out, out_stride);
+    else
+        hipLaunchKernelGGL(splitk_reduce_kernel, grid, block, 0, s, static_cast<const float *>(d_partial), P, M, N,
+                           d_bias, d_out, out_stride);
+    CI_LAUNCH_CHECK("splitk_reduce_kernel");
+    return CI_OK;
+}

@@ -1,0 +1,129 @@
+"""Fused decompress + linear on the GPU.
+
+Call signatures follow comp_inference/linear_triton.py:229-246 (`fused_rans_linear_triton`) and
+:1189-1206 (`fused_rans_linear_triton_uncoalesced`).  The kernels are HIP (csrc/linear.hip): the
+weight is decoded tile by tile inside the GEMV/GEMM and never written to memory.
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+import torch
+
+from . import _lib
+from ._lib import check, lib, ptr
+
+
+class _Scratch:
+    """Grow-only fp32 scratch for split-K partials, one per device
+    (the reference keeps a class-level buffer too, comp_inference/pytorch_runtime.py:386-394)."""
+    _buf: dict = {}
+
+    @classmethod
+    def get(cls, nbytes: int, device) -> torch.Tensor | None:
+        if nbytes == 0:
+            return None
+        b = cls._buf.get(device)
+        if b is None or b.numel() < nbytes:
+            b = torch.empty(nbytes, dtype=torch.uint8, device=device)
+            cls._buf[device] = b
+        return b
+
+
+def _prep_x(x: torch.Tensor, K: int):
+    if x.dtype != torch.bfloat16:
+        x = x.to(torch.bfloat16)  # the kernel computes on bf16 (comp_inference/linear_triton.py:431-436)
+    x2 = x.reshape(-1, K)
+    if x2.stride(-1) != 1:
+        x2 = x2.contiguous()
+    return x2
+
+
+def _pick_workspace(workspace, need: int, dev):
+    """A caller-supplied workspace is used when it is large enough for this library's fp32
+    partials; the reference sizes it for its own bf16 partials, which may be smaller."""
+    if need == 0:
+        return None, 0
+    if workspace is not None and workspace.is_cuda and workspace.is_contiguous() \
+            and workspace.numel() * workspace.element_size() >= need:
+        return workspace, workspace.numel() * workspace.element_size()
+    buf = _Scratch.get(need, dev)
+    return buf, buf.numel()
+
+
+def _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, meta0, meta1, tile_k,
+         tile_n, mantissas, bias, out, workspace, dense: bool):
+    K, N = int(weight_shape[0]), int(weight_shape[1])
+    _lib.require_device(x)
+    dev = x.device
+    x2 = _prep_x(x, K)
+    M = x2.shape[0]
+    if out is None:
+        result = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+    else:
+        if out.dtype != torch.bfloat16 or not out.is_cuda:
+            raise RuntimeError("out must be a bfloat16 GPU tensor")
+        result = out.view(M, N) if out.is_contiguous() else out
+        if result.stride(-1) != 1:
+            raise RuntimeError("out must have unit stride in its last dimension")
+    stream_t = _lib.as_u8(compressed_data, dev)
+    man = _lib.as_u8(mantissas, dev).view(-1)
+    need_man = (-(-K // tile_k)) * (-(-N // tile_n)) * tile_k * tile_n
+    if man.numel() < need_man:
+        man = torch.nn.functional.pad(man, (0, need_man - man.numel()))
+    need = lib().ci_fused_linear_workspace_bytes(M, K, N, int(tile_k), int(tile_n), int(dense))
+    ws, ws_bytes = _pick_workspace(workspace, need, dev)
+    b = None
+    if bias is not None:
+        b = bias.to(device=dev, dtype=torch.bfloat16).contiguous()
+    fn = lib().ci_fused_linear_dense if dense else lib().ci_fused_linear_ilp2
+    # device copies must stay referenced until the launch has been enqueued
+    st, tb, sm = _lib.as_u32(initial_states, dev), _lib.as_u32(tables, dev), _lib.as_u8(slot_map, dev)
+    m0, m1 = _lib.as_u32(meta0, dev), _lib.as_u32(meta1, dev)
+    check(fn(ptr(x2), M, K, N, x2.stride(0), ptr(stream_t), C.c_uint64(stream_t.numel()),
+             ptr(st), ptr(tb), ptr(sm), ptr(m0), ptr(m1), ptr(man), int(tile_k), int(tile_n), ptr(b), ptr(result), result.stride(0), ptr(ws),
+             C.c_size_t(ws_bytes), _lib.stream_handle(dev)))
+    if out is not None:
+        return out
+    return result.view(*x.shape[:-1], N)
+
+
+def fused_rans_linear(x, compressed_data, initial_states, tables, slot_map, weight_shape, tile_offsets,
+                      tile_max_lens, tile_k, tile_n, mantissas, accum_block_size=32, bias=None, out=None,
+                      SPLIT_K=8, workspace=None):
+    """x[..., K] @ W[K, N] (+ bias) with W in the tiled two-streams-per-column format
+    (comp_inference/linear_triton.py:229-315).  `accum_block_size` and `SPLIT_K` are accepted for
+    signature compatibility: the kernel always gives every tile its own wavefront and sums the
+    per-tile partials in a fixed order, which is the finest split the format allows."""
+    return _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, tile_offsets,
+                tile_max_lens, tile_k, tile_n, mantissas, bias, out, workspace, dense=False)
+
+
+def fused_rans_linear_uncoalesced(x, compressed_data, initial_states, tables, slot_map, weight_shape,
+                                  stream_offsets, stream_sizes, tile_k, tile_n, mantissas,
+                                  accum_block_size=32, bias=None, out=None, SPLIT_K=8, workspace=None):
+    """Same for the dense one-stream-per-column layout (comp_inference/linear_triton.py:1189-1265)."""
+    return _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, stream_offsets,
+                stream_sizes, tile_k, tile_n, mantissas, bias, out, workspace, dense=True)
+
+
+def splitk_reduce(workspace: torch.Tensor, bias=None, out=None):
+    """out = sum over dim 0 of a [SPLIT_K, M, N] workspace (+ bias), fp32 accumulate, one rounding
+    to bf16: the reduction the reference performs with torch.sum
+    (comp_inference/linear_triton.py:303-314).  Accepts bf16 or fp32 partials."""
+    _lib.require_device(workspace)
+    dev = workspace.device
+    P, M, N = workspace.shape
+    ws = workspace.contiguous()
+    if ws.dtype not in (torch.bfloat16, torch.float32):
+        raise RuntimeError("workspace must be bfloat16 or float32")
+    result = out if out is not None else torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+    b = bias.to(device=dev, dtype=torch.bfloat16).contiguous() if bias is not None else None
+    check(lib().ci_splitk_reduce(ptr(ws), int(ws.dtype == torch.bfloat16), P, M, N, ptr(b), ptr(result),
+                                 result.stride(0), _lib.stream_handle(dev)))
+    return result
+
+
+# Names under which the reference exports these ops (comp_inference/__init__.py:39-42).
+fused_rans_linear_triton = fused_rans_linear
+fused_rans_linear_triton_uncoalesced = fused_rans_linear_uncoalesced

@@ -1,0 +1,109 @@
+/*
+ * comp_inference_hip.h -- C ABI of libcomp_inference_hip.so (MI355X / gfx950).
+ *
+ * This library stands where the reference's pybind11/CUDA extension `comp_inference.ccore`
+ * (src/python_bindings.cpp:59-472) and its Triton kernels stand: rANS coding of the bf16
+ * exponent plane and the fused decode kernels.  Every entry point takes plain pointers and
+ * sizes; "d_" arguments are device pointers, "h_" arguments are host pointers.  Kernels are
+ * enqueued on the given hipStream_t and, unless a function says otherwise, the call does not
+ * wait for them (the reference's ops run on the current torch stream without a sync,
+ * src/cuda/rans_host.cuh:823-834).
+ *
+ * Return value: 0 on success, a CI_ERR_* code otherwise; ci_last_error() then holds a
+ * message (thread local).  The reference reports the same conditions as C++ exceptions that
+ * pybind11 turns into RuntimeError (src/cuda/rans_host.cuh:12-20, :441-445, :462-467).
+ *
+ * Coder parameters are the reference's RansConfig8 (src/cuda/rans_host.cuh:22-24): 8-bit
+ * symbols, 12-bit probabilities, byte I/O, 32-bit state with lower bound 2^16.
+ */
+#ifndef COMP_INFERENCE_HIP_H
+#define COMP_INFERENCE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CI_OK 0
+#define CI_ERR_ARG 1      /* bad shape, size, alignment or null pointer            */
+#define CI_ERR_HIP 2      /* a HIP runtime call or kernel launch failed            */
+#define CI_ERR_CAPACITY 3 /* a buffer handed in by the caller is too small         */
+#define CI_ERR_DEVICE 4   /* current device is not gfx950                          */
+#define CI_ERR_ENCODE 5   /* a stream outgrew the per-stream capacity              */
+
+typedef void *ci_stream_t; /* a hipStream_t; NULL = the null stream */
+
+/* Message of the last failing call on this thread ("" if none). */
+const char *ci_last_error(void);
+
+/* ABI version of this header (bumped when a signature changes). */
+int ci_abi_version(void);
+
+/* CI_OK if the current HIP device is a gfx950; CI_ERR_DEVICE otherwise.  There is no
+ * fallback path: on any other device the library refuses to run. */
+int ci_check_device(void);
+
+/* ---------------------------------------------------------------------------------------
+ * Geometry of a tiled encoding (src/cuda/rans_host.cuh:447-471).  ilp2 != 0: two streams
+ * per column per tile (the default format); ilp2 == 0: one stream per column per tile (the
+ * dense / "uncoalesced" format).  capacity = bytes reserved per stream in the scratch buffer.
+ * ------------------------------------------------------------------------------------- */
+typedef struct ci_tiling {
+    uint32_t K, N, tile_height, tile_width;
+    uint32_t num_tiles_k, num_tiles_n, num_tiles;
+    uint32_t streams_per_tile, num_streams;
+    uint32_t capacity;
+} ci_tiling;
+
+int ci_tiling_init(ci_tiling *t, uint32_t K, uint32_t N, uint32_t tile_height,
+                   uint32_t tile_width, int ilp2);
+
+/* ---------------------------------------------------------------------------------------
+ * Encoder, default format.  Replaces RansManager::compress_tiled_ilp2
+ * (src/cuda/rans_ops.cu:205-410) = kernel rans_compress_kernel_tiled_ilp2
+ * (src/cuda/rans_kernels.cuh:76-188) + the host interleave loop (src/cuda/rans_ops.cu:328-375),
+ * which here runs on the GPU as a second kernel.
+ *
+ * Step 1, ci_encode_tiled_ilp2: encodes d_symbols (u8 [K,N] row major) into d_scratch
+ * (num_streams * capacity bytes), fills d_states / d_sizes (num_streams each) and
+ * d_tile_offsets / d_tile_max_lens (num_tiles each), waits for the stream and returns the
+ * packed length in *h_stream_len.  CI_ERR_ENCODE if any stream outgrew `capacity` (the
+ * reference loses that flag in a by-value kernel argument, src/cuda/rans_kernels.cuh:144-146).
+ * Step 2, ci_pack_tiled_ilp2: writes the packed stream (exactly *h_stream_len bytes) into
+ * d_stream.  Streams of columns >= N get state 2^16 and size 0.
+ * ------------------------------------------------------------------------------------- */
+int ci_encode_tiled_ilp2(const uint8_t *d_symbols, const ci_tiling *t, const uint16_t *h_freqs,
+                         const uint16_t *h_cdf, uint8_t *d_scratch, size_t scratch_bytes,
+                         uint32_t *d_states, uint32_t *d_sizes, uint32_t *d_tile_offsets,
+                         uint32_t *d_tile_max_lens, uint64_t *h_stream_len, ci_stream_t stream);
+
+int ci_pack_tiled_ilp2(const uint8_t *d_scratch, const ci_tiling *t, const uint32_t *d_sizes,
+                       const uint32_t *d_tile_offsets, const uint32_t *d_tile_max_lens,
+                       uint8_t *d_stream, uint64_t stream_len, ci_stream_t stream);
+
+/* Host-side decoder tables (src/cuda/rans_host.cuh:476-488): tables[s] = freq | cdf << 16,
+ * slot_map[cdf[s] + j] = s.  h_tables: 256 entries, h_slot_map: 4096 entries. */
+int ci_build_tables(const uint16_t *h_freqs, const uint16_t *h_cdf, uint32_t *h_tables,
+                    uint8_t *h_slot_map);
+
+/* ---------------------------------------------------------------------------------------
+ * Stand-alone decoder, default format.  Replaces rans_decomp_triton_tiled /
+ * rans_decompress_tiled_kernel_triton_ilp2 (comp_inference/rans_triton.py:34-168).
+ * Output: the exponent plane, u8 [K,N] row major.
+ * d_man_tiled != NULL additionally merges the tile-interleaved sign|mantissa plane
+ * (comp_inference/comp_inference.py:35-64) and writes bf16 bit patterns to d_out_bf16
+ * (the reference does this merge as separate torch ops, comp_inference/comp_inference.py:694-708).
+ * ------------------------------------------------------------------------------------- */
+int ci_decode_tiled_ilp2(const uint8_t *d_stream, uint64_t stream_len, const uint32_t *d_states,
+                         const uint32_t *d_tables, const uint8_t *d_slot_map,
+                         const uint32_t *d_tile_offsets, const uint32_t *d_tile_max_lens,
+                         uint32_t K, uint32_t N, uint32_t tile_height, uint32_t tile_width,
+                         uint8_t *d_out_exp, const uint8_t *d_man_tiled, uint16_t *d_out_bf16,
+                         ci_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* COMP_INFERENCE_HIP_H */

@@ -1,0 +1,143 @@
+"""GPU parity: HIP encoder and decoders against the CPU oracle, bit exact, through the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import bf16_bits, make_weight_kn, zipf_bytes
+
+pytestmark = pytest.mark.gpu
+
+
+def _t32(a):
+    return torch.from_numpy(np.ascontiguousarray(a).view(np.int32))
+
+
+def _np32(t):
+    return t.cpu().view(torch.int32).numpy().view(np.uint32)
+
+
+def _encode_both(oracle, sym, th, tw):
+    from comp_inference_amd import ccore, get_rans_lut
+
+    f, c = oracle.get_lut(sym)
+    ft, ct = get_rans_lut(torch.from_numpy(sym))
+    assert np.array_equal(ft.view(torch.int16).numpy().view(np.uint16), f)
+    assert np.array_equal(ct.view(torch.int16).numpy().view(np.uint16), c)
+    ref = oracle.encode_tiled_ilp2(sym, f, c, th, tw)
+    got = ccore.RansManager(sym.size).compress_tiled(torch.from_numpy(sym), ft, ct, th, tw)
+    return ref, got
+
+
+@pytest.mark.parametrize("K,N,th,tw", [
+    (1024, 64, 1024, 32), (2048, 96, 1024, 32), (1300, 80, 1024, 32), (512, 64, 256, 32),
+    (96, 100, 32, 32), (256, 128, 64, 16), (384, 256, 128, 64), (256, 256, 256, 128),
+])
+def test_encoder_matches_oracle(oracle, K, N, th, tw):
+    sym = zipf_bytes(K * N, 2.0, K + N).reshape(K, N)
+    ref, got = _encode_both(oracle, sym, th, tw)
+    assert got.success and got.num_streams == ref.num_streams
+    assert np.array_equal(_np32(got.states), ref.states)
+    assert np.array_equal(_np32(got.output_sizes), ref.sizes)
+    assert np.array_equal(_np32(got.tile_offsets), ref.tile_offsets)
+    assert np.array_equal(_np32(got.tile_max_lens), ref.tile_max_lens)
+    assert np.array_equal(got.stream.numpy(), ref.stream)
+    assert np.array_equal(_np32(got.tables), ref.tables)
+    assert np.array_equal(got.slot_map.numpy(), ref.slot_map)
+    assert (got.num_tiles_k, got.num_tiles_n) == (ref.num_tiles_k, ref.num_tiles_n)
+
+
+@pytest.mark.parametrize("K,N,th,tw", [
+    (1024, 64, 1024, 32), (4096, 512, 1024, 32), (1300, 80, 1024, 32), (1000, 70, 512, 32),
+    (96, 100, 32, 32), (256, 128, 64, 16), (384, 256, 128, 64), (256, 256, 256, 128),
+])
+def test_tiled_decode_matches_oracle(oracle, K, N, th, tw):
+    from comp_inference_amd import rans_decomp_triton_tiled
+
+    w = make_weight_kn(N, K, seed=K * 7 + N)
+    e, m = oracle.split_bf16(bf16_bits(w))
+    f, c = oracle.get_lut(e)
+    enc = oracle.encode_tiled_ilp2(e, f, c, th, tw)
+    dev = "cuda"
+    args = (torch.from_numpy(enc.stream).to(dev), _t32(enc.states).to(dev), _t32(enc.tables).to(dev),
+            torch.from_numpy(enc.slot_map).to(dev), (K, N), _t32(enc.tile_offsets).to(dev),
+            _t32(enc.tile_max_lens).to(dev))
+    out = rans_decomp_triton_tiled(*args, tile_k=th, tile_n=tw)
+    assert out.dtype == torch.uint8 and tuple(out.shape) == (K, N)
+    assert np.array_equal(out.cpu().numpy(), e)
+    # merged output: bit-exact bf16 weight
+    man = oracle.interleave_plane(m, th, tw)
+    wout = rans_decomp_triton_tiled(*args, tile_k=th, tile_n=tw, mantissas=torch.from_numpy(man).to(dev))
+    assert np.array_equal(bf16_bits(wout), bf16_bits(w))
+
+
+def test_tiled_decode_state_count_mismatch_raises():
+    from comp_inference_amd import rans_decomp_triton_tiled
+
+    z8 = torch.zeros(64, dtype=torch.uint8, device="cuda")
+    z32 = torch.zeros(63, dtype=torch.int32, device="cuda")
+    with pytest.raises(ValueError, match="Initial states size mismatch"):
+        rans_decomp_triton_tiled(z8, z32, z32, z8, (1024, 32), z32, z32)
+
+
+def test_deep_tile_takes_global_path(oracle):
+    """Nearly incompressible symbols: tile bodies too deep for the LDS staging area."""
+    from comp_inference_amd import rans_decomp_triton_tiled
+
+    K, N = 1024, 64
+    sym = np.random.default_rng(5).integers(0, 256, size=(K, N), dtype=np.uint8)
+    f, c = oracle.get_lut(sym)
+    enc = oracle.encode_tiled_ilp2(sym, f, c, 1024, 32)
+    assert enc.tile_max_lens.max() * 64 > 14336
+    dev = "cuda"
+    out = rans_decomp_triton_tiled(torch.from_numpy(enc.stream).to(dev), _t32(enc.states).to(dev),
+                                   _t32(enc.tables).to(dev), torch.from_numpy(enc.slot_map).to(dev), (K, N),
+                                   _t32(enc.tile_offsets).to(dev), _t32(enc.tile_max_lens).to(dev))
+    assert np.array_equal(out.cpu().numpy(), sym)
+
+
+@pytest.mark.parametrize("K,N,th,tw", [(1024, 64, 1024, 32), (700, 50, 256, 32), (256, 128, 64, 16)])
+def test_dense_encode_decode(oracle, K, N, th, tw):
+    from comp_inference_amd import ccore, rans_decomp_tiled_uncoalesced
+
+    sym = zipf_bytes(K * N, 1.5, 3).reshape(K, N)
+    f, c = oracle.get_lut(sym)
+    ref = oracle.encode_tiled_dense(sym, f, c, th, tw)
+    got = ccore.RansManager().compress_tiled_uncoalesced(torch.from_numpy(sym), torch.from_numpy(f.view(np.int16)).view(torch.uint16),
+                                                         torch.from_numpy(c.view(np.int16)).view(torch.uint16), th, tw)
+    assert np.array_equal(got.stream.numpy(), ref.stream)
+    assert np.array_equal(_np32(got.states), ref.states)
+    assert np.array_equal(_np32(got.stream_offsets), ref.stream_offsets)
+    assert np.array_equal(_np32(got.output_sizes), ref.sizes)
+    dev = "cuda"
+    out = rans_decomp_tiled_uncoalesced(got.stream.to(dev), got.states, got.tables, got.slot_map, (K, N),
+                                        got.stream_offsets, got.output_sizes, tile_k=th, tile_n=tw)
+    assert np.array_equal(out.cpu().numpy(), sym)
+
+
+@pytest.mark.parametrize("K,N", [(300, 8), (512, 33), (1500, 16), (70000, 1)])
+def test_flat_encode_decode(oracle, K, N):
+    from comp_inference_amd import ccore, rans_decomp_triton
+
+    sym = zipf_bytes(K * N, 4.0, 11).reshape(K, N)
+    f, c = oracle.get_lut(sym)
+    ref = oracle.encode_flat(sym, f, c, 512)
+    got = ccore.RansManager().compress(torch.from_numpy(sym), torch.from_numpy(f.view(np.int16)).view(torch.uint16),
+                                       torch.from_numpy(c.view(np.int16)).view(torch.uint16), 512)
+    assert got.num_streams == ref.num_streams
+    assert got.states.dtype == torch.int32
+    assert np.array_equal(got.states.numpy().view(np.uint32), ref.states)
+    assert np.array_equal(got.output_sizes.numpy().view(np.uint32), ref.sizes)
+    assert np.array_equal(got.stream.numpy(), ref.stream)
+    assert np.array_equal(got.checkpoints.view(torch.int64).numpy().view(np.uint64), ref.checkpoints)
+    dev = "cuda"
+    out = rans_decomp_triton(got.stream.to(dev), got.states.to(dev), got.tables.to(dev), got.slot_map.to(dev),
+                             got.output_sizes.to(dev), (K, N))
+    assert np.array_equal(out.cpu().numpy(), sym)
+    # the extension's own flat decoder writes symbol i of stream g at g + i * streams
+    flat = torch.empty(K * N, dtype=torch.uint8, device=dev)
+    ccore.decompress(got.stream.to(dev), got.states.to(dev), got.output_sizes.to(dev), got.num_streams,
+                     got.tables.to(dev), got.slot_map.to(dev), flat)
+    want = oracle.decode_flat_strided(ref.stream, ref.states, ref.sizes, ref.tables, ref.slot_map, K * N)
+    assert np.array_equal(flat.cpu().numpy(), want)
+    if K <= 512:
+        assert np.array_equal(want.reshape(K, N), sym)

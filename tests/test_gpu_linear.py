@@ -1,0 +1,120 @@
+"""GPU parity of the fused decompress-linear: against torch.matmul on the oracle-decoded weight,
+with the tolerance the reference's own test uses (tests/test_mat_mul.py:220: atol=rtol=1e-2)."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import bf16_bits, bits_to_bf16, make_weight_kn, make_x
+
+pytestmark = pytest.mark.gpu
+ATOL = RTOL = 1e-2
+
+
+def _t32(a):
+    return torch.from_numpy(np.ascontiguousarray(a).view(np.int32))
+
+
+def _compress(oracle, w, th, tw):
+    enc, man = oracle.compress_bf16(bf16_bits(w), th, tw)
+    K, N = w.shape
+    wdec = bits_to_bf16(oracle.decompress_bf16(enc, man, K, N))
+    assert torch.equal(wdec.view(torch.int16), w.view(torch.int16))
+    return enc, man, wdec
+
+
+def _call(enc, man, x, K, N, th, tw, **kw):
+    from comp_inference_amd import fused_rans_linear_triton
+
+    dev = "cuda"
+    return fused_rans_linear_triton(
+        x.to(dev), torch.from_numpy(enc.stream).to(dev), _t32(enc.states).to(dev), _t32(enc.tables).to(dev),
+        torch.from_numpy(enc.slot_map).to(dev), (K, N), _t32(enc.tile_offsets).to(dev),
+        _t32(enc.tile_max_lens).to(dev), th, tw, torch.from_numpy(man).to(dev), **kw)
+
+
+@pytest.mark.parametrize("M", [1, 4, 16, 33, 64, 100])
+@pytest.mark.parametrize("K,N,th,tw", [(4096, 256, 1024, 32), (3072, 128, 512, 32)])
+def test_fused_linear_fast_path(oracle, M, K, N, th, tw):
+    w = make_weight_kn(N, K, seed=1)
+    enc, man, wdec = _compress(oracle, w, th, tw)
+    x = make_x(M, K, seed=2)
+    got = _call(enc, man, x, K, N, th, tw).float().cpu()
+    want = torch.matmul(x.float(), wdec.float())
+    assert got.shape == (M, N)
+    assert torch.allclose(got, want, atol=ATOL, rtol=RTOL), (got - want).abs().max()
+
+
+@pytest.mark.parametrize("K,N,th,tw,M", [
+    (14336, 64, 1024, 32, 1),    # 14 k-tiles: two partial sums + reduction kernel
+    (14336, 64, 1024, 32, 5),
+    (1300, 80, 1024, 32, 3),     # ragged K and N
+    (1000, 70, 512, 32, 2),
+    (9000, 32, 1024, 32, 1),
+    (256, 128, 64, 16, 4),       # other tile widths: generic kernel
+    (384, 256, 128, 64, 9),
+    (256, 256, 256, 128, 1),
+])
+def test_fused_linear_shapes(oracle, K, N, th, tw, M):
+    w = make_weight_kn(N, K, seed=K + N)
+    enc, man, wdec = _compress(oracle, w, th, tw)
+    x = make_x(M, K, seed=M)
+    got = _call(enc, man, x, K, N, th, tw).float().cpu()
+    want = torch.matmul(x.float(), wdec.float())
+    assert torch.allclose(got, want, atol=ATOL, rtol=RTOL), (got - want).abs().max()
+
+
+def test_fused_linear_bias_out_and_batch_shape(oracle):
+    K, N, th, tw = 2048, 96, 1024, 32
+    w = make_weight_kn(N, K, seed=9)
+    enc, man, wdec = _compress(oracle, w, th, tw)
+    x = make_x(6, K, seed=3).view(2, 3, K)
+    bias = make_x(1, N, seed=4).view(N)
+    got = _call(enc, man, x, K, N, th, tw, bias=bias.cuda())
+    assert got.shape == (2, 3, N) and got.dtype == torch.bfloat16
+    want = (torch.matmul(x.float(), wdec.float()).to(torch.bfloat16) + bias).float()
+    assert torch.allclose(got.float().cpu(), want, atol=ATOL, rtol=RTOL)
+    out = torch.zeros(6, N, dtype=torch.bfloat16, device="cuda")
+    ret = _call(enc, man, x, K, N, th, tw, bias=bias.cuda(), out=out)
+    assert ret is out
+    assert torch.equal(out.view(2, 3, N), got)
+
+
+def test_fused_linear_is_deterministic(oracle):
+    K, N, th, tw = 14336, 64, 1024, 32
+    w = make_weight_kn(N, K, seed=21)
+    enc, man, _ = _compress(oracle, w, th, tw)
+    x = make_x(1, K, seed=22)
+    a = _call(enc, man, x, K, N, th, tw)
+    b = _call(enc, man, x, K, N, th, tw)
+    assert torch.equal(a, b)
+
+
+def test_fused_linear_dense_layout(oracle):
+    from comp_inference_amd import fused_rans_linear_triton_uncoalesced
+
+    K, N, th, tw, M = 1024, 64, 512, 32, 3
+    w = make_weight_kn(N, K, seed=31)
+    e, m = oracle.split_bf16(bf16_bits(w))
+    f, c = oracle.get_lut(e)
+    enc = oracle.encode_tiled_dense(e, f, c, th, tw)
+    man = oracle.interleave_plane(m, th, tw)
+    x = make_x(M, K, seed=32)
+    dev = "cuda"
+    got = fused_rans_linear_triton_uncoalesced(
+        x.to(dev), torch.from_numpy(enc.stream).to(dev), _t32(enc.states).to(dev), _t32(enc.tables).to(dev),
+        torch.from_numpy(enc.slot_map).to(dev), (K, N), _t32(enc.stream_offsets).to(dev), _t32(enc.sizes).to(dev),
+        th, tw, torch.from_numpy(man).to(dev))
+    want = torch.matmul(x.float(), w.float())
+    assert torch.allclose(got.float().cpu(), want, atol=ATOL, rtol=RTOL)
+
+
+def test_splitk_reduce_matches_torch_sum():
+    from comp_inference_amd import splitk_reduce
+
+    g = torch.Generator("cpu").manual_seed(0)
+    ws = torch.randn(8, 5, 96, generator=g).to(torch.bfloat16).cuda()
+    bias = torch.randn(96, generator=g).to(torch.bfloat16).cuda()
+    want = torch.sum(ws, dim=0)
+    want += bias
+    got = splitk_reduce(ws, bias=bias)
+    assert torch.equal(got, want)
