@@ -1,0 +1,252 @@
+#!/usr/bin/env python3
+"""Benchmark of the compressed-weight hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Workload (one "step"): stand-alone rANS decode of the seven weight tensors of one
+Llama-3-8B-shaped decoder layer (q, k, v, o, gate, up, down), bf16 N(0, 0.02) from seed 1,
+default format (1024x32 tiles, two streams per column, 12-bit per-tensor table).  All inputs are
+resident in HBM before the timed region.  `value` = exponent-plane bytes decoded per second.
+
+The JSON line also carries
+  roofline      decode kernel, algorithmic bytes per launch / measured launch time vs 8 TB/s HBM
+  cpu_baseline  the CPU oracle decoding the same streams on the host cores (bounded sample)
+  fused_gemv    fused decompress-GEMV/GEMM on the gate projection for M = 1, 4, 16, 64:
+                time, share of the HBM roofline on compressed bytes, and torch.matmul (hipBLASLt)
+                on the uncompressed bf16 weight for comparison
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+LAYER = [("q", 4096, 4096), ("k", 1024, 4096), ("v", 1024, 4096), ("o", 4096, 4096),
+         ("gate", 14336, 4096), ("up", 14336, 4096), ("down", 4096, 14336)]  # (name, out, in)
+
+
+def log(msg: str) -> None:
+    print(msg, file=sys.stderr, flush=True)
+
+
+def make_layer(seed: int):
+    """Weights drawn in the listed order from one generator, nn.Linear orientation [out, in]."""
+    g = torch.Generator("cpu").manual_seed(seed)
+    return [(name, (torch.randn(o, i, generator=g, dtype=torch.float32) * 0.02).to(torch.bfloat16))
+            for name, o, i in LAYER]
+
+
+class Compressed:
+    """One weight in the default format, resident on the GPU."""
+
+    def __init__(self, name: str, w_out_in: torch.Tensor, dev, th: int = 1024, tw: int = 32):
+        import comp_inference_amd as ci
+
+        w = w_out_in.t().contiguous()  # [K, N] as the reference encodes it
+        self.name, self.K, self.N, self.th, self.tw = name, w.shape[0], w.shape[1], th, tw
+        exp, man = ci.extract_exp_and_mantissa(w)
+        f, c = ci.get_rans_lut(exp)
+        r = ci.ccore.RansManager(exp.numel()).compress_tiled(exp, f, c, th, tw)
+        self.host = r
+        self.exp_host = exp.numpy()
+        self.stream = r.stream.to(dev)
+        self.states = r.states.to(dev)
+        self.tables = r.tables.to(dev)
+        self.slot_map = r.slot_map.to(dev)
+        self.tile_offsets = r.tile_offsets.to(dev)
+        self.tile_max_lens = r.tile_max_lens.to(dev)
+        self.man = ci.interleave_mantissas(man, th, tw).to(dev)
+        self.n_streams = r.num_streams
+        self.n_tiles = r.num_tiles_k * r.num_tiles_n
+
+    # algorithmic bytes of one stand-alone decode: stream + states + per-tile metadata + tables in,
+    # exponent plane out
+    def decode_bytes(self) -> int:
+        return self.stream.numel() + 4 * self.n_streams + 8 * self.n_tiles + 1024 + 4096 + self.K * self.N
+
+    # algorithmic bytes of one fused linear at M rows
+    def linear_bytes(self, M: int) -> int:
+        return (self.stream.numel() + self.man.numel() + 4 * self.n_streams + 8 * self.n_tiles + 5120
+                + 2 * M * self.K + 2 * M * self.N)
+
+    def decode(self):
+        import comp_inference_amd as ci
+
+        return ci.rans_decomp_tiled(self.stream, self.states, self.tables, self.slot_map, (self.K, self.N),
+                                    self.tile_offsets, self.tile_max_lens, tile_k=self.th, tile_n=self.tw)
+
+    def linear(self, x):
+        import comp_inference_amd as ci
+
+        return ci.fused_rans_linear(x, self.stream, self.states, self.tables, self.slot_map, (self.K, self.N),
+                                    self.tile_offsets, self.tile_max_lens, self.th, self.tw, self.man)
+
+
+def event_times_us(fn, warmup: int, iters: int):
+    """Per-call GPU time with events on the stream the kernels are launched on."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    out = []
+    for _ in range(iters):
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        fn()
+        e.record()
+        e.synchronize()
+        out.append(s.elapsed_time(e) * 1e3)
+    return out
+
+
+def batched_time_us(fn, warmup: int, iters: int) -> float:
+    """Average GPU time per call with `iters` calls enqueued back to back between two events, so
+    that host launch latency is not part of the figure."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    s.record()
+    for _ in range(iters):
+        fn()
+    e.record()
+    e.synchronize()
+    return s.elapsed_time(e) * 1e3 / iters
+
+
+def cpu_baseline(layer: list[Compressed], budget_s: float = 15.0):
+    """CPU oracle decoding the same streams, all host cores (OpenMP), median of repeated passes
+    over the whole layer within a time budget."""
+    from oracle import rans_oracle as ro
+
+    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else os.cpu_count()
+    cores = min(cores or 1, int(os.environ.get("OMP_NUM_THREADS", cores or 1)))
+    args = [(c.host.stream.numpy(), c.host.states.view(torch.int32).numpy().view(np.uint32),
+             c.host.tables.view(torch.int32).numpy().view(np.uint32), c.host.slot_map.numpy(),
+             c.host.tile_offsets.view(torch.int32).numpy().view(np.uint32),
+             c.host.tile_max_lens.view(torch.int32).numpy().view(np.uint32), c.K, c.N, c.th, c.tw) for c in layer]
+    total = sum(c.K * c.N for c in layer)
+    times = []
+    t_start = time.time()
+    checked = False
+    while len(times) < 13 and (time.time() - t_start < budget_s or len(times) < 3):
+        t0 = time.time()
+        outs = [ro.decode_tiled_ilp2(*a) for a in args]
+        times.append(time.time() - t0)
+        if not checked:  # the baseline must be decoding the right thing
+            assert all(np.array_equal(o, c.exp_host) for o, c in zip(outs, layer))
+            checked = True
+    med = float(np.median(times[1:])) if len(times) > 1 else times[0]
+    return {"value": round(total / med / 1e9, 3), "unit": "GB/s", "cores": int(cores), "kind": "port",
+            "sample": f"whole layer ({total / 1e6:.0f} M symbols), {len(times)} passes, median, OpenMP over tiles"}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-gemv", action="store_true")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print("bench.py measures one GPU: this path has no multi-GPU part (run with --gpus 1)", file=sys.stderr)
+        return 2
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (gfx950)", file=sys.stderr)
+        return 2
+
+    import comp_inference_amd as ci  # noqa: F401  (fails loudly if the HIP library is missing)
+
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    log("generating and compressing one layer (seed 1) ...")
+    layer = [Compressed(n, w, dev) for n, w in make_layer(1)]
+    total_syms = sum(c.K * c.N for c in layer)
+    total_stream = sum(c.stream.numel() for c in layer)
+
+    # bit-exact check of what is about to be timed
+    for c in layer:
+        assert np.array_equal(c.decode().cpu().numpy(), c.exp_host), f"decode mismatch on {c.name}"
+
+    def step():
+        for c in layer:
+            c.decode()
+
+    # --- timed region: W warm-up steps, then exactly K steps between two synchronisations
+    for _ in range(a.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / a.steps
+    value = total_syms / (ms_per_step * 1e-3) / 1e9
+
+    # --- decode kernel roofline: per-launch durations by events on the launch stream
+    per_kernel = {}
+    kern_us_total = 0.0
+    for c in layer:
+        us = float(np.median(event_times_us(c.decode, 5, 30)))
+        per_kernel[c.name] = round(us, 2)
+        kern_us_total += us
+    algo_bytes = sum(c.decode_bytes() for c in layer)
+    achieved = algo_bytes / (kern_us_total * 1e-6) / 1e9
+    roofline = {"bound": "hbm", "kernel": "decode_tiled32_kernel", "achieved": round(achieved, 1),
+                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "bytes_per_launch_avg": int(algo_bytes / len(layer)),
+                "launch_us_avg": round(kern_us_total / len(layer), 2), "launch_us": per_kernel,
+                "compressed_read_GBs": round(total_stream / (kern_us_total * 1e-6) / 1e9, 1)}
+
+    out = {"metric": "decoded GB/s", "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": a.steps,
+           "warmup": a.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+           "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+           "config": {"workload": "standalone rANS decode of one Llama-3-8B-shaped layer (q,k,v,o,gate,up,down), "
+                                  "bf16 N(0,0.02) seed 1, tile 1024x32, two streams per column, 12-bit tables",
+                      "symbols_per_step": total_syms, "compressed_stream_bytes": total_stream,
+                      "exponent_plane_ratio": round(total_syms / total_stream, 3)},
+           "roofline": roofline}
+
+    # --- fused decompress-GEMV/GEMM on the gate projection
+    if not a.no_gemv:
+        gate = next(c for c in layer if c.name == "gate")
+        g = torch.Generator("cpu").manual_seed(2)
+        x_all = torch.randn(64, gate.K, generator=g, dtype=torch.float32).to(torch.bfloat16).to(dev)
+        w_dense = ci.rans_decomp_tiled(gate.stream, gate.states, gate.tables, gate.slot_map, (gate.K, gate.N),
+                                       gate.tile_offsets, gate.tile_max_lens, mantissas=gate.man)
+        rows = []
+        for M in (1, 4, 16, 64):
+            x = x_all[:M].contiguous()
+            got = gate.linear(x).float()
+            want = torch.matmul(x, w_dense).float()
+            ok = bool(torch.allclose(got, want, atol=1e-2, rtol=1e-2))
+            us = batched_time_us(lambda: gate.linear(x), 25, 100)
+            us_ref = batched_time_us(lambda: torch.matmul(x, w_dense), 25, 100)
+            nbytes = gate.linear_bytes(M)
+            rows.append({"M": M, "us": round(us, 2), "allclose_1e-2": ok,
+                         "hbm_frac_compressed_bytes": round(nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+                         "effective_weight_GBs": round(2 * gate.K * gate.N / (us * 1e-6) / 1e9, 1),
+                         "mfma_TFLOPs": round(2 * M * gate.K * gate.N / (us * 1e-6) / 1e12, 2),
+                         "torch_matmul_bf16_us": round(us_ref, 2),
+                         "torch_matmul_weight_GBs": round(2 * gate.K * gate.N / (us_ref * 1e-6) / 1e9, 1)})
+        out["fused_gemv"] = {"layer": "gate K=4096 N=14336", "bytes_M1": gate.linear_bytes(1), "rows": rows}
+
+    if not a.no_cpu_baseline:
+        log("timing the CPU oracle ...")
+        out["cpu_baseline"] = cpu_baseline(layer)
+
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

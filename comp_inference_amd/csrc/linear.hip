@@ -67,50 +67,99 @@ __device__ __forceinline__ uint16_t finish_bf16(float acc, const uint16_t *bias,
 }
 
 // Two decoded symbols (top bytes of w0, w1) + two sign|mantissa bytes -> two bf16 in one dword
-// (row of w0 in the low half).
-__device__ __forceinline__ uint32_t pack_bf16_pair(uint32_t w0, uint32_t w1, uint32_t m0, uint32_t m1) {
+// (row of w0 in the low half).  The sign|mantissa bytes are byte `b` of m0 / m1, chosen by
+// man_sel = 0x04040000 + b * 0x01010101.
+__device__ __forceinline__ uint32_t pack_bf16_pair(uint32_t w0, uint32_t w1, uint32_t m0, uint32_t m1,
+                                                   uint32_t man_sel = 0x04040000u) {
     const uint32_t e = __builtin_amdgcn_perm(w1, w0, 0x070C030Cu) >> 1;  // s1 << 23 | s0 << 7
-    const uint32_t mm = __builtin_amdgcn_perm(m1, m0, 0x04040000u);       // [m1 m1 m0 m0]
+    const uint32_t mm = __builtin_amdgcn_perm(m1, m0, man_sel);           // [m1 m1 m0 m0]
     return (e & 0x7F807F80u) | (mm & 0x807F807Fu);
 }
 
-// Eight decode steps + operand assembly + MFMA for one block of 8 rows per half tile.
-// kFull: the whole tile lies inside [K,N] and the lane takes every step.
-template <int MB, bool kFull, typename Bytes>
-__device__ __forceinline__ void linear_tile(Bytes &src, uint32_t x, const uint2 *tab, const LinearArgs &a,
-                                            uint32_t half, uint32_t my_steps, const uint8_t *man,
-                                            const uint16_t *xrow[MB], bool m_ok[MB], uint32_t k0,
-                                            f32x16 acc[MB]) {
+// Fast path: the whole tile lies inside [K,N], its body is staged in LDS and x rows can be read
+// with 16-byte loads.  The sign|mantissa bytes and the x fragment of the next block of 8 rows are
+// requested before the current block is decoded, so their latency hides behind the decode chain.
+template <int MB>
+__device__ __forceinline__ void linear_tile_fast(LdsBytes &src, uint32_t x, const uint2 *tab, uint32_t half,
+                                                 const uint8_t *man, uint32_t lane_col, const uint16_t *xrow[MB],
+                                                 const bool m_ok[MB], f32x16 acc[MB]) {
+    // The sign|mantissa byte of this lane's column is fetched as the aligned dword that holds it
+    // (four neighbouring lanes share the dword) and picked out by the byte permute that packs it.
+    const uint32_t *man4 = reinterpret_cast<const uint32_t *>(man - (lane_col & 3));
+    const uint32_t man_sel = 0x04040000u + (lane_col & 3) * 0x01010101u;
+    // two operand buffers used alternately, so the prefetched values are consumed in place
+    uint32_t mb[2][8];
+    u32x4 xv[2][MB];
+    auto request = [&](uint32_t i, int buf) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) mb[buf][j] = man4[(size_t)(i + j) * 8];
+#pragma unroll
+        for (int b = 0; b < MB; ++b) {
+            xv[buf][b] = (u32x4){0, 0, 0, 0};
+            if (m_ok[b]) xv[buf][b] = *reinterpret_cast<const u32x4 *>(xrow[b] + i);
+        }
+    };
+    auto block = [&](int buf) {
+        uint32_t w[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            w[j] = decode_symbol(x, tab);
+            src.renorm(x);
+            src.renorm(x);
+        }
+        u32x4 wv;
+#pragma unroll
+        for (int p = 0; p < 4; ++p)
+            wv[p] = pack_bf16_pair(w[2 * p], w[2 * p + 1], mb[buf][2 * p], mb[buf][2 * p + 1], man_sel);
+#pragma unroll
+        for (int b = 0; b < MB; ++b)
+            acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, wv),
+                                                             __builtin_bit_cast(bf16x8, xv[buf][b]), acc[b], 0, 0, 0);
+    };
+    // A request past the end of the half tile re-reads block 0 instead of branching (in range,
+    // result unused).
+    request(0, 0);
+    uint32_t i = 0;
+    for (; i + 16 <= half; i += 16) {
+        request(i + 8, 1);
+        block(0);
+        request(i + 16 < half ? i + 16 : 0, 0);
+        block(1);
+    }
+    if (i < half) block(0);
+}
+
+// General path: ragged tiles (rows >= K, columns >= N), unaligned x, or a tile body read from
+// global memory.  Same arithmetic, every access guarded.
+template <int MB, typename Bytes>
+__device__ __forceinline__ void linear_tile_guarded(Bytes &src, uint32_t x, const uint2 *tab, uint32_t K,
+                                                    uint32_t half, uint32_t my_steps, const uint8_t *man,
+                                                    const uint16_t *xrow[MB], const bool m_ok[MB], uint32_t k0,
+                                                    f32x16 acc[MB]) {
     for (uint32_t i = 0; i < half; i += 8) {
-        // x fragment: 8 consecutive k of row m for this lane's half tile
         u32x4 xv[MB];
 #pragma unroll
         for (int b = 0; b < MB; ++b) {
             xv[b] = (u32x4){0, 0, 0, 0};
             if (m_ok[b]) {
-                if (kFull && a.x_vec_ok) {
-                    xv[b] = *reinterpret_cast<const u32x4 *>(xrow[b] + k0 + i);
-                } else {
 #pragma unroll
-                    for (int j = 0; j < 8; ++j) {
-                        const uint32_t k = k0 + i + j;
-                        const uint32_t v = k < a.K ? xrow[b][k] : 0u;
-                        xv[b][j / 2] |= v << (16 * (j & 1));
-                    }
+                for (int j = 0; j < 8; ++j) {
+                    const uint32_t k = k0 + i + j;
+                    const uint32_t v = k < K ? xrow[b][i + j] : 0u;
+                    xv[b][j / 2] |= v << (16 * (j & 1));
                 }
             }
         }
         uint32_t mb[8], w[8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) mb[j] = (kFull || i + j < my_steps) ? man[(size_t)(i + j) * 32] : 0u;
-#pragma unroll
         for (int j = 0; j < 8; ++j) {
-            if (kFull || i + j < my_steps) {
+            mb[j] = 0;
+            w[j] = 0;
+            if (i + j < my_steps) {
+                mb[j] = man[(size_t)(i + j) * 32];
                 w[j] = decode_symbol(x, tab);
                 src.renorm(x);
                 src.renorm(x);
-            } else {
-                w[j] = 0;
             }
         }
         u32x4 wv;
@@ -163,27 +212,28 @@ __global__ __launch_bounds__(kLinMaxWaves *kWave) void fused_linear32_kernel(Lin
         uint32_t my_steps = 0;
         if (col0 + c < a.N && k0 < a.K) my_steps = min(half, a.K - k0);
         const bool full = __builtin_amdgcn_ballot_w64(my_steps != half) == 0;
-        const uint16_t *xrow[MB];
+        const uint16_t *xrow[MB];  // row m of x, already advanced to this lane's first k
         bool m_ok[MB];
 #pragma unroll
         for (int b = 0; b < MB; ++b) {
             const uint32_t m = m_base + b * 32 + c;
             m_ok[b] = m < a.M;
-            xrow[b] = a.x + (size_t)(m_ok[b] ? m : 0) * a.x_stride;
+            xrow[b] = a.x + (size_t)(m_ok[b] ? m : 0) * a.x_stride + k0;
         }
         const uint8_t *man = a.man_tiled + (size_t)tile * a.th * 32 + (size_t)hsel * half * 32 + c;
         uint32_t x = a.states[(size_t)tile * 64 + lane];
+        const bool aligned_man = (reinterpret_cast<uintptr_t>(a.man_tiled) & 3) == 0;
         if (in_lds) {
             LdsBytes src;
             src.init(stage, depth, 64, lane);
-            if (full)
-                linear_tile<MB, true>(src, x, tab, a, half, my_steps, man, xrow, m_ok, k0, acc);
+            if (full && a.x_vec_ok && aligned_man)
+                linear_tile_fast<MB>(src, x, tab, half, man, c, xrow, m_ok, acc);
             else
-                linear_tile<MB, false>(src, x, tab, a, half, my_steps, man, xrow, m_ok, k0, acc);
+                linear_tile_guarded<MB>(src, x, tab, a.K, half, my_steps, man, xrow, m_ok, k0, acc);
         } else {
             GlobalBytes src;
             src.init(a.stream + base, depth, 64, lane);
-            linear_tile<MB, false>(src, x, tab, a, half, my_steps, man, xrow, m_ok, k0, acc);
+            linear_tile_guarded<MB>(src, x, tab, a.K, half, my_steps, man, xrow, m_ok, k0, acc);
         }
     }
 

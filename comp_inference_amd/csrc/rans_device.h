@@ -56,21 +56,19 @@ __device__ __forceinline__ uint32_t decode_symbol(uint32_t &x, const uint2 *tab)
 // dependency chain).  An exhausted stream walks to negative offsets; LDS reads outside the
 // allocation return zero, and a well-formed stream never asks for those bytes.
 struct LdsBytes {
-    const uint8_t *base;
-    uint32_t pos;
-    uint32_t nxt;
+    const uint8_t *cur;  // LDS address of the next byte of this lane's stream
+    uint32_t nxt;        // that byte, already read
     uint32_t row_bytes;
     __device__ __forceinline__ void init(const uint8_t *b, uint32_t depth, uint32_t rb, uint32_t q) {
-        base = b;
         row_bytes = rb;
-        pos = (depth - 1) * rb + q;
-        nxt = depth ? base[pos] : 0;
+        cur = b + (depth - 1) * rb + q;
+        nxt = depth ? *cur : 0;
     }
     __device__ __forceinline__ void renorm(uint32_t &x) {
         if (x < kRansL) {
             x = (x << 8) | nxt;
-            pos -= row_bytes;
-            nxt = base[pos];
+            cur -= row_bytes;
+            nxt = *cur;
         }
     }
 };

@@ -103,6 +103,116 @@ int ci_decode_tiled_ilp2(const uint8_t *d_stream, uint64_t stream_len, const uin
                          uint8_t *d_out_exp, const uint8_t *d_man_tiled, uint16_t *d_out_bf16,
                          ci_stream_t stream);
 
+/* Bytes of scratch the encoders need for `num_streams` streams of `capacity` bytes (a small
+ * header for flags and totals precedes the per-stream slices). */
+size_t ci_encode_scratch_bytes(uint32_t num_streams, uint32_t capacity);
+
+/* ---------------------------------------------------------------------------------------
+ * Encoder, dense ("uncoalesced") format: one stream per (tile, column) over the full tile
+ * height, streams concatenated byte-exact.  Replaces RansManager::compress_tiled_uncoalesced
+ * (src/cuda/rans_ops.cu:74-203) = kernel rans_compress_kernel_tiled_uncoalesced
+ * (src/cuda/rans_kernels.cuh:7-74) + the host packing loop (src/cuda/rans_ops.cu:165-176).
+ * Same two-step protocol as the default format; d_stream_offsets has num_streams entries.
+ * The tiling must come from ci_tiling_init(..., ilp2 = 0).
+ * ------------------------------------------------------------------------------------- */
+int ci_encode_tiled_dense(const uint8_t *d_symbols, const ci_tiling *t, const uint16_t *h_freqs,
+                          const uint16_t *h_cdf, uint8_t *d_scratch, size_t scratch_bytes,
+                          uint32_t *d_states, uint32_t *d_sizes, uint32_t *d_stream_offsets,
+                          uint64_t *h_stream_len, ci_stream_t stream);
+
+int ci_pack_tiled_dense(const uint8_t *d_scratch, const ci_tiling *t, const uint32_t *d_sizes,
+                        const uint32_t *d_stream_offsets, uint8_t *d_stream, uint64_t stream_len,
+                        ci_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Encoder, flat (legacy) format.  Replaces RansManager::compress (src/cuda/rans_ops.cu:16-72)
+ * = StreamConfigurator::suggest (src/cuda/rans_host.cuh:161-183) + kernel rans_compress_kernel
+ * (src/cuda/rans_kernels.cuh:393-509).  num_streams = ceil(K / min_block_size) * N; stream g
+ * covers the 512-row segment g / N of column g % N (the kernel's segment length is fixed at
+ * 512 whatever min_block_size says, src/cuda/rans_kernels.cuh:421).  d_checkpoints receives
+ * num_streams * 128 u64 entries: {state, bytes written} before symbols 0, 128, 256, 384 of each
+ * segment at [(i / 128) * num_streams + g], zero elsewhere.  ci_pack_flat writes byte j of
+ * stream g at [j * num_streams + g], max_len rows (src/cuda/rans_ops.cu:51-65).
+ * ------------------------------------------------------------------------------------- */
+int ci_flat_geometry(uint32_t K, uint32_t N, uint32_t min_block_size, uint32_t *num_streams,
+                     uint32_t *capacity);
+
+int ci_encode_flat(const uint8_t *d_symbols, uint32_t K, uint32_t N, uint32_t num_streams,
+                   uint32_t capacity, const uint16_t *h_freqs, const uint16_t *h_cdf,
+                   uint8_t *d_scratch, size_t scratch_bytes, uint32_t *d_states, uint32_t *d_sizes,
+                   uint64_t *d_checkpoints, uint32_t *h_max_len, ci_stream_t stream);
+
+int ci_pack_flat(const uint8_t *d_scratch, uint32_t num_streams, uint32_t capacity,
+                 const uint32_t *d_sizes, uint32_t max_len, uint8_t *d_stream, ci_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Flat decoders.
+ * ci_decode_flat_strided replaces the free function decompress() behind ccore.decompress
+ * (src/python_bindings.cpp:61-78, src/cuda/rans_ops.cu:619-629, kernel
+ * src/cuda/rans_kernels.cuh:626-708): every stream decodes ceil(out_len / num_streams) symbols,
+ * symbol i of stream g goes to d_out[g + i * num_streams] (writes past out_len are dropped).
+ * ci_decode_flat_segmented replaces rans_decomp_triton (comp_inference/rans_triton.py:172-271):
+ * stream g decodes the 512-row segment g / N of column g % N into u8 [K,N].
+ * ------------------------------------------------------------------------------------- */
+int ci_decode_flat_strided(const uint8_t *d_stream, uint64_t stream_len, const uint32_t *d_states,
+                           const uint32_t *d_sizes, uint32_t num_streams, const uint32_t *d_tables,
+                           const uint8_t *d_slot_map, uint64_t out_len, uint8_t *d_out,
+                           ci_stream_t stream);
+
+int ci_decode_flat_segmented(const uint8_t *d_stream, uint64_t stream_len, const uint32_t *d_states,
+                             const uint32_t *d_sizes, uint32_t num_streams, const uint32_t *d_tables,
+                             const uint8_t *d_slot_map, uint32_t K, uint32_t N, uint8_t *d_out,
+                             ci_stream_t stream);
+
+/* Stand-alone decoder of the dense tiled format (byte order as the reference's fused kernels
+ * read it, comp_inference/linear_triton.py:1103-1108, :1147-1170).  Outputs as
+ * ci_decode_tiled_ilp2. */
+int ci_decode_tiled_dense(const uint8_t *d_stream, uint64_t stream_len, const uint32_t *d_states,
+                          const uint32_t *d_tables, const uint8_t *d_slot_map,
+                          const uint32_t *d_stream_offsets, const uint32_t *d_stream_sizes,
+                          uint32_t K, uint32_t N, uint32_t tile_height, uint32_t tile_width,
+                          uint8_t *d_out_exp, const uint8_t *d_man_tiled, uint16_t *d_out_bf16,
+                          ci_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Fused decompress + linear:  out[M,N] (bf16) = x[M,K] (bf16) * W[K,N] (+ bias), W given as
+ * coded exponent plane + tile-interleaved raw sign|mantissa plane, never written to memory.
+ * ci_fused_linear_ilp2 replaces fused_rans_linear_triton / fused_rans_matmul_kernel_ilp2_splitk
+ * (comp_inference/linear_triton.py:229-552); ci_fused_linear_dense replaces
+ * fused_rans_linear_triton_uncoalesced (comp_inference/linear_triton.py:1045-1265).
+ * x_stride / out_stride are row strides in elements.  d_bias may be NULL.  Products are
+ * accumulated in fp32; partial sums over K are combined in a fixed order, so results are
+ * reproducible run to run.  d_workspace must hold ci_fused_linear_workspace_bytes(...) bytes
+ * (0 when one workgroup spans all of K); it carries the fp32 split-K partials that
+ * the reduction kernel sums (the reference keeps bf16 partials and sums them with torch.sum,
+ * comp_inference/linear_triton.py:257-264, :303-314).
+ * ------------------------------------------------------------------------------------- */
+size_t ci_fused_linear_workspace_bytes(uint32_t M, uint32_t K, uint32_t N, uint32_t tile_height,
+                                       uint32_t tile_width, int dense);
+
+int ci_fused_linear_ilp2(const uint16_t *d_x, uint32_t M, uint32_t K, uint32_t N, uint32_t x_stride,
+                         const uint8_t *d_stream, uint64_t stream_len, const uint32_t *d_states,
+                         const uint32_t *d_tables, const uint8_t *d_slot_map,
+                         const uint32_t *d_tile_offsets, const uint32_t *d_tile_max_lens,
+                         const uint8_t *d_man_tiled, uint32_t tile_height, uint32_t tile_width,
+                         const uint16_t *d_bias, uint16_t *d_out, uint32_t out_stride,
+                         void *d_workspace, size_t workspace_bytes, ci_stream_t stream);
+
+int ci_fused_linear_dense(const uint16_t *d_x, uint32_t M, uint32_t K, uint32_t N, uint32_t x_stride,
+                          const uint8_t *d_stream, uint64_t stream_len, const uint32_t *d_states,
+                          const uint32_t *d_tables, const uint8_t *d_slot_map,
+                          const uint32_t *d_stream_offsets, const uint32_t *d_stream_sizes,
+                          const uint8_t *d_man_tiled, uint32_t tile_height, uint32_t tile_width,
+                          const uint16_t *d_bias, uint16_t *d_out, uint32_t out_stride,
+                          void *d_workspace, size_t workspace_bytes, ci_stream_t stream);
+
+/* Split-K reduction on its own: d_out[m][n] = bf16(sum_p partial[p][m][n]) (+ bias, added in
+ * fp32 and rounded once more, as torch's in-place bf16 add does).  Replaces
+ * torch.sum(workspace, dim=0) (+= bias) of comp_inference/linear_triton.py:303-314;
+ * partial_is_bf16 != 0 reads the reference's bf16 [P,M,N] workspace layout, 0 reads fp32. */
+int ci_splitk_reduce(const void *d_partial, int partial_is_bf16, uint32_t P, uint32_t M, uint32_t N,
+                     const uint16_t *d_bias, uint16_t *d_out, uint32_t out_stride, ci_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

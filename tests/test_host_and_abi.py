@@ -1,0 +1,115 @@
+"""Host-side logic that needs no GPU, and the C ABI: the shared library loads and exports every
+function that include/comp_inference_hip.h declares (no compute calls here)."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import bf16_bits, bits_to_bf16, make_weight_kn, make_x
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_functions():
+    text = open(os.path.join(ROOT, "include", "comp_inference_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ci_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from comp_inference_amd import _lib
+
+    lib = _lib.lib()
+    names = _declared_functions()
+    assert len(names) >= 15
+    for n in names:
+        assert hasattr(lib, n), f"{n} is declared in the header but not exported"
+
+
+def test_every_exported_entry_point_is_declared():
+    import subprocess
+
+    from comp_inference_amd import _lib
+
+    out = subprocess.run(["nm", "-D", "--defined-only", _lib.LIB_PATH], capture_output=True, text=True).stdout
+    exported = sorted(set(re.findall(r"\bT (ci_[a-z0-9_]+)", out)))
+    assert exported == _declared_functions()
+
+
+def test_host_only_entry_points_run_without_gpu():
+    from comp_inference_amd import _lib
+
+    lib = _lib.lib()
+    assert lib.ci_abi_version() >= 1
+    t = _lib.Tiling()
+    assert lib.ci_tiling_init(ctypes.byref(t), 4096, 14336, 1024, 32, 1) == 0
+    assert (t.num_tiles_k, t.num_tiles_n, t.num_tiles, t.num_streams) == (4, 448, 1792, 114688)
+    assert t.capacity == int(512 * 1.25) + 64  # src/cuda/rans_host.cuh:470-471
+    assert lib.ci_tiling_init(ctypes.byref(t), 128256, 4096, 1024, 32, 1) == 0
+    assert (t.num_tiles_k, t.num_tiles) == (126, 16128)
+    # tile height not a multiple of 16 is refused with the reference's message (rans_host.cuh:441-445)
+    assert lib.ci_tiling_init(ctypes.byref(t), 4096, 4096, 24, 32, 1) != 0
+    assert b"tile height" in lib.ci_last_error()
+    assert lib.ci_tiling_init(ctypes.byref(t), 0, 4096, 1024, 32, 1) != 0
+    # decoder tables built on the host equal the oracle's
+    from oracle import rans_oracle as ro
+
+    f, c = ro.get_lut(np.arange(256, dtype=np.uint8).repeat(3))
+    tables, slot_map = np.zeros(256, np.uint32), np.zeros(4096, np.uint8)
+    vp = lambda a: a.ctypes.data_as(ctypes.c_void_p)
+    assert lib.ci_build_tables(vp(f), vp(c), vp(tables), vp(slot_map)) == 0
+    to, so = ro.build_tables(f, c)
+    assert np.array_equal(tables, to) and np.array_equal(slot_map, so)
+    bad = c.copy()
+    bad[255] = 4095
+    f2 = f.copy()
+    f2[255] = 9
+    assert lib.ci_build_tables(vp(f2), vp(bad), vp(tables), vp(slot_map)) != 0
+
+
+def test_ops_refuse_cpu_tensors():
+    """There is no CPU path: ops given host tensors raise instead of computing."""
+    from comp_inference_amd import ccore, fused_rans_linear_triton, rans_decomp_triton_tiled
+
+    z8, z32 = torch.zeros(64, dtype=torch.uint8), torch.zeros(64, dtype=torch.int32)
+    with pytest.raises(RuntimeError):
+        rans_decomp_triton_tiled(z8, z32, z32, z8, (1024, 32), z32, z32)
+    with pytest.raises(RuntimeError):
+        fused_rans_linear_triton(torch.zeros(1, 1024, dtype=torch.bfloat16), z8, z32, z32, z8, (1024, 32), z32, z32,
+                                 1024, 32, z8)
+    with pytest.raises(RuntimeError, match="GPU"):
+        ccore.decompress(z8, z32, z32, 64, z32, z8, z8)
+    if not torch.cuda.is_available():
+        with pytest.raises(RuntimeError):
+            ccore.RansManager().compress_tiled(torch.zeros(1024, 32, dtype=torch.uint8), z32, z32, 1024, 32)
+
+
+def test_reference_numerics_restatement_is_within_the_reference_tolerance(oracle):
+    """The reference rounds each product to bf16 and stores bf16 split partials; its own test
+    accepts atol=rtol=1e-2 against an fp32 matmul (tests/test_mat_mul.py:220)."""
+    K, N, M = 2048, 64, 4
+    w = make_weight_kn(N, K, 3)
+    x = make_x(M, K, 4)
+    ref = bits_to_bf16(oracle.linear_reference_numerics(bf16_bits(x), bf16_bits(w), None, 1024, 8)).float()
+    f32 = torch.from_numpy(oracle.linear_f32(bf16_bits(x), bf16_bits(w)))
+    f64 = (x.double() @ w.double()).float()
+    assert torch.allclose(f32, f64, atol=1e-4, rtol=1e-4)
+    assert torch.allclose(ref, f64, atol=1e-2, rtol=1e-2)
+    bias = make_x(1, N, 5).view(N)
+    refb = bits_to_bf16(oracle.linear_reference_numerics(bf16_bits(x), bf16_bits(w), bf16_bits(bias), 1024, 8))
+    assert torch.equal(refb, (ref.to(torch.bfloat16) + bias))
+
+
+def test_embedding_oracle_equals_table_lookup(oracle):
+    K, N, th, tw = 1300, 64, 512, 32
+    table = make_weight_kn(N, K, 7)  # [K, N]
+    enc, man = oracle.compress_bf16(bf16_bits(table), th, tw)
+    ids = np.array([0, 1, 255, 256, 511, 512, 1023, 1024, 1299, 1300, -1, 7, 7], np.int64)
+    got = oracle.embedding_gather(ids, enc, man, K, N)
+    want = np.zeros((ids.size, N), np.uint16)
+    ok = (ids >= 0) & (ids < K)
+    want[ok] = bf16_bits(table)[ids[ok]]
+    assert np.array_equal(got, want)
