@@ -16,6 +16,12 @@ from .comp_inference import (
     reconstruct_from_exp_and_mantissa,
     uninterleave_mantissas,
 )
+from .embedding_hip import (
+    fused_rans_embedding,
+    fused_rans_embedding_triton,
+    fused_rans_embedding_triton_uncoalesced,
+    fused_rans_embedding_uncoalesced,
+)
 from .linear_hip import (
     fused_rans_linear,
     fused_rans_linear_triton,

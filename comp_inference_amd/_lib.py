@@ -34,6 +34,7 @@ def lib() -> C.CDLL:
         _lib.ci_last_error.restype = C.c_char_p
         _lib.ci_encode_scratch_bytes.restype = C.c_size_t
         _lib.ci_fused_linear_workspace_bytes.restype = C.c_size_t
+        _lib.ci_fused_embedding_workspace_bytes.restype = C.c_size_t
     return _lib
 
 

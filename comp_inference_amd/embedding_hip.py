@@ -1,0 +1,74 @@
+"""Fused decompress + embedding gather on the GPU.
+
+Call signatures follow comp_inference/embedding_triton.py:278-291 (`fused_rans_embedding_triton`)
+and :431-444 (`fused_rans_embedding_triton_uncoalesced`); the kernels are HIP (csrc/embedding.hip).
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+import torch
+
+from . import _lib
+from ._lib import check, lib, ptr
+from .linear_hip import _Scratch
+
+
+def _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, meta0, meta1, tile_k, tile_n,
+         mantissas, out, dense: bool):
+    K, N = int(weight_shape[0]), int(weight_shape[1])  # K = vocabulary, N = hidden
+    _lib.require_device(x)
+    dev = x.device
+    ids = x.reshape(-1)
+    if ids.dtype != torch.int64:
+        ids = ids.to(torch.int64)
+    ids = ids.contiguous()
+    n = ids.numel()
+    if out is None:
+        result = torch.empty((n, N), device=dev, dtype=torch.bfloat16)
+    else:
+        if out.dtype != torch.bfloat16 or not out.is_cuda:
+            raise RuntimeError("out must be a bfloat16 GPU tensor")
+        result = out.view(n, N)
+    stream_t = _lib.as_u8(compressed_data, dev)
+    man = _lib.as_u8(mantissas, dev).view(-1)
+    need_man = (-(-K // tile_k)) * (-(-N // tile_n)) * tile_k * tile_n
+    if man.numel() < need_man:
+        man = torch.nn.functional.pad(man, (0, need_man - man.numel()))
+    # device copies must stay referenced until the launch has been enqueued
+    st, tb, sm = _lib.as_u32(initial_states, dev), _lib.as_u32(tables, dev), _lib.as_u8(slot_map, dev)
+    m0, m1 = _lib.as_u32(meta0, dev), _lib.as_u32(meta1, dev)
+    if dense:
+        check(lib().ci_fused_embedding_dense(
+            ptr(ids), n, ptr(stream_t), C.c_uint64(stream_t.numel()), ptr(st), ptr(tb), ptr(sm), ptr(m0), ptr(m1),
+            ptr(man), K, N, int(tile_k), int(tile_n), ptr(result), result.stride(0), _lib.stream_handle(dev)))
+    else:
+        need = lib().ci_fused_embedding_workspace_bytes(n, K, int(tile_k))
+        ws = _Scratch.get(need, ("emb", dev))
+        check(lib().ci_fused_embedding_ilp2(
+            ptr(ids), n, ptr(stream_t), C.c_uint64(stream_t.numel()), ptr(st), ptr(tb), ptr(sm), ptr(m0), ptr(m1),
+            ptr(man), K, N, int(tile_k), int(tile_n), ptr(result), result.stride(0), ptr(ws),
+            C.c_size_t(ws.numel() if ws is not None else 0), _lib.stream_handle(dev)))
+    if out is not None:
+        return out.view(*x.shape, N)
+    return result.view(*x.shape, N)
+
+
+def fused_rans_embedding(x, compressed_data, initial_states, tables, slot_map, weight_shape, tile_offsets,
+                         tile_max_lens, tile_k, tile_n, mantissas, out=None):
+    """table[x] for a table in the tiled two-streams-per-column format; ids outside the table give
+    zero rows (comp_inference/embedding_triton.py:204-210, :278-330)."""
+    return _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, tile_offsets, tile_max_lens,
+                tile_k, tile_n, mantissas, out, dense=False)
+
+
+def fused_rans_embedding_uncoalesced(x, compressed_data, initial_states, tables, slot_map, weight_shape,
+                                     stream_offsets, stream_sizes, tile_k, tile_n, mantissas, out=None):
+    """Same for the dense one-stream-per-column layout (comp_inference/embedding_triton.py:431-483)."""
+    return _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, stream_offsets, stream_sizes,
+                tile_k, tile_n, mantissas, out, dense=True)
+
+
+# Names under which the reference exports these ops (comp_inference/__init__.py:49-52).
+fused_rans_embedding_triton = fused_rans_embedding
+fused_rans_embedding_triton_uncoalesced = fused_rans_embedding_uncoalesced

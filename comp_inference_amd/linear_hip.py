@@ -20,13 +20,15 @@ class _Scratch:
     _buf: dict = {}
 
     @classmethod
-    def get(cls, nbytes: int, device) -> torch.Tensor | None:
+    def get(cls, nbytes: int, key) -> torch.Tensor | None:
+        """`key` is a device, or a (tag, device) pair for a scratch area of its own."""
         if nbytes == 0:
             return None
-        b = cls._buf.get(device)
+        device = key[1] if isinstance(key, tuple) else key
+        b = cls._buf.get(key)
         if b is None or b.numel() < nbytes:
             b = torch.empty(nbytes, dtype=torch.uint8, device=device)
-            cls._buf[device] = b
+            cls._buf[key] = b
         return b
 
 

@@ -213,6 +213,33 @@ int ci_fused_linear_dense(const uint16_t *d_x, uint32_t M, uint32_t K, uint32_t 
 int ci_splitk_reduce(const void *d_partial, int partial_is_bf16, uint32_t P, uint32_t M, uint32_t N,
                      const uint16_t *d_bias, uint16_t *d_out, uint32_t out_stride, ci_stream_t stream);
 
+/* ---------------------------------------------------------------------------------------
+ * Fused decompress + gather:  out[t, 0..N) (bf16) = table[ids[t], 0..N) for a table [K,N] stored
+ * like a weight (K = vocabulary rows, not transposed); ids outside [0,K) give zero rows.
+ * ci_fused_embedding_ilp2 replaces fused_rans_embedding_triton / fused_rans_embedding_kernel_ilp2
+ * (comp_inference/embedding_triton.py:170-330); ci_fused_embedding_dense replaces
+ * fused_rans_embedding_triton_uncoalesced (comp_inference/embedding_triton.py:333-483).
+ * d_ids: int64.  out_stride: row stride of d_out in elements.  The default-format entry point
+ * sorts the ids on the device and needs ci_fused_embedding_workspace_bytes(...) bytes of
+ * scratch (sorted ids, their output rows, one start index per half tile of rows).
+ * ------------------------------------------------------------------------------------- */
+size_t ci_fused_embedding_workspace_bytes(uint32_t n_ids, uint32_t K, uint32_t tile_height);
+
+int ci_fused_embedding_ilp2(const int64_t *d_ids, uint32_t n_ids, const uint8_t *d_stream,
+                            uint64_t stream_len, const uint32_t *d_states, const uint32_t *d_tables,
+                            const uint8_t *d_slot_map, const uint32_t *d_tile_offsets,
+                            const uint32_t *d_tile_max_lens, const uint8_t *d_man_tiled, uint32_t K,
+                            uint32_t N, uint32_t tile_height, uint32_t tile_width, uint16_t *d_out,
+                            uint32_t out_stride, void *d_workspace, size_t workspace_bytes,
+                            ci_stream_t stream);
+
+int ci_fused_embedding_dense(const int64_t *d_ids, uint32_t n_ids, const uint8_t *d_stream,
+                             uint64_t stream_len, const uint32_t *d_states, const uint32_t *d_tables,
+                             const uint8_t *d_slot_map, const uint32_t *d_stream_offsets,
+                             const uint32_t *d_stream_sizes, const uint8_t *d_man_tiled, uint32_t K,
+                             uint32_t N, uint32_t tile_height, uint32_t tile_width, uint16_t *d_out,
+                             uint32_t out_stride, ci_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,94 @@
+"""GPU parity of the fused decompress-gather: bit exact against table[ids] and against the oracle's
+literal restatement of the reference kernel."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import bf16_bits, make_weight_kn
+
+pytestmark = pytest.mark.gpu
+
+
+def _t32(a):
+    return torch.from_numpy(np.ascontiguousarray(a).view(np.int32))
+
+
+def _gather(enc, man, ids, K, N, th, tw, **kw):
+    from comp_inference_amd import fused_rans_embedding_triton
+
+    dev = "cuda"
+    return fused_rans_embedding_triton(
+        ids.to(dev), torch.from_numpy(enc.stream).to(dev), _t32(enc.states).to(dev), _t32(enc.tables).to(dev),
+        torch.from_numpy(enc.slot_map).to(dev), (K, N), _t32(enc.tile_offsets).to(dev),
+        _t32(enc.tile_max_lens).to(dev), th, tw, torch.from_numpy(man).to(dev), **kw)
+
+
+def _expected(table, ids):
+    K, N = table.shape
+    flat = ids.reshape(-1)
+    want = torch.zeros(flat.numel(), N, dtype=torch.bfloat16)
+    ok = (flat >= 0) & (flat < K)
+    want[ok] = table[flat[ok]]
+    return want.view(*ids.shape, N)
+
+
+@pytest.mark.parametrize("K,N,th,tw", [(1300, 128, 1024, 32), (2048, 96, 1024, 32), (700, 64, 256, 32),
+                                       (300, 40, 64, 16), (512, 128, 128, 64)])
+def test_embedding_matches_table_and_oracle(oracle, K, N, th, tw):
+    table = make_weight_kn(N, K, seed=K)  # [K, N], rows are vocabulary entries
+    enc, man = oracle.compress_bf16(bf16_bits(table), th, tw)
+    rng = np.random.default_rng(4)
+    ids = np.concatenate([rng.integers(0, K, 200), [0, K - 1, K, -1, 5, 5, 5, th // 2 - 1, th // 2, min(K - 1, th)]])
+    ids_t = torch.from_numpy(ids.astype(np.int64))
+    got = _gather(enc, man, ids_t, K, N, th, tw)
+    assert got.shape == (ids.size, N) and got.dtype == torch.bfloat16
+    want = _expected(table, ids_t)
+    assert torch.equal(got.cpu().view(torch.int16), want.view(torch.int16))
+    ref = oracle.embedding_gather(ids, enc, man, K, N)
+    assert np.array_equal(bf16_bits(got), ref)
+
+
+def test_embedding_single_id_2d_shape_and_out(oracle):
+    K, N, th, tw = 1300, 128, 1024, 32
+    table = make_weight_kn(N, K, seed=3)
+    enc, man = oracle.compress_bf16(bf16_bits(table), th, tw)
+    one = torch.tensor([777], dtype=torch.int64)
+    assert torch.equal(_gather(enc, man, one, K, N, th, tw).cpu().view(torch.int16),
+                       table[777:778].view(torch.int16))
+    ids = torch.tensor([[1, 2, 1299], [1024, 0, 511]], dtype=torch.int64)
+    out = torch.full((6, N), 7.0, dtype=torch.bfloat16, device="cuda")
+    got = _gather(enc, man, ids, K, N, th, tw, out=out)
+    assert got.shape == (2, 3, N)
+    assert torch.equal(out.cpu().view(torch.int16), _expected(table, ids).view(6, N).view(torch.int16))
+    # int32 ids are accepted
+    got32 = _gather(enc, man, ids.to(torch.int32), K, N, th, tw)
+    assert torch.equal(got32.cpu().view(torch.int16), _expected(table, ids).view(torch.int16))
+
+
+def test_embedding_more_ids_than_one_sort_pass(oracle):
+    K, N, th, tw = 640, 64, 128, 32
+    table = make_weight_kn(N, K, seed=8)
+    enc, man = oracle.compress_bf16(bf16_bits(table), th, tw)
+    rng = np.random.default_rng(0)
+    p = 1.0 / np.arange(1, K + 1) ** 1.1
+    ids = torch.from_numpy(rng.choice(K, 20000, p=p / p.sum()).astype(np.int64))
+    got = _gather(enc, man, ids, K, N, th, tw)
+    assert torch.equal(got.cpu().view(torch.int16), table[ids].view(torch.int16))
+
+
+def test_embedding_dense_layout(oracle):
+    from comp_inference_amd import fused_rans_embedding_triton_uncoalesced
+
+    K, N, th, tw = 600, 64, 256, 32
+    table = make_weight_kn(N, K, seed=12)
+    e, m = oracle.split_bf16(bf16_bits(table))
+    f, c = oracle.get_lut(e)
+    enc = oracle.encode_tiled_dense(e, f, c, th, tw)
+    man = oracle.interleave_plane(m, th, tw)
+    ids = torch.tensor([0, 599, 600, 255, 256, 300, 300], dtype=torch.int64)
+    dev = "cuda"
+    got = fused_rans_embedding_triton_uncoalesced(
+        ids.to(dev), torch.from_numpy(enc.stream).to(dev), _t32(enc.states).to(dev), _t32(enc.tables).to(dev),
+        torch.from_numpy(enc.slot_map).to(dev), (K, N), _t32(enc.stream_offsets).to(dev), _t32(enc.sizes).to(dev),
+        th, tw, torch.from_numpy(man).to(dev))
+    assert torch.equal(got.cpu().view(torch.int16), _expected(table, ids).view(torch.int16))
