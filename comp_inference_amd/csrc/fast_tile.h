@@ -1,0 +1,214 @@
+// Hand-scheduled gfx950 inner loops for the default format (32-column tiles, body staged in LDS).
+//
+// State representation inside these loops
+//   X   = 8 * rANS state.  Bits 3..14 are the slot, bits 15.. the quotient; the low three bits
+//         carry nothing (renormalisation may leave byte fragments there, every consumer masks
+//         or shifts them away).  With this scaling the LDS address of the 8-byte slot-table
+//         entry is X & 0x7ff8: one instruction on the serial chain instead of two.
+//   tab = slot table with .x = 8*freq | symbol << 24, .y = 8*(slot - cdf), at LDS address 0.
+//   q   = LDS address of the byte after the next one of this lane's stream.  The tile body is
+//         staged transposed (each lane's bytes contiguous, ascending with the stored row), so
+//         consuming k bytes is q -= k, done with subtract-with-borrow on the compare results.
+//   n1, n2 = the next two stream bytes (at q+1 and q), read one step ahead.
+//
+// One decode step is branch free.  t = freq * (X >> 15) + bias needs 0, 1 or 2 more bytes
+// (t >= 2^16, t < 2^16, t < 2^8 in unscaled terms); both candidates are formed and selected:
+//   X = t < 2^8 ? (t << 16 | n1 << 8 | n2) : t < 2^16 ? (t << 8 | n1) : t
+// The serial chain per symbol is v_and -> ds_read_b64 -> v_mad_u32_u24 -> v_cmp -> 2 x v_cndmask;
+// everything else is placed in the latency shadow of the table read.
+//
+// Inline-asm rule kept throughout: no LDS or global load issued inside an asm statement is
+// still in flight when the statement ends (the compiler does not know about them and may
+// reuse or copy their destination registers).
+#pragma once
+#include "rans_device.h"
+
+namespace ci {
+
+constexpr uint32_t kFastStride = 228;  // bytes of LDS per lane (57 dwords: odd, so lanes spread over banks)
+constexpr uint32_t kFastStageBytes = 64 * kFastStride;
+
+// Slot table for the scaled state (see above).  Frequencies are at most 4096, so 8*freq fits
+// the 24-bit multiplier with the symbol parked in the top byte.
+__device__ __forceinline__ void build_slot_table_x8(uint2 *tab, const uint32_t *__restrict__ tables,
+                                                    const uint8_t *__restrict__ slot_map, int tid,
+                                                    int nthreads) {
+    const uint32_t *sm4 = reinterpret_cast<const uint32_t *>(slot_map);
+    for (int g = tid; g < (int)kProbScale / 4; g += nthreads) {
+        uint32_t four = sm4[g];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            uint32_t slot = (uint32_t)g * 4 + j;
+            uint32_t s = (four >> (8 * j)) & 0xFFu;
+            uint32_t pk = tables[s];
+            tab[slot] = make_uint2(((pk & 0xFFFFu) << 3) | (s << 24), (slot - (pk >> 16)) << 3);
+        }
+    }
+}
+
+// Stage a tile body (rows of 64 bytes, row r at src + 64 r) into LDS transposed:
+// dst[lane * kFastStride + r] = src[64 r + lane].  16 rows per pass, 16-byte global loads.
+__device__ __forceinline__ void stage_transposed(uint8_t *dst, const uint8_t *__restrict__ src, uint32_t depth,
+                                                 int lane) {
+    const uint32_t g = lane & 3, rr = lane >> 2;
+    for (uint32_t r0 = 0; r0 < depth; r0 += 16) {
+        const uint32_t r = r0 + rr;
+        if (r < depth) {
+            const u32x4 v = *reinterpret_cast<const u32x4 *>(src + (size_t)r * 64 + g * 16);
+            uint8_t *d = dst + (g * 16) * kFastStride + r;
+#pragma unroll
+            for (int j = 0; j < 16; ++j) d[j * kFastStride] = (uint8_t)(v[j / 4] >> (8 * (j & 3)));
+        }
+    }
+}
+
+// ---- assembly building blocks ----------------------------------------------------------------
+// Fixed temporaries (declared as clobbers by every user):
+//   v[96:97], v[98:99]  slot-table entries of the even / odd step of a pair
+//   v100 address, v101 quotient, v102 n1 << 3, v103 n2 << 3, v104 t, v105 t<<8|n1, v106 ..<<8|n2
+//   s[20:21] second compare
+// Operands by name: X q n1 n2 (lane state), L8 B8 (scaled 2^16 and 2^8 in SGPRs).
+
+// Issue the table read and prepare everything that does not depend on it.
+#define CI_STEP_ISSUE(E)                       \
+    "v_and_b32 v100, 0x7ff8, %[X]\n"           \
+    "ds_read_b64 " E ", v100\n"                \
+    "v_lshrrev_b32 v101, 15, %[X]\n"           \
+    "s_waitcnt lgkmcnt(1)\n"                   \
+    "v_lshlrev_b32 v102, 3, %[n1]\n"           \
+    "v_lshlrev_b32 v103, 3, %[n2]\n"
+
+// Consume the table entry (ELO/EHI = its two dwords): new state, pointer, next two bytes.
+#define CI_STEP_FINISH(ELO, EHI)                        \
+    "s_waitcnt lgkmcnt(0)\n"                            \
+    "v_mad_u32_u24 v104, " ELO ", v101, " EHI "\n"      \
+    "v_cmp_gt_u32 vcc, %[L8], v104\n"                   \
+    "v_cmp_gt_u32 s[20:21], %[B8], v104\n"              \
+    "v_lshl_or_b32 v105, v104, 8, v102\n"               \
+    "v_lshl_or_b32 v106, v105, 8, v103\n"               \
+    "v_cndmask_b32 %[X], v104, v105, vcc\n"             \
+    "v_subbrev_co_u32 %[q], vcc, 0, %[q], vcc\n"        \
+    "v_cndmask_b32 %[X], %[X], v106, s[20:21]\n"        \
+    "v_subbrev_co_u32 %[q], vcc, 0, %[q], s[20:21]\n"   \
+    "ds_read_u8 %[n1], %[q] offset:1\n"                 \
+    "ds_read_u8 %[n2], %[q]\n"
+
+#define CI_STEP_CLOBBERS                                                                                  \
+    "vcc", "s20", "s21", "v96", "v97", "v98", "v99", "v100", "v101", "v102", "v103", "v104", "v105", "v106", \
+        "memory"
+
+// Two decoded symbols (top bytes of ELO0, ELO1) and their sign|mantissa bytes (byte %[msel] of the
+// dwords M0, M1) -> one dword holding two bf16 (first row in the low half).  v107/v136 temporaries.
+#define CI_PACK(ELO0, ELO1, M0, M1, WV)                       \
+    "v_perm_b32 v107, " ELO1 ", " ELO0 ", %[selE]\n"          \
+    "v_lshrrev_b32 v107, 1, v107\n"                           \
+    "v_perm_b32 v136, " M1 ", " M0 ", %[msel]\n"              \
+    "v_and_or_b32 " WV ", v136, %[mask], v107\n"
+
+// Advance the per-lane load offsets to the block after the current one (wrapping to block 0
+// after the last, so the loads stay inside the tile) -- s23 counts the blocks requested so far.
+#define CI_NEXT_BLOCK_OFFSETS                  \
+    "s_add_u32 s23, s23, 1\n"                  \
+    "s_cmp_eq_u32 s23, %[nblk]\n"              \
+    "s_cselect_b32 s24, %[wrapM], 0x100\n"     \
+    "s_cselect_b32 s25, %[wrapX], 16\n"        \
+    "v_add_u32 %[moff], s24, %[moff]\n"        \
+    "v_add_u32 %[xoff], s25, %[xoff]\n"
+
+// Sign|mantissa dwords of rows 0..4 / rows 5..7 + the x fragment of one block into buffer
+// (M0..M7, XR).
+#define CI_LOAD_LO(M0, M1, M2, M3, M4)                              \
+    "global_load_dword " M0 ", %[moff], %[mbase]\n"                 \
+    "global_load_dword " M1 ", %[moff], %[mbase] offset:32\n"       \
+    "global_load_dword " M2 ", %[moff], %[mbase] offset:64\n"       \
+    "global_load_dword " M3 ", %[moff], %[mbase] offset:96\n"       \
+    "global_load_dword " M4 ", %[moff], %[mbase] offset:128\n"
+#define CI_LOAD_HI(M5, M6, M7, XR)                                  \
+    "global_load_dword " M5 ", %[moff], %[mbase] offset:160\n"      \
+    "global_load_dword " M6 ", %[moff], %[mbase] offset:192\n"      \
+    "global_load_dword " M7 ", %[moff], %[mbase] offset:224\n"      \
+    "global_load_dwordx4 " XR ", %[xoff], %[xbase]\n"
+
+// Eight decode steps of one block.  C* = registers of the block being decoded, N* = buffer
+// being filled for the block after it (which is also the buffer the previous block used).
+// TAIL = what runs in the shadow of step 0: nothing for the first block, otherwise the last
+// pack of the previous block and its MFMA.
+#define CI_BLOCK(TAIL, C0, C1, C2, C3, C4, C5, C6, C7, N0, N1, N2, N3, N4, N5, N6, N7, NX)      \
+    CI_STEP_ISSUE("v[96:97]") TAIL CI_STEP_FINISH("v96", "v97")                                  \
+    CI_STEP_ISSUE("v[98:99]") CI_NEXT_BLOCK_OFFSETS CI_LOAD_LO(N0, N1, N2, N3, N4)               \
+    CI_STEP_FINISH("v98", "v99")                                                                 \
+    CI_STEP_ISSUE("v[140:141]") "s_waitcnt vmcnt(5)\n" CI_PACK("v96", "v98", C0, C1, "v132")     \
+    CI_STEP_FINISH("v140", "v141")                                                               \
+    CI_STEP_ISSUE("v[142:143]") CI_LOAD_HI(N5, N6, N7, NX) CI_STEP_FINISH("v142", "v143")        \
+    CI_STEP_ISSUE("v[96:97]") CI_PACK("v140", "v142", C2, C3, "v133") CI_STEP_FINISH("v96", "v97") \
+    CI_STEP_ISSUE("v[98:99]") CI_STEP_FINISH("v98", "v99")                                       \
+    CI_STEP_ISSUE("v[140:141]") CI_PACK("v96", "v98", C4, C5, "v134") CI_STEP_FINISH("v140", "v141") \
+    CI_STEP_ISSUE("v[142:143]") CI_STEP_FINISH("v142", "v143")
+
+// Last pack of a block whose buffer is (.., M6, M7, XR) and the block's MFMA.
+#define CI_TAIL(M6, M7, XR)                                             \
+    CI_PACK("v140", "v142", M6, M7, "v135")                             \
+    "s_nop 1\n"                                                         \
+    "v_mfma_f32_32x32x16_bf16 %[acc], v[132:135], " XR ", %[acc]\n"
+
+// (argument lists are expanded before CI_BLOCK counts them)
+#define CI_BLOCK_X(...) CI_BLOCK(__VA_ARGS__)
+#define CI_BUF_A "v108", "v109", "v110", "v111", "v112", "v113", "v114", "v115"
+#define CI_BUF_B "v116", "v117", "v118", "v119", "v120", "v121", "v122", "v123"
+
+// Per-lane decoder state of the hand-scheduled loops.
+struct FastLane {
+    uint32_t X, q, n1, n2;
+    // `stage` = this wave's staging area, q_lane = this lane's stream inside the tile.
+    __device__ __forceinline__ void init(const uint8_t *stage, uint32_t depth, uint32_t q_lane, uint32_t state) {
+        X = state << 3;
+        const uint8_t *col = stage + q_lane * kFastStride;
+        q = (uint32_t)(uintptr_t)col + depth - 2;  // low 32 bits of an LDS pointer are its LDS address
+        n1 = depth >= 1 ? col[depth - 1] : 0;
+        n2 = depth >= 2 ? col[depth - 2] : 0;
+    }
+};
+
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+
+// Whole-tile loop of the fused linear for M <= 32: `nblocks` (even, >= 2) blocks of 8 rows per
+// half tile.  mbase/moff: tile's sign|mantissa plane (uniform base, per-lane byte offset of the
+// aligned dword holding this lane's byte of the first row).  xbase/xoff: x (uniform base, per-lane
+// byte offset of the first of this lane's 8 consecutive k).  acc accumulates W^T-tile x x^T.
+__device__ __forceinline__ void linear_tile_asm(FastLane &st, f32x16_t &acc, uint64_t mbase, uint32_t moff,
+                                                uint64_t xbase, uint32_t xoff, uint32_t man_sel,
+                                                uint32_t nblocks) {
+    const uint32_t wrap_m = 0u - (nblocks - 1) * 256u, wrap_x = 0u - (nblocks - 1) * 16u;
+    asm volatile(
+        "s_mov_b32 s23, 0\n"
+        "s_lshr_b32 s22, %[nblk], 1\n"
+        "s_sub_u32 s22, s22, 1\n"
+        // block 0 into buffer A
+        CI_LOAD_LO("v108", "v109", "v110", "v111", "v112")
+        CI_LOAD_HI("v113", "v114", "v115", "v[124:127]")
+        CI_BLOCK_X("", CI_BUF_A, CI_BUF_B, "v[128:131]")
+        CI_BLOCK_X(CI_TAIL("v114", "v115", "v[124:127]"), CI_BUF_B, CI_BUF_A, "v[124:127]")
+        "ci_lin_loop%=:\n"
+        "s_cmp_eq_u32 s22, 0\n"
+        "s_cbranch_scc1 ci_lin_done%=\n"
+        CI_BLOCK_X(CI_TAIL("v122", "v123", "v[128:131]"), CI_BUF_A, CI_BUF_B, "v[128:131]")
+        CI_BLOCK_X(CI_TAIL("v114", "v115", "v[124:127]"), CI_BUF_B, CI_BUF_A, "v[124:127]")
+        "s_sub_u32 s22, s22, 1\n"
+        "s_branch ci_lin_loop%=\n"
+        "ci_lin_done%=:\n"
+        "s_waitcnt vmcnt(0) lgkmcnt(0)\n"
+        CI_TAIL("v122", "v123", "v[128:131]")
+        "s_nop 15\n"
+        "s_nop 15\n"
+        : [X] "+v"(st.X), [q] "+v"(st.q), [n1] "+v"(st.n1), [n2] "+v"(st.n2), [acc] "+v"(acc), [moff] "+v"(moff),
+          [xoff] "+v"(xoff)
+        : [L8] "s"(kRansL << 3), [B8] "s"(256u << 3), [selE] "s"(0x070C030Cu), [mask] "s"(0x807F807Fu),
+          [msel] "v"(man_sel), [mbase] "s"(mbase), [xbase] "s"(xbase), [nblk] "s"(nblocks), [wrapM] "s"(wrap_m),
+          [wrapX] "s"(wrap_x)
+        : CI_STEP_CLOBBERS, "scc", "s22", "s23", "s24", "s25", "v107", "v108", "v109", "v110", "v111", "v112",
+          "v113", "v114", "v115", "v116", "v117", "v118", "v119", "v120", "v121", "v122", "v123", "v124", "v125",
+          "v126", "v127", "v128", "v129", "v130", "v131", "v132", "v133", "v134", "v135", "v136", "v140", "v141",
+          "v142", "v143");
+}
+
+}  // namespace ci

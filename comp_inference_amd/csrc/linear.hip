@@ -19,11 +19,11 @@
 // splitk_reduce_kernel sums them in index order.
 #include "ci_common.h"
 #include "rans_device.h"
+#include "fast_tile.h"
 
 namespace ci {
 
 constexpr int kLinMaxWaves = 8;
-constexpr uint32_t kLinStageBytes = 14336;  // 224 byte rows per tile in LDS
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -46,8 +46,7 @@ struct LinearArgs {
     uint16_t *out;    // [M][N]
     uint32_t out_stride;
     uint32_t th, tw, tiles_n, tiles_k, kw, nw, P;
-    uint32_t stage_bytes;
-    int x_vec_ok;  // x rows may be read with 16-byte loads
+    int fast_ok;  // x rows may be read with 16-byte loads at 32-bit offsets, sign|mantissa plane dword aligned
 };
 
 __device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {
@@ -76,78 +75,20 @@ __device__ __forceinline__ uint32_t pack_bf16_pair(uint32_t w0, uint32_t w1, uin
     return (e & 0x7F807F80u) | (mm & 0x807F807Fu);
 }
 
-// Fast path: the whole tile lies inside [K,N], its body is staged in LDS and x rows can be read
-// with 16-byte loads.  The sign|mantissa bytes and the x fragment of the next block of 8 rows are
-// requested before the current block is decoded, so their latency hides behind the decode chain.
-template <int MB>
-__device__ __forceinline__ void linear_tile_fast(LdsBytes &src, uint32_t x, const uint2 *tab, uint32_t half,
-                                                 const uint8_t *man, uint32_t lane_col, const uint16_t *xrow[MB],
-                                                 const bool m_ok[MB], f32x16 acc[MB]) {
-    // The sign|mantissa byte of this lane's column is fetched as the aligned dword that holds it
-    // (four neighbouring lanes share the dword) and picked out by the byte permute that packs it.
-    const uint32_t *man4 = reinterpret_cast<const uint32_t *>(man - (lane_col & 3));
-    const uint32_t man_sel = 0x04040000u + (lane_col & 3) * 0x01010101u;
-    // two operand buffers used alternately, so the prefetched values are consumed in place
-    uint32_t mb[2][8];
-    u32x4 xv[2][MB];
-    auto request = [&](uint32_t i, int buf) {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) mb[buf][j] = man4[(size_t)(i + j) * 8];
-#pragma unroll
-        for (int b = 0; b < MB; ++b) {
-            xv[buf][b] = (u32x4){0, 0, 0, 0};
-            if (m_ok[b]) xv[buf][b] = *reinterpret_cast<const u32x4 *>(xrow[b] + i);
-        }
-    };
-    auto block = [&](int buf) {
-        uint32_t w[8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            w[j] = decode_symbol(x, tab);
-            src.renorm(x);
-            src.renorm(x);
-        }
-        u32x4 wv;
-#pragma unroll
-        for (int p = 0; p < 4; ++p)
-            wv[p] = pack_bf16_pair(w[2 * p], w[2 * p + 1], mb[buf][2 * p], mb[buf][2 * p + 1], man_sel);
-#pragma unroll
-        for (int b = 0; b < MB; ++b)
-            acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, wv),
-                                                             __builtin_bit_cast(bf16x8, xv[buf][b]), acc[b], 0, 0, 0);
-    };
-    // A request past the end of the half tile re-reads block 0 instead of branching (in range,
-    // result unused).
-    request(0, 0);
-    uint32_t i = 0;
-    for (; i + 16 <= half; i += 16) {
-        request(i + 8, 1);
-        block(0);
-        request(i + 16 < half ? i + 16 : 0, 0);
-        block(1);
-    }
-    if (i < half) block(0);
-}
-
-// General path: ragged tiles (rows >= K, columns >= N), unaligned x, or a tile body read from
-// global memory.  Same arithmetic, every access guarded.
-template <int MB, typename Bytes>
-__device__ __forceinline__ void linear_tile_guarded(Bytes &src, uint32_t x, const uint2 *tab, uint32_t K,
+// General path: ragged tiles (rows >= K, columns >= N), unaligned x, odd block counts, or a tile
+// body too deep for the staging area.  Same arithmetic on the scaled state, bytes read where they
+// lie in global memory, every access guarded.
+__device__ __forceinline__ void linear_tile_guarded(GlobalBytes &src, uint32_t X, const uint2 *tab, uint32_t K,
                                                     uint32_t half, uint32_t my_steps, const uint8_t *man,
-                                                    const uint16_t *xrow[MB], const bool m_ok[MB], uint32_t k0,
-                                                    f32x16 acc[MB]) {
+                                                    const uint16_t *xrow, bool m_ok, uint32_t k0, f32x16 &acc) {
     for (uint32_t i = 0; i < half; i += 8) {
-        u32x4 xv[MB];
+        u32x4 xv = (u32x4){0, 0, 0, 0};
+        if (m_ok) {
 #pragma unroll
-        for (int b = 0; b < MB; ++b) {
-            xv[b] = (u32x4){0, 0, 0, 0};
-            if (m_ok[b]) {
-#pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const uint32_t k = k0 + i + j;
-                    const uint32_t v = k < K ? xrow[b][i + j] : 0u;
-                    xv[b][j / 2] |= v << (16 * (j & 1));
-                }
+            for (int j = 0; j < 8; ++j) {
+                const uint32_t k = k0 + i + j;
+                const uint32_t v = k < K ? xrow[i + j] : 0u;
+                xv[j / 2] |= v << (16 * (j & 1));
             }
         }
         uint32_t mb[8], w[8];
@@ -157,112 +98,103 @@ __device__ __forceinline__ void linear_tile_guarded(Bytes &src, uint32_t x, cons
             w[j] = 0;
             if (i + j < my_steps) {
                 mb[j] = man[(size_t)(i + j) * 32];
-                w[j] = decode_symbol(x, tab);
-                src.renorm(x);
-                src.renorm(x);
+                w[j] = decode_symbol_scaled(X, tab);
+                src.renorm_scaled(X);
+                src.renorm_scaled(X);
             }
         }
         u32x4 wv;
 #pragma unroll
         for (int p = 0; p < 4; ++p) wv[p] = pack_bf16_pair(w[2 * p], w[2 * p + 1], mb[2 * p], mb[2 * p + 1]);
-#pragma unroll
-        for (int b = 0; b < MB; ++b)
-            acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, wv),
-                                                             __builtin_bit_cast(bf16x8, xv[b]), acc[b], 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, wv), __builtin_bit_cast(bf16x8, xv),
+                                                      acc, 0, 0, 0);
     }
 }
 
-// grid: (ceil(tiles_n / nw), P, ceil(M / (32 * MB)))   block: kw * nw waves
-template <int MB>
+// grid: (ceil(tiles_n / nw), P, ceil(M / 32))   block: kw * nw waves
 __global__ __launch_bounds__(kLinMaxWaves *kWave) void fused_linear32_kernel(LinearArgs a) {
     extern __shared__ __align__(16) uint8_t lds[];
     uint2 *tab = reinterpret_cast<uint2 *>(lds);
     const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
     const int nthreads = blockDim.x;
-    uint8_t *stage = lds + kSlotTableBytes + (size_t)wave * a.stage_bytes;
+    uint8_t *stage = lds + kSlotTableBytes + (size_t)wave * kFastStageBytes;
 
-    build_slot_table(tab, a.tables, a.slot_map, tid, nthreads);
+    build_slot_table_x8(tab, a.tables, a.slot_map, tid, nthreads);
 
     const uint32_t kidx = wave % a.kw, nidx = wave / a.kw;
     const uint32_t tk = blockIdx.y * a.kw + kidx, tn = blockIdx.x * a.nw + nidx;
     const bool have_tile = tk < a.tiles_k && tn < a.tiles_n;
     const uint32_t tile = tk * a.tiles_n + tn;
-    uint32_t depth = 0;
+    const uint32_t half = a.th / 2, hsel = lane / 32, c = lane % 32;
+    const uint32_t col0 = tn * 32, k0 = tk * a.th + hsel * half;
+    uint32_t depth = 0, my_steps = 0;
     uint64_t base = 0;
-    bool in_lds = false;
+    bool fast = false;
     if (have_tile) {
         base = a.tile_offsets[tile];
         depth = a.tile_max_lens[tile];
         if (base + (uint64_t)depth * 64 > a.stream_len) depth = 0;
-        in_lds = depth * 64u <= a.stage_bytes;
-        if (in_lds) stage_to_lds(stage, a.stream + base, depth * 64u, lane);
+        if (col0 + c < a.N && k0 < a.K) my_steps = min(half, a.K - k0);
+        const bool full = __builtin_amdgcn_ballot_w64(my_steps != half) == 0;
+        // the hand-scheduled loop wants: a full tile, a body that fits one lane stride, an even
+        // number of 8-row blocks, 16-byte readable x rows and a dword-aligned sign|mantissa plane
+        fast = full && a.fast_ok && depth >= 2 && depth < kFastStride && half % 16 == 0 &&
+               (uint32_t)(uintptr_t)tab == 0;
+        if (fast) stage_transposed(stage, a.stream + base, depth, lane);
     }
     __syncthreads();
 
-    const uint32_t half = a.th / 2, hsel = lane / 32, c = lane % 32;
-    const uint32_t m_base = blockIdx.z * 32 * MB;
-    f32x16 acc[MB];
+    const uint32_t m = blockIdx.z * 32 + c;  // row of x this lane feeds to the MFMA
+    const bool m_ok = m < a.M;
+    f32x16 acc;
 #pragma unroll
-    for (int b = 0; b < MB; ++b)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) acc[b][v] = 0.f;
+    for (int v = 0; v < 16; ++v) acc[v] = 0.f;
 
     if (have_tile) {
-        const uint32_t col0 = tn * 32, k0 = tk * a.th + hsel * half;
-        uint32_t my_steps = 0;
-        if (col0 + c < a.N && k0 < a.K) my_steps = min(half, a.K - k0);
-        const bool full = __builtin_amdgcn_ballot_w64(my_steps != half) == 0;
-        const uint16_t *xrow[MB];  // row m of x, already advanced to this lane's first k
-        bool m_ok[MB];
-#pragma unroll
-        for (int b = 0; b < MB; ++b) {
-            const uint32_t m = m_base + b * 32 + c;
-            m_ok[b] = m < a.M;
-            xrow[b] = a.x + (size_t)(m_ok[b] ? m : 0) * a.x_stride + k0;
-        }
-        const uint8_t *man = a.man_tiled + (size_t)tile * a.th * 32 + (size_t)hsel * half * 32 + c;
-        uint32_t x = a.states[(size_t)tile * 64 + lane];
-        const bool aligned_man = (reinterpret_cast<uintptr_t>(a.man_tiled) & 3) == 0;
-        if (in_lds) {
-            LdsBytes src;
-            src.init(stage, depth, 64, lane);
-            if (full && a.x_vec_ok && aligned_man)
-                linear_tile_fast<MB>(src, x, tab, half, man, c, xrow, m_ok, acc);
-            else
-                linear_tile_guarded<MB>(src, x, tab, a.K, half, my_steps, man, xrow, m_ok, k0, acc);
+        const uint32_t xrow_elems = (m_ok ? m : 0) * a.x_stride + k0;  // rows past M re-read row 0: their
+                                                                       // accumulator columns are never stored
+        const size_t man_tile = (size_t)tile * a.th * 32;
+        const uint32_t state = a.states[(size_t)tile * 64 + lane];
+        if (fast) {
+            FastLane st;
+            st.init(stage, depth, lane, state);
+            const uint64_t mbase = reinterpret_cast<uint64_t>(a.man_tiled + man_tile);
+            // readfirstlane returns a signed int: widen through uint32_t, not by sign extension
+            const uint32_t mb_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(mbase >> 32));
+            const uint32_t mb_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)mbase);
+            const uint64_t mb_u = ((uint64_t)mb_hi << 32) | (uint64_t)mb_lo;
+            const uint32_t moff = hsel * half * 32 + (c & ~3u);
+            const uint32_t man_sel = 0x04040000u + (c & 3u) * 0x01010101u;
+            linear_tile_asm(st, acc, mb_u, moff, reinterpret_cast<uint64_t>(a.x), xrow_elems * 2u, man_sel, half / 8);
         } else {
             GlobalBytes src;
             src.init(a.stream + base, depth, 64, lane);
-            linear_tile_guarded<MB>(src, x, tab, a.K, half, my_steps, man, xrow, m_ok, k0, acc);
+            linear_tile_guarded(src, state << 3, tab, a.K, half, my_steps,
+                                a.man_tiled + man_tile + (size_t)hsel * half * 32 + c, a.x + xrow_elems, m_ok, k0, acc);
         }
     }
 
     // Sum the kw accumulators of each column tile in k order.  The staging area is free now;
-    // every wave stores its fragment as [v][lane] floats (4 KB per m-block).
+    // every wave stores its fragment as [v][lane] floats (4 KB).
     __syncthreads();
     float *red = reinterpret_cast<float *>(lds + kSlotTableBytes);
-    const uint32_t frag = 16 * kWave;  // floats per wave per m-block
+    const uint32_t frag = 16 * kWave;
 #pragma unroll
-    for (int b = 0; b < MB; ++b) {
-        if (b > 0) __syncthreads();
+    for (int v = 0; v < 16; ++v) red[(size_t)wave * frag + v * kWave + lane] = acc[v];
+    __syncthreads();
+    if (kidx == 0 && tn < a.tiles_n) {
 #pragma unroll
-        for (int v = 0; v < 16; ++v) red[(size_t)wave * frag + v * kWave + lane] = acc[b][v];
-        __syncthreads();
-        if (kidx == 0 && tn < a.tiles_n) {
-            const uint32_t m = m_base + b * 32 + c;
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                float s = 0.f;
-                for (uint32_t kk = 0; kk < a.kw; ++kk) s += red[(size_t)(nidx * a.kw + kk) * frag + v * kWave + lane];
-                // MFMA 32x32 result layout: register v of lane l is row (v/4)*8 + (l/32)*4 + v%4
-                // (= column of the tile), column l%32 (= row m of x)
-                const uint32_t n = tn * 32 + (v / 4) * 8 + hsel * 4 + (v % 4);
-                if (m < a.M && n < a.N) {
-                    if (a.P == 1)
-                        a.out[(size_t)m * a.out_stride + n] = finish_bf16(s, a.bias, n);
-                    else
-                        a.partial[((size_t)blockIdx.y * a.M + m) * a.N + n] = s;
-                }
+        for (int v = 0; v < 16; ++v) {
+            float s = 0.f;
+            for (uint32_t kk = 0; kk < a.kw; ++kk) s += red[(size_t)(nidx * a.kw + kk) * frag + v * kWave + lane];
+            // MFMA 32x32 result layout: register v of lane l is row (v/4)*8 + (l/32)*4 + v%4
+            // (= column of the tile), column l%32 (= row m of x)
+            const uint32_t n = tn * 32 + (v / 4) * 8 + hsel * 4 + (v % 4);
+            if (m_ok && n < a.N) {
+                if (a.P == 1)
+                    a.out[(size_t)m * a.out_stride + n] = finish_bf16(s, a.bias, n);
+                else
+                    a.partial[((size_t)blockIdx.y * a.M + m) * a.N + n] = s;
             }
         }
     }
@@ -429,8 +361,8 @@ static int fused_linear_impl(const uint16_t *d_x, uint32_t M, uint32_t K, uint32
     a.tw = tw;
     a.tiles_n = ceil_div(N, tw);
     a.tiles_k = ceil_div(K, th);
-    a.stage_bytes = kLinStageBytes;
-    a.x_vec_ok = aligned(d_x, 16) && x_stride % 8 == 0 && th % 16 == 0;
+    a.fast_ok = aligned(d_x, 16) && x_stride % 8 == 0 && aligned(d_man_tiled, 4) &&
+                (uint64_t)M * x_stride * 2 < (1ull << 31);
     const LinearPlan p = plan_linear(K, th, tw, a.tiles_n, dense, aligned(d_stream, 16));
     a.kw = p.kw;
     a.nw = p.nw;
@@ -445,23 +377,15 @@ static int fused_linear_impl(const uint16_t *d_x, uint32_t M, uint32_t K, uint32
 
     if (p.fast) {
         const uint32_t waves = p.kw * p.nw;
-        const uint32_t lds_bytes = kSlotTableBytes + waves * a.stage_bytes;
+        const uint32_t lds_bytes = kSlotTableBytes + waves * kFastStageBytes;
         static bool attr_set = false;
         if (!attr_set) {
-            CI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(fused_linear32_kernel<1>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit));
-            CI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(fused_linear32_kernel<2>),
+            CI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(fused_linear32_kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit));
             attr_set = true;
         }
-        const dim3 block(waves * kWave);
-        if (M <= 32) {
-            hipLaunchKernelGGL(fused_linear32_kernel<1>, dim3(ceil_div(a.tiles_n, p.nw), p.P, 1), block, lds_bytes,
-                               s, a);
-        } else {
-            hipLaunchKernelGGL(fused_linear32_kernel<2>, dim3(ceil_div(a.tiles_n, p.nw), p.P, ceil_div(M, 64)),
-                               block, lds_bytes, s, a);
-        }
+        hipLaunchKernelGGL(fused_linear32_kernel, dim3(ceil_div(a.tiles_n, p.nw), p.P, ceil_div(M, 32)),
+                           dim3(waves * kWave), lds_bytes, s, a);
         CI_LAUNCH_CHECK("fused_linear32_kernel");
     } else {
         const uint64_t streams = (uint64_t)a.tiles_k * a.tiles_n * (dense ? 1 : 2) * tw;

@@ -50,6 +50,14 @@ __device__ __forceinline__ uint32_t decode_symbol(uint32_t &x, const uint2 *tab)
     return e.x;
 }
 
+// The same step on the table built for the scaled state X = 8 * state (fast_tile.h); X stays
+// scaled.  Renormalisation on a scaled state: see renorm_scaled of the byte sources.
+__device__ __forceinline__ uint32_t decode_symbol_scaled(uint32_t &X, const uint2 *tab) {
+    uint2 e = tab[(X >> 3) & kProbMask];
+    X = __umul24(e.x, X >> (kProbBits + 3)) + e.y;
+    return e.x;
+}
+
 // Byte source: a tile body staged in LDS exactly as stored (rows of `row_bytes`, every stream
 // bottom-aligned).  `pos` is the byte offset of the next byte of this lane's stream and `nxt`
 // holds that byte already (read one step ahead so that the LDS latency stays off the state
@@ -88,6 +96,12 @@ struct GlobalBytes {
     __device__ __forceinline__ void renorm(uint32_t &x) {
         if (x < kRansL && row >= 0) {
             x = (x << 8) | base[(uint32_t)row * row_bytes];
+            row -= 1;
+        }
+    }
+    __device__ __forceinline__ void renorm_scaled(uint32_t &X) {
+        if (X < (kRansL << 3) && row >= 0) {
+            X = (X << 8) | ((uint32_t)base[(uint32_t)row * row_bytes] << 3);
             row -= 1;
         }
     }
