@@ -7,6 +7,7 @@
 // in LDS with 16-byte coalesced loads and then runs the sequential decode out of LDS.
 #include "ci_common.h"
 #include "rans_device.h"
+#include "fast_tile.h"
 
 namespace ci {
 
@@ -108,6 +109,68 @@ __global__ __launch_bounds__(kDecWaves *kWave) void decode_tiled32_kernel(Decode
     }
 }
 
+// Exponent-plane output through the hand-scheduled loop (fast_tile.h): scaled state, tile body
+// staged transposed.  Tiles that do not qualify (ragged, odd half height, body deeper than a
+// lane stride) take the same arithmetic with guarded byte reads from global memory.
+__global__ __launch_bounds__(kDecWaves *kWave) void decode_tiled32_fast_kernel(DecodeArgs a) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    uint2 *tab = reinterpret_cast<uint2 *>(lds);
+    const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
+    uint8_t *stage = lds + kSlotTableBytes + (size_t)wave * kFastStageBytes;
+
+    const uint32_t tile = blockIdx.x * kDecWaves + wave;
+    const bool have_tile = tile < a.num_tiles;
+    const uint32_t tk = have_tile ? tile / a.tiles_n : 0, tn = have_tile ? tile % a.tiles_n : 0;
+    const uint32_t half = a.th / 2, hsel = lane / 32, c = lane % 32;
+    const uint32_t row0 = tk * a.th, col0 = tn * 32, my_row0 = row0 + hsel * half;
+    uint32_t depth = 0, my_steps = 0;
+    uint64_t base = 0;
+    bool fast = false;
+    StageRegs body;
+    if (have_tile) {
+        base = a.tile_offsets[tile];
+        depth = a.tile_max_lens[tile];
+        if (base + (uint64_t)depth * 64 > a.stream_len) depth = 0;
+        if (col0 + c < a.N && my_row0 < a.K) my_steps = min(half, a.K - my_row0);
+        const bool full = __builtin_amdgcn_ballot_w64(my_steps != half) == 0;
+        fast = full && depth >= 2 && depth < kFastStride && half % 2 == 0 && half >= 2 &&
+               (uint64_t)a.K * a.N < (1ull << 32) && (uint32_t)(uintptr_t)tab == 0;
+        if (fast) stage_fetch(body, a.stream + base, 0, depth, lane);
+    }
+    build_slot_table_x8(tab, a.tables, a.slot_map, tid, kDecWaves * kWave);
+    if (fast) {
+        stage_commit(body, stage, 0, depth, lane);
+        for (int grp = 1; grp < kStageGroups; ++grp)
+            if ((uint32_t)grp * 128 < depth) {
+                stage_fetch(body, a.stream + base, grp * 128, depth, lane);
+                stage_commit(body, stage, grp * 128, depth, lane);
+            }
+    }
+    __syncthreads();
+    if (!have_tile) return;
+
+    const uint32_t state = a.states[(size_t)tile * 64 + lane];
+    if (fast) {
+        FastLane st;
+        st.init(stage, depth, lane, state);
+        const uint64_t ob = reinterpret_cast<uint64_t>(a.out_exp + (size_t)row0 * a.N + col0);
+        // readfirstlane returns a signed int: widen through uint32_t
+        const uint32_t ob_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(ob >> 32));
+        const uint32_t ob_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)ob);
+        decode_tile_asm(st, ((uint64_t)ob_hi << 32) | (uint64_t)ob_lo, hsel * half * a.N + c, a.N, half / 2);
+    } else {
+        GlobalBytes src;
+        src.init(a.stream + base, depth, 64, lane);
+        uint32_t X = state << 3;
+        uint8_t *o = a.out_exp + (size_t)my_row0 * a.N + col0 + c;
+        for (uint32_t i = 0; i < my_steps; ++i) {
+            o[(size_t)i * a.N] = (uint8_t)(decode_symbol_scaled(X, tab) >> 24);
+            src.renorm_scaled(X);
+            src.renorm_scaled(X);
+        }
+    }
+}
+
 // Any tile width: one thread per stream, bytes read where they lie.  Used for widths other
 // than 32 (the reference's tests sweep 16..128, tests/test_mat_mul.py:263-264).
 template <bool kMerge>
@@ -193,12 +256,14 @@ extern "C" int ci_decode_tiled_ilp2(const uint8_t *d_stream, uint64_t stream_len
             CI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(decode_tiled32_kernel<true>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes));
             hipLaunchKernelGGL(decode_tiled32_kernel<true>, grid, block, lds_bytes, s, a);
+            CI_LAUNCH_CHECK("decode_tiled32_kernel");
         } else {
-            CI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(decode_tiled32_kernel<false>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes));
-            hipLaunchKernelGGL(decode_tiled32_kernel<false>, grid, block, lds_bytes, s, a);
+            const uint32_t fast_lds = kSlotTableBytes + kDecWaves * kFastStageBytes;
+            CI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(decode_tiled32_fast_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, fast_lds));
+            hipLaunchKernelGGL(decode_tiled32_fast_kernel, grid, block, fast_lds, s, a);
+            CI_LAUNCH_CHECK("decode_tiled32_fast_kernel");
         }
-        CI_LAUNCH_CHECK("decode_tiled32_kernel");
     } else {
         a.stage_bytes = 0;
         const uint64_t streams = (uint64_t)a.num_tiles * 2 * tile_width;

@@ -47,17 +47,37 @@ __device__ __forceinline__ void build_slot_table_x8(uint2 *tab, const uint32_t *
 }
 
 // Stage a tile body (rows of 64 bytes, row r at src + 64 r) into LDS transposed:
-// dst[lane * kFastStride + r] = src[64 r + lane].  16 rows per pass, 16-byte global loads.
-__device__ __forceinline__ void stage_transposed(uint8_t *dst, const uint8_t *__restrict__ src, uint32_t depth,
-                                                 int lane) {
+// dst[lane * kFastStride + r] = src[64 r + lane].  Split in two so that all global loads of the
+// body are issued in groups of eight (128 rows) and other work -- the slot-table build -- can
+// run under the first group: stage_fetch issues the loads, stage_commit writes LDS.
+constexpr int kStagePasses = 8;                       // 16 rows per pass, 128 rows per group
+constexpr int kStageGroups = (kFastStride + 127) / 128;
+struct StageRegs {
+    u32x4 v[kStagePasses];
+};
+
+// `row0` = first row of the group (a multiple of 128).
+__device__ __forceinline__ void stage_fetch(StageRegs &regs, const uint8_t *__restrict__ src, uint32_t row0,
+                                            uint32_t depth, int lane) {
     const uint32_t g = lane & 3, rr = lane >> 2;
-    for (uint32_t r0 = 0; r0 < depth; r0 += 16) {
-        const uint32_t r = r0 + rr;
+#pragma unroll
+    for (int p = 0; p < kStagePasses; ++p) {
+        const uint32_t r = row0 + p * 16 + rr;
+        regs.v[p] = (u32x4){0, 0, 0, 0};
+        if (r < depth) regs.v[p] = *reinterpret_cast<const u32x4 *>(src + (size_t)r * 64 + g * 16);
+    }
+}
+
+__device__ __forceinline__ void stage_commit(const StageRegs &regs, uint8_t *dst, uint32_t row0, uint32_t depth,
+                                             int lane) {
+    const uint32_t g = lane & 3, rr = lane >> 2;
+#pragma unroll
+    for (int p = 0; p < kStagePasses; ++p) {
+        const uint32_t r = row0 + p * 16 + rr;
         if (r < depth) {
-            const u32x4 v = *reinterpret_cast<const u32x4 *>(src + (size_t)r * 64 + g * 16);
             uint8_t *d = dst + (g * 16) * kFastStride + r;
 #pragma unroll
-            for (int j = 0; j < 16; ++j) d[j * kFastStride] = (uint8_t)(v[j / 4] >> (8 * (j & 3)));
+            for (int j = 0; j < 16; ++j) d[j * kFastStride] = (uint8_t)(regs.v[p][j / 4] >> (8 * (j & 3)));
         }
     }
 }
@@ -209,6 +229,54 @@ __device__ __forceinline__ void linear_tile_asm(FastLane &st, f32x16_t &acc, uin
           "v113", "v114", "v115", "v116", "v117", "v118", "v119", "v120", "v121", "v122", "v123", "v124", "v125",
           "v126", "v127", "v128", "v129", "v130", "v131", "v132", "v133", "v134", "v135", "v136", "v140", "v141",
           "v142", "v143");
+}
+
+// Symbol of the step that used table entry ELO -> one byte at obase + off; off advances a row.
+#define CI_STORE_SYM(ELO)                                  \
+    "v_lshrrev_b32 v107, 24, " ELO "\n"                    \
+    "global_store_byte %[off], v107, %[obase]\n"           \
+    "v_add_u32 %[off], %[stride], %[off]\n"
+
+// Stand-alone decode of one half tile per lane: `npairs` >= 1 pairs of steps, symbol i stored at
+// obase + off + i * stride (bytes).  The store of a symbol sits in the shadow of the next step.
+__device__ __forceinline__ void decode_tile_asm(FastLane &st, uint64_t obase, uint32_t off, uint32_t stride,
+                                                uint32_t npairs) {
+    asm volatile(
+        "s_sub_u32 s22, %[npairs], 1\n"
+        CI_STEP_ISSUE("v[96:97]") CI_STEP_FINISH("v96", "v97")
+        "ci_dec_loop%=:\n"
+        "s_cmp_eq_u32 s22, 0\n"
+        "s_cbranch_scc1 ci_dec_done%=\n"
+        CI_STEP_ISSUE("v[98:99]") CI_STORE_SYM("v96") CI_STEP_FINISH("v98", "v99")
+        CI_STEP_ISSUE("v[96:97]") CI_STORE_SYM("v98") CI_STEP_FINISH("v96", "v97")
+        "s_sub_u32 s22, s22, 1\n"
+        "s_branch ci_dec_loop%=\n"
+        "ci_dec_done%=:\n"
+        CI_STEP_ISSUE("v[98:99]") CI_STORE_SYM("v96") CI_STEP_FINISH("v98", "v99")
+        CI_STORE_SYM("v98")
+        "s_waitcnt vmcnt(0) lgkmcnt(0)\n"
+        : [X] "+v"(st.X), [q] "+v"(st.q), [n1] "+v"(st.n1), [n2] "+v"(st.n2), [off] "+v"(off)
+        : [L8] "s"(kRansL << 3), [B8] "s"(256u << 3), [obase] "s"(obase), [stride] "s"(stride), [npairs] "s"(npairs)
+        : CI_STEP_CLOBBERS, "scc", "s22", "v107");
+}
+
+// Advance the lane's stream by n >= 1 symbols; returns the table word (symbol in the top byte) of
+// the last one.  n must be the same for every lane of the wave.
+__device__ __forceinline__ uint32_t advance_asm(FastLane &st, uint32_t n) {
+    uint32_t e;
+    asm volatile(
+        "s_mov_b32 s22, %[n]\n"
+        "ci_adv_loop%=:\n"
+        CI_STEP_ISSUE("v[96:97]") CI_STEP_FINISH("v96", "v97")
+        "s_sub_u32 s22, s22, 1\n"
+        "s_cmp_lg_u32 s22, 0\n"
+        "s_cbranch_scc1 ci_adv_loop%=\n"
+        "s_waitcnt lgkmcnt(0)\n"
+        "v_mov_b32 %[e], v96\n"
+        : [X] "+v"(st.X), [q] "+v"(st.q), [n1] "+v"(st.n1), [n2] "+v"(st.n2), [e] "=&v"(e)
+        : [L8] "s"(kRansL << 3), [B8] "s"(256u << 3), [n] "s"(n)
+        : CI_STEP_CLOBBERS, "scc", "s22");
+    return e;
 }
 
 }  // namespace ci

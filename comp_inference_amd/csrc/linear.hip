@@ -119,8 +119,6 @@ __global__ __launch_bounds__(kLinMaxWaves *kWave) void fused_linear32_kernel(Lin
     const int nthreads = blockDim.x;
     uint8_t *stage = lds + kSlotTableBytes + (size_t)wave * kFastStageBytes;
 
-    build_slot_table_x8(tab, a.tables, a.slot_map, tid, nthreads);
-
     const uint32_t kidx = wave % a.kw, nidx = wave / a.kw;
     const uint32_t tk = blockIdx.y * a.kw + kidx, tn = blockIdx.x * a.nw + nidx;
     const bool have_tile = tk < a.tiles_k && tn < a.tiles_n;
@@ -130,6 +128,7 @@ __global__ __launch_bounds__(kLinMaxWaves *kWave) void fused_linear32_kernel(Lin
     uint32_t depth = 0, my_steps = 0;
     uint64_t base = 0;
     bool fast = false;
+    StageRegs body;
     if (have_tile) {
         base = a.tile_offsets[tile];
         depth = a.tile_max_lens[tile];
@@ -140,7 +139,16 @@ __global__ __launch_bounds__(kLinMaxWaves *kWave) void fused_linear32_kernel(Lin
         // number of 8-row blocks, 16-byte readable x rows and a dword-aligned sign|mantissa plane
         fast = full && a.fast_ok && depth >= 2 && depth < kFastStride && half % 16 == 0 &&
                (uint32_t)(uintptr_t)tab == 0;
-        if (fast) stage_transposed(stage, a.stream + base, depth, lane);
+        if (fast) stage_fetch(body, a.stream + base, 0, depth, lane);
+    }
+    build_slot_table_x8(tab, a.tables, a.slot_map, tid, nthreads);  // runs under the body loads
+    if (fast) {
+        stage_commit(body, stage, 0, depth, lane);
+        for (int grp = 1; grp < kStageGroups; ++grp)
+            if ((uint32_t)grp * 128 < depth) {
+                stage_fetch(body, a.stream + base, grp * 128, depth, lane);
+                stage_commit(body, stage, grp * 128, depth, lane);
+            }
     }
     __syncthreads();
 
