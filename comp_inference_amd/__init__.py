@@ -36,3 +36,23 @@ from .rans_hip import (
     rans_decomp_triton,
     rans_decomp_triton_tiled,
 )
+from .transposed_linear_hip import (
+    fused_rans_linear_transposed,
+    fused_rans_linear_transposed_triton,
+    fused_rans_linear_transposed_triton_uncoalesced,
+    fused_rans_linear_transposed_uncoalesced,
+)
+from .pytorch_runtime import (
+    RansEmbedding,
+    RansLinear,
+    RansLMHead,
+    RansWorkspace,
+    load_compressed_model_with_auto_model,
+    swap_in_rans_modules,
+)
+from .rans_saving import (
+    pack_and_save_tensors,
+    parse_rans_info,
+    rans_tensors_for_module,
+    save_rans_model_package,
+)

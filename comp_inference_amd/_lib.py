@@ -35,6 +35,7 @@ def lib() -> C.CDLL:
         _lib.ci_encode_scratch_bytes.restype = C.c_size_t
         _lib.ci_fused_linear_workspace_bytes.restype = C.c_size_t
         _lib.ci_fused_embedding_workspace_bytes.restype = C.c_size_t
+        _lib.ci_fused_linear_transposed_workspace_bytes.restype = C.c_size_t
     return _lib
 
 

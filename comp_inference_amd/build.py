@@ -13,7 +13,7 @@ import sys
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libcomp_inference_hip.so")
-SOURCES = ["api.hip", "encode.hip", "decode.hip", "linear.hip", "embedding.hip", "legacy.hip"]
+SOURCES = ["api.hip", "encode.hip", "decode.hip", "linear.hip", "embedding.hip", "transposed.hip", "legacy.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",

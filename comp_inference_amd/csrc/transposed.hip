@@ -1,0 +1,309 @@
+// Fused decompress + linear against a weight stored row-per-output ("transposed", the layout of
+// an embedding table reused as LM head) on gfx950.
+//
+// out[M, V] = x[M, H] * W^T with W tiled as [V rows, H columns].  Replaces
+// fused_rans_linear_transposed_triton / fused_rans_matmul_transposed_kernel_ilp2_splitk
+// (comp_inference/transposed_linear_triton.py:187-435) and the dense variant (:660-883).
+//
+// The reference gives every 64 output rows their own program, which first discards all decode
+// steps above its rows.  Here one wavefront walks one tile exactly once: at step i lane (half, c)
+// holds W[v_i, c]; the products with x[m, c] are summed over the 32 lanes of the half with a DPP
+// reduction and lane 31 / 63 writes the partial sum of output row v_i for this column tile.
+// Partials go to a workspace [tiles_n][M][V] (fp32) and are summed in tile order by the split-K
+// reduction kernel, so the result does not depend on scheduling.
+#include "ci_common.h"
+#include "rans_device.h"
+#include "fast_tile.h"
+
+namespace ci {
+
+constexpr int kTrWaves = 8;
+constexpr int kTrRows = 4;  // rows of x handled per pass
+
+struct TransArgs {
+    const uint16_t *x;
+    uint32_t M, H, V, x_stride;  // M = rows of this pass (<= kTrRows)
+    const uint8_t *stream;
+    uint64_t stream_len;
+    const uint32_t *states;
+    const uint32_t *tables;
+    const uint8_t *slot_map;
+    const uint32_t *tile_offsets;
+    const uint32_t *tile_max_lens;
+    const uint32_t *stream_offsets;  // dense layout
+    const uint32_t *stream_sizes;    // dense layout
+    const uint8_t *man_tiled;
+    float *partial;  // [P][M][V]
+    uint32_t th, tw, tiles_n, tiles_k, num_tiles;
+};
+
+template <int kCtrl>
+__device__ __forceinline__ float dpp_add(float v) {
+    const int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(v), kCtrl, 0xF, 0xF, false);
+    return v + __int_as_float(moved);
+}
+
+// Sum over each group of 32 lanes; the total is valid in lane 31 of the group.
+__device__ __forceinline__ float sum32_to_last_lane(float v) {
+    v = dpp_add<0xB1>(v);   // quad_perm [1,0,3,2]
+    v = dpp_add<0x4E>(v);   // quad_perm [2,3,0,1]
+    v = dpp_add<0x141>(v);  // row_half_mirror
+    v = dpp_add<0x140>(v);  // row_mirror: every lane of a 16-lane row holds the row total
+    // row_bcast15: lane 15 of each row is added into the following row (rows 1 and 3 complete a group)
+    const int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x142, 0xA, 0xF, false);
+    return v + __int_as_float(moved);
+}
+
+__device__ __forceinline__ float weight_f32(uint32_t sym, uint32_t man) {
+    return __uint_as_float(((man & 0x80u) << 24) | (sym << 23) | ((man & 0x7Fu) << 16));
+}
+
+// grid: ceil(num_tiles / kTrWaves); one wave per tile
+template <int MB>
+__global__ __launch_bounds__(kTrWaves *kWave) void trans32_kernel(TransArgs a) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    uint2 *tab = reinterpret_cast<uint2 *>(lds);
+    const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
+    uint8_t *stage = lds + kSlotTableBytes + (size_t)wave * kFastStageBytes;
+
+    const uint32_t tile = blockIdx.x * kTrWaves + wave;
+    const bool have_tile = tile < a.num_tiles;
+    const uint32_t tk = have_tile ? tile / a.tiles_n : 0, tn = have_tile ? tile % a.tiles_n : 0;
+    const uint32_t half = a.th / 2, hsel = lane / 32, c = lane % 32;
+    const uint32_t v0 = tk * a.th + hsel * half, h = tn * 32 + c;
+    uint32_t depth = 0, my_steps = 0;
+    uint64_t base = 0;
+    bool fast = false;
+    StageRegs body;
+    if (have_tile) {
+        base = a.tile_offsets[tile];
+        depth = a.tile_max_lens[tile];
+        if (base + (uint64_t)depth * 64 > a.stream_len) depth = 0;
+        if (v0 < a.V) my_steps = min(half, a.V - v0);  // rows of this lane's half (same for its 32 lanes)
+        const bool full = __builtin_amdgcn_ballot_w64(my_steps != half || h >= a.H) == 0;
+        fast = full && depth >= 2 && depth < kFastStride && (uint32_t)(uintptr_t)tab == 0;
+        if (fast) stage_fetch(body, a.stream + base, 0, depth, lane);
+    }
+    build_slot_table_x8(tab, a.tables, a.slot_map, tid, kTrWaves * kWave);
+    if (fast) {
+        stage_commit(body, stage, 0, depth, lane);
+        for (int grp = 1; grp < kStageGroups; ++grp)
+            if ((uint32_t)grp * 128 < depth) {
+                stage_fetch(body, a.stream + base, grp * 128, depth, lane);
+                stage_commit(body, stage, grp * 128, depth, lane);
+            }
+    }
+    __syncthreads();
+    if (!have_tile) return;
+
+    float xs[MB];
+#pragma unroll
+    for (int m = 0; m < MB; ++m)
+        xs[m] = (m < (int)a.M && h < a.H) ? __uint_as_float((uint32_t)a.x[(size_t)m * a.x_stride + h] << 16) : 0.f;
+    const uint8_t *man = a.man_tiled + (size_t)tile * a.th * 32 + (size_t)hsel * half * 32 + c;
+    float *dst = a.partial + (size_t)tn * a.M * a.V + v0;  // + m * V + i
+    const uint32_t state = a.states[(size_t)tile * 64 + lane];
+    // In the last k-tile the bottom half has fewer rows than the top half: the wave runs to the
+    // top half's count, lanes past their own count (or past the last column) contribute zero.
+    const uint32_t n_wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)my_steps);
+    const bool writer = c == 31, col_ok = h < a.H;
+
+    auto emit = [&](uint32_t i, uint32_t sym, bool live) {
+        const float w = live ? weight_f32(sym, man[(size_t)i * 32]) : 0.f;
+#pragma unroll
+        for (int m = 0; m < MB; ++m) {
+            const float s = sum32_to_last_lane(w * xs[m]);
+            if (writer && m < (int)a.M && i < my_steps) dst[(size_t)m * a.V + i] = s;
+        }
+    };
+
+    if (fast) {
+        FastLane st;
+        st.init(stage, depth, lane, state);
+        for (uint32_t i = 0; i < half; ++i) emit(i, advance_asm(st, 1) >> 24, true);
+    } else {
+        GlobalBytes src;
+        src.init(a.stream + base, depth, 64, lane);
+        uint32_t X = state << 3;
+        for (uint32_t i = 0; i < n_wave; ++i) {
+            uint32_t sym = 0;
+            const bool live = col_ok && i < my_steps;
+            if (live) {
+                sym = decode_symbol_scaled(X, tab) >> 24;
+                src.renorm_scaled(X);
+                src.renorm_scaled(X);
+            }
+            emit(i, sym, live);
+        }
+    }
+}
+
+// Any tile width and the dense layout: one thread per (tile, half): it decodes the tile's columns
+// one after the other and accumulates their products into its own rows of the tile's partial, so
+// the summation order is fixed.  Slow; kept for format coverage.
+template <bool kDense>
+__global__ __launch_bounds__(256) void trans_generic_kernel(TransArgs a) {
+    __shared__ uint2 tab[kProbScale];
+    build_slot_table(tab, a.tables, a.slot_map, threadIdx.x, 256);
+    __syncthreads();
+    const uint32_t spt = kDense ? 1u : 2u;
+    const uint64_t id = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (id >= (uint64_t)a.num_tiles * spt) return;
+    const uint32_t tile = (uint32_t)(id / spt), hsel = (uint32_t)(id % spt);
+    const uint32_t tk = tile / a.tiles_n, tn = tile % a.tiles_n;
+    const uint32_t span = kDense ? a.th : a.th / 2, v0 = tk * a.th + hsel * span;
+    if (v0 >= a.V) return;
+    const uint32_t rows = min(span, a.V - v0);
+    float *dst = a.partial + (size_t)tn * a.M * a.V + v0;
+    for (uint32_t m = 0; m < a.M; ++m)
+        for (uint32_t i = 0; i < rows; ++i) dst[(size_t)m * a.V + i] = 0.f;
+    for (uint32_t c = 0; c < a.tw; ++c) {  // columns of the tile in order: a fixed summation order
+        const uint32_t h = tn * a.tw + c;
+        if (h >= a.H) break;
+        const uint8_t *man = a.man_tiled + (size_t)tile * a.th * a.tw + (size_t)hsel * span * a.tw + c;
+        uint32_t x;
+        auto run = [&](auto &src) {
+            for (uint32_t i = 0; i < rows; ++i) {
+                const uint32_t sym = decode_symbol(x, tab) >> 24;
+                src.renorm(x);
+                src.renorm(x);
+                const float w = weight_f32(sym, man[(size_t)i * a.tw]);
+                for (uint32_t m = 0; m < a.M; ++m)
+                    dst[(size_t)m * a.V + i] += w * __uint_as_float((uint32_t)a.x[(size_t)m * a.x_stride + h] << 16);
+            }
+        };
+        if (kDense) {
+            const uint32_t sid = tile * a.tw + c;
+            x = a.states[sid];
+            const uint64_t off = a.stream_offsets[sid];
+            uint32_t size = a.stream_sizes[sid];
+            if (off + size > a.stream_len) size = 0;
+            DenseBytes src;
+            src.init(a.stream + off, size);
+            run(src);
+        } else {
+            const uint32_t q = hsel * a.tw + c;
+            x = a.states[(size_t)tile * 2 * a.tw + q];
+            uint64_t base = a.tile_offsets[tile];
+            uint32_t depth = a.tile_max_lens[tile];
+            if (base + (uint64_t)depth * 2 * a.tw > a.stream_len) depth = 0;
+            GlobalBytes src;
+            src.init(a.stream + base, depth, 2 * a.tw, q);
+            run(src);
+        }
+    }
+}
+
+}  // namespace ci
+
+using namespace ci;
+
+extern "C" size_t ci_fused_linear_transposed_workspace_bytes(uint32_t M, uint32_t H, uint32_t V,
+                                                             uint32_t tile_width) {
+    if (tile_width == 0) return 0;
+    const uint32_t rows = M < (uint32_t)kTrRows ? M : (uint32_t)kTrRows;
+    return (size_t)ceil_div(H, tile_width) * rows * V * sizeof(float);
+}
+
+static int transposed_impl(const uint16_t *d_x, uint32_t M, uint32_t H, uint32_t V, uint32_t x_stride,
+                           const uint8_t *d_stream, uint64_t stream_len, const uint32_t *d_states,
+                           const uint32_t *d_tables, const uint8_t *d_slot_map, const uint32_t *d_meta0,
+                           const uint32_t *d_meta1, const uint8_t *d_man_tiled, uint32_t th, uint32_t tw,
+                           const uint16_t *d_bias, uint16_t *d_out, uint32_t out_stride, void *d_workspace,
+                           size_t workspace_bytes, bool dense, ci_stream_t stream) {
+    if (M == 0 || V == 0) return CI_OK;
+    if (H == 0) return fail(CI_ERR_ARG, "transposed linear: hidden size is 0");
+    if (!d_x || !d_states || !d_tables || !d_slot_map || !d_meta0 || !d_meta1 || !d_man_tiled || !d_out)
+        return fail(CI_ERR_ARG, "transposed linear: null pointer");
+    if (stream_len && !d_stream) return fail(CI_ERR_ARG, "transposed linear: null stream");
+    if (th == 0 || tw == 0 || (!dense && (th & 1))) return fail(CI_ERR_ARG, "transposed linear: bad tile shape");
+    if (x_stride < H || out_stride < V) return fail(CI_ERR_ARG, "transposed linear: row stride shorter than the row");
+    if (!aligned(d_slot_map, 4)) return fail(CI_ERR_ARG, "transposed linear: slot_map must be 4-byte aligned");
+    const size_t need = ci_fused_linear_transposed_workspace_bytes(M, H, V, tw);
+    if (!d_workspace || workspace_bytes < need)
+        return fail(CI_ERR_CAPACITY, "transposed linear: workspace needs %zu bytes, got %zu", need, workspace_bytes);
+    if (!aligned(d_workspace, 4)) return fail(CI_ERR_ARG, "transposed linear: workspace must be 4-byte aligned");
+
+    TransArgs a;
+    a.H = H;
+    a.V = V;
+    a.x_stride = x_stride;
+    a.stream = d_stream;
+    a.stream_len = stream_len;
+    a.states = d_states;
+    a.tables = d_tables;
+    a.slot_map = d_slot_map;
+    a.tile_offsets = dense ? nullptr : d_meta0;
+    a.tile_max_lens = dense ? nullptr : d_meta1;
+    a.stream_offsets = dense ? d_meta0 : nullptr;
+    a.stream_sizes = dense ? d_meta1 : nullptr;
+    a.man_tiled = d_man_tiled;
+    a.partial = static_cast<float *>(d_workspace);
+    a.th = th;
+    a.tw = tw;
+    a.tiles_n = ceil_div(H, tw);  // column tiles run along the hidden dimension
+    a.tiles_k = ceil_div(V, th);
+    a.num_tiles = a.tiles_n * a.tiles_k;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const bool fast = !dense && tw == 32 && aligned(d_stream, 16);
+    static bool attr_set = false;
+    if (fast && !attr_set) {
+        CI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(trans32_kernel<1>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit));
+        CI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(trans32_kernel<kTrRows>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit));
+        attr_set = true;
+    }
+    // passes of kTrRows rows of x reuse the workspace one after another on the stream
+    for (uint32_t m0 = 0; m0 < M; m0 += kTrRows) {
+        a.x = d_x + (size_t)m0 * x_stride;
+        a.M = M - m0 < (uint32_t)kTrRows ? M - m0 : (uint32_t)kTrRows;
+        if (fast) {
+            const uint32_t lds_bytes = kSlotTableBytes + kTrWaves * kFastStageBytes;
+            const dim3 grid(ceil_div(a.num_tiles, kTrWaves)), block(kTrWaves * kWave);
+            if (a.M == 1)
+                hipLaunchKernelGGL(trans32_kernel<1>, grid, block, lds_bytes, s, a);
+            else
+                hipLaunchKernelGGL(trans32_kernel<kTrRows>, grid, block, lds_bytes, s, a);
+            CI_LAUNCH_CHECK("trans32_kernel");
+        } else {
+            const uint64_t threads = (uint64_t)a.num_tiles * (dense ? 1 : 2);
+            const dim3 grid((uint32_t)((threads + 255) / 256)), block(256);
+            if (dense)
+                hipLaunchKernelGGL(trans_generic_kernel<true>, grid, block, 0, s, a);
+            else
+                hipLaunchKernelGGL(trans_generic_kernel<false>, grid, block, 0, s, a);
+            CI_LAUNCH_CHECK("trans_generic_kernel");
+        }
+        int rc = ci_splitk_reduce(a.partial, 0, a.tiles_n, a.M, V, d_bias, d_out + (size_t)m0 * out_stride, out_stride,
+                                  stream);
+        if (rc) return rc;
+    }
+    return CI_OK;
+}
+
+extern "C" int ci_fused_linear_transposed_ilp2(const uint16_t *d_x, uint32_t M, uint32_t H, uint32_t V,
+                                               uint32_t x_stride, const uint8_t *d_stream, uint64_t stream_len,
+                                               const uint32_t *d_states, const uint32_t *d_tables,
+                                               const uint8_t *d_slot_map, const uint32_t *d_tile_offsets,
+                                               const uint32_t *d_tile_max_lens, const uint8_t *d_man_tiled,
+                                               uint32_t tile_height, uint32_t tile_width, const uint16_t *d_bias,
+                                               uint16_t *d_out, uint32_t out_stride, void *d_workspace,
+                                               size_t workspace_bytes, ci_stream_t stream) {
+    return transposed_impl(d_x, M, H, V, x_stride, d_stream, stream_len, d_states, d_tables, d_slot_map,
+                           d_tile_offsets, d_tile_max_lens, d_man_tiled, tile_height, tile_width, d_bias, d_out,
+                           out_stride, d_workspace, workspace_bytes, false, stream);
+}
+
+extern "C" int ci_fused_linear_transposed_dense(const uint16_t *d_x, uint32_t M, uint32_t H, uint32_t V,
+                                                uint32_t x_stride, const uint8_t *d_stream, uint64_t stream_len,
+                                                const uint32_t *d_states, const uint32_t *d_tables,
+                                                const uint8_t *d_slot_map, const uint32_t *d_stream_offsets,
+                                                const uint32_t *d_stream_sizes, const uint8_t *d_man_tiled,
+                                                uint32_t tile_height, uint32_t tile_width, const uint16_t *d_bias,
+                                                uint16_t *d_out, uint32_t out_stride, void *d_workspace,
+                                                size_t workspace_bytes, ci_stream_t stream) {
+    return transposed_impl(d_x, M, H, V, x_stride, d_stream, stream_len, d_states, d_tables, d_slot_map,
+                           d_stream_offsets, d_stream_sizes, d_man_tiled, tile_height, tile_width, d_bias, d_out,
+                           out_stride, d_workspace, workspace_bytes, true, stream);
+}

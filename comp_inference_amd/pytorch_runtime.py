@@ -1,0 +1,236 @@
+"""Inference modules that keep their weights compressed, mirroring
+comp_inference/pytorch_runtime.py:386-642 of the reference: `RansWorkspace`, `RansLinear`,
+`RansLMHead`, `RansEmbedding` (same constructor arguments and buffer names/dtypes, so a package
+written by the reference loads by key) and the model loader.
+"""
+from __future__ import annotations
+
+import json
+import os
+
+import torch
+import torch.nn as nn
+
+from .embedding_hip import fused_rans_embedding
+from .linear_hip import fused_rans_linear
+from .transposed_linear_hip import fused_rans_linear_transposed
+
+
+class RansWorkspace:
+    """Grow-only split-K workspace shared by all layers (comp_inference/pytorch_runtime.py:386-394)."""
+    _buffer = None
+
+    @classmethod
+    def get_workspace(cls, M, N, split_k, device):
+        elements = M * N * split_k
+        if cls._buffer is None or cls._buffer.numel() < elements or cls._buffer.device != torch.device(device):
+            cls._buffer = torch.zeros(elements * 2, device=device, dtype=torch.bfloat16)
+        return cls._buffer[:elements].view(split_k, M, N)
+
+
+def _register_rans_buffers(mod: nn.Module) -> None:
+    # names and dtypes as comp_inference/pytorch_runtime.py:413-424; the slot map is stored as
+    # uint8 in every package (comp_inference/rans_saving.py:406-408) and arrives as such
+    mod.register_buffer("rans_exp_stream", torch.empty(0, dtype=torch.uint8))
+    mod.register_buffer("rans_exp_states", torch.empty(0, dtype=torch.uint32))
+    mod.register_buffer("rans_exp_tables", torch.empty(0, dtype=torch.uint32))
+    mod.register_buffer("rans_exp_slot_map", torch.empty(0, dtype=torch.uint16))
+    mod.register_buffer("rans_exp_tile_offsets", torch.empty(0, dtype=torch.uint32))
+    mod.register_buffer("rans_exp_tile_max_lens", torch.empty(0, dtype=torch.uint32))
+    mod.register_buffer("rans_man_raw", torch.empty(0, dtype=torch.uint8))
+    mod.register_buffer("rans_info", torch.empty(0, dtype=torch.int32))
+
+
+def _load_from_compressed(mod: nn.Module, src: nn.Module) -> None:
+    """Fill the buffers from a module compressed with rans_compress_module_weight."""
+    if getattr(src, "exponent_uncoalesced_interleaving", False):
+        raise ValueError("the runtime modules take the default (tile-interleaved) format")
+    mod.rans_exp_stream = src.exponent_compressed_weight.clone()
+    mod.rans_exp_states = src.exponent_states.clone()
+    mod.rans_exp_tables = src.exponent_tables.clone()
+    mod.rans_exp_slot_map = src.exponent_slot_map.clone()
+    mod.rans_exp_tile_offsets = src.exponent_tile_offsets.clone()
+    mod.rans_exp_tile_max_lens = src.exponent_tile_max_lens.clone()
+    mod.rans_man_raw = src.mantissa_raw.clone()
+    mod.tile_k, mod.tile_n = int(src.exponent_tile_height), int(src.exponent_tile_width)
+
+
+class RansLinear(nn.Module):
+    """comp_inference/pytorch_runtime.py:397-459.  Weight stored as [K=in, N=out]."""
+
+    def __init__(self, in_features: int, out_features: int, tile_k: int = 1024, tile_n: int = 32,
+                 split_k: int = 1, has_bias: bool = False):
+        super().__init__()
+        self.in_features, self.out_features = in_features, out_features
+        self.tile_k, self.tile_n, self.split_k = tile_k, tile_n, split_k
+        _register_rans_buffers(self)
+        if has_bias:
+            self.register_buffer("bias", torch.empty(out_features, dtype=torch.bfloat16))
+        else:
+            self.bias = None
+
+    @classmethod
+    def from_compressed(cls, src: nn.Module, bias=None, split_k: int = 1) -> "RansLinear":
+        K, N = src.input_shape
+        mod = cls(K, N, split_k=split_k, has_bias=bias is not None)
+        _load_from_compressed(mod, src)
+        if bias is not None:
+            mod.bias = bias.detach().to(torch.bfloat16).clone()
+        return mod
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        device = x.device
+        return fused_rans_linear(
+            x=x,
+            compressed_data=self.rans_exp_stream.to(device, non_blocking=True),
+            initial_states=self.rans_exp_states.to(device, non_blocking=True),
+            tables=self.rans_exp_tables.to(device, non_blocking=True),
+            slot_map=self.rans_exp_slot_map.to(device, non_blocking=True),
+            weight_shape=(self.in_features, self.out_features),
+            tile_offsets=self.rans_exp_tile_offsets.to(device, non_blocking=True),
+            tile_max_lens=self.rans_exp_tile_max_lens.to(device, non_blocking=True),
+            tile_k=self.tile_k, tile_n=self.tile_n,
+            mantissas=self.rans_man_raw.to(device, non_blocking=True),
+            SPLIT_K=self.split_k,
+            bias=self.bias.to(device, non_blocking=True) if self.bias is not None else None)
+
+
+class RansLMHead(nn.Module):
+    """comp_inference/pytorch_runtime.py:462-505.  Weight stored as [out=vocab, in=hidden]: the
+    embedding table's layout, so a tied head shares the table's buffers."""
+
+    def __init__(self, in_features: int, out_features: int, tile_k: int = 1024, tile_n: int = 32):
+        super().__init__()
+        self.in_features, self.out_features = in_features, out_features
+        self.tile_k, self.tile_n = tile_k, tile_n
+        _register_rans_buffers(self)
+
+    @classmethod
+    def from_compressed(cls, src: nn.Module) -> "RansLMHead":
+        V, H = src.input_shape
+        mod = cls(H, V)
+        _load_from_compressed(mod, src)
+        return mod
+
+    def tie_to(self, emb: "RansEmbedding") -> None:
+        for name in ("rans_exp_stream", "rans_exp_states", "rans_exp_tables", "rans_exp_slot_map",
+                     "rans_exp_tile_offsets", "rans_exp_tile_max_lens", "rans_man_raw", "rans_info"):
+            setattr(self, name, getattr(emb, name))
+        self.tile_k, self.tile_n = emb.tile_k, emb.tile_n
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        device = x.device
+        return fused_rans_linear_transposed(
+            x=x,
+            compressed_data=self.rans_exp_stream.to(device, non_blocking=True),
+            initial_states=self.rans_exp_states.to(device, non_blocking=True),
+            tables=self.rans_exp_tables.to(device, non_blocking=True),
+            slot_map=self.rans_exp_slot_map.to(device, non_blocking=True),
+            weight_shape=(self.out_features, self.in_features),
+            tile_offsets=self.rans_exp_tile_offsets.to(device, non_blocking=True),
+            tile_max_lens=self.rans_exp_tile_max_lens.to(device, non_blocking=True),
+            tile_n=self.tile_n, tile_k=self.tile_k,
+            mantissas=self.rans_man_raw.to(device, non_blocking=True),
+            workspace=None, SPLIT_K=1, bias=None)
+
+
+class RansEmbedding(nn.Module):
+    """comp_inference/pytorch_runtime.py:508-549.  Table stored as [vocab, dim], not transposed."""
+
+    def __init__(self, num_embeddings: int, embedding_dim: int, tile_k: int = 1024, tile_n: int = 32):
+        super().__init__()
+        self.num_embeddings, self.embedding_dim = num_embeddings, embedding_dim
+        self.tile_k, self.tile_n = tile_k, tile_n
+        _register_rans_buffers(self)
+
+    @classmethod
+    def from_compressed(cls, src: nn.Module) -> "RansEmbedding":
+        V, H = src.input_shape
+        mod = cls(V, H)
+        _load_from_compressed(mod, src)
+        return mod
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        device = x.device
+        return fused_rans_embedding(
+            x=x,
+            compressed_data=self.rans_exp_stream.to(device, non_blocking=True),
+            initial_states=self.rans_exp_states.to(device, non_blocking=True),
+            tables=self.rans_exp_tables.to(device, non_blocking=True),
+            slot_map=self.rans_exp_slot_map.to(device, non_blocking=True),
+            weight_shape=(self.num_embeddings, self.embedding_dim),
+            tile_offsets=self.rans_exp_tile_offsets.to(device, non_blocking=True),
+            tile_max_lens=self.rans_exp_tile_max_lens.to(device, non_blocking=True),
+            tile_k=self.tile_k, tile_n=self.tile_n,
+            mantissas=self.rans_man_raw.to(device, non_blocking=True))
+
+
+def swap_in_rans_modules(model: nn.Module, state_dict: dict, quant_config: dict | None = None,
+                         split_k: int = 1) -> nn.Module:
+    """Replace every nn.Linear / nn.Embedding / lm_head whose `<name>.rans_exp_stream` key exists in
+    `state_dict` by its compressed counterpart and assign all matching tensors
+    (comp_inference/pytorch_runtime.py:563-637).  Works on any already constructed model, so no
+    network access is needed."""
+    quant_config = quant_config or {}
+    layer_configs = quant_config.get("layer_configs", {})
+    default_th = quant_config.get("default_tile_height", 1024)
+    default_tw = quant_config.get("default_tile_width", 32)
+
+    def tile_of(name):
+        cfg = layer_configs.get(name, {})
+        return cfg.get("tile_height", default_th), cfg.get("tile_width", default_tw)
+
+    replacements = []
+    for name, module in model.named_modules():
+        if "lm_head" in name or isinstance(module, (RansLinear, RansEmbedding, RansLMHead)):
+            continue
+        if f"{name}.rans_exp_stream" not in state_dict:
+            continue
+        th, tw = tile_of(name)
+        if isinstance(module, nn.Linear):
+            replacements.append((name, RansLinear(module.in_features, module.out_features, th, tw, split_k,
+                                                  module.bias is not None)))
+        elif isinstance(module, nn.Embedding):
+            replacements.append((name, RansEmbedding(module.num_embeddings, module.embedding_dim, th, tw)))
+    for name, new_layer in replacements:
+        parent_name, _, child = name.rpartition(".")
+        parent = model.get_submodule(parent_name) if parent_name else model
+        setattr(parent, child, new_layer)
+    if hasattr(model, "lm_head") and "lm_head.rans_exp_stream" in state_dict:
+        th, tw = tile_of("lm_head")
+        model.lm_head = RansLMHead(model.lm_head.in_features, model.lm_head.out_features, tile_k=th, tile_n=tw)
+
+    targets = dict(model.named_buffers())
+    targets.update(dict(model.named_parameters()))
+    for name, tensor in targets.items():
+        if name in state_dict:
+            tensor.data = state_dict[name].contiguous()
+    return model
+
+
+def load_compressed_model_with_auto_model(model_id: str, safetensors_path: str, split_k: int = 1,
+                                          compile_model: bool = False, model: nn.Module | None = None):
+    """comp_inference/pytorch_runtime.py:552-642.  `model_id` may be a local directory holding
+    config.json (the model is then built from the config alone, no download); pass `model` to
+    swap modules in a model built elsewhere."""
+    from safetensors.torch import load_file
+
+    quant_config = {}
+    if model is None:
+        from transformers import AutoConfig, AutoModelForCausalLM
+
+        if os.path.isdir(model_id):
+            config = AutoConfig.from_pretrained(model_id)
+            model = AutoModelForCausalLM.from_config(config, torch_dtype=torch.bfloat16)
+        else:
+            model = AutoModelForCausalLM.from_pretrained(model_id, torch_dtype=torch.bfloat16)
+        quant_config = getattr(model.config, "quantization_config", {}) or {}
+        if not isinstance(quant_config, dict):
+            quant_config = quant_config.to_dict()
+    else:
+        cfg_path = os.path.join(os.path.dirname(safetensors_path), "config.json")
+        if os.path.exists(cfg_path):
+            quant_config = json.load(open(cfg_path)).get("quantization_config", {})
+    state_dict = load_file(safetensors_path, device="cpu")
+    model = swap_in_rans_modules(model, state_dict, quant_config, split_k)
+    return model.cuda()

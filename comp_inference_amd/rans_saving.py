@@ -1,0 +1,123 @@
+"""safetensors package of a compressed model: tensor names, dtypes and the `rans_info` record of
+comp_inference/rans_saving.py:352-481, the `quantization_config` block of :19-109, the file-level
+metadata of :238-242.
+"""
+from __future__ import annotations
+
+import json
+import os
+
+import torch
+from safetensors.torch import save_file
+
+RANS_INFO_FIELDS = ("version", "numel", "exp_compressed", "exp_streams", "man_compressed", "man_streams",
+                    "rank", "num_tiles_n", "num_tiles_k", "tile_height", "tile_width")
+
+
+def _cpu(t: torch.Tensor, dtype) -> torch.Tensor:
+    t = t.detach().cpu()
+    if t.dtype != dtype:
+        t = t.to(torch.int64).to(dtype) if dtype == torch.uint32 else t.to(dtype)
+    return t.contiguous()
+
+
+def rans_tensors_for_module(base_name: str, module) -> dict:
+    """Tensors of one compressed module under `<base_name>rans_*` keys
+    (comp_inference/rans_saving.py:352-481); base_name ends with '.'."""
+    out = {}
+    p = base_name
+    out[p + "rans_exp_stream"] = _cpu(module.exponent_compressed_weight, torch.uint8)
+    out[p + "rans_exp_states"] = _cpu(module.exponent_states, torch.uint32)
+    out[p + "rans_exp_tables"] = _cpu(module.exponent_tables, torch.uint32)
+    out[p + "rans_exp_slot_map"] = _cpu(module.exponent_slot_map, torch.uint8)
+    if getattr(module, "exponent_uncoalesced_interleaving", False):
+        out[p + "rans_exp_stream_offsets"] = _cpu(module.exponent_stream_offsets, torch.uint32)
+    else:
+        out[p + "rans_exp_tile_offsets"] = _cpu(module.exponent_tile_offsets, torch.uint32)
+        out[p + "rans_exp_tile_max_lens"] = _cpu(module.exponent_tile_max_lens, torch.uint32)
+    out[p + "rans_man_raw"] = _cpu(module.mantissa_raw, torch.uint8)
+    shape = list(getattr(module, "input_shape", [module.expanded_size]))
+    info = [1, module.expanded_size, 1, module.exponent_num_streams, 0, 0, len(shape),
+            module.exponent_num_tiles_n, module.exponent_num_tiles_k, module.exponent_tile_height,
+            module.exponent_tile_width] + shape
+    out[p + "rans_info"] = torch.tensor(info, dtype=torch.int32)
+    bias = getattr(module, "bias", None)
+    if bias is not None:
+        out[p + "bias"] = bias.detach().cpu()
+    return out
+
+
+def parse_rans_info(info: torch.Tensor) -> dict:
+    vals = [int(v) for v in info.tolist()]
+    d = dict(zip(RANS_INFO_FIELDS, vals))
+    d["shape"] = vals[len(RANS_INFO_FIELDS):len(RANS_INFO_FIELDS) + d["rank"]]
+    return d
+
+
+def collect_tensors(model, tied_lm_head: bool = False) -> dict:
+    tensors, handled = {}, set()
+    if tied_lm_head:
+        handled.update({"lm_head.weight", "model.lm_head.weight"})
+    for name, module in model.named_modules():
+        if getattr(module, "compressed", None) == "rans_bfloat16":
+            if tied_lm_head and "lm_head" in name:
+                continue
+            tensors.update(rans_tensors_for_module(name + ".", module))
+            handled.update({f"{name}.weight", f"{name}.bias"})
+    for pname, param in model.named_parameters():
+        if pname not in handled:
+            tensors[pname] = param.data.cpu().contiguous()
+    return tensors
+
+
+def pack_and_save_tensors(model, output_path: str, fuse: bool = False, tied_lm_head: bool = False):
+    """comp_inference/rans_saving.py:177-245."""
+    tensors = collect_tensors(model, tied_lm_head)
+    metadata = {"format": "pt", "compression_method": "rans_bfloat16", "fused_projections": str(fuse)}
+    save_file(tensors, output_path, metadata=metadata)
+    return tensors
+
+
+def quantization_config_for(model, fuse: bool = False, tied_lm_head: bool = False) -> dict:
+    """comp_inference/rans_saving.py:33-98."""
+    layer_configs = {}
+    for name, module in model.named_modules():
+        if tied_lm_head and "lm_head" in name:
+            continue
+        if getattr(module, "compressed", None) != "rans_bfloat16":
+            continue
+        if fuse:
+            if "gate_proj" in name:
+                name = name.replace("gate_proj", "gate_up_proj")
+            elif "q_proj" in name:
+                name = name.replace("q_proj", "qkv_proj")
+        layer_configs[name] = {
+            "tile_height": int(getattr(module, "exponent_tile_height", 1024)),
+            "tile_width": int(getattr(module, "exponent_tile_width", 32)),
+            "uncoalesced_interleaving": bool(getattr(module, "exponent_uncoalesced_interleaving", False)),
+        }
+    return {"quant_method": "rans", "compression": "rans_bfloat16", "layer_configs": layer_configs,
+            "default_tile_height": 1024, "default_tile_width": 32, "fused_projections": fuse}
+
+
+def save_rans_model_package(model, tokenizer, output_dir: str, fuse: bool = False, tied_lm_head: bool = False):
+    """config.json (+ tokenizer) + model.safetensors (comp_inference/rans_saving.py:19-109).
+    As in the reference, an unfused package goes to `<output_dir>_unfused`."""
+    if not fuse:
+        output_dir = output_dir + "_unfused"
+    os.makedirs(output_dir, exist_ok=True)
+    qc = quantization_config_for(model, fuse, tied_lm_head)
+    config = getattr(model, "config", None)
+    if config is not None and hasattr(config, "save_pretrained"):
+        config.quantization_config = qc
+        config.save_pretrained(output_dir)
+    else:
+        cfg = dict(config) if isinstance(config, dict) else {}
+        cfg["quantization_config"] = qc
+        with open(os.path.join(output_dir, "config.json"), "w") as f:
+            json.dump(cfg, f, indent=2)
+    if tokenizer is not None:
+        tokenizer.save_pretrained(output_dir)
+    path = os.path.join(output_dir, "model.safetensors")
+    pack_and_save_tensors(model, path, fuse=fuse, tied_lm_head=tied_lm_head)
+    return output_dir

@@ -1,0 +1,72 @@
+"""Fused decompress + linear against a row-per-output weight (LM head sharing the embedding
+table's layout).  Call signatures follow comp_inference/transposed_linear_triton.py:361-377
+(`fused_rans_linear_transposed_triton`) and :813-829 (`..._uncoalesced`); the kernels are HIP
+(csrc/transposed.hip).
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+import torch
+
+from . import _lib
+from ._lib import check, lib, ptr
+from .linear_hip import _Scratch, _prep_x
+
+
+def _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, meta0, meta1, tile_k, tile_n,
+         mantissas, bias, out, dense: bool):
+    V, H = int(weight_shape[0]), int(weight_shape[1])  # weight is [vocab, hidden]
+    _lib.require_device(x)
+    dev = x.device
+    x2 = _prep_x(x, H)
+    M = x2.shape[0]
+    if out is None:
+        result = torch.empty((M, V), dtype=torch.bfloat16, device=dev)
+    else:
+        if out.dtype != torch.bfloat16 or not out.is_cuda:
+            raise RuntimeError("out must be a bfloat16 GPU tensor")
+        result = out.view(M, V)
+    stream_t = _lib.as_u8(compressed_data, dev)
+    man = _lib.as_u8(mantissas, dev).view(-1)
+    need_man = (-(-V // tile_k)) * (-(-H // tile_n)) * tile_k * tile_n
+    if man.numel() < need_man:
+        man = torch.nn.functional.pad(man, (0, need_man - man.numel()))
+    need = lib().ci_fused_linear_transposed_workspace_bytes(M, H, V, int(tile_n))
+    ws = _Scratch.get(need, ("lmhead", dev))
+    b = bias.to(device=dev, dtype=torch.bfloat16).contiguous() if bias is not None else None
+    # device copies must stay referenced until the launch has been enqueued
+    st, tb, sm = _lib.as_u32(initial_states, dev), _lib.as_u32(tables, dev), _lib.as_u8(slot_map, dev)
+    m0, m1 = _lib.as_u32(meta0, dev), _lib.as_u32(meta1, dev)
+    fn = lib().ci_fused_linear_transposed_dense if dense else lib().ci_fused_linear_transposed_ilp2
+    check(fn(ptr(x2), M, H, V, x2.stride(0), ptr(stream_t), C.c_uint64(stream_t.numel()), ptr(st), ptr(tb),
+             ptr(sm), ptr(m0), ptr(m1), ptr(man), int(tile_k), int(tile_n), ptr(b), ptr(result),
+             result.stride(0), ptr(ws), C.c_size_t(ws.numel()), _lib.stream_handle(dev)))
+    if out is not None:
+        return out
+    return result.view(*x.shape[:-1], V)
+
+
+def fused_rans_linear_transposed(x, compressed_data, initial_states, tables, slot_map, weight_shape,
+                                 tile_offsets, tile_max_lens, tile_k, tile_n, mantissas, workspace=None,
+                                 bias=None, out=None, SPLIT_K=8):
+    """x[..., H] @ W[V, H]^T (+ bias), W in the tiled two-streams-per-column format
+    (comp_inference/transposed_linear_triton.py:361-435).  `workspace` and `SPLIT_K` are accepted
+    for signature compatibility; the library keeps its own fp32 scratch (one partial per column
+    tile, summed in tile order)."""
+    return _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, tile_offsets, tile_max_lens,
+                tile_k, tile_n, mantissas, bias, out, dense=False)
+
+
+def fused_rans_linear_transposed_uncoalesced(x, compressed_data, initial_states, tables, slot_map, weight_shape,
+                                             stream_offsets, stream_sizes, tile_k, tile_n, mantissas,
+                                             workspace=None, bias=None, out=None, SPLIT_K=8):
+    """Same for the dense one-stream-per-column layout
+    (comp_inference/transposed_linear_triton.py:813-883)."""
+    return _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, stream_offsets, stream_sizes,
+                tile_k, tile_n, mantissas, bias, out, dense=True)
+
+
+# Names under which the reference exports these ops (comp_inference/__init__.py:44-47).
+fused_rans_linear_transposed_triton = fused_rans_linear_transposed
+fused_rans_linear_transposed_triton_uncoalesced = fused_rans_linear_transposed_uncoalesced

@@ -240,6 +240,36 @@ int ci_fused_embedding_dense(const int64_t *d_ids, uint32_t n_ids, const uint8_t
                              uint32_t N, uint32_t tile_height, uint32_t tile_width, uint16_t *d_out,
                              uint32_t out_stride, ci_stream_t stream);
 
+/* ---------------------------------------------------------------------------------------
+ * Fused decompress + linear against a row-per-output weight:  out[M,V] (bf16) = x[M,H] * W^T
+ * (+ bias) with W [V,H] stored like an embedding table (tiles of tile_height rows of V by
+ * tile_width columns of H).  ci_fused_linear_transposed_ilp2 replaces
+ * fused_rans_linear_transposed_triton (comp_inference/transposed_linear_triton.py:187-435);
+ * ci_fused_linear_transposed_dense replaces its _uncoalesced variant (:660-883).
+ * d_workspace: ci_fused_linear_transposed_workspace_bytes(...) bytes of fp32 partials, one slice
+ * per column tile, summed in tile order (the reference zeroes a bf16 workspace and sums it with
+ * torch.sum, comp_inference/transposed_linear_triton.py:384, :424-435).
+ * ------------------------------------------------------------------------------------- */
+size_t ci_fused_linear_transposed_workspace_bytes(uint32_t M, uint32_t H, uint32_t V, uint32_t tile_width);
+
+int ci_fused_linear_transposed_ilp2(const uint16_t *d_x, uint32_t M, uint32_t H, uint32_t V,
+                                    uint32_t x_stride, const uint8_t *d_stream, uint64_t stream_len,
+                                    const uint32_t *d_states, const uint32_t *d_tables,
+                                    const uint8_t *d_slot_map, const uint32_t *d_tile_offsets,
+                                    const uint32_t *d_tile_max_lens, const uint8_t *d_man_tiled,
+                                    uint32_t tile_height, uint32_t tile_width, const uint16_t *d_bias,
+                                    uint16_t *d_out, uint32_t out_stride, void *d_workspace,
+                                    size_t workspace_bytes, ci_stream_t stream);
+
+int ci_fused_linear_transposed_dense(const uint16_t *d_x, uint32_t M, uint32_t H, uint32_t V,
+                                     uint32_t x_stride, const uint8_t *d_stream, uint64_t stream_len,
+                                     const uint32_t *d_states, const uint32_t *d_tables,
+                                     const uint8_t *d_slot_map, const uint32_t *d_stream_offsets,
+                                     const uint32_t *d_stream_sizes, const uint8_t *d_man_tiled,
+                                     uint32_t tile_height, uint32_t tile_width, const uint16_t *d_bias,
+                                     uint16_t *d_out, uint32_t out_stride, void *d_workspace,
+                                     size_t workspace_bytes, ci_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,125 @@
+"""Module level: compress -> package -> load -> forward, on the GPU.  Checks the attribute names
+the compressor attaches, the safetensors keys / dtypes / rans_info record, and that a model whose
+layers were swapped for the compressed modules reproduces the uncompressed model."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+
+pytestmark = pytest.mark.gpu
+
+
+class Tiny(nn.Module):
+    def __init__(self, V=1300, H=128, F=256):
+        super().__init__()
+        self.embed_tokens = nn.Embedding(V, H)
+        self.up_proj = nn.Linear(H, F, bias=True)
+        self.down_proj = nn.Linear(F, H, bias=False)
+        self.norm = nn.LayerNorm(H)
+        self.lm_head = nn.Linear(H, V, bias=False)
+
+    def forward(self, ids):
+        h = self.embed_tokens(ids)
+        h = h + self.down_proj(torch.nn.functional.silu(self.up_proj(h)))
+        return self.lm_head(self.norm(h))
+
+
+def _make(seed=0):
+    torch.manual_seed(seed)
+    m = Tiny().to(torch.bfloat16)
+    with torch.no_grad():
+        for p in m.parameters():
+            if p.ndim == 2:
+                p.mul_(0.3)
+    return m
+
+
+def test_compress_attributes_and_roundtrip():
+    from comp_inference_amd import rans_compress_module_weight, rans_decompress_module_weight
+
+    lin = nn.Linear(256, 128, bias=False).to(torch.bfloat16)
+    w = lin.weight.detach().clone()
+    rans_compress_module_weight(lin, tile_height=128, tile_width=32)
+    assert not hasattr(lin, "weight") and lin.compressed == "rans_bfloat16"
+    assert lin.input_shape == [256, 128] and lin.expanded_size == 256 * 128
+    for attr in ("exponent_compressed_weight", "exponent_states", "exponent_output_sizes", "exponent_tables",
+                 "exponent_slot_map", "exponent_tile_offsets", "exponent_tile_max_lens", "mantissa_raw",
+                 "exponent_freqs", "exponent_cdf"):
+        assert hasattr(lin, attr), attr
+    assert (lin.exponent_num_tiles_k, lin.exponent_num_tiles_n) == (2, 4)
+    assert lin.exponent_states.dtype == torch.uint32 and lin.exponent_slot_map.dtype == torch.uint8
+    rans_decompress_module_weight(lin)
+    assert isinstance(lin.weight, nn.Parameter)
+    assert torch.equal(lin.weight.detach().cpu().view(torch.int16), w.t().contiguous().view(torch.int16))
+    with pytest.raises(ValueError):
+        rans_compress_module_weight(nn.Linear(64, 64, bias=False).to(torch.bfloat16), tile_height=1024)
+
+
+def test_package_roundtrip_and_forward(tmp_path):
+    import comp_inference_amd as ci
+    from safetensors import safe_open
+
+    ref = _make()
+    ids = torch.tensor([[0, 5, 1299, 640, 5]])
+    want = ref.cuda()(ids.cuda()).float().cpu()
+    ref = ref.cpu()
+
+    comp = _make()
+    ci.rans_compress_module_weight(comp.embed_tokens, tile_height=256, tile_width=32, transpose_weight=False)
+    ci.rans_compress_module_weight(comp.lm_head, tile_height=256, tile_width=32, transpose_weight=False)
+    for name in ("up_proj", "down_proj"):
+        ci.rans_compress_module_weight(getattr(comp, name), tile_height=64, tile_width=32)
+    out_dir = ci.save_rans_model_package(comp, None, str(tmp_path / "pkg"))
+    assert out_dir.endswith("_unfused")
+    cfg = json.load(open(os.path.join(out_dir, "config.json")))["quantization_config"]
+    assert cfg["quant_method"] == "rans" and cfg["compression"] == "rans_bfloat16"
+    assert cfg["layer_configs"]["up_proj"] == {"tile_height": 64, "tile_width": 32, "uncoalesced_interleaving": False}
+    path = os.path.join(out_dir, "model.safetensors")
+    with safe_open(path, "pt") as f:
+        keys = set(f.keys())
+        assert f.metadata() == {"format": "pt", "compression_method": "rans_bfloat16", "fused_projections": "False"}
+        for mod in ("embed_tokens", "up_proj", "down_proj", "lm_head"):
+            for suffix, dt in (("rans_exp_stream", torch.uint8), ("rans_exp_states", torch.uint32),
+                               ("rans_exp_tables", torch.uint32), ("rans_exp_slot_map", torch.uint8),
+                               ("rans_exp_tile_offsets", torch.uint32), ("rans_exp_tile_max_lens", torch.uint32),
+                               ("rans_man_raw", torch.uint8), ("rans_info", torch.int32)):
+                assert f"{mod}.{suffix}" in keys
+                assert f.get_tensor(f"{mod}.{suffix}").dtype == dt
+        assert "up_proj.bias" in keys and "norm.weight" in keys and "up_proj.weight" not in keys
+        info = ci.parse_rans_info(f.get_tensor("up_proj.rans_info"))
+        assert info["version"] == 1 and info["shape"] == [128, 256] and info["numel"] == 128 * 256
+        assert (info["tile_height"], info["tile_width"], info["num_tiles_k"], info["num_tiles_n"]) == (64, 32, 2, 8)
+
+    fresh = _make(seed=123)  # different weights: everything must come from the package
+    model = ci.load_compressed_model_with_auto_model("unused", path, model=fresh)
+    assert isinstance(model.up_proj, ci.RansLinear) and isinstance(model.embed_tokens, ci.RansEmbedding)
+    assert isinstance(model.lm_head, ci.RansLMHead) and model.up_proj.tile_k == 64
+    got = model(ids.cuda()).float().cpu()
+    assert torch.allclose(got, want, atol=3e-2, rtol=3e-2), (got - want).abs().max()
+
+
+def test_modules_from_compressed():
+    import comp_inference_amd as ci
+
+    torch.manual_seed(1)
+    lin = nn.Linear(512, 96, bias=True).to(torch.bfloat16)
+    x = torch.randn(3, 512).to(torch.bfloat16)
+    want = lin(x).float()
+    bias = lin.bias.detach().clone()
+    ci.rans_compress_module_weight(lin, tile_height=256, tile_width=32)
+    rl = ci.RansLinear.from_compressed(lin, bias=bias)
+    got = rl(x.cuda()).float().cpu()
+    assert torch.allclose(got, want, atol=2e-2, rtol=2e-2)
+    emb = nn.Embedding(700, 64).to(torch.bfloat16)
+    table = emb.weight.detach().clone()
+    ci.rans_compress_module_weight(emb, tile_height=256, tile_width=32, transpose_weight=False)
+    re = ci.RansEmbedding.from_compressed(emb)
+    ids = torch.tensor([0, 699, 300, 300])
+    assert torch.equal(re(ids.cuda()).cpu().view(torch.int16), table[ids].view(torch.int16))
+    head = ci.RansLMHead(64, 700)
+    head.tie_to(re)
+    h = torch.randn(2, 64).to(torch.bfloat16)
+    assert torch.allclose(head(h.cuda()).float().cpu(), h.float() @ table.float().t(), atol=2e-2, rtol=2e-2)
