@@ -32,6 +32,7 @@ from .linear_hip import (
 from .rans_hip import (
     rans_decomp_flat,
     rans_decomp_tiled,
+    rans_decomp_tiled_batch,
     rans_decomp_tiled_uncoalesced,
     rans_decomp_triton,
     rans_decomp_triton_tiled,

@@ -112,13 +112,12 @@ __global__ __launch_bounds__(kDecWaves *kWave) void decode_tiled32_kernel(Decode
 // Exponent-plane output through the hand-scheduled loop (fast_tile.h): scaled state, tile body
 // staged transposed.  Tiles that do not qualify (ragged, odd half height, body deeper than a
 // lane stride) take the same arithmetic with guarded byte reads from global memory.
-__global__ __launch_bounds__(kDecWaves *kWave) void decode_tiled32_fast_kernel(DecodeArgs a) {
-    extern __shared__ __align__(16) uint8_t lds[];
+__device__ __forceinline__ void decode_tiles_fast(const DecodeArgs &a, uint32_t block, uint8_t *lds) {
     uint2 *tab = reinterpret_cast<uint2 *>(lds);
     const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
     uint8_t *stage = lds + kSlotTableBytes + (size_t)wave * kFastStageBytes;
 
-    const uint32_t tile = blockIdx.x * kDecWaves + wave;
+    const uint32_t tile = block * kDecWaves + wave;
     const bool have_tile = tile < a.num_tiles;
     const uint32_t tk = have_tile ? tile / a.tiles_n : 0, tn = have_tile ? tile % a.tiles_n : 0;
     const uint32_t half = a.th / 2, hsel = lane / 32, c = lane % 32;
@@ -171,6 +170,28 @@ __global__ __launch_bounds__(kDecWaves *kWave) void decode_tiled32_fast_kernel(D
     }
 }
 
+__global__ __launch_bounds__(kDecWaves *kWave) void decode_tiled32_fast_kernel(DecodeArgs a) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    decode_tiles_fast(a, blockIdx.x, lds);
+}
+
+// Several tensors in one launch: a stand-alone decode is a chain of tile_height / 2 dependent
+// steps per wave whatever the tensor's size, so small tensors launched one by one leave most of
+// the chip idle.  Workgroups are assigned to tensors by a prefix table in the kernel arguments.
+constexpr int kDecBatchMax = 16;
+struct DecodeBatchArgs {
+    DecodeArgs item[kDecBatchMax];
+    uint32_t first_block[kDecBatchMax + 1];
+    uint32_t n;
+};
+
+__global__ __launch_bounds__(kDecWaves *kWave) void decode_tiled32_batch_kernel(DecodeBatchArgs b) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    uint32_t i = 0;
+    while (i + 1 < b.n && blockIdx.x >= b.first_block[i + 1]) ++i;
+    decode_tiles_fast(b.item[i], blockIdx.x - b.first_block[i], lds);
+}
+
 // Any tile width: one thread per stream, bytes read where they lie.  Used for widths other
 // than 32 (the reference's tests sweep 16..128, tests/test_mat_mul.py:263-264).
 template <bool kMerge>
@@ -210,6 +231,64 @@ __global__ __launch_bounds__(256) void decode_tiled_generic_kernel(DecodeArgs a)
 }  // namespace ci
 
 using namespace ci;
+
+extern "C" int ci_decode_tiled_ilp2_batch(const ci_decode_item *h_items, uint32_t n_items, ci_stream_t stream) {
+    if (n_items == 0) return CI_OK;
+    if (!h_items) return fail(CI_ERR_ARG, "ci_decode_tiled_ilp2_batch: null item list");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const uint32_t fast_lds = kSlotTableBytes + kDecWaves * kFastStageBytes;
+    CI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(decode_tiled32_batch_kernel),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, fast_lds));
+    uint32_t done = 0;
+    while (done < n_items) {
+        DecodeBatchArgs b;
+        b.n = 0;
+        uint32_t blocks = 0;
+        for (; done < n_items && b.n < (uint32_t)kDecBatchMax; ++done) {
+            const ci_decode_item &it = h_items[done];
+            if (it.K == 0 || it.N == 0) continue;
+            // items the batched kernel cannot take go through the single-tensor entry point
+            if (it.tile_width != 32 || !aligned(it.d_stream, 16)) {
+                int rc = ci_decode_tiled_ilp2(it.d_stream, it.stream_len, it.d_states, it.d_tables, it.d_slot_map,
+                                              it.d_tile_offsets, it.d_tile_max_lens, it.K, it.N, it.tile_height,
+                                              it.tile_width, it.d_out_exp, nullptr, nullptr, stream);
+                if (rc) return rc;
+                continue;
+            }
+            if (!it.d_states || !it.d_tables || !it.d_slot_map || !it.d_tile_offsets || !it.d_tile_max_lens ||
+                !it.d_out_exp || (it.stream_len && !it.d_stream))
+                return fail(CI_ERR_ARG, "ci_decode_tiled_ilp2_batch: null pointer in item %u", done);
+            if (it.tile_height == 0 || (it.tile_height & 1) || !aligned(it.d_slot_map, 4))
+                return fail(CI_ERR_ARG, "ci_decode_tiled_ilp2_batch: bad tile height or slot_map alignment in item %u", done);
+            DecodeArgs &a = b.item[b.n];
+            a.stream = it.d_stream;
+            a.stream_len = it.stream_len;
+            a.states = it.d_states;
+            a.tables = it.d_tables;
+            a.slot_map = it.d_slot_map;
+            a.tile_offsets = it.d_tile_offsets;
+            a.tile_max_lens = it.d_tile_max_lens;
+            a.K = it.K;
+            a.N = it.N;
+            a.th = it.tile_height;
+            a.tw = 32;
+            a.tiles_n = ceil_div(it.N, 32);
+            a.num_tiles = ceil_div(it.K, it.tile_height) * a.tiles_n;
+            a.out_exp = it.d_out_exp;
+            a.man_tiled = nullptr;
+            a.out_bf16 = nullptr;
+            a.stage_bytes = 0;
+            b.first_block[b.n] = blocks;
+            blocks += ceil_div(a.num_tiles, kDecWaves);
+            ++b.n;
+        }
+        if (b.n == 0) continue;
+        b.first_block[b.n] = blocks;
+        hipLaunchKernelGGL(decode_tiled32_batch_kernel, dim3(blocks), dim3(kDecWaves * kWave), fast_lds, s, b);
+        CI_LAUNCH_CHECK("decode_tiled32_batch_kernel");
+    }
+    return CI_OK;
+}
 
 extern "C" int ci_decode_tiled_ilp2(const uint8_t *d_stream, uint64_t stream_len,
                                     const uint32_t *d_states, const uint32_t *d_tables,

@@ -52,6 +52,43 @@ def rans_decomp_tiled(compressed_streams, initial_states, tables, slot_map, outp
     return out
 
 
+class _DecodeItem(C.Structure):
+    _fields_ = [("d_stream", C.c_void_p), ("stream_len", C.c_uint64), ("d_states", C.c_void_p),
+                ("d_tables", C.c_void_p), ("d_slot_map", C.c_void_p), ("d_tile_offsets", C.c_void_p),
+                ("d_tile_max_lens", C.c_void_p), ("K", C.c_uint32), ("N", C.c_uint32),
+                ("tile_height", C.c_uint32), ("tile_width", C.c_uint32), ("d_out_exp", C.c_void_p)]
+
+
+def rans_decomp_tiled_batch(items, tile_k=1024, tile_n=32):
+    """Decode several tensors with one launch.  `items` is a sequence of tuples
+    (compressed_streams, initial_states, tables, slot_map, output_shape, tile_offsets, tile_max_lens)
+    -- the positional arguments of rans_decomp_tiled -- all on the same GPU; returns the list of
+    exponent planes.  A stand-alone decode takes tile_k / 2 dependent steps per wavefront whatever
+    the tensor's size, so decoding a layer's tensors together keeps the whole chip busy."""
+    items = list(items)
+    if not items:
+        return []
+    _lib.require_device(items[0][0])
+    dev = items[0][0].device
+    arr = (_DecodeItem * len(items))()
+    keep, outs = [], []
+    for i, (cs, st, tb, sm, shape, to, tl) in enumerate(items):
+        K, N = int(shape[0]), int(shape[1])
+        expected = (-(-N // tile_n)) * (-(-K // tile_k)) * tile_n * 2
+        if st.numel() != expected:
+            raise ValueError(f"Initial states size mismatch. Expected {expected}")
+        t = (_lib.as_u8(cs, dev), _lib.as_u32(st, dev), _lib.as_u32(tb, dev), _lib.as_u8(sm, dev),
+             _lib.as_u32(to, dev), _lib.as_u32(tl, dev))
+        out = torch.empty((K, N), device=dev, dtype=torch.uint8)
+        keep.append(t)
+        outs.append(out)
+        arr[i] = _DecodeItem(t[0].data_ptr() if t[0].numel() else None, t[0].numel(), t[1].data_ptr(),
+                             t[2].data_ptr(), t[3].data_ptr(), t[4].data_ptr(), t[5].data_ptr(), K, N,
+                             int(tile_k), int(tile_n), out.data_ptr())
+    check(lib().ci_decode_tiled_ilp2_batch(arr, len(items), _lib.stream_handle(dev)))
+    return outs
+
+
 def rans_decomp_flat(compressed_streams, initial_states, tables, slot_map, stream_sizes, output_shape):
     """Decode the flat format (512-row segments per column) into u8[K,N]
     (comp_inference/rans_triton.py:243-271)."""

@@ -270,6 +270,26 @@ int ci_fused_linear_transposed_dense(const uint16_t *d_x, uint32_t M, uint32_t H
                                      uint16_t *d_out, uint32_t out_stride, void *d_workspace,
                                      size_t workspace_bytes, ci_stream_t stream);
 
+/* ---------------------------------------------------------------------------------------
+ * Stand-alone decode of several tensors in one launch (exponent planes only).  No counterpart
+ * in the reference, which decodes tensor by tensor (comp_inference/comp_inference.py:633-647):
+ * one decode is a chain of tile_height / 2 dependent steps per wavefront however small the
+ * tensor, so a model's tensors are best decoded together.  Items are plain host structs.
+ * ------------------------------------------------------------------------------------- */
+typedef struct ci_decode_item {
+    const uint8_t *d_stream;
+    uint64_t stream_len;
+    const uint32_t *d_states;
+    const uint32_t *d_tables;
+    const uint8_t *d_slot_map;
+    const uint32_t *d_tile_offsets;
+    const uint32_t *d_tile_max_lens;
+    uint32_t K, N, tile_height, tile_width;
+    uint8_t *d_out_exp;
+} ci_decode_item;
+
+int ci_decode_tiled_ilp2_batch(const ci_decode_item *h_items, uint32_t n_items, ci_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

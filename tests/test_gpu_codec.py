@@ -70,6 +70,31 @@ def test_tiled_decode_matches_oracle(oracle, K, N, th, tw):
     assert np.array_equal(bf16_bits(wout), bf16_bits(w))
 
 
+def test_batched_decode_matches_oracle(oracle):
+    """Several tensors of different shapes (ragged ones included) decoded by one launch."""
+    from comp_inference_amd import rans_decomp_tiled_batch
+
+    dev = "cuda"
+    shapes = [(2048, 96), (1024, 32), (1300, 80), (4096, 512), (1024, 2048), (512, 40)] * 3  # > 16 items
+    items, want = [], []
+    for i, (K, N) in enumerate(shapes):
+        w = make_weight_kn(N, K, seed=100 + i)
+        e, _ = oracle.split_bf16(bf16_bits(w))
+        f, c = oracle.get_lut(e)
+        enc = oracle.encode_tiled_ilp2(e, f, c, 1024, 32)
+        items.append((torch.from_numpy(enc.stream).to(dev), _t32(enc.states).to(dev), _t32(enc.tables).to(dev),
+                      torch.from_numpy(enc.slot_map).to(dev), (K, N), _t32(enc.tile_offsets).to(dev),
+                      _t32(enc.tile_max_lens).to(dev)))
+        want.append(oracle.decode_tiled_ilp2(enc.stream, enc.states, enc.tables, enc.slot_map, enc.tile_offsets,
+                                             enc.tile_max_lens, K, N, 1024, 32))
+        assert np.array_equal(want[-1], e)
+    outs = rans_decomp_tiled_batch(items, tile_k=1024, tile_n=32)
+    assert len(outs) == len(shapes)
+    for o, w_, (K, N) in zip(outs, want, shapes):
+        assert o.shape == (K, N) and np.array_equal(o.cpu().numpy(), w_)
+    assert rans_decomp_tiled_batch([]) == []
+
+
 def test_tiled_decode_state_count_mismatch_raises():
     from comp_inference_amd import rans_decomp_triton_tiled
 
