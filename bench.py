@@ -32,8 +32,8 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 # HBM bytes of one batched decode launch on this workload, from rocprofv3 FETCH_SIZE and WRITE_SIZE
 # passes scaled by what the same counters read for a plain copy of known size (profiles/ holds the
-# runs); None until measured for the kernel named in `roofline`.
-MEASURED_TRAFFIC_BYTES = None
+# runs): 37927.4 KiB x 1.9992 fetched + 212992.1 KiB x 1.0 written.
+MEASURED_TRAFFIC_BYTES = 295_748_896
 LAYER = [("q", 4096, 4096), ("k", 1024, 4096), ("v", 1024, 4096), ("o", 4096, 4096),
          ("gate", 14336, 4096), ("up", 14336, 4096), ("down", 4096, 14336)]  # (name, out, in)
 
@@ -160,6 +160,9 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-gemv", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run three 64 MiB device-to-device copies, so that a counter run has a "
+                         "kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU part (run with --gpus 1)", file=sys.stderr)
@@ -172,6 +175,13 @@ def main() -> int:
 
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
+    if a.copy_calibration:
+        src = torch.full((64 << 20,), 7, device=dev, dtype=torch.uint8)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     log("generating and compressing one layer (seed 1) ...")
     layer = [Compressed(n, w, dev) for n, w in make_layer(1)]
     total_syms = sum(c.K * c.N for c in layer)
@@ -195,18 +205,21 @@ def main() -> int:
     for _ in range(a.warmup):
         step()
     torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
+    ev0.record()  # on the current stream, which is the stream the library launches on
     for _ in range(a.steps):
         step()
+    ev1.record()
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / a.steps
+    launch_us = ev0.elapsed_time(ev1) * 1e3 / a.steps  # one decode launch per step, back to back
     value = total_syms / (ms_per_step * 1e-3) / 1e9
 
     # --- decode kernel roofline: per-launch durations by events on the launch stream
     per_kernel = {}
     for c in layer:
         per_kernel[c.name] = round(float(np.median(event_times_us(c.decode, 5, 30))), 2)
-    launch_us = float(np.mean(event_times_us(step, 5, max(30, a.steps))))
     algo_bytes = sum(c.decode_bytes() for c in layer)
     achieved = algo_bytes / (launch_us * 1e-6) / 1e9
     roofline = {"bound": "hbm", "kernel": "decode_tiled32_batch_kernel", "achieved": round(achieved, 1),
