@@ -112,46 +112,33 @@ __global__ __launch_bounds__(kDecWaves *kWave) void decode_tiled32_kernel(Decode
 // Exponent-plane output through the hand-scheduled loop (fast_tile.h): scaled state, tile body
 // staged transposed.  Tiles that do not qualify (ragged, odd half height, body deeper than a
 // lane stride) take the same arithmetic with guarded byte reads from global memory.
-__device__ __forceinline__ void decode_tiles_fast(const DecodeArgs &a, uint32_t block, uint8_t *lds) {
-    uint2 *tab = reinterpret_cast<uint2 *>(lds);
-    const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
-    uint8_t *stage = lds + kSlotTableBytes + (size_t)wave * kFastStageBytes;
-
-    const uint32_t tile = block * kDecWaves + wave;
-    const bool have_tile = tile < a.num_tiles;
-    const uint32_t tk = have_tile ? tile / a.tiles_n : 0, tn = have_tile ? tile % a.tiles_n : 0;
+template <uint32_t kStride>
+__device__ __forceinline__ void decode_one_tile(const DecodeArgs &a, uint32_t tile, const uint2 *tab,
+                                                uint8_t *stage, int lane) {
+    const uint32_t tk = tile / a.tiles_n, tn = tile % a.tiles_n;
     const uint32_t half = a.th / 2, hsel = lane / 32, c = lane % 32;
     const uint32_t row0 = tk * a.th, col0 = tn * 32, my_row0 = row0 + hsel * half;
-    uint32_t depth = 0, my_steps = 0;
-    uint64_t base = 0;
-    bool fast = false;
-    StageRegs body;
-    if (have_tile) {
-        base = a.tile_offsets[tile];
-        depth = a.tile_max_lens[tile];
-        if (base + (uint64_t)depth * 64 > a.stream_len) depth = 0;
-        if (col0 + c < a.N && my_row0 < a.K) my_steps = min(half, a.K - my_row0);
-        const bool full = __builtin_amdgcn_ballot_w64(my_steps != half) == 0;
-        fast = full && depth >= 2 && depth < kFastStride && half % 2 == 0 && half >= 2 &&
-               (uint64_t)a.K * a.N < (1ull << 32) && (uint32_t)(uintptr_t)tab == 0;
-        if (fast) stage_fetch(body, a.stream + base, 0, depth, lane);
-    }
-    build_slot_table_x8(tab, a.tables, a.slot_map, tid, kDecWaves * kWave);
+    const uint64_t base = a.tile_offsets[tile];
+    uint32_t depth = a.tile_max_lens[tile];
+    const uint32_t state = a.states[(size_t)tile * 64 + lane];
+    // A body that would run past the stream is treated as empty rather than read.
+    if (base + (uint64_t)depth * 64 > a.stream_len) depth = 0;
+    uint32_t my_steps = 0;
+    if (col0 + c < a.N && my_row0 < a.K) my_steps = min(half, a.K - my_row0);
+    const bool full = __builtin_amdgcn_ballot_w64(my_steps != half) == 0;
+    const bool fast = full && depth >= 2 && depth < kStride && half % 2 == 0 && half >= 2 &&
+                      (uint64_t)a.K * a.N < (1ull << 32) && (uint32_t)(uintptr_t)tab == 0;
     if (fast) {
-        stage_commit(body, stage, 0, depth, lane);
-        for (int grp = 1; grp < kStageGroups; ++grp)
+        StageRegs body;
+#pragma unroll
+        for (int grp = 0; grp < stage_groups(kStride); ++grp)
             if ((uint32_t)grp * 128 < depth) {
                 stage_fetch(body, a.stream + base, grp * 128, depth, lane);
-                stage_commit(body, stage, grp * 128, depth, lane);
+                stage_commit<kStride>(body, stage, grp * 128, depth, lane);
             }
-    }
-    __syncthreads();
-    if (!have_tile) return;
-
-    const uint32_t state = a.states[(size_t)tile * 64 + lane];
-    if (fast) {
+        // LDS operations of one wavefront complete in order: the reads below see the writes above
         FastLane st;
-        st.init(stage, depth, lane, state);
+        st.init<kStride>(stage, depth, lane, state);
         const uint64_t ob = reinterpret_cast<uint64_t>(a.out_exp + (size_t)row0 * a.N + col0);
         // readfirstlane returns a signed int: widen through uint32_t
         const uint32_t ob_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(ob >> 32));
@@ -170,26 +157,66 @@ __device__ __forceinline__ void decode_tiles_fast(const DecodeArgs &a, uint32_t 
     }
 }
 
-__global__ __launch_bounds__(kDecWaves *kWave) void decode_tiled32_fast_kernel(DecodeArgs a) {
-    extern __shared__ __align__(16) uint8_t lds[];
-    decode_tiles_fast(a, blockIdx.x, lds);
+// Wavefront `wave` of workgroup `j` (of the `n_wg` that share this tensor) decodes the tiles
+// (slot * n_wg + j), slot = wave, wave + kWaves, ...: a workgroup's concurrent tiles are n_wg
+// apart, so every workgroup gets the same number of tiles to within one.
+template <int kWaves, uint32_t kStride>
+__device__ __forceinline__ void decode_wave_tiles(const DecodeArgs &a, uint32_t j, uint32_t n_wg, const uint2 *tab,
+                                                  uint8_t *lds, int wave, int lane) {
+    static_assert(kSlotTableBytes + (uint32_t)kWaves * 64u * kStride + 64u <= kLdsLimit, "staging areas exceed the LDS");
+    if (wave >= kWaves) return;
+    uint8_t *stage = lds + kSlotTableBytes + (size_t)wave * 64 * kStride;
+    for (uint32_t slot = wave;; slot += kWaves) {
+        const uint64_t tile = (uint64_t)slot * n_wg + j;
+        if (tile >= a.num_tiles) break;
+        decode_one_tile<kStride>(a, (uint32_t)tile, tab, stage, lane);
+    }
 }
 
-// Several tensors in one launch: a stand-alone decode is a chain of tile_height / 2 dependent
-// steps per wave whatever the tensor's size, so small tensors launched one by one leave most of
-// the chip idle.  Workgroups are assigned to tensors by a prefix table in the kernel arguments.
+// Several tensors in one launch, workgroups resident for the whole launch.  A stand-alone decode
+// is a chain of tile_height / 2 dependent steps per wavefront whatever the tensor's size, so what
+// counts is wavefronts in flight per SIMD: the whole LDS goes to the slot table plus as many
+// transposed tile bodies as fit, one workgroup per CU, and each wavefront walks a list of tiles.
+// How many bodies fit depends on the deepest body among the workgroup's tiles, which the
+// workgroup finds out first: 11 wavefronts x 186 bytes per lane, 10 x 204 or 8 x 255.
+// Workgroups are assigned to tensors by a prefix table in the kernel arguments.
 constexpr int kDecBatchMax = 16;
+constexpr int kPersistWaves = 11;
+constexpr uint32_t kDepthShallow = 186, kDepthMedium = 204, kDepthDeep = 255;
 struct DecodeBatchArgs {
     DecodeArgs item[kDecBatchMax];
     uint32_t first_block[kDecBatchMax + 1];
     uint32_t n;
 };
 
-__global__ __launch_bounds__(kDecWaves *kWave) void decode_tiled32_batch_kernel(DecodeBatchArgs b) {
+__global__ __launch_bounds__(kPersistWaves *kWave) void decode_tiled32_persist_kernel(DecodeBatchArgs b) {
     extern __shared__ __align__(16) uint8_t lds[];
+    uint2 *tab = reinterpret_cast<uint2 *>(lds);
+    uint32_t *flags = reinterpret_cast<uint32_t *>(lds + kLdsLimit - 64);  // beyond every staging area
+    const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
     uint32_t i = 0;
     while (i + 1 < b.n && blockIdx.x >= b.first_block[i + 1]) ++i;
-    decode_tiles_fast(b.item[i], blockIdx.x - b.first_block[i], lds);
+    const DecodeArgs &a = b.item[i];
+    const uint32_t j = blockIdx.x - b.first_block[i], n_wg = b.first_block[i + 1] - b.first_block[i];
+
+    uint32_t deepest = 0;
+    for (uint64_t t = (uint64_t)tid * n_wg + j; t < a.num_tiles; t += (uint64_t)kPersistWaves * kWave * n_wg)
+        deepest = max(deepest, a.tile_max_lens[t]);
+    build_slot_table_x8(tab, a.tables, a.slot_map, tid, kPersistWaves * kWave);
+    const uint32_t mine = (__builtin_amdgcn_ballot_w64(deepest >= kDepthShallow) ? 1u : 0u) |
+                          (__builtin_amdgcn_ballot_w64(deepest >= kDepthMedium) ? 2u : 0u);
+    if (lane == 0) flags[wave] = mine;
+    __syncthreads();
+    uint32_t any = 0;
+#pragma unroll
+    for (int w = 0; w < kPersistWaves; ++w) any |= flags[w];
+    any = (uint32_t)__builtin_amdgcn_readfirstlane((int)any);
+    if (any & 2u)
+        decode_wave_tiles<8, kDepthDeep>(a, j, n_wg, tab, lds, wave, lane);
+    else if (any & 1u)
+        decode_wave_tiles<10, kDepthMedium>(a, j, n_wg, tab, lds, wave, lane);
+    else
+        decode_wave_tiles<kPersistWaves, kDepthShallow>(a, j, n_wg, tab, lds, wave, lane);
 }
 
 // Any tile width: one thread per stream, bytes read where they lie.  Used for widths other
@@ -232,18 +259,68 @@ __global__ __launch_bounds__(256) void decode_tiled_generic_kernel(DecodeArgs a)
 
 using namespace ci;
 
+// Number of CUs of the current device (one resident workgroup each for the persistent kernel).
+static int cu_count(uint32_t *out) {
+    int dev = 0, n = 0;
+    CI_HIP(hipGetDevice(&dev));
+    CI_HIP(hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev));
+    *out = n > 0 ? (uint32_t)n : 1u;
+    return CI_OK;
+}
+
+// Launch the persistent kernel over the (already checked) tensors of `b`: the device's CUs are
+// divided among the tensors in proportion to their tile counts.
+static int launch_persist(DecodeBatchArgs &b, hipStream_t s) {
+    uint32_t cus = 0;
+    if (int rc = cu_count(&cus)) return rc;
+    uint64_t total = 0;
+    for (uint32_t i = 0; i < b.n; ++i) total += b.item[i].num_tiles;
+    // Never more workgroups than CUs (one is resident per CU; a workgroup too many would run alone
+    // after all the others): floor of the proportional share, then hand out what is left to the
+    // tensors with the most tiles per workgroup.
+    uint32_t share[kDecBatchMax], used = 0;
+    for (uint32_t i = 0; i < b.n; ++i) {
+        const uint64_t tiles = b.item[i].num_tiles;
+        uint64_t sh = tiles * cus / total;  // total >= 1: empty tensors are not in b
+        sh = sh < 1 ? 1 : sh;
+        share[i] = (uint32_t)(sh > tiles ? tiles : sh);
+        used += share[i];
+    }
+    while (used < cus) {
+        int best = -1;
+        for (uint32_t i = 0; i < b.n; ++i)
+            if (share[i] < b.item[i].num_tiles &&
+                (best < 0 || (uint64_t)b.item[i].num_tiles * share[best] > (uint64_t)b.item[best].num_tiles * share[i]))
+                best = (int)i;
+        if (best < 0) break;  // every tensor already has one workgroup per tile
+        ++share[best];
+        ++used;
+    }
+    uint32_t blocks = 0;
+    for (uint32_t i = 0; i < b.n; ++i) {
+        b.first_block[i] = blocks;
+        blocks += share[i];
+    }
+    b.first_block[b.n] = blocks;
+    static bool attr_set = false;  // a per-function attribute; setting it again is harmless
+    if (!attr_set) {
+        CI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(decode_tiled32_persist_kernel),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit));
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(decode_tiled32_persist_kernel, dim3(blocks), dim3(kPersistWaves * kWave), kLdsLimit, s, b);
+    CI_LAUNCH_CHECK("decode_tiled32_persist_kernel");
+    return CI_OK;
+}
+
 extern "C" int ci_decode_tiled_ilp2_batch(const ci_decode_item *h_items, uint32_t n_items, ci_stream_t stream) {
     if (n_items == 0) return CI_OK;
     if (!h_items) return fail(CI_ERR_ARG, "ci_decode_tiled_ilp2_batch: null item list");
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const uint32_t fast_lds = kSlotTableBytes + kDecWaves * kFastStageBytes;
-    CI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(decode_tiled32_batch_kernel),
-                               hipFuncAttributeMaxDynamicSharedMemorySize, fast_lds));
     uint32_t done = 0;
     while (done < n_items) {
         DecodeBatchArgs b;
         b.n = 0;
-        uint32_t blocks = 0;
         for (; done < n_items && b.n < (uint32_t)kDecBatchMax; ++done) {
             const ci_decode_item &it = h_items[done];
             if (it.K == 0 || it.N == 0) continue;
@@ -278,14 +355,10 @@ extern "C" int ci_decode_tiled_ilp2_batch(const ci_decode_item *h_items, uint32_
             a.man_tiled = nullptr;
             a.out_bf16 = nullptr;
             a.stage_bytes = 0;
-            b.first_block[b.n] = blocks;
-            blocks += ceil_div(a.num_tiles, kDecWaves);
             ++b.n;
         }
         if (b.n == 0) continue;
-        b.first_block[b.n] = blocks;
-        hipLaunchKernelGGL(decode_tiled32_batch_kernel, dim3(blocks), dim3(kDecWaves * kWave), fast_lds, s, b);
-        CI_LAUNCH_CHECK("decode_tiled32_batch_kernel");
+        if (int rc = launch_persist(b, s)) return rc;
     }
     return CI_OK;
 }
@@ -337,11 +410,10 @@ extern "C" int ci_decode_tiled_ilp2(const uint8_t *d_stream, uint64_t stream_len
             hipLaunchKernelGGL(decode_tiled32_kernel<true>, grid, block, lds_bytes, s, a);
             CI_LAUNCH_CHECK("decode_tiled32_kernel");
         } else {
-            const uint32_t fast_lds = kSlotTableBytes + kDecWaves * kFastStageBytes;
-            CI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(decode_tiled32_fast_kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, fast_lds));
-            hipLaunchKernelGGL(decode_tiled32_fast_kernel, grid, block, fast_lds, s, a);
-            CI_LAUNCH_CHECK("decode_tiled32_fast_kernel");
+            DecodeBatchArgs b;
+            b.n = 1;
+            b.item[0] = a;
+            if (int rc = launch_persist(b, s)) return rc;
         }
     } else {
         a.stage_bytes = 0;

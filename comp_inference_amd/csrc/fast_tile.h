@@ -52,6 +52,7 @@ __device__ __forceinline__ void build_slot_table_x8(uint2 *tab, const uint32_t *
 // run under the first group: stage_fetch issues the loads, stage_commit writes LDS.
 constexpr int kStagePasses = 8;                       // 16 rows per pass, 128 rows per group
 constexpr int kStageGroups = (kFastStride + 127) / 128;
+constexpr int stage_groups(uint32_t stride) { return (int)((stride + 127) / 128); }
 struct StageRegs {
     u32x4 v[kStagePasses];
 };
@@ -68,6 +69,7 @@ __device__ __forceinline__ void stage_fetch(StageRegs &regs, const uint8_t *__re
     }
 }
 
+template <uint32_t kStride = kFastStride>
 __device__ __forceinline__ void stage_commit(const StageRegs &regs, uint8_t *dst, uint32_t row0, uint32_t depth,
                                              int lane) {
     const uint32_t g = lane & 3, rr = lane >> 2;
@@ -75,9 +77,9 @@ __device__ __forceinline__ void stage_commit(const StageRegs &regs, uint8_t *dst
     for (int p = 0; p < kStagePasses; ++p) {
         const uint32_t r = row0 + p * 16 + rr;
         if (r < depth) {
-            uint8_t *d = dst + (g * 16) * kFastStride + r;
+            uint8_t *d = dst + (g * 16) * kStride + r;
 #pragma unroll
-            for (int j = 0; j < 16; ++j) d[j * kFastStride] = (uint8_t)(regs.v[p][j / 4] >> (8 * (j & 3)));
+            for (int j = 0; j < 16; ++j) d[j * kStride] = (uint8_t)(regs.v[p][j / 4] >> (8 * (j & 3)));
         }
     }
 }
@@ -180,9 +182,11 @@ __device__ __forceinline__ void stage_commit(const StageRegs &regs, uint8_t *dst
 struct FastLane {
     uint32_t X, q, n1, n2;
     // `stage` = this wave's staging area, q_lane = this lane's stream inside the tile.
+    // kStride = bytes of LDS per lane in the staging area (must exceed the tile's depth).
+    template <uint32_t kStride = kFastStride>
     __device__ __forceinline__ void init(const uint8_t *stage, uint32_t depth, uint32_t q_lane, uint32_t state) {
         X = state << 3;
-        const uint8_t *col = stage + q_lane * kFastStride;
+        const uint8_t *col = stage + q_lane * kStride;
         q = (uint32_t)(uintptr_t)col + depth - 2;  // low 32 bits of an LDS pointer are its LDS address
         n1 = depth >= 1 ? col[depth - 1] : 0;
         n2 = depth >= 2 ? col[depth - 2] : 0;

@@ -95,6 +95,29 @@ def test_batched_decode_matches_oracle(oracle):
     assert rans_decomp_tiled_batch([]) == []
 
 
+@pytest.mark.parametrize("n_sym", [4, 5, 6, 8, 9, 12, 40])
+def test_decode_body_depth_classes(oracle, n_sym):
+    """Uniform symbols over n_sym values give bodies of about 64 * log2(n_sym) rows: below, between and
+    above the depths at which the decoder changes how many tile bodies it keeps in LDS; the last
+    values are deeper than any staging area.  One half of the tensor is near-constant so that shallow
+    and deep tiles meet in one launch."""
+    from comp_inference_amd import rans_decomp_tiled, rans_decomp_tiled_batch
+
+    rng = np.random.default_rng(n_sym)
+    K, N = 3072, 96
+    e = rng.integers(100, 100 + n_sym, size=(K, N), dtype=np.uint8)
+    e[:1024] = np.where(rng.random((1024, N)) < 0.95, 120, e[:1024]).astype(np.uint8)
+    f, c = oracle.get_lut(e)
+    enc = oracle.encode_tiled_ilp2(e, f, c, 1024, 32)
+    dev = "cuda"
+    args = (torch.from_numpy(enc.stream).to(dev), _t32(enc.states).to(dev), _t32(enc.tables).to(dev),
+            torch.from_numpy(enc.slot_map).to(dev), (K, N), _t32(enc.tile_offsets).to(dev),
+            _t32(enc.tile_max_lens).to(dev))
+    assert np.array_equal(rans_decomp_tiled(*args, tile_k=1024, tile_n=32).cpu().numpy(), e)
+    a, b = rans_decomp_tiled_batch([args, args], tile_k=1024, tile_n=32)
+    assert np.array_equal(a.cpu().numpy(), e) and np.array_equal(b.cpu().numpy(), e)
+
+
 def test_tiled_decode_state_count_mismatch_raises():
     from comp_inference_amd import rans_decomp_triton_tiled
 
