@@ -52,10 +52,11 @@ def make_layer(seed: int):
 class Compressed:
     """One weight in the default format, resident on the GPU."""
 
-    def __init__(self, name: str, w_out_in: torch.Tensor, dev, th: int = 1024, tw: int = 32):
+    def __init__(self, name: str, w_out_in: torch.Tensor, dev, th: int = 1024, tw: int = 32, transpose: bool = True):
         import comp_inference_amd as ci
 
-        w = w_out_in.t().contiguous()  # [K, N] as the reference encodes it
+        # linear weights are encoded as [K, N] = [in, out]; an embedding table as it is
+        w = w_out_in.t().contiguous() if transpose else w_out_in.contiguous()
         self.name, self.K, self.N, self.th, self.tw = name, w.shape[0], w.shape[1], th, tw
         exp, man = ci.extract_exp_and_mantissa(w)
         f, c = ci.get_rans_lut(exp)
@@ -160,6 +161,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-gemv", action="store_true")
+    ap.add_argument("--no-embedding", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three 64 MiB device-to-device copies, so that a counter run has a "
                          "kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
@@ -222,7 +224,7 @@ def main() -> int:
         per_kernel[c.name] = round(float(np.median(event_times_us(c.decode, 5, 30))), 2)
     algo_bytes = sum(c.decode_bytes() for c in layer)
     achieved = algo_bytes / (launch_us * 1e-6) / 1e9
-    roofline = {"bound": "hbm", "kernel": "decode_tiled32_batch_kernel", "achieved": round(achieved, 1),
+    roofline = {"bound": "hbm", "kernel": "decode_tiled32_persist_kernel", "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                 "traffic": MEASURED_TRAFFIC_BYTES, "bytes_per_launch": int(algo_bytes),
                 "launch_us": round(launch_us, 2), "single_tensor_launch_us": per_kernel,
@@ -260,6 +262,33 @@ def main() -> int:
                          "torch_matmul_bf16_us": round(us_ref, 2),
                          "torch_matmul_weight_GBs": round(2 * gate.K * gate.N / (us_ref * 1e-6) / 1e9, 1)})
         out["fused_gemv"] = {"layer": "gate K=4096 N=14336", "bytes_M1": gate.linear_bytes(1), "rows": rows}
+
+    # --- fused decompress-gather on a 128256 x 4096 table, 2048 Zipf(1.1) ids
+    if not a.no_embedding:
+        log("generating and compressing the embedding table (seed 3) ...")
+        V, H, T = 128256, 4096, 2048
+        g = torch.Generator("cpu").manual_seed(3)
+        table = (torch.randn(V, H, generator=g, dtype=torch.float32) * 0.02).to(torch.bfloat16)
+        emb = Compressed("embed", table, dev, transpose=False)
+        p = np.arange(1, V + 1, dtype=np.float64) ** -1.1
+        ids_np = np.random.default_rng(4).choice(V, T, p=p / p.sum())
+        ids = torch.from_numpy(ids_np).to(dev)
+
+        def gather():
+            return ci.fused_rans_embedding(ids, emb.stream, emb.states, emb.tables, emb.slot_map, (V, H),
+                                           emb.tile_offsets, emb.tile_max_lens, emb.th, emb.tw, emb.man)
+
+        exact = bool(torch.equal(gather().cpu().view(torch.int16), table[torch.from_numpy(ids_np)].view(torch.int16)))
+        us = batched_time_us(gather, 10, 50)
+        table_dev = table.to(dev)
+        us_ref = batched_time_us(lambda: table_dev[ids], 10, 50)
+        out["fused_embedding"] = {"table": f"{V}x{H} bf16 N(0,0.02) seed 3", "ids": f"{T} Zipf(1.1) seed 4",
+                                  "distinct_ids": int(np.unique(ids_np).size), "bit_exact": exact, "us": round(us, 1),
+                                  "rows_per_s": round(T / (us * 1e-6), 1),
+                                  "gathered_GBs": round(T * H * 2 / (us * 1e-6) / 1e9, 2),
+                                  "compressed_table_bytes": int(emb.stream.numel() + emb.man.numel()),
+                                  "torch_index_bf16_us": round(us_ref, 1)}
+        del emb, table_dev, table
 
     if not a.no_cpu_baseline:
         log("timing the CPU oracle ...")
