@@ -129,13 +129,7 @@ __device__ __forceinline__ void decode_one_tile(const DecodeArgs &a, uint32_t ti
     const bool fast = full && depth >= 2 && depth < kStride && half % 2 == 0 && half >= 2 &&
                       (uint64_t)a.K * a.N < (1ull << 32) && (uint32_t)(uintptr_t)tab == 0;
     if (fast) {
-        StageRegs body;
-#pragma unroll
-        for (int grp = 0; grp < stage_groups(kStride); ++grp)
-            if ((uint32_t)grp * 128 < depth) {
-                stage_fetch(body, a.stream + base, grp * 128, depth, lane);
-                stage_commit<kStride>(body, stage, grp * 128, depth, lane);
-            }
+        stage_body<kStride>(stage, a.stream + base, depth, lane);
         // LDS operations of one wavefront complete in order: the reads below see the writes above
         FastLane st;
         st.init<kStride>(stage, depth, lane, state);
@@ -163,9 +157,8 @@ __device__ __forceinline__ void decode_one_tile(const DecodeArgs &a, uint32_t ti
 template <int kWaves, uint32_t kStride>
 __device__ __forceinline__ void decode_wave_tiles(const DecodeArgs &a, uint32_t j, uint32_t n_wg, const uint2 *tab,
                                                   uint8_t *lds, int wave, int lane) {
-    static_assert(kSlotTableBytes + (uint32_t)kWaves * 64u * kStride + 64u <= kLdsLimit, "staging areas exceed the LDS");
     if (wave >= kWaves) return;
-    uint8_t *stage = lds + kSlotTableBytes + (size_t)wave * 64 * kStride;
+    uint8_t *stage = persist_stage<kWaves, kStride>(lds, wave);
     for (uint32_t slot = wave;; slot += kWaves) {
         const uint64_t tile = (uint64_t)slot * n_wg + j;
         if (tile >= a.num_tiles) break;
@@ -173,16 +166,11 @@ __device__ __forceinline__ void decode_wave_tiles(const DecodeArgs &a, uint32_t 
     }
 }
 
-// Several tensors in one launch, workgroups resident for the whole launch.  A stand-alone decode
-// is a chain of tile_height / 2 dependent steps per wavefront whatever the tensor's size, so what
-// counts is wavefronts in flight per SIMD: the whole LDS goes to the slot table plus as many
-// transposed tile bodies as fit, one workgroup per CU, and each wavefront walks a list of tiles.
-// How many bodies fit depends on the deepest body among the workgroup's tiles, which the
-// workgroup finds out first: 11 wavefronts x 186 bytes per lane, 10 x 204 or 8 x 255.
-// Workgroups are assigned to tensors by a prefix table in the kernel arguments.
+// Several tensors in one launch, workgroups resident for the whole launch (fast_tile.h).  A
+// stand-alone decode is a chain of tile_height / 2 dependent steps per wavefront whatever the
+// tensor's size, so small tensors launched one by one leave most of the chip idle.  Workgroups are
+// assigned to tensors by a prefix table in the kernel arguments.
 constexpr int kDecBatchMax = 16;
-constexpr int kPersistWaves = 11;
-constexpr uint32_t kDepthShallow = 186, kDepthMedium = 204, kDepthDeep = 255;
 struct DecodeBatchArgs {
     DecodeArgs item[kDecBatchMax];
     uint32_t first_block[kDecBatchMax + 1];
@@ -191,29 +179,17 @@ struct DecodeBatchArgs {
 
 __global__ __launch_bounds__(kPersistWaves *kWave) void decode_tiled32_persist_kernel(DecodeBatchArgs b) {
     extern __shared__ __align__(16) uint8_t lds[];
-    uint2 *tab = reinterpret_cast<uint2 *>(lds);
-    uint32_t *flags = reinterpret_cast<uint32_t *>(lds + kLdsLimit - 64);  // beyond every staging area
+    const uint2 *tab = reinterpret_cast<const uint2 *>(lds);
     const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
     uint32_t i = 0;
     while (i + 1 < b.n && blockIdx.x >= b.first_block[i + 1]) ++i;
     const DecodeArgs &a = b.item[i];
     const uint32_t j = blockIdx.x - b.first_block[i], n_wg = b.first_block[i + 1] - b.first_block[i];
 
-    uint32_t deepest = 0;
-    for (uint64_t t = (uint64_t)tid * n_wg + j; t < a.num_tiles; t += (uint64_t)kPersistWaves * kWave * n_wg)
-        deepest = max(deepest, a.tile_max_lens[t]);
-    build_slot_table_x8(tab, a.tables, a.slot_map, tid, kPersistWaves * kWave);
-    const uint32_t mine = (__builtin_amdgcn_ballot_w64(deepest >= kDepthShallow) ? 1u : 0u) |
-                          (__builtin_amdgcn_ballot_w64(deepest >= kDepthMedium) ? 2u : 0u);
-    if (lane == 0) flags[wave] = mine;
-    __syncthreads();
-    uint32_t any = 0;
-#pragma unroll
-    for (int w = 0; w < kPersistWaves; ++w) any |= flags[w];
-    any = (uint32_t)__builtin_amdgcn_readfirstlane((int)any);
-    if (any & 2u)
+    const uint32_t cls = persist_prologue(lds, a.tables, a.slot_map, a.tile_max_lens, a.num_tiles, j, n_wg);
+    if (cls == 2u)
         decode_wave_tiles<8, kDepthDeep>(a, j, n_wg, tab, lds, wave, lane);
-    else if (any & 1u)
+    else if (cls == 1u)
         decode_wave_tiles<10, kDepthMedium>(a, j, n_wg, tab, lds, wave, lane);
     else
         decode_wave_tiles<kPersistWaves, kDepthShallow>(a, j, n_wg, tab, lds, wave, lane);

@@ -84,6 +84,57 @@ __device__ __forceinline__ void stage_commit(const StageRegs &regs, uint8_t *dst
     }
 }
 
+// ---- workgroups resident for a whole launch ------------------------------------------------------
+// The kernels built on the loops below are bound by wavefronts in flight, not by memory: the whole
+// LDS goes to the slot table plus as many transposed tile bodies as fit, one workgroup per CU, and
+// every wavefront walks a list of tiles.  How many bodies fit depends on the deepest body among the
+// workgroup's tiles: 11 wavefronts x 186 bytes per lane, 10 x 204 or 8 x 255.
+constexpr int kPersistWaves = 11;
+constexpr uint32_t kDepthShallow = 186, kDepthMedium = 204, kDepthDeep = 255;
+
+// Builds the slot table and classifies the workgroup's tiles (j, j + n_wg, ...) by their deepest
+// body: returns 0 (all below kDepthShallow), 1 (all below kDepthMedium) or 2.  Contains the only
+// workgroup barrier of such a kernel; blockDim.x must be kPersistWaves * 64.
+__device__ __forceinline__ uint32_t persist_prologue(uint8_t *lds, const uint32_t *__restrict__ tables,
+                                                     const uint8_t *__restrict__ slot_map,
+                                                     const uint32_t *__restrict__ tile_max_lens, uint32_t num_tiles,
+                                                     uint32_t j, uint32_t n_wg) {
+    const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+    uint32_t *flags = reinterpret_cast<uint32_t *>(lds + kLdsLimit - 64);  // beyond every staging area
+    uint32_t deepest = 0;
+    for (uint64_t t = (uint64_t)tid * n_wg + j; t < num_tiles; t += (uint64_t)kPersistWaves * 64 * n_wg)
+        deepest = max(deepest, tile_max_lens[t]);
+    build_slot_table_x8(reinterpret_cast<uint2 *>(lds), tables, slot_map, tid, kPersistWaves * 64);
+    const uint32_t mine = (__builtin_amdgcn_ballot_w64(deepest >= kDepthShallow) ? 1u : 0u) |
+                          (__builtin_amdgcn_ballot_w64(deepest >= kDepthMedium) ? 2u : 0u);
+    if (lane == 0) flags[wave] = mine;
+    __syncthreads();
+    uint32_t any = 0;
+#pragma unroll
+    for (int w = 0; w < kPersistWaves; ++w) any |= flags[w];
+    any = (uint32_t)__builtin_amdgcn_readfirstlane((int)any);
+    return (any & 2u) ? 2u : (any & 1u);
+}
+
+// Staging area of wavefront `wave` when kWaves wavefronts of kStride bytes per lane share the LDS.
+template <int kWaves, uint32_t kStride>
+__device__ __forceinline__ uint8_t *persist_stage(uint8_t *lds, int wave) {
+    static_assert(kSlotTableBytes + (uint32_t)kWaves * 64u * kStride + 64u <= kLdsLimit, "staging areas exceed the LDS");
+    return lds + kSlotTableBytes + (size_t)wave * 64 * kStride;
+}
+
+// Stage a whole tile body (depth < kStride rows) for the hand-scheduled loops.
+template <uint32_t kStride>
+__device__ __forceinline__ void stage_body(uint8_t *stage, const uint8_t *__restrict__ src, uint32_t depth, int lane) {
+    StageRegs body;
+#pragma unroll
+    for (int grp = 0; grp < stage_groups(kStride); ++grp)
+        if ((uint32_t)grp * 128 < depth) {
+            stage_fetch(body, src, grp * 128, depth, lane);
+            stage_commit<kStride>(body, stage, grp * 128, depth, lane);
+        }
+}
+
 // ---- assembly building blocks ----------------------------------------------------------------
 // Fixed temporaries (declared as clobbers by every user):
 //   v[96:97], v[98:99]  slot-table entries of the even / odd step of a pair
@@ -178,6 +229,20 @@ __device__ __forceinline__ void stage_commit(const StageRegs &regs, uint8_t *dst
 #define CI_BUF_A "v108", "v109", "v110", "v111", "v112", "v113", "v114", "v115"
 #define CI_BUF_B "v116", "v117", "v118", "v119", "v120", "v121", "v122", "v123"
 
+// Eight decode steps whose weights leave the statement: W0..W3 = four dwords of two bf16 each
+// (rows 0/1, 2/3, 4/5, 6/7 of the block), from the sign|mantissa dwords M0..M7 of those rows.
+#define CI_BLOCK8_OUT                                                                                      \
+    CI_STEP_ISSUE("v[96:97]") CI_STEP_FINISH("v96", "v97")                                                 \
+    CI_STEP_ISSUE("v[98:99]") CI_STEP_FINISH("v98", "v99")                                                 \
+    CI_STEP_ISSUE("v[140:141]") CI_PACK("v96", "v98", "%[m0]", "%[m1]", "%[w0]") CI_STEP_FINISH("v140", "v141") \
+    CI_STEP_ISSUE("v[142:143]") CI_STEP_FINISH("v142", "v143")                                             \
+    CI_STEP_ISSUE("v[96:97]") CI_PACK("v140", "v142", "%[m2]", "%[m3]", "%[w1]") CI_STEP_FINISH("v96", "v97")  \
+    CI_STEP_ISSUE("v[98:99]") CI_STEP_FINISH("v98", "v99")                                                 \
+    CI_STEP_ISSUE("v[140:141]") CI_PACK("v96", "v98", "%[m4]", "%[m5]", "%[w2]") CI_STEP_FINISH("v140", "v141") \
+    CI_STEP_ISSUE("v[142:143]") CI_STEP_FINISH("v142", "v143")                                             \
+    CI_PACK("v140", "v142", "%[m6]", "%[m7]", "%[w3]")                                                     \
+    "s_waitcnt lgkmcnt(0)\n"
+
 // Per-lane decoder state of the hand-scheduled loops.
 struct FastLane {
     uint32_t X, q, n1, n2;
@@ -262,6 +327,20 @@ __device__ __forceinline__ void decode_tile_asm(FastLane &st, uint64_t obase, ui
         : [X] "+v"(st.X), [q] "+v"(st.q), [n1] "+v"(st.n1), [n2] "+v"(st.n2), [off] "+v"(off)
         : [L8] "s"(kRansL << 3), [B8] "s"(256u << 3), [obase] "s"(obase), [stride] "s"(stride), [npairs] "s"(npairs)
         : CI_STEP_CLOBBERS, "scc", "s22", "v107");
+}
+
+// Eight symbols of this lane's stream as bf16 weights: w[d] = rows 2d (low half) and 2d + 1 of the
+// block.  m[r] = aligned dword holding this lane's sign|mantissa byte of row r, man_sel = the
+// per-lane byte selector 0x04040000 + (column & 3) * 0x01010101.
+__device__ __forceinline__ void decode8_weights_asm(FastLane &st, const uint32_t (&m)[8], uint32_t man_sel,
+                                                    uint32_t (&w)[4]) {
+    asm volatile(CI_BLOCK8_OUT
+                 : [X] "+v"(st.X), [q] "+v"(st.q), [n1] "+v"(st.n1), [n2] "+v"(st.n2), [w0] "=&v"(w[0]),
+                   [w1] "=&v"(w[1]), [w2] "=&v"(w[2]), [w3] "=&v"(w[3])
+                 : [L8] "s"(kRansL << 3), [B8] "s"(256u << 3), [selE] "s"(0x070C030Cu), [mask] "s"(0x807F807Fu),
+                   [msel] "v"(man_sel), [m0] "v"(m[0]), [m1] "v"(m[1]), [m2] "v"(m[2]), [m3] "v"(m[3]), [m4] "v"(m[4]),
+                   [m5] "v"(m[5]), [m6] "v"(m[6]), [m7] "v"(m[7])
+                 : CI_STEP_CLOBBERS, "v107", "v136", "v140", "v141", "v142", "v143");
 }
 
 // Advance the lane's stream by n >= 1 symbols; returns the table word (symbol in the top byte) of

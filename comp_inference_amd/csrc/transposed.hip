@@ -7,8 +7,9 @@
 //
 // The reference gives every 64 output rows their own program, which first discards all decode
 // steps above its rows.  Here one wavefront walks one tile exactly once: at step i lane (half, c)
-// holds W[v_i, c]; the products with x[m, c] are summed over the 32 lanes of the half with a DPP
-// reduction and lane 31 / 63 writes the partial sum of output row v_i for this column tile.
+// holds W[v_i, c]; the products with x[m, c] are summed over the 32 lanes of the half -- eight rows
+// at a time, with a cross-lane reduction that folds the eight sums together -- and written as the
+// partial sum of output row v_i for this column tile.
 // Partials go to a workspace [tiles_n][M][V] (fp32) and are summed in tile order by the split-K
 // reduction kernel, so the result does not depend on scheduling.
 #include "ci_common.h"
@@ -17,7 +18,6 @@
 
 namespace ci {
 
-constexpr int kTrWaves = 8;
 constexpr int kTrRows = 4;  // rows of x handled per pass
 
 struct TransArgs {
@@ -58,84 +58,139 @@ __device__ __forceinline__ float weight_f32(uint32_t sym, uint32_t man) {
     return __uint_as_float(((man & 0x80u) << 24) | (sym << 23) | ((man & 0x7Fu) << 16));
 }
 
-// grid: ceil(num_tiles / kTrWaves); one wave per tile
-template <int MB>
-__global__ __launch_bounds__(kTrWaves *kWave) void trans32_kernel(TransArgs a) {
-    extern __shared__ __align__(16) uint8_t lds[];
-    uint2 *tab = reinterpret_cast<uint2 *>(lds);
-    const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
-    uint8_t *stage = lds + kSlotTableBytes + (size_t)wave * kFastStageBytes;
+// a + b after exchanging the second 16-lane row of `a` with the first 16-lane row of `b`: lanes of
+// the first row of each 32-lane group end up with a[l] + a[l + 16], lanes of the second row with
+// b[l - 16] + b[l].
+__device__ __forceinline__ float swap16_add(float a, float b) {
+    const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
 
-    const uint32_t tile = blockIdx.x * kTrWaves + wave;
-    const bool have_tile = tile < a.num_tiles;
-    const uint32_t tk = have_tile ? tile / a.tiles_n : 0, tn = have_tile ? tile % a.tiles_n : 0;
+// Sums of eight values per lane over the 32 lanes of each half wave, all eight at once: every
+// level adds lane pairs and at the same time halves the number of values a lane carries, so the
+// whole reduction is 19 instructions instead of 8 x 5.  On return every lane of the quad
+// (r, b8, b4) -- r = 16-lane row of the half, b8 = 8-lane group of the row, b4 = quad of the group --
+// holds the total of value 4 * b4 + 2 * b8 + r.
+__device__ __forceinline__ float reduce8_over32(const float (&p)[8], bool b8, bool b4) {
+    const float s0 = swap16_add(p[0], p[1]), s1 = swap16_add(p[2], p[3]);
+    const float s2 = swap16_add(p[4], p[5]), s3 = swap16_add(p[6], p[7]);
+    // every cross-lane add runs on all lanes; only the choice between two results is per lane
+    const float a0 = dpp_add<0x128>(s0), a1 = dpp_add<0x128>(s1);  // row_ror:8
+    const float a2 = dpp_add<0x128>(s2), a3 = dpp_add<0x128>(s3);
+    const float t0 = b8 ? a1 : a0, t1 = b8 ? a3 : a2;
+    const float c0 = dpp_add<0x104>(t0), c1 = dpp_add<0x114>(t1);  // row_shl:4, row_shr:4
+    float u = b4 ? c1 : c0;
+    u = dpp_add<0x4E>(u);     // quad_perm [2,3,0,1]
+    return dpp_add<0xB1>(u);  // quad_perm [1,0,3,2]
+}
+
+// One tile: wave walks it once.  Fast path: blocks of eight steps through the hand-scheduled
+// loop, products and the eight-at-once reduction in between; otherwise a guarded step at a time.
+template <int MB, uint32_t kStride>
+__device__ __forceinline__ void trans_one_tile(const TransArgs &a, uint32_t tile, const uint2 *tab, uint8_t *stage,
+                                               int lane) {
+    const uint32_t tk = tile / a.tiles_n, tn = tile % a.tiles_n;
     const uint32_t half = a.th / 2, hsel = lane / 32, c = lane % 32;
     const uint32_t v0 = tk * a.th + hsel * half, h = tn * 32 + c;
-    uint32_t depth = 0, my_steps = 0;
-    uint64_t base = 0;
-    bool fast = false;
-    StageRegs body;
-    if (have_tile) {
-        base = a.tile_offsets[tile];
-        depth = a.tile_max_lens[tile];
-        if (base + (uint64_t)depth * 64 > a.stream_len) depth = 0;
-        if (v0 < a.V) my_steps = min(half, a.V - v0);  // rows of this lane's half (same for its 32 lanes)
-        const bool full = __builtin_amdgcn_ballot_w64(my_steps != half || h >= a.H) == 0;
-        fast = full && depth >= 2 && depth < kFastStride && (uint32_t)(uintptr_t)tab == 0;
-        if (fast) stage_fetch(body, a.stream + base, 0, depth, lane);
-    }
-    build_slot_table_x8(tab, a.tables, a.slot_map, tid, kTrWaves * kWave);
-    if (fast) {
-        stage_commit(body, stage, 0, depth, lane);
-        for (int grp = 1; grp < kStageGroups; ++grp)
-            if ((uint32_t)grp * 128 < depth) {
-                stage_fetch(body, a.stream + base, grp * 128, depth, lane);
-                stage_commit(body, stage, grp * 128, depth, lane);
-            }
-    }
-    __syncthreads();
-    if (!have_tile) return;
-
-    float xs[MB];
-#pragma unroll
-    for (int m = 0; m < MB; ++m)
-        xs[m] = (m < (int)a.M && h < a.H) ? __uint_as_float((uint32_t)a.x[(size_t)m * a.x_stride + h] << 16) : 0.f;
-    const uint8_t *man = a.man_tiled + (size_t)tile * a.th * 32 + (size_t)hsel * half * 32 + c;
-    float *dst = a.partial + (size_t)tn * a.M * a.V + v0;  // + m * V + i
+    const uint64_t base = a.tile_offsets[tile];
+    uint32_t depth = a.tile_max_lens[tile];
     const uint32_t state = a.states[(size_t)tile * 64 + lane];
+    if (base + (uint64_t)depth * 64 > a.stream_len) depth = 0;
+    uint32_t my_steps = 0;
+    if (v0 < a.V) my_steps = min(half, a.V - v0);  // rows of this lane's half (same for its 32 lanes)
+    const bool full = __builtin_amdgcn_ballot_w64(my_steps != half || h >= a.H) == 0;
+    const bool fast = full && depth >= 2 && depth < kStride && half % 8 == 0 && (uint32_t)(uintptr_t)tab == 0;
+
+    uint32_t xb[MB];  // bf16 bits of x[m, h]
+#pragma unroll
+    for (int m = 0; m < MB; ++m) xb[m] = (m < (int)a.M && h < a.H) ? a.x[(size_t)m * a.x_stride + h] : 0u;
+    const uint8_t *man_tile = a.man_tiled + (size_t)tile * a.th * 32 + (size_t)hsel * half * 32;
+    float *dst = a.partial + (size_t)tn * a.M * a.V + v0;  // + m * V + i
+
+    if (fast) {
+        stage_body<kStride>(stage, a.stream + base, depth, lane);
+        FastLane st;
+        st.init<kStride>(stage, depth, lane, state);
+        const uint32_t man_sel = 0x04040000u + (c & 3u) * 0x01010101u;
+        const uint32_t *mrow = reinterpret_cast<const uint32_t *>(man_tile + (c & ~3u));  // + 8 dwords per row
+        const bool b8 = (lane & 8) != 0, b4 = (lane & 4) != 0;
+        const uint32_t j = 4u * b4 + 2u * b8 + ((lane >> 4) & 1u);  // which of the 8 rows this quad ends up with
+        const bool writer = (lane & 3) == 0;
+        const uint32_t nblk = half / 8;
+        uint32_t mcur[8], mnext[8];
+#pragma unroll
+        for (int r = 0; r < 8; ++r) mcur[r] = mrow[r * 8];
+        for (uint32_t blk = 0; blk < nblk; ++blk) {
+            // rows of the next block (the last block re-reads its own: stays inside the tile)
+            const uint32_t *nrow = mrow + (size_t)(blk + 1 < nblk ? blk + 1 : blk) * 64;
+#pragma unroll
+            for (int r = 0; r < 8; ++r) mnext[r] = nrow[r * 8];
+            uint32_t w[4];
+            decode8_weights_asm(st, mcur, man_sel, w);
+#pragma unroll
+            for (int m = 0; m < MB; ++m) {
+                const float xf = __uint_as_float(xb[m] << 16);
+                float p[8];
+#pragma unroll
+                for (int d = 0; d < 4; ++d) {  // a bf16 x bf16 product is exact in fp32
+                    p[2 * d] = __uint_as_float(w[d] << 16) * xf;
+                    p[2 * d + 1] = __uint_as_float(w[d] & 0xFFFF0000u) * xf;
+                }
+                const float total = reduce8_over32(p, b8, b4);
+                if (writer && m < (int)a.M) dst[(size_t)m * a.V + blk * 8 + j] = total;
+            }
+#pragma unroll
+            for (int r = 0; r < 8; ++r) mcur[r] = mnext[r];
+        }
+        return;
+    }
+
     // In the last k-tile the bottom half has fewer rows than the top half: the wave runs to the
     // top half's count, lanes past their own count (or past the last column) contribute zero.
     const uint32_t n_wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)my_steps);
     const bool writer = c == 31, col_ok = h < a.H;
-
-    auto emit = [&](uint32_t i, uint32_t sym, bool live) {
-        const float w = live ? weight_f32(sym, man[(size_t)i * 32]) : 0.f;
+    const uint8_t *man = man_tile + c;
+    GlobalBytes src;
+    src.init(a.stream + base, depth, 64, lane);
+    uint32_t X = state << 3;
+    for (uint32_t i = 0; i < n_wave; ++i) {
+        float w = 0.f;
+        if (col_ok && i < my_steps) {
+            const uint32_t sym = decode_symbol_scaled(X, tab) >> 24;
+            src.renorm_scaled(X);
+            src.renorm_scaled(X);
+            w = weight_f32(sym, man[(size_t)i * 32]);
+        }
 #pragma unroll
         for (int m = 0; m < MB; ++m) {
-            const float s = sum32_to_last_lane(w * xs[m]);
+            const float s = sum32_to_last_lane(w * __uint_as_float(xb[m] << 16));
             if (writer && m < (int)a.M && i < my_steps) dst[(size_t)m * a.V + i] = s;
         }
-    };
-
-    if (fast) {
-        FastLane st;
-        st.init(stage, depth, lane, state);
-        for (uint32_t i = 0; i < half; ++i) emit(i, advance_asm(st, 1) >> 24, true);
-    } else {
-        GlobalBytes src;
-        src.init(a.stream + base, depth, 64, lane);
-        uint32_t X = state << 3;
-        for (uint32_t i = 0; i < n_wave; ++i) {
-            uint32_t sym = 0;
-            const bool live = col_ok && i < my_steps;
-            if (live) {
-                sym = decode_symbol_scaled(X, tab) >> 24;
-                src.renorm_scaled(X);
-                src.renorm_scaled(X);
-            }
-            emit(i, sym, live);
-        }
     }
+}
+
+template <int MB, int kWaves, uint32_t kStride>
+__device__ __forceinline__ void trans_wave_tiles(const TransArgs &a, const uint2 *tab, uint8_t *lds, int wave, int lane) {
+    if (wave >= kWaves) return;
+    uint8_t *stage = persist_stage<kWaves, kStride>(lds, wave);
+    for (uint64_t tile = (uint64_t)wave * gridDim.x + blockIdx.x; tile < a.num_tiles; tile += (uint64_t)kWaves * gridDim.x)
+        trans_one_tile<MB, kStride>(a, (uint32_t)tile, tab, stage, lane);
+}
+
+// grid: at most one workgroup per CU, resident for the whole launch (fast_tile.h); workgroup j
+// takes the tiles j, j + gridDim.x, ...
+template <int MB>
+__global__ __launch_bounds__(kPersistWaves *kWave) void trans32_kernel(TransArgs a) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    const uint2 *tab = reinterpret_cast<const uint2 *>(lds);
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    const uint32_t cls = persist_prologue(lds, a.tables, a.slot_map, a.tile_max_lens, a.num_tiles, blockIdx.x, gridDim.x);
+    if (cls == 2u)
+        trans_wave_tiles<MB, 8, kDepthDeep>(a, tab, lds, wave, lane);
+    else if (cls == 1u)
+        trans_wave_tiles<MB, 10, kDepthMedium>(a, tab, lds, wave, lane);
+    else
+        trans_wave_tiles<MB, kPersistWaves, kDepthShallow>(a, tab, lds, wave, lane);
 }
 
 // Any tile width and the dense layout: one thread per (tile, half): it decodes the tile's columns
@@ -245,7 +300,14 @@ static int transposed_impl(const uint16_t *d_x, uint32_t M, uint32_t H, uint32_t
     a.tiles_k = ceil_div(V, th);
     a.num_tiles = a.tiles_n * a.tiles_k;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const bool fast = !dense && tw == 32 && aligned(d_stream, 16);
+    const bool fast = !dense && tw == 32 && aligned(d_stream, 16) && aligned(d_man_tiled, 4);
+    uint32_t cus = 1;
+    if (fast) {
+        int dev = 0, n = 0;
+        CI_HIP(hipGetDevice(&dev));
+        CI_HIP(hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev));
+        cus = n > 0 ? (uint32_t)n : 1u;
+    }
     static bool attr_set = false;
     if (fast && !attr_set) {
         CI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(trans32_kernel<1>),
@@ -259,12 +321,11 @@ static int transposed_impl(const uint16_t *d_x, uint32_t M, uint32_t H, uint32_t
         a.x = d_x + (size_t)m0 * x_stride;
         a.M = M - m0 < (uint32_t)kTrRows ? M - m0 : (uint32_t)kTrRows;
         if (fast) {
-            const uint32_t lds_bytes = kSlotTableBytes + kTrWaves * kFastStageBytes;
-            const dim3 grid(ceil_div(a.num_tiles, kTrWaves)), block(kTrWaves * kWave);
+            const dim3 grid(a.num_tiles < cus ? a.num_tiles : cus), block(kPersistWaves * kWave);
             if (a.M == 1)
-                hipLaunchKernelGGL(trans32_kernel<1>, grid, block, lds_bytes, s, a);
+                hipLaunchKernelGGL(trans32_kernel<1>, grid, block, kLdsLimit, s, a);
             else
-                hipLaunchKernelGGL(trans32_kernel<kTrRows>, grid, block, lds_bytes, s, a);
+                hipLaunchKernelGGL(trans32_kernel<kTrRows>, grid, block, kLdsLimit, s, a);
             CI_LAUNCH_CHECK("trans32_kernel");
         } else {
             const uint64_t threads = (uint64_t)a.num_tiles * (dense ? 1 : 2);
