@@ -7,18 +7,23 @@
 //
 // The reference starts one program per (token, column tile) and discards row % (th/2) decode
 // steps in each.  Here the ids are sorted once (one workgroup, bitonic sort in LDS); a "bucket"
-// is one half tile of rows, i.e. the row range of one stream.  Each wavefront owns one bucket
-// of two neighbouring column tiles (32 + 32 lanes, all on the same half), walks the two half
+// is one half tile of rows, i.e. the row range of one stream.  A work item is one bucket of two
+// neighbouring column tiles (32 + 32 lanes, all on the same half): a wavefront walks the two half
 // tiles once up to the deepest requested row and writes every requested row on the way as one
-// 128-byte store.  Buckets nobody asked for exit before touching the stream.
+// 128-byte store.  Items of buckets nobody asked for are skipped before touching the stream.
 #include "ci_common.h"
 #include "rans_device.h"
+#include "fast_tile.h"
 
 namespace ci {
 
 constexpr uint32_t kEmbChunk = 8192;  // ids sorted per pass (64 KB of LDS)
-constexpr int kEmbWaves = 4;
-constexpr uint32_t kEmbStageBytes = 14336;
+constexpr uint32_t kEmbRun = 64;      // most requests one wavefront serves for one bucket
+
+__host__ __device__ inline uint32_t emb_max_chunks(uint32_t n_ids, uint32_t n_buckets) {
+    const uint32_t by_bucket = n_ids < n_buckets + 1 ? n_ids : n_buckets + 1;
+    return n_ids / kEmbRun + by_bucket + 1;
+}
 
 struct EmbedArgs {
     const int64_t *ids;
@@ -38,12 +43,12 @@ struct EmbedArgs {
     uint32_t out_stride;
     uint32_t *keys;          // workspace: sorted row ids (invalid = 0xFFFFFFFF, sorted last)
     uint32_t *pos;           // workspace: output row of each sorted id
-    uint32_t *bucket_start;  // workspace: n_buckets + 2 entries (last real one = first invalid)
+    uint32_t *chunk_start;   // workspace: first sorted request of every chunk, then n_ids; [-1] = chunk count
+                             // (bucket n_buckets collects the invalid ids)
     uint32_t n_pad;          // n_ids rounded up to a power of two
-    uint32_t stage_bytes;
 };
 
-// One workgroup: sort (id, position) by id, then mark where every bucket starts.
+// One workgroup: sort (id, position) by id, then list the chunks of requests.
 __global__ __launch_bounds__(1024) void embed_sort_kernel(EmbedArgs a) {
     extern __shared__ __align__(16) uint8_t lds[];
     uint32_t *key = reinterpret_cast<uint32_t *>(lds);
@@ -76,99 +81,209 @@ __global__ __launch_bounds__(1024) void embed_sort_kernel(EmbedArgs a) {
             }
             __syncthreads();
         }
-    const uint32_t nb = a.n_buckets + 1;  // bucket n_buckets collects the invalid ids
     for (uint32_t i = tid; i < a.n_ids; i += 1024) {
         a.keys[i] = key[i];
         a.pos[i] = val[i];
-        const uint32_t b = key[i] == 0xFFFFFFFFu ? a.n_buckets : key[i] / half;
-        const uint32_t pb = i == 0 ? 0 : (key[i - 1] == 0xFFFFFFFFu ? a.n_buckets : key[i - 1] / half);
-        if (i == 0)
-            for (uint32_t bb = 0; bb <= b; ++bb) a.bucket_start[bb] = 0;
-        else
-            for (uint32_t bb = pb + 1; bb <= b; ++bb) a.bucket_start[bb] = i;
     }
+    // Chunks: runs of sorted requests of one bucket, cut at every multiple of kEmbRun, so that a
+    // bucket many ids fall into is served by several wavefronts.  Request i opens a chunk if it is
+    // the first of its bucket or i is a multiple of kEmbRun; the chunk list is the compaction of
+    // those i: each thread counts its own consecutive requests, an inclusive scan over the 1024
+    // counts gives the offsets.
+    auto bucket_of = [&](uint32_t i) { return key[i] == 0xFFFFFFFFu ? a.n_buckets : key[i] / half; };
+    auto opens = [&](uint32_t i) {
+        return i < a.n_ids && (i == 0 || i % kEmbRun == 0 || bucket_of(i) != bucket_of(i - 1));
+    };
+    uint32_t *scan = key + 2 * a.n_pad;  // 1024 counters behind the two sort arrays
+    const uint32_t per = (a.n_pad + 1023) / 1024;
+    uint32_t mine = 0;
+    for (uint32_t u = 0; u < per; ++u) mine += opens(tid * per + u) ? 1u : 0u;
+    scan[tid] = mine;
     __syncthreads();
-    // buckets after the last occupied one, and the end marker
-    if (tid == 0) {
-        const uint32_t kl = a.n_ids ? key[a.n_ids - 1] : 0;
-        const uint32_t bl = a.n_ids == 0 ? 0 : (kl == 0xFFFFFFFFu ? a.n_buckets : kl / half);
-        for (uint32_t bb = (a.n_ids ? bl + 1 : 0); bb <= nb; ++bb) a.bucket_start[bb] = a.n_ids;
+    for (uint32_t d = 1; d < 1024; d <<= 1) {
+        const uint32_t add = tid >= d ? scan[tid - d] : 0u;
+        __syncthreads();
+        scan[tid] += add;
+        __syncthreads();
+    }
+    uint32_t at = scan[tid] - mine;
+    for (uint32_t u = 0; u < per; ++u) {
+        const uint32_t i = tid * per + u;
+        if (opens(i)) a.chunk_start[at++] = i;
+    }
+    if (tid == 1023) {
+        a.chunk_start[scan[1023]] = a.n_ids;  // end marker
+        a.chunk_start[-1] = scan[1023];       // number of chunks
     }
 }
 
-// grid: (n_buckets + 1, ceil(tiles_n / (2 * kEmbWaves)))   block: kEmbWaves waves
-__global__ __launch_bounds__(kEmbWaves *kWave) void embed_gather32_kernel(EmbedArgs a) {
-    extern __shared__ __align__(16) uint8_t lds[];
-    const uint32_t b = blockIdx.x;
-    const uint32_t lo = a.bucket_start[b], hi = a.bucket_start[b + 1];
-    if (lo >= hi) return;  // uniform for the workgroup: nobody asked for this bucket
-    const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
-    const uint32_t c = lane % 32, side = lane / 32;
-    const uint32_t tn = (blockIdx.y * kEmbWaves + wave) * 2 + side;
-    const uint32_t col = tn * 32 + c;
-    const bool col_ok = tn < a.tiles_n && col < a.N;
+// Stage the `hsel` halves (32 columns each) of two tile bodies side by side, transposed: LDS column
+// side * 32 + c holds column hsel * 32 + c of body `side`, one byte per stored row.  Same lane
+// roles as stage_fetch / stage_commit: lane = 4 * row + (16-byte group), groups 0,1 = body A, 2,3 = B.
+__device__ __forceinline__ void stage_fetch_pair(StageRegs &regs, const uint8_t *__restrict__ src_a, uint32_t depth_a,
+                                                 const uint8_t *__restrict__ src_b, uint32_t depth_b, uint32_t hsel,
+                                                 uint32_t row0, int lane) {
+    const uint32_t g = lane & 3, rr = lane >> 2;
+    const uint8_t *src = (g < 2 ? src_a : src_b) + hsel * 32 + (g & 1) * 16;
+    const uint32_t depth = g < 2 ? depth_a : depth_b;
+#pragma unroll
+    for (int p = 0; p < kStagePasses; ++p) {
+        const uint32_t r = row0 + p * 16 + rr;
+        regs.v[p] = (u32x4){0, 0, 0, 0};
+        if (r < depth) regs.v[p] = *reinterpret_cast<const u32x4 *>(src + (size_t)r * 64);
+    }
+}
 
+// One chunk of requests (all in one bucket = half tile of rows) for two neighbouring column tiles:
+// lanes 0..31 the first tile's 32 streams of that half, lanes 32..63 the second tile's.  Walks the
+// streams once, to the chunk's deepest row, and writes every requested row on the way as one
+// 128-byte store.
+template <uint32_t kStride>
+__device__ __forceinline__ void embed_one_item(const EmbedArgs &a, uint32_t chunk, uint32_t pair, const uint2 *tab,
+                                               uint8_t *stage, int lane) {
+    const uint32_t lo = a.chunk_start[chunk], hi = a.chunk_start[chunk + 1];
+    if (lo >= hi || hi > a.n_ids) return;
+    const uint32_t key0 = a.keys[lo];
+    const uint32_t b = key0 == 0xFFFFFFFFu ? a.n_buckets : min(key0 / (a.th / 2), a.n_buckets - 1);
+    const uint32_t c = lane % 32, side = lane / 32;
+    const uint32_t tn = pair * 2 + side, col = tn * 32 + c;
+    const bool col_ok = tn < a.tiles_n && col < a.N;
     if (b == a.n_buckets) {  // ids outside the table: zero rows
         for (uint32_t j = lo; j < hi; ++j)
             if (col_ok) a.out[(size_t)a.pos[j] * a.out_stride + col] = 0;
         return;
     }
-
-    uint2 *tab = reinterpret_cast<uint2 *>(lds);
-    // two tile bodies per wave, side by side
-    uint8_t *stage = lds + kSlotTableBytes + ((size_t)wave * 2 + side) * a.stage_bytes;
-    build_slot_table(tab, a.tables, a.slot_map, tid, kEmbWaves * kWave);
-
     const uint32_t half = a.th / 2, tk = b / 2, hsel = b & 1;
-    const uint32_t tile = tk * a.tiles_n + (tn < a.tiles_n ? tn : 0);
-    uint32_t depth = 0;
-    uint64_t base = 0;
-    if (tn < a.tiles_n) {
-        base = a.tile_offsets[tile];
-        depth = a.tile_max_lens[tile];
-        if (base + (uint64_t)depth * 64 > a.stream_len) depth = 0;
-    }
-    // both halves of the wave must agree on the byte source; fall back together
-    const bool fits = __builtin_amdgcn_ballot_w64(depth * 64u > a.stage_bytes) == 0;
-    if (fits && tn < a.tiles_n) {
-        // 32 lanes copy one body: 16 bytes per lane per pass
-        for (uint32_t off = c * 16; off < depth * 64u; off += 32 * 16)
-            *reinterpret_cast<u32x4 *>(stage + off) = *reinterpret_cast<const u32x4 *>(a.stream + base + off);
-    }
-    __syncthreads();
-
+    const uint32_t tile_a = tk * a.tiles_n + pair * 2;
+    const bool have_b = pair * 2 + 1 < a.tiles_n;
+    const uint32_t tile_b = have_b ? tile_a + 1 : tile_a;
+    uint64_t base_a = a.tile_offsets[tile_a], base_b = a.tile_offsets[tile_b];
+    uint32_t depth_a = a.tile_max_lens[tile_a], depth_b = a.tile_max_lens[tile_b];
+    if (base_a + (uint64_t)depth_a * 64 > a.stream_len) depth_a = 0;
+    if (base_b + (uint64_t)depth_b * 64 > a.stream_len) depth_b = 0;
+    const uint32_t tile = side ? tile_b : tile_a, depth = side ? depth_b : depth_a;
+    const uint64_t base = side ? base_b : base_a;
     const uint32_t q = hsel * 32 + c;  // this lane's stream inside its tile
-    uint32_t x = tn < a.tiles_n ? a.states[(size_t)tile * 64 + q] : kRansL;
+    const uint32_t state = a.states[(size_t)tile * 64 + q];
     const uint32_t bucket_row0 = b * half;
     const uint8_t *man = a.man_tiled + (size_t)tile * a.th * 32 + (size_t)hsel * half * 32 + c;
-    const uint32_t last_row = a.keys[hi - 1] - bucket_row0;  // deepest requested row of the bucket
-
-    auto walk = [&](auto &src) {
-        uint32_t j = lo;
-        uint32_t want = a.keys[j] - bucket_row0;
-        for (uint32_t i = 0; i <= last_row; ++i) {
-            const uint32_t sym = decode_symbol(x, tab) >> 24;
-            src.renorm(x);
-            src.renorm(x);
-            if (i == want) {  // wave uniform
-                const uint16_t v = (uint16_t)assemble_bf16(sym, man[(size_t)i * 32]);
-                do {
-                    if (col_ok) a.out[(size_t)a.pos[j] * a.out_stride + col] = v;
-                    ++j;
-                    want = j < hi ? a.keys[j] - bucket_row0 : 0xFFFFFFFFu;
-                } while (want == i);
+    const bool fast = __builtin_amdgcn_ballot_w64(!col_ok) == 0 && depth_a >= 2 && depth_b >= 2 &&
+                      depth_a < kStride && depth_b < kStride && (uint32_t)(uintptr_t)tab == 0;
+    uint32_t j = lo;
+    if (fast) {
+        StageRegs body;
+        const uint32_t deepest = max(depth_a, depth_b), my_depth = (lane & 2) ? depth_b : depth_a;
+#pragma unroll
+        for (int grp = 0; grp < stage_groups(kStride); ++grp)
+            if ((uint32_t)grp * 128 < deepest) {
+                stage_fetch_pair(body, a.stream + base_a, depth_a, a.stream + base_b, depth_b, hsel, grp * 128, lane);
+                stage_commit<kStride>(body, stage, grp * 128, my_depth, lane);
+            }
+        FastLane st;
+        st.init<kStride>(stage, depth, lane, state);
+        // Requests are taken 64 at a time (one sorted key and output row per lane, read back with
+        // readlane) and their sign|mantissa bytes eight at a time, one group ahead of the decoding,
+        // so that no load sits on the chain of decode steps.
+        uint32_t done = 0, sym = 0;  // rows decoded so far, symbol of row done - 1
+        for (uint32_t jb = lo; jb < hi; jb += 64) {
+            const uint32_t nb = min(64u, hi - jb);
+            const uint32_t my_row = (uint32_t)lane < nb ? a.keys[jb + lane] - bucket_row0 : 0u;
+            const uint32_t my_pos = (uint32_t)lane < nb ? a.pos[jb + lane] : 0u;
+            constexpr int kG = 8;
+            uint32_t row_cur[kG] = {}, row_next[kG] = {};
+            uint8_t man_cur[kG] = {}, man_next[kG] = {};
+            auto fetch = [&](uint32_t first, uint32_t(&rows)[kG], uint8_t(&mans)[kG]) {
+#pragma unroll
+                for (int u = 0; u < kG; ++u) {
+                    const uint32_t idx = min(first + u, nb - 1);  // wave uniform
+                    rows[u] = min((uint32_t)__builtin_amdgcn_readlane((int)my_row, (int)idx), half - 1);
+                    mans[u] = man[(size_t)rows[u] * 32];
+                }
+            };
+            fetch(0, row_cur, man_cur);
+            for (uint32_t s0 = 0; s0 < nb; s0 += kG) {
+                if (s0 + kG < nb) fetch(s0 + kG, row_next, man_next);
+#pragma unroll
+                for (int u = 0; u < kG; ++u)
+                    if (s0 + u < nb) {
+                        const uint32_t want = row_cur[u];
+                        if (want + 1 > done) {  // wave uniform; sorted keys make the step count >= 1
+                            sym = advance_asm(st, want + 1 - done) >> 24;
+                            done = want + 1;
+                        }
+                        const uint32_t p = (uint32_t)__builtin_amdgcn_readlane((int)my_pos, (int)(s0 + u));
+                        a.out[(size_t)p * a.out_stride + col] = (uint16_t)assemble_bf16(sym, man_cur[u]);
+                    }
+#pragma unroll
+                for (int u = 0; u < kG; ++u) {
+                    row_cur[u] = row_next[u];
+                    man_cur[u] = man_next[u];
+                }
             }
         }
-    };
-    if (fits) {
-        LdsBytes src;
-        src.init(stage, depth, 64, q);
-        walk(src);
-    } else {
-        GlobalBytes src;
-        src.init(a.stream + base, depth, 64, q);
-        walk(src);
+        return;
     }
+    GlobalBytes src;
+    src.init(a.stream + base, depth, 64, q);
+    uint32_t X = state << 3;
+    const uint32_t last_row = a.keys[hi - 1] - bucket_row0;  // deepest requested row of the bucket
+    uint32_t want = a.keys[j] - bucket_row0;
+    for (uint32_t i = 0; i <= last_row; ++i) {
+        uint32_t sym = 0;
+        if (col_ok) {
+            sym = decode_symbol_scaled(X, tab) >> 24;
+            src.renorm_scaled(X);
+            src.renorm_scaled(X);
+        }
+        if (i == want) {  // wave uniform
+            const uint16_t v = col_ok ? (uint16_t)assemble_bf16(sym, man[(size_t)i * 32]) : 0;
+            do {
+                if (col_ok) a.out[(size_t)a.pos[j] * a.out_stride + col] = v;
+                ++j;
+                want = j < hi ? a.keys[j] - bucket_row0 : 0xFFFFFFFFu;
+            } while (want == i);
+        }
+    }
+}
+
+template <int kWaves, uint32_t kStride>
+__device__ __forceinline__ void embed_wave_items(const EmbedArgs &a, const uint2 *tab, uint8_t *lds, int wave, int lane) {
+    if (wave >= kWaves) return;
+    uint8_t *stage = persist_stage<kWaves, kStride>(lds, wave);
+    const uint32_t pairs = (a.tiles_n + 1) / 2;
+    const uint64_t n_items = (uint64_t)min(a.chunk_start[-1], emb_max_chunks(a.n_ids, a.n_buckets)) * pairs;
+    for (uint64_t item = (uint64_t)wave * gridDim.x + blockIdx.x; item < n_items; item += (uint64_t)kWaves * gridDim.x)
+        embed_one_item<kStride>(a, (uint32_t)(item / pairs), (uint32_t)(item % pairs), tab, stage, lane);
+}
+
+// grid: at most one workgroup per CU, resident for the whole launch (fast_tile.h).  Work items are
+// (chunk of requests, pair of column tiles), chunk-major, so the items of one requested row spread
+// over as many workgroups as there are pairs.
+__global__ __launch_bounds__(kPersistWaves *kWave) void embed_gather32_kernel(EmbedArgs a) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    const uint2 *tab = reinterpret_cast<const uint2 *>(lds);
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    const uint32_t pairs = (a.tiles_n + 1) / 2;
+    const uint64_t n_items = (uint64_t)min(a.chunk_start[-1], emb_max_chunks(a.n_ids, a.n_buckets)) * pairs;
+    uint32_t deepest = 0;
+    for (uint64_t item = (uint64_t)threadIdx.x * gridDim.x + blockIdx.x; item < n_items;
+         item += (uint64_t)kPersistWaves * kWave * gridDim.x) {
+        const uint32_t lo = a.chunk_start[item / pairs], pair = (uint32_t)(item % pairs);
+        if (lo >= a.n_ids) continue;
+        const uint32_t key0 = a.keys[lo];
+        if (key0 == 0xFFFFFFFFu) continue;  // the chunks of invalid ids touch no tile
+        const uint32_t b = min(key0 / (a.th / 2), a.n_buckets - 1);
+        const uint32_t tile_a = (b / 2) * a.tiles_n + pair * 2;
+        deepest = max(deepest, a.tile_max_lens[tile_a]);
+        if (pair * 2 + 1 < a.tiles_n) deepest = max(deepest, a.tile_max_lens[tile_a + 1]);
+    }
+    const uint32_t cls = persist_classify(lds, a.tables, a.slot_map, deepest);
+    if (cls == 2u)
+        embed_wave_items<8, kDepthDeep>(a, tab, lds, wave, lane);
+    else if (cls == 1u)
+        embed_wave_items<10, kDepthMedium>(a, tab, lds, wave, lane);
+    else
+        embed_wave_items<kPersistWaves, kDepthShallow>(a, tab, lds, wave, lane);
 }
 
 // Any tile width and the dense layout: one thread per (token, column), discarding the rows above
@@ -234,7 +349,7 @@ extern "C" size_t ci_fused_embedding_workspace_bytes(uint32_t n_ids, uint32_t K,
     if (tile_height < 2) return 0;
     const uint32_t chunk = n_ids < kEmbChunk ? n_ids : kEmbChunk;
     const uint32_t n_buckets = ceil_div(K, tile_height / 2);
-    return (size_t)chunk * 8 + (size_t)(n_buckets + 3) * 4;
+    return (size_t)chunk * 8 + (size_t)(emb_max_chunks(chunk, n_buckets) + 2) * 4;
 }
 
 static int embedding_impl(const int64_t *d_ids, uint32_t n_ids, const uint8_t *d_stream, uint64_t stream_len,
@@ -267,7 +382,6 @@ static int embedding_impl(const int64_t *d_ids, uint32_t n_ids, const uint8_t *d
     a.tw = tw;
     a.tiles_n = ceil_div(N, tw);
     a.out_stride = out_stride;
-    a.stage_bytes = kEmbStageBytes;
 
     const bool fast = !dense && tw == 32 && aligned(d_stream, 16);
     if (!fast) {
@@ -292,7 +406,7 @@ static int embedding_impl(const int64_t *d_ids, uint32_t n_ids, const uint8_t *d
     const uint32_t chunk_cap = n_ids < kEmbChunk ? n_ids : kEmbChunk;
     a.keys = static_cast<uint32_t *>(d_workspace);
     a.pos = a.keys + chunk_cap;
-    a.bucket_start = a.pos + chunk_cap;
+    a.chunk_start = a.pos + chunk_cap + 1;  // one word in front holds the count
     static bool attr_set = false;
     if (!attr_set) {
         CI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(embed_gather32_kernel),
@@ -301,17 +415,21 @@ static int embedding_impl(const int64_t *d_ids, uint32_t n_ids, const uint8_t *d
                                    hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit));
         attr_set = true;
     }
-    const uint32_t gather_lds = kSlotTableBytes + kEmbWaves * 2 * a.stage_bytes;
+    int dev = 0, cus = 0;
+    CI_HIP(hipGetDevice(&dev));
+    CI_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    // as many work items as chunks x pairs of column tiles; the chunk count is known on the device only
     // chunks run one after another on the stream and reuse the workspace
     for (uint32_t first = 0; first < n_ids; first += kEmbChunk) {
         a.ids = d_ids + first;
         a.n_ids = n_ids - first < kEmbChunk ? n_ids - first : kEmbChunk;
         a.out = d_out + (size_t)first * out_stride;
         a.n_pad = next_pow2(a.n_ids);
-        hipLaunchKernelGGL(embed_sort_kernel, dim3(1), dim3(1024), a.n_pad * 8, s, a);
+        hipLaunchKernelGGL(embed_sort_kernel, dim3(1), dim3(1024), a.n_pad * 8 + 4096, s, a);
         CI_LAUNCH_CHECK("embed_sort_kernel");
-        hipLaunchKernelGGL(embed_gather32_kernel, dim3(a.n_buckets + 1, ceil_div(a.tiles_n, 2 * kEmbWaves)),
-                           dim3(kEmbWaves * kWave), gather_lds, s, a);
+        const uint64_t most = (uint64_t)emb_max_chunks(a.n_ids, a.n_buckets) * ceil_div(a.tiles_n, 2u);
+        const uint32_t gather_grid = (uint32_t)(most < (uint64_t)(cus > 0 ? cus : 1) ? most : (uint64_t)(cus > 0 ? cus : 1));
+        hipLaunchKernelGGL(embed_gather32_kernel, dim3(gather_grid), dim3(kPersistWaves * kWave), kLdsLimit, s, a);
         CI_LAUNCH_CHECK("embed_gather32_kernel");
     }
     return CI_OK;

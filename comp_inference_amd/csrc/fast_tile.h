@@ -92,18 +92,14 @@ __device__ __forceinline__ void stage_commit(const StageRegs &regs, uint8_t *dst
 constexpr int kPersistWaves = 11;
 constexpr uint32_t kDepthShallow = 186, kDepthMedium = 204, kDepthDeep = 255;
 
-// Builds the slot table and classifies the workgroup's tiles (j, j + n_wg, ...) by their deepest
-// body: returns 0 (all below kDepthShallow), 1 (all below kDepthMedium) or 2.  Contains the only
-// workgroup barrier of such a kernel; blockDim.x must be kPersistWaves * 64.
-__device__ __forceinline__ uint32_t persist_prologue(uint8_t *lds, const uint32_t *__restrict__ tables,
-                                                     const uint8_t *__restrict__ slot_map,
-                                                     const uint32_t *__restrict__ tile_max_lens, uint32_t num_tiles,
-                                                     uint32_t j, uint32_t n_wg) {
+// Builds the slot table and classifies the workgroup by the deepest tile body it will meet
+// (`deepest` = this thread's maximum over its share of the workgroup's tiles): returns 0 (all below
+// kDepthShallow), 1 (all below kDepthMedium) or 2.  Contains the only workgroup barrier of such a
+// kernel; blockDim.x must be kPersistWaves * 64.
+__device__ __forceinline__ uint32_t persist_classify(uint8_t *lds, const uint32_t *__restrict__ tables,
+                                                     const uint8_t *__restrict__ slot_map, uint32_t deepest) {
     const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
     uint32_t *flags = reinterpret_cast<uint32_t *>(lds + kLdsLimit - 64);  // beyond every staging area
-    uint32_t deepest = 0;
-    for (uint64_t t = (uint64_t)tid * n_wg + j; t < num_tiles; t += (uint64_t)kPersistWaves * 64 * n_wg)
-        deepest = max(deepest, tile_max_lens[t]);
     build_slot_table_x8(reinterpret_cast<uint2 *>(lds), tables, slot_map, tid, kPersistWaves * 64);
     const uint32_t mine = (__builtin_amdgcn_ballot_w64(deepest >= kDepthShallow) ? 1u : 0u) |
                           (__builtin_amdgcn_ballot_w64(deepest >= kDepthMedium) ? 2u : 0u);
@@ -114,6 +110,17 @@ __device__ __forceinline__ uint32_t persist_prologue(uint8_t *lds, const uint32_
     for (int w = 0; w < kPersistWaves; ++w) any |= flags[w];
     any = (uint32_t)__builtin_amdgcn_readfirstlane((int)any);
     return (any & 2u) ? 2u : (any & 1u);
+}
+
+// The same for a workgroup that takes the tiles j, j + n_wg, ... of one tensor.
+__device__ __forceinline__ uint32_t persist_prologue(uint8_t *lds, const uint32_t *__restrict__ tables,
+                                                     const uint8_t *__restrict__ slot_map,
+                                                     const uint32_t *__restrict__ tile_max_lens, uint32_t num_tiles,
+                                                     uint32_t j, uint32_t n_wg) {
+    uint32_t deepest = 0;
+    for (uint64_t t = (uint64_t)threadIdx.x * n_wg + j; t < num_tiles; t += (uint64_t)kPersistWaves * 64 * n_wg)
+        deepest = max(deepest, tile_max_lens[t]);
+    return persist_classify(lds, tables, slot_map, deepest);
 }
 
 // Staging area of wavefront `wave` when kWaves wavefronts of kStride bytes per lane share the LDS.
@@ -347,6 +354,7 @@ __device__ __forceinline__ void decode8_weights_asm(FastLane &st, const uint32_t
 // the last one.  n must be the same for every lane of the wave.
 __device__ __forceinline__ uint32_t advance_asm(FastLane &st, uint32_t n) {
     uint32_t e;
+    n = (uint32_t)__builtin_amdgcn_readfirstlane((int)n);  // the loop counter is scalar
     asm volatile(
         "s_mov_b32 s22, %[n]\n"
         "ci_adv_loop%=:\n"

@@ -76,6 +76,20 @@ def test_embedding_more_ids_than_one_sort_pass(oracle):
     assert torch.equal(got.cpu().view(torch.int16), table[ids].view(torch.int16))
 
 
+def test_embedding_hot_bucket_is_split_between_wavefronts(oracle):
+    """Thousands of requests for one half tile of rows (with duplicates, invalid ids between them):
+    the requests are served in runs of 64 by different wavefronts, each decoding from the top."""
+    K, N, th, tw = 2048, 128, 1024, 32
+    table = make_weight_kn(N, K, seed=21)
+    enc, man = oracle.compress_bf16(bf16_bits(table), th, tw)
+    rng = np.random.default_rng(21)
+    ids = np.concatenate([rng.integers(0, 400, 3000), rng.integers(500, 530, 300), [-5, K + 7, 2047, 1024, 1535, 1536]])
+    rng.shuffle(ids)
+    ids_t = torch.from_numpy(ids.astype(np.int64))
+    got = _gather(enc, man, ids_t, K, N, th, tw)
+    assert torch.equal(got.cpu().view(torch.int16), _expected(table, ids_t).view(torch.int16))
+
+
 def test_embedding_dense_layout(oracle):
     from comp_inference_amd import fused_rans_embedding_triton_uncoalesced
 
