@@ -191,9 +191,12 @@ __device__ __forceinline__ void stage_body(uint8_t *stage, const uint8_t *__rest
     "s_add_u32 s23, s23, 1\n"                  \
     "s_cmp_eq_u32 s23, %[nblk]\n"              \
     "s_cselect_b32 s24, %[wrapM], 0x100\n"     \
-    "s_cselect_b32 s25, %[wrapX], 16\n"        \
+    "s_cselect_b32 s25, %[wrapX], %[xstep]\n"  \
     "v_add_u32 %[moff], s24, %[moff]\n"        \
     "v_add_u32 %[xoff], s25, %[xoff]\n"
+// the same step for the x rows 32..63 of a 64-row pass
+#define CI_NEXT_BLOCK_OFFSETS2 "v_add_u32 %[xoff2], s25, %[xoff2]\n"
+#define CI_LOAD_X2(XR2) "global_load_dwordx4 " XR2 ", %[xoff2], %[xbase]\n"
 
 // Sign|mantissa dwords of rows 0..4 / rows 5..7 + the x fragment of one block into buffer
 // (M0..M7, XR).
@@ -213,13 +216,14 @@ __device__ __forceinline__ void stage_body(uint8_t *stage, const uint8_t *__rest
 // being filled for the block after it (which is also the buffer the previous block used).
 // TAIL = what runs in the shadow of step 0: nothing for the first block, otherwise the last
 // pack of the previous block and its MFMA.
-#define CI_BLOCK(TAIL, C0, C1, C2, C3, C4, C5, C6, C7, N0, N1, N2, N3, N4, N5, N6, N7, NX)      \
+// EXTRA_OFFS / EXTRA_LOAD: nothing, or the offset step and load of a second x fragment.
+#define CI_BLOCK(TAIL, EXTRA_OFFS, EXTRA_LOAD, C0, C1, C2, C3, C4, C5, C6, C7, N0, N1, N2, N3, N4, N5, N6, N7, NX) \
     CI_STEP_ISSUE("v[96:97]") TAIL CI_STEP_FINISH("v96", "v97")                                  \
-    CI_STEP_ISSUE("v[98:99]") CI_NEXT_BLOCK_OFFSETS CI_LOAD_LO(N0, N1, N2, N3, N4)               \
+    CI_STEP_ISSUE("v[98:99]") CI_NEXT_BLOCK_OFFSETS EXTRA_OFFS CI_LOAD_LO(N0, N1, N2, N3, N4)    \
     CI_STEP_FINISH("v98", "v99")                                                                 \
     CI_STEP_ISSUE("v[140:141]") "s_waitcnt vmcnt(5)\n" CI_PACK("v96", "v98", C0, C1, "v132")     \
     CI_STEP_FINISH("v140", "v141")                                                               \
-    CI_STEP_ISSUE("v[142:143]") CI_LOAD_HI(N5, N6, N7, NX) CI_STEP_FINISH("v142", "v143")        \
+    CI_STEP_ISSUE("v[142:143]") CI_LOAD_HI(N5, N6, N7, NX) EXTRA_LOAD CI_STEP_FINISH("v142", "v143") \
     CI_STEP_ISSUE("v[96:97]") CI_PACK("v140", "v142", C2, C3, "v133") CI_STEP_FINISH("v96", "v97") \
     CI_STEP_ISSUE("v[98:99]") CI_STEP_FINISH("v98", "v99")                                       \
     CI_STEP_ISSUE("v[140:141]") CI_PACK("v96", "v98", C4, C5, "v134") CI_STEP_FINISH("v140", "v141") \
@@ -230,6 +234,9 @@ __device__ __forceinline__ void stage_body(uint8_t *stage, const uint8_t *__rest
     CI_PACK("v140", "v142", M6, M7, "v135")                             \
     "s_nop 1\n"                                                         \
     "v_mfma_f32_32x32x16_bf16 %[acc], v[132:135], " XR ", %[acc]\n"
+// ... and a second MFMA of the same weights with the x fragment of rows 32..63
+#define CI_TAIL2(M6, M7, XR, XR2) \
+    CI_TAIL(M6, M7, XR) "v_mfma_f32_32x32x16_bf16 %[acc2], v[132:135], " XR2 ", %[acc2]\n"
 
 // (argument lists are expanded before CI_BLOCK counts them)
 #define CI_BLOCK_X(...) CI_BLOCK(__VA_ARGS__)
@@ -270,11 +277,12 @@ typedef float f32x16_t __attribute__((ext_vector_type(16)));
 // Whole-tile loop of the fused linear for M <= 32: `nblocks` (even, >= 2) blocks of 8 rows per
 // half tile.  mbase/moff: tile's sign|mantissa plane (uniform base, per-lane byte offset of the
 // aligned dword holding this lane's byte of the first row).  xbase/xoff: x (uniform base, per-lane
-// byte offset of the first of this lane's 8 consecutive k).  acc accumulates W^T-tile x x^T.
+// byte offset of the first of this lane's 8 consecutive k), xstep = bytes from one block's
+// fragment to the next (16 in a plain row of x).  acc accumulates W^T-tile x x^T.
 __device__ __forceinline__ void linear_tile_asm(FastLane &st, f32x16_t &acc, uint64_t mbase, uint32_t moff,
-                                                uint64_t xbase, uint32_t xoff, uint32_t man_sel,
+                                                uint64_t xbase, uint32_t xoff, uint32_t xstep, uint32_t man_sel,
                                                 uint32_t nblocks) {
-    const uint32_t wrap_m = 0u - (nblocks - 1) * 256u, wrap_x = 0u - (nblocks - 1) * 16u;
+    const uint32_t wrap_m = 0u - (nblocks - 1) * 256u, wrap_x = 0u - (nblocks - 1) * xstep;
     asm volatile(
         "s_mov_b32 s23, 0\n"
         "s_lshr_b32 s22, %[nblk], 1\n"
@@ -282,13 +290,13 @@ __device__ __forceinline__ void linear_tile_asm(FastLane &st, f32x16_t &acc, uin
         // block 0 into buffer A
         CI_LOAD_LO("v108", "v109", "v110", "v111", "v112")
         CI_LOAD_HI("v113", "v114", "v115", "v[124:127]")
-        CI_BLOCK_X("", CI_BUF_A, CI_BUF_B, "v[128:131]")
-        CI_BLOCK_X(CI_TAIL("v114", "v115", "v[124:127]"), CI_BUF_B, CI_BUF_A, "v[124:127]")
+        CI_BLOCK_X("", "", "", CI_BUF_A, CI_BUF_B, "v[128:131]")
+        CI_BLOCK_X(CI_TAIL("v114", "v115", "v[124:127]"), "", "", CI_BUF_B, CI_BUF_A, "v[124:127]")
         "ci_lin_loop%=:\n"
         "s_cmp_eq_u32 s22, 0\n"
         "s_cbranch_scc1 ci_lin_done%=\n"
-        CI_BLOCK_X(CI_TAIL("v122", "v123", "v[128:131]"), CI_BUF_A, CI_BUF_B, "v[128:131]")
-        CI_BLOCK_X(CI_TAIL("v114", "v115", "v[124:127]"), CI_BUF_B, CI_BUF_A, "v[124:127]")
+        CI_BLOCK_X(CI_TAIL("v122", "v123", "v[128:131]"), "", "", CI_BUF_A, CI_BUF_B, "v[128:131]")
+        CI_BLOCK_X(CI_TAIL("v114", "v115", "v[124:127]"), "", "", CI_BUF_B, CI_BUF_A, "v[124:127]")
         "s_sub_u32 s22, s22, 1\n"
         "s_branch ci_lin_loop%=\n"
         "ci_lin_done%=:\n"
@@ -300,11 +308,52 @@ __device__ __forceinline__ void linear_tile_asm(FastLane &st, f32x16_t &acc, uin
           [xoff] "+v"(xoff)
         : [L8] "s"(kRansL << 3), [B8] "s"(256u << 3), [selE] "s"(0x070C030Cu), [mask] "s"(0x807F807Fu),
           [msel] "v"(man_sel), [mbase] "s"(mbase), [xbase] "s"(xbase), [nblk] "s"(nblocks), [wrapM] "s"(wrap_m),
-          [wrapX] "s"(wrap_x)
+          [wrapX] "s"(wrap_x), [xstep] "s"(xstep)
         : CI_STEP_CLOBBERS, "scc", "s22", "s23", "s24", "s25", "v107", "v108", "v109", "v110", "v111", "v112",
           "v113", "v114", "v115", "v116", "v117", "v118", "v119", "v120", "v121", "v122", "v123", "v124", "v125",
           "v126", "v127", "v128", "v129", "v130", "v131", "v132", "v133", "v134", "v135", "v136", "v140", "v141",
           "v142", "v143");
+}
+
+// The same loop for up to 64 rows of x: a second x fragment (rows 32..63, per-lane offset xoff2,
+// buffers v[144:147] / v[148:151]) and a second accumulator fed with the same decoded weights.
+__device__ __forceinline__ void linear_tile_asm2(FastLane &st, f32x16_t &acc, f32x16_t &acc2, uint64_t mbase,
+                                                 uint32_t moff, uint64_t xbase, uint32_t xoff, uint32_t xoff2,
+                                                 uint32_t xstep, uint32_t man_sel, uint32_t nblocks) {
+    const uint32_t wrap_m = 0u - (nblocks - 1) * 256u, wrap_x = 0u - (nblocks - 1) * xstep;
+    asm volatile(
+        "s_mov_b32 s23, 0\n"
+        "s_lshr_b32 s22, %[nblk], 1\n"
+        "s_sub_u32 s22, s22, 1\n"
+        // block 0 into buffer A
+        CI_LOAD_LO("v108", "v109", "v110", "v111", "v112")
+        CI_LOAD_HI("v113", "v114", "v115", "v[124:127]") CI_LOAD_X2("v[144:147]")
+        CI_BLOCK_X("", CI_NEXT_BLOCK_OFFSETS2, CI_LOAD_X2("v[148:151]"), CI_BUF_A, CI_BUF_B, "v[128:131]")
+        CI_BLOCK_X(CI_TAIL2("v114", "v115", "v[124:127]", "v[144:147]"), CI_NEXT_BLOCK_OFFSETS2,
+                   CI_LOAD_X2("v[144:147]"), CI_BUF_B, CI_BUF_A, "v[124:127]")
+        "ci_lin2_loop%=:\n"
+        "s_cmp_eq_u32 s22, 0\n"
+        "s_cbranch_scc1 ci_lin2_done%=\n"
+        CI_BLOCK_X(CI_TAIL2("v122", "v123", "v[128:131]", "v[148:151]"), CI_NEXT_BLOCK_OFFSETS2,
+                   CI_LOAD_X2("v[148:151]"), CI_BUF_A, CI_BUF_B, "v[128:131]")
+        CI_BLOCK_X(CI_TAIL2("v114", "v115", "v[124:127]", "v[144:147]"), CI_NEXT_BLOCK_OFFSETS2,
+                   CI_LOAD_X2("v[144:147]"), CI_BUF_B, CI_BUF_A, "v[124:127]")
+        "s_sub_u32 s22, s22, 1\n"
+        "s_branch ci_lin2_loop%=\n"
+        "ci_lin2_done%=:\n"
+        "s_waitcnt vmcnt(0) lgkmcnt(0)\n"
+        CI_TAIL2("v122", "v123", "v[128:131]", "v[148:151]")
+        "s_nop 15\n"
+        "s_nop 15\n"
+        : [X] "+v"(st.X), [q] "+v"(st.q), [n1] "+v"(st.n1), [n2] "+v"(st.n2), [acc] "+v"(acc), [acc2] "+v"(acc2),
+          [moff] "+v"(moff), [xoff] "+v"(xoff), [xoff2] "+v"(xoff2)
+        : [L8] "s"(kRansL << 3), [B8] "s"(256u << 3), [selE] "s"(0x070C030Cu), [mask] "s"(0x807F807Fu),
+          [msel] "v"(man_sel), [mbase] "s"(mbase), [xbase] "s"(xbase), [nblk] "s"(nblocks), [wrapM] "s"(wrap_m),
+          [wrapX] "s"(wrap_x), [xstep] "s"(xstep)
+        : CI_STEP_CLOBBERS, "scc", "s22", "s23", "s24", "s25", "v107", "v108", "v109", "v110", "v111", "v112",
+          "v113", "v114", "v115", "v116", "v117", "v118", "v119", "v120", "v121", "v122", "v123", "v124", "v125",
+          "v126", "v127", "v128", "v129", "v130", "v131", "v132", "v133", "v134", "v135", "v136", "v140", "v141",
+          "v142", "v143", "v144", "v145", "v146", "v147", "v148", "v149", "v150", "v151");
 }
 
 // Symbol of the step that used table entry ELO -> one byte at obase + off; off advances a row.

@@ -47,7 +47,24 @@ struct LinearArgs {
     uint32_t out_stride;
     uint32_t th, tw, tiles_n, tiles_k, kw, nw, P;
     int fast_ok;  // x rows may be read with 16-byte loads at 32-bit offsets, sign|mantissa plane dword aligned
+    // x rearranged so that one MFMA operand load reads whole cache lines: fragment (group g of 32 rows,
+    // block kb of 8 k, row mm) = 16 bytes at ((g * K/8 + kb) * 32 + mm) * 16, rows >= M zero; or null
+    const uint16_t *xf;
 };
+
+// x [M, K] -> the fragment order described at LinearArgs::xf.  In a plain row-major x the 64 lanes of
+// one operand load touch 64 different cache lines (16 bytes of each); with many rows that traffic, not
+// the decoding, bounds the kernel.
+__global__ __launch_bounds__(256) void x_fragments_kernel(const uint16_t *__restrict__ x, uint32_t M, uint32_t K,
+                                                          uint32_t x_stride, u32x4 *__restrict__ xf,
+                                                          uint32_t total) {
+    const uint32_t e = blockIdx.x * 256 + threadIdx.x;
+    if (e >= total) return;
+    const uint32_t kbs = K / 8, mm = e % 32, kb = (e / 32) % kbs, g = e / (32 * kbs), row = g * 32 + mm;
+    u32x4 v = (u32x4){0, 0, 0, 0};
+    if (row < M) v = *reinterpret_cast<const u32x4 *>(x + (size_t)row * x_stride + (size_t)kb * 8);
+    xf[e] = v;
+}
 
 __device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {
     uint32_t u = __float_as_uint(f);
@@ -111,7 +128,10 @@ __device__ __forceinline__ void linear_tile_guarded(GlobalBytes &src, uint32_t X
     }
 }
 
-// grid: (ceil(tiles_n / nw), P, ceil(M / 32))   block: kw * nw waves
+// grid: (ceil(tiles_n / nw), P, ceil(M / (32 * MB)))   block: kw * nw waves
+// MB = 32-row groups of x per pass over the weight: 1, or 2 (M > 32: the weight is decoded once per
+// 64 rows and feeds two accumulators).
+template <int MB>
 __global__ __launch_bounds__(kLinMaxWaves *kWave) void fused_linear32_kernel(LinearArgs a) {
     extern __shared__ __align__(16) uint8_t lds[];
     uint2 *tab = reinterpret_cast<uint2 *>(lds);
@@ -152,15 +172,16 @@ __global__ __launch_bounds__(kLinMaxWaves *kWave) void fused_linear32_kernel(Lin
     }
     __syncthreads();
 
-    const uint32_t m = blockIdx.z * 32 + c;  // row of x this lane feeds to the MFMA
-    const bool m_ok = m < a.M;
-    f32x16 acc;
+    const uint32_t m = blockIdx.z * (32 * MB) + c;  // row of x this lane feeds to the (first) MFMA
+    const bool m_ok = m < a.M, m2_ok = MB == 2 && m + 32 < a.M;
+    f32x16 acc, acc2;
 #pragma unroll
-    for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+    for (int v = 0; v < 16; ++v) acc[v] = acc2[v] = 0.f;
 
     if (have_tile) {
         const uint32_t xrow_elems = (m_ok ? m : 0) * a.x_stride + k0;  // rows past M re-read row 0: their
                                                                        // accumulator columns are never stored
+        const uint32_t xrow2_elems = (m2_ok ? m + 32 : 0) * a.x_stride + k0;
         const size_t man_tile = (size_t)tile * a.th * 32;
         const uint32_t state = a.states[(size_t)tile * 64 + lane];
         if (fast) {
@@ -173,36 +194,58 @@ __global__ __launch_bounds__(kLinMaxWaves *kWave) void fused_linear32_kernel(Lin
             const uint64_t mb_u = ((uint64_t)mb_hi << 32) | (uint64_t)mb_lo;
             const uint32_t moff = hsel * half * 32 + (c & ~3u);
             const uint32_t man_sel = 0x04040000u + (c & 3u) * 0x01010101u;
-            linear_tile_asm(st, acc, mb_u, moff, reinterpret_cast<uint64_t>(a.x), xrow_elems * 2u, man_sel, half / 8);
+            uint64_t xb = reinterpret_cast<uint64_t>(a.x);
+            uint32_t xo = xrow_elems * 2u, xo2 = xrow2_elems * 2u, xstep = 16;
+            if (a.xf) {  // fragment order: this lane's row slot c of group g, block k0 / 8 onwards
+                const uint32_t kbs = a.K / 8, g = blockIdx.z * MB;
+                xb = reinterpret_cast<uint64_t>(a.xf);
+                xo = ((g * kbs + k0 / 8) * 32 + c) * 16;
+                xo2 = xo + kbs * 32 * 16;
+                xstep = 32 * 16;
+            }
+            if (MB == 2)
+                linear_tile_asm2(st, acc, acc2, mb_u, moff, xb, xo, xo2, xstep, man_sel, half / 8);
+            else
+                linear_tile_asm(st, acc, mb_u, moff, xb, xo, xstep, man_sel, half / 8);
         } else {
+            const uint8_t *man = a.man_tiled + man_tile + (size_t)hsel * half * 32 + c;
             GlobalBytes src;
             src.init(a.stream + base, depth, 64, lane);
-            linear_tile_guarded(src, state << 3, tab, a.K, half, my_steps,
-                                a.man_tiled + man_tile + (size_t)hsel * half * 32 + c, a.x + xrow_elems, m_ok, k0, acc);
+            linear_tile_guarded(src, state << 3, tab, a.K, half, my_steps, man, a.x + xrow_elems, m_ok, k0, acc);
+            if (MB == 2) {  // the guarded path simply walks the tile again for the second group of rows
+                src.init(a.stream + base, depth, 64, lane);
+                linear_tile_guarded(src, state << 3, tab, a.K, half, my_steps, man, a.x + xrow2_elems, m2_ok, k0, acc2);
+            }
         }
     }
 
     // Sum the kw accumulators of each column tile in k order.  The staging area is free now;
-    // every wave stores its fragment as [v][lane] floats (4 KB).
+    // every wave stores its fragment(s) as [v][lane] floats (4 KB each).
     __syncthreads();
     float *red = reinterpret_cast<float *>(lds + kSlotTableBytes);
     const uint32_t frag = 16 * kWave;
 #pragma unroll
-    for (int v = 0; v < 16; ++v) red[(size_t)wave * frag + v * kWave + lane] = acc[v];
-    __syncthreads();
-    if (kidx == 0 && tn < a.tiles_n) {
+    for (int g = 0; g < MB; ++g) {
+        const f32x16 &part = g ? acc2 : acc;
+        const uint32_t mg = m + 32 * g;
+        if (g) __syncthreads();
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            float s = 0.f;
-            for (uint32_t kk = 0; kk < a.kw; ++kk) s += red[(size_t)(nidx * a.kw + kk) * frag + v * kWave + lane];
-            // MFMA 32x32 result layout: register v of lane l is row (v/4)*8 + (l/32)*4 + v%4
-            // (= column of the tile), column l%32 (= row m of x)
-            const uint32_t n = tn * 32 + (v / 4) * 8 + hsel * 4 + (v % 4);
-            if (m_ok && n < a.N) {
-                if (a.P == 1)
-                    a.out[(size_t)m * a.out_stride + n] = finish_bf16(s, a.bias, n);
-                else
-                    a.partial[((size_t)blockIdx.y * a.M + m) * a.N + n] = s;
+        for (int v = 0; v < 16; ++v) red[(size_t)wave * frag + v * kWave + lane] = part[v];
+        __syncthreads();
+        if (kidx == 0 && tn < a.tiles_n) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                float s = 0.f;
+                for (uint32_t kk = 0; kk < a.kw; ++kk) s += red[(size_t)(nidx * a.kw + kk) * frag + v * kWave + lane];
+                // MFMA 32x32 result layout: register v of lane l is row (v/4)*8 + (l/32)*4 + v%4
+                // (= column of the tile), column l%32 (= row m of x)
+                const uint32_t n = tn * 32 + (v / 4) * 8 + hsel * 4 + (v % 4);
+                if (mg < a.M && n < a.N) {
+                    if (a.P == 1)
+                        a.out[(size_t)mg * a.out_stride + n] = finish_bf16(s, a.bias, n);
+                    else
+                        a.partial[((size_t)blockIdx.y * a.M + mg) * a.N + n] = s;
+                }
             }
         }
     }
@@ -294,6 +337,14 @@ __global__ __launch_bounds__(256) void splitk_reduce_bf16_kernel(const uint16_t 
     out[(size_t)m * out_stride + n] = finish_bf16(s, bias, n);
 }
 
+// Rows of x from which the fragment copy pays (below, the lanes past M re-read row 0 and one operand
+// load touches only M + 1 cache lines), and its size.
+constexpr uint32_t kFragMinRows = 17;
+static size_t x_fragment_bytes(uint32_t M, uint32_t K, bool fast_plan) {
+    if (!fast_plan || M < kFragMinRows || K % 8) return 0;
+    return (size_t)ceil_div(M, 32u) * 32 * K * 2;
+}
+
 struct LinearPlan {
     bool fast;
     uint32_t kw, nw, P;
@@ -328,7 +379,8 @@ extern "C" size_t ci_fused_linear_workspace_bytes(uint32_t M, uint32_t K, uint32
     const LinearPlan fast = plan_linear(K, tile_height, tile_width, ceil_div(N, tile_width), dense != 0, true);
     const LinearPlan slow = plan_linear(K, tile_height, tile_width, ceil_div(N, tile_width), dense != 0, false);
     const uint32_t P = fast.P > slow.P ? fast.P : slow.P;
-    return P > 1 ? (size_t)P * M * N * sizeof(float) : 0;
+    const size_t partial = P > 1 ? (size_t)P * M * N * sizeof(float) : 0;
+    return ((partial + 15) & ~(size_t)15) + x_fragment_bytes(M, K, fast.fast);
 }
 
 static int fused_linear_impl(const uint16_t *d_x, uint32_t M, uint32_t K, uint32_t N, uint32_t x_stride,
@@ -376,11 +428,26 @@ static int fused_linear_impl(const uint16_t *d_x, uint32_t M, uint32_t K, uint32
     a.nw = p.nw;
     a.P = p.P;
     a.partial = static_cast<float *>(d_workspace);
+    size_t partial_bytes = 0;
     if (p.P > 1) {
-        const size_t need = (size_t)p.P * M * N * sizeof(float);
-        if (!d_workspace || workspace_bytes < need)
-            return fail(CI_ERR_CAPACITY, "fused linear: workspace needs %zu bytes, got %zu", need, workspace_bytes);
+        partial_bytes = (size_t)p.P * M * N * sizeof(float);
+        if (!d_workspace || workspace_bytes < partial_bytes)
+            return fail(CI_ERR_CAPACITY, "fused linear: workspace needs %zu bytes, got %zu", partial_bytes, workspace_bytes);
         if (!aligned(d_workspace, 4)) return fail(CI_ERR_ARG, "fused linear: workspace must be 4-byte aligned");
+    }
+    // the fragment copy of x goes behind the partials when the caller's workspace has room for it
+    a.xf = nullptr;
+    const size_t frag_bytes = x_fragment_bytes(M, K, p.fast && a.fast_ok);
+    if (frag_bytes && frag_bytes < (1ull << 31) && d_workspace) {
+        uint8_t *at = static_cast<uint8_t *>(d_workspace) + ((partial_bytes + 15) & ~(size_t)15);
+        at += (16 - (reinterpret_cast<uintptr_t>(at) & 15)) & 15;
+        if (at + frag_bytes <= static_cast<uint8_t *>(d_workspace) + workspace_bytes) {
+            const uint32_t total = (uint32_t)(frag_bytes / 16);
+            hipLaunchKernelGGL(x_fragments_kernel, dim3(ceil_div(total, 256u)), dim3(256), 0, s, d_x, M, K, x_stride,
+                               reinterpret_cast<u32x4 *>(at), total);
+            CI_LAUNCH_CHECK("x_fragments_kernel");
+            a.xf = reinterpret_cast<const uint16_t *>(at);
+        }
     }
 
     if (p.fast) {
@@ -388,12 +455,18 @@ static int fused_linear_impl(const uint16_t *d_x, uint32_t M, uint32_t K, uint32
         const uint32_t lds_bytes = kSlotTableBytes + waves * kFastStageBytes;
         static bool attr_set = false;
         if (!attr_set) {
-            CI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(fused_linear32_kernel),
+            CI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(fused_linear32_kernel<1>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit));
+            CI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(fused_linear32_kernel<2>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit));
             attr_set = true;
         }
-        hipLaunchKernelGGL(fused_linear32_kernel, dim3(ceil_div(a.tiles_n, p.nw), p.P, ceil_div(M, 32)),
-                           dim3(waves * kWave), lds_bytes, s, a);
+        const dim3 block(waves * kWave);
+        if (M > 32)
+            hipLaunchKernelGGL(fused_linear32_kernel<2>, dim3(ceil_div(a.tiles_n, p.nw), p.P, ceil_div(M, 64)), block,
+                               lds_bytes, s, a);
+        else
+            hipLaunchKernelGGL(fused_linear32_kernel<1>, dim3(ceil_div(a.tiles_n, p.nw), p.P, 1), block, lds_bytes, s, a);
         CI_LAUNCH_CHECK("fused_linear32_kernel");
     } else {
         const uint64_t streams = (uint64_t)a.tiles_k * a.tiles_n * (dense ? 1 : 2) * tw;

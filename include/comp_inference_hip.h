@@ -183,9 +183,11 @@ int ci_decode_tiled_dense(const uint8_t *d_stream, uint64_t stream_len, const ui
  * x_stride / out_stride are row strides in elements.  d_bias may be NULL.  Products are
  * accumulated in fp32; partial sums over K are combined in a fixed order, so results are
  * reproducible run to run.  d_workspace must hold ci_fused_linear_workspace_bytes(...) bytes
- * (0 when one workgroup spans all of K); it carries the fp32 split-K partials that
+ * (0 for few rows when one workgroup spans all of K); it carries the fp32 split-K partials that
  * the reduction kernel sums (the reference keeps bf16 partials and sums them with torch.sum,
- * comp_inference/linear_triton.py:257-264, :303-314).
+ * comp_inference/linear_triton.py:257-264, :303-314) and, for more than 16 rows of x, a copy of
+ * x in the order the matrix cores read it.  A workspace with room for the partials only is
+ * accepted: x is then read in place.
  * ------------------------------------------------------------------------------------- */
 size_t ci_fused_linear_workspace_bytes(uint32_t M, uint32_t K, uint32_t N, uint32_t tile_height,
                                        uint32_t tile_width, int dense);

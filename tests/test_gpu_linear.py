@@ -47,6 +47,8 @@ def test_fused_linear_fast_path(oracle, M, K, N, th, tw):
 @pytest.mark.parametrize("K,N,th,tw,M", [
     (14336, 64, 1024, 32, 1),    # 14 k-tiles: two partial sums + reduction kernel
     (14336, 64, 1024, 32, 5),
+    (14336, 64, 1024, 32, 40),   # two 32-row groups per pass + reduction kernel
+    (1300, 80, 1024, 32, 50),    # two 32-row groups on the guarded path
     (1300, 80, 1024, 32, 3),     # ragged K and N
     (1000, 70, 512, 32, 2),
     (9000, 32, 1024, 32, 1),
