@@ -40,8 +40,7 @@ def log(msg):
 
 
 def rmsnorm(x, eps):
-    xf = x.float()
-    return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)).to(torch.bfloat16)
+    return F.rms_norm(x, (x.shape[-1],), eps=eps)  # norm weights are 1
 
 
 def rope(x, cos, sin):
@@ -81,21 +80,14 @@ class Decoder:
         """h [T, H]; pos int64 [T] (device).  Attention reads the whole cache, masked by position."""
         s = Shape
         qkv = self.ops["qkv"][l](rmsnorm(h, s.eps))
-        q, k, v = qkv.split((s.heads * s.head_dim, s.kv_heads * s.head_dim, s.kv_heads * s.head_dim), dim=-1)
-        cos, sin = self.cos.index_select(0, pos), self.sin.index_select(0, pos)
-        q = rope(q.reshape(T, s.heads, s.head_dim), cos, sin)
-        k = rope(k.reshape(T, s.kv_heads, s.head_dim), cos, sin)
-        self.k[l].index_copy_(1, pos, k.transpose(0, 1))
-        self.v[l].index_copy_(1, pos, v.reshape(T, s.kv_heads, s.head_dim).transpose(0, 1))
-        g = s.heads // s.kv_heads
-        qh = q.transpose(0, 1).reshape(s.kv_heads, g * T, s.head_dim)           # [kv, g*T, d] (head-major)
-        scores = torch.matmul(qh, self.k[l].transpose(1, 2)).float() / math.sqrt(s.head_dim)
+        qkv = qkv.view(T, s.heads + 2 * s.kv_heads, s.head_dim)
+        qk = rope(qkv[:, :s.heads + s.kv_heads], self.cos.index_select(0, pos), self.sin.index_select(0, pos))
+        self.k[l].index_copy_(1, pos, qk[:, s.heads:].transpose(0, 1))
+        self.v[l].index_copy_(1, pos, qkv[:, s.heads + s.kv_heads:].transpose(0, 1))
         allowed = self.positions[None, :] <= pos[:, None]                        # [T, max_len]
-        scores = scores.view(s.kv_heads, g, T, self.max_len).masked_fill(~allowed[None, None], float("-inf"))
-        att = torch.softmax(scores, dim=-1).to(torch.bfloat16).view(s.kv_heads, g * T, self.max_len)
-        ctx = torch.matmul(att, self.v[l]).view(s.kv_heads, g, T, s.head_dim)   # [kv, g, T, d]
-        ctx = ctx.permute(2, 0, 1, 3).reshape(T, s.heads * s.head_dim)
-        h = h + self.ops["o"][l](ctx)
+        ctx = F.scaled_dot_product_attention(qk[:, :s.heads].transpose(0, 1)[None], self.k[l][None], self.v[l][None],
+                                             attn_mask=allowed[None, None], enable_gqa=True)[0]  # [heads, T, d]
+        h = h + self.ops["o"][l](ctx.transpose(0, 1).reshape(T, s.heads * s.head_dim))
         gu = self.ops["gate_up"][l](rmsnorm(h, s.eps))
         gate, up = gu.split((s.ffn, s.ffn), dim=-1)
         return h + self.ops["down"][l](F.silu(gate) * up)
@@ -153,6 +145,17 @@ def generate(dec: Decoder, prompt, n_new, use_graph):
         graph.replay()
     torch.cuda.synchronize()
     return out.tolist(), time.perf_counter() - t0
+
+
+def teacher_forced(dec: Decoder, prompt, ids):
+    """Logits [len(ids), V] of every decode step when the given ids are fed, whatever the model itself
+    would have chosen: the comparison that one flipped argmax does not derail."""
+    dev = dec.dev
+    P = prompt.numel()
+    rows = [dec.forward(prompt, torch.arange(P, device=dev))]
+    for t, tok in enumerate(ids[:-1]):
+        rows.append(dec.forward(torch.tensor([tok], device=dev), torch.tensor([P + t], device=dev)))
+    return torch.stack(rows)
 
 
 def build(n_layers, dev, tile_k, tile_n, gen):
@@ -242,6 +245,14 @@ def run(n_layers=32, n_prompt=128, n_new=256, tile_k=1024, tile_n=32, gen="cpu")
             res[name] = (ids, sec)
             del dec
     base = res["reference_bf16"][0]
+    with torch.no_grad():
+        log("teacher-forced comparison ...")
+        lr = teacher_forced(Decoder(ref, n_layers, max_len, dev), prompt, base)
+        lc = teacher_forced(Decoder(comp, n_layers, max_len, dev), prompt, base)
+    forced_same = int((lr.argmax(-1) == lc.argmax(-1)).sum())
+    logit_err = float((lr - lc).abs().max())
+    top2 = lr.topk(2, dim=-1).values
+    min_gap = float((top2[:, 0] - top2[:, 1]).min())
 
     def agree(ids):
         n = 0
@@ -261,6 +272,9 @@ def run(n_layers=32, n_prompt=128, n_new=256, tile_k=1024, tile_n=32, gen="cpu")
         "tok_per_s_reference_bf16_eager": round(n_new / res["reference_bf16"][1], 2),
         "ids_equal_to_reference": res["compressed_eager"][0] == base,
         "ids_matching_prefix": agree(res["compressed_eager"][0]),
+        "teacher_forced_top1_agreement": f"{forced_same}/{n_new}",
+        "teacher_forced_max_abs_logit_diff": round(logit_err, 5),
+        "reference_smallest_top1_top2_logit_gap": round(min_gap, 6),
         "graph_ids_equal_eager_ids": res["compressed_graph"][0] == res["compressed_eager"][0],
         "reference_graph_ids_equal_eager_ids": res["reference_bf16_graph"][0] == base,
         "first_ids": res["compressed_eager"][0][:8],
