@@ -88,32 +88,40 @@ __global__ __launch_bounds__(1024) void embed_sort_kernel(EmbedArgs a) {
     // Chunks: runs of sorted requests of one bucket, cut at every multiple of kEmbRun, so that a
     // bucket many ids fall into is served by several wavefronts.  Request i opens a chunk if it is
     // the first of its bucket or i is a multiple of kEmbRun; the chunk list is the compaction of
-    // those i: each thread counts its own consecutive requests, an inclusive scan over the 1024
-    // counts gives the offsets.
+    // those i: each thread counts its own consecutive requests, a scan over the counts gives the
+    // offsets.
     auto bucket_of = [&](uint32_t i) { return key[i] == 0xFFFFFFFFu ? a.n_buckets : key[i] / half; };
     auto opens = [&](uint32_t i) {
         return i < a.n_ids && (i == 0 || i % kEmbRun == 0 || bucket_of(i) != bucket_of(i - 1));
     };
-    uint32_t *scan = key + 2 * a.n_pad;  // 1024 counters behind the two sort arrays
+    uint32_t *wave_total = key + 2 * a.n_pad;  // 16 counters behind the two sort arrays
     const uint32_t per = (a.n_pad + 1023) / 1024;
     uint32_t mine = 0;
     for (uint32_t u = 0; u < per; ++u) mine += opens(tid * per + u) ? 1u : 0u;
-    scan[tid] = mine;
-    __syncthreads();
-    for (uint32_t d = 1; d < 1024; d <<= 1) {
-        const uint32_t add = tid >= d ? scan[tid - d] : 0u;
-        __syncthreads();
-        scan[tid] += add;
-        __syncthreads();
+    // inclusive scan inside the wavefront, then over the 16 wavefront totals
+    uint32_t incl = mine;
+    const uint32_t lane = tid % 64, wv = tid / 64;
+#pragma unroll
+    for (uint32_t d = 1; d < 64; d <<= 1) {
+        const uint32_t up = (uint32_t)__shfl_up((int)incl, d, 64);
+        if (lane >= d) incl += up;
     }
-    uint32_t at = scan[tid] - mine;
+    if (lane == 63) wave_total[wv] = incl;
+    __syncthreads();
+    uint32_t before = 0, total = 0;
+    for (uint32_t w = 0; w < 16; ++w) {
+        const uint32_t t = wave_total[w];
+        if (w < wv) before += t;
+        total += t;
+    }
+    uint32_t at = before + incl - mine;
     for (uint32_t u = 0; u < per; ++u) {
         const uint32_t i = tid * per + u;
         if (opens(i)) a.chunk_start[at++] = i;
     }
-    if (tid == 1023) {
-        a.chunk_start[scan[1023]] = a.n_ids;  // end marker
-        a.chunk_start[-1] = scan[1023];       // number of chunks
+    if (tid == 0) {
+        a.chunk_start[total] = a.n_ids;  // end marker
+        a.chunk_start[-1] = total;       // number of chunks
     }
 }
 
