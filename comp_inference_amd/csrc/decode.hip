@@ -2,16 +2,14 @@
 //
 // Work decomposition for the default 32-column tile: one wavefront per tile.  Lanes 0..31
 // own the top-half streams of columns 0..31, lanes 32..63 the bottom-half streams, so one
-// stored byte row (64 bytes) is one byte per lane.  Eight waves (eight neighbouring column
-// tiles) form a workgroup and share one LDS slot table; each wave stages its whole tile body
-// in LDS with 16-byte coalesced loads and then runs the sequential decode out of LDS.
+// stored byte row (64 bytes) is one byte per lane.  One workgroup per CU stays resident for the
+// launch and shares one LDS slot table; each wavefront stages a whole tile body in LDS with
+// 16-byte coalesced loads, runs the sequential decode out of LDS and takes the next tile.
 #include "ci_common.h"
 #include "rans_device.h"
 #include "fast_tile.h"
 
 namespace ci {
-
-constexpr int kDecWaves = 8;
 
 struct DecodeArgs {
     const uint8_t *stream;
@@ -25,94 +23,14 @@ struct DecodeArgs {
     uint8_t *out_exp;
     const uint8_t *man_tiled;
     uint16_t *out_bf16;
-    uint32_t stage_bytes;  // LDS bytes per wave for the tile body
+    uint32_t man_aligned;  // sign|mantissa plane may be read as dwords
 };
 
-// The decode loop of one lane.  kFull: every lane takes all `half` steps (no row or column
-// masking).  kMerge: emit bf16 instead of the exponent byte.
-template <bool kFull, bool kMerge, typename Bytes>
-__device__ __forceinline__ void decode_lane(Bytes &src, uint32_t x, const uint2 *tab, uint32_t half,
-                                            uint32_t my_steps, uint8_t *out_row0, uint32_t lane_off,
-                                            uint32_t N, const uint8_t *man_row0, uint32_t man_off,
-                                            uint16_t *out16_row0) {
-    for (uint32_t i = 0; i < half; ++i) {
-        if (kFull || i < my_steps) {
-            uint32_t w = decode_symbol(x, tab);
-            uint32_t sym = w >> 24;
-            src.renorm(x);
-            src.renorm(x);
-            if (kMerge) {
-                uint32_t man = man_row0[(size_t)i * 32 + man_off];
-                out16_row0[(size_t)i * N + lane_off] = (uint16_t)assemble_bf16(sym, man);
-            } else {
-                out_row0[(size_t)i * N + lane_off] = (uint8_t)sym;
-            }
-        }
-    }
-}
-
-template <bool kMerge>
-__global__ __launch_bounds__(kDecWaves *kWave) void decode_tiled32_kernel(DecodeArgs a) {
-    extern __shared__ __align__(16) uint8_t lds[];
-    uint2 *tab = reinterpret_cast<uint2 *>(lds);
-    const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
-    uint8_t *stage = lds + kSlotTableBytes + (size_t)wave * a.stage_bytes;
-
-    build_slot_table(tab, a.tables, a.slot_map, tid, kDecWaves * kWave);
-
-    const uint32_t tile = blockIdx.x * kDecWaves + wave;
-    const bool have_tile = tile < a.num_tiles;
-    uint32_t depth = 0;
-    uint64_t base = 0;
-    bool in_lds = false;
-    if (have_tile) {
-        base = a.tile_offsets[tile];
-        depth = a.tile_max_lens[tile];
-        // A body that would run past the stream is treated as empty rather than read.
-        if (base + (uint64_t)depth * 64 > a.stream_len) depth = 0;
-        in_lds = depth * 64u <= a.stage_bytes;
-        if (in_lds) stage_to_lds(stage, a.stream + base, depth * 64u, lane);
-    }
-    __syncthreads();
-    if (!have_tile) return;
-
-    const uint32_t tk = tile / a.tiles_n, tn = tile % a.tiles_n;
-    const uint32_t half = a.th / 2, hsel = lane / 32, c = lane % 32;
-    const uint32_t row0 = tk * a.th, col0 = tn * 32;
-    const uint32_t my_row0 = row0 + hsel * half;
-    uint32_t my_steps = 0;
-    if (col0 + c < a.N && my_row0 < a.K) my_steps = min(half, a.K - my_row0);
-    const bool full = __builtin_amdgcn_ballot_w64(my_steps != half) == 0;
-
-    uint32_t x = a.states[(size_t)tile * 64 + lane];
-    // wave-uniform row base + 32-bit per-lane offset keeps the address math scalar
-    uint8_t *out_row0 = kMerge ? nullptr : a.out_exp + (size_t)row0 * a.N + col0;
-    uint16_t *out16_row0 = kMerge ? a.out_bf16 + (size_t)row0 * a.N + col0 : nullptr;
-    const uint32_t lane_off = hsel * half * a.N + c;
-    const uint8_t *man_row0 = kMerge ? a.man_tiled + (size_t)tile * a.th * 32 : nullptr;
-    const uint32_t man_off = hsel * half * 32 + c;
-
-    if (in_lds) {
-        LdsBytes src;
-        src.init(stage, depth, 64, lane);
-        if (full)
-            decode_lane<true, kMerge>(src, x, tab, half, my_steps, out_row0, lane_off, a.N, man_row0,
-                                      man_off, out16_row0);
-        else
-            decode_lane<false, kMerge>(src, x, tab, half, my_steps, out_row0, lane_off, a.N, man_row0,
-                                       man_off, out16_row0);
-    } else {
-        GlobalBytes src;
-        src.init(a.stream + base, depth, 64, lane);
-        decode_lane<false, kMerge>(src, x, tab, half, my_steps, out_row0, lane_off, a.N, man_row0,
-                                   man_off, out16_row0);
-    }
-}
-
-// Exponent-plane output through the hand-scheduled loop (fast_tile.h): scaled state, tile body
-// staged transposed.  Tiles that do not qualify (ragged, odd half height, body deeper than a
-// lane stride) take the same arithmetic with guarded byte reads from global memory.
-template <uint32_t kStride>
+// One tile through the hand-scheduled loops (fast_tile.h): scaled state, tile body staged
+// transposed.  kMerge = false writes the exponent plane; kMerge = true joins it with the tile's
+// sign|mantissa bytes and writes bf16.  Tiles that do not qualify (ragged, odd block counts, body
+// deeper than a lane stride) take the same arithmetic with guarded byte reads from global memory.
+template <uint32_t kStride, bool kMerge>
 __device__ __forceinline__ void decode_one_tile(const DecodeArgs &a, uint32_t tile, const uint2 *tab,
                                                 uint8_t *stage, int lane) {
     const uint32_t tk = tile / a.tiles_n, tn = tile % a.tiles_n;
@@ -126,27 +44,58 @@ __device__ __forceinline__ void decode_one_tile(const DecodeArgs &a, uint32_t ti
     uint32_t my_steps = 0;
     if (col0 + c < a.N && my_row0 < a.K) my_steps = min(half, a.K - my_row0);
     const bool full = __builtin_amdgcn_ballot_w64(my_steps != half) == 0;
-    const bool fast = full && depth >= 2 && depth < kStride && half % 2 == 0 && half >= 2 &&
-                      (uint64_t)a.K * a.N < (1ull << 32) && (uint32_t)(uintptr_t)tab == 0;
+    const bool fast = full && depth >= 2 && depth < kStride && half % (kMerge ? 8 : 2) == 0 && half >= 2 &&
+                      (uint64_t)a.K * a.N < (1ull << (kMerge ? 31 : 32)) && (uint32_t)(uintptr_t)tab == 0 &&
+                      (!kMerge || a.man_aligned);
+    const uint8_t *man_half = kMerge ? a.man_tiled + (size_t)tile * a.th * 32 + (size_t)hsel * half * 32 : nullptr;
     if (fast) {
         stage_body<kStride>(stage, a.stream + base, depth, lane);
         // LDS operations of one wavefront complete in order: the reads below see the writes above
         FastLane st;
         st.init<kStride>(stage, depth, lane, state);
-        const uint64_t ob = reinterpret_cast<uint64_t>(a.out_exp + (size_t)row0 * a.N + col0);
-        // readfirstlane returns a signed int: widen through uint32_t
-        const uint32_t ob_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(ob >> 32));
-        const uint32_t ob_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)ob);
-        decode_tile_asm(st, ((uint64_t)ob_hi << 32) | (uint64_t)ob_lo, hsel * half * a.N + c, a.N, half / 2);
+        if (kMerge) {
+            // blocks of eight rows: sign|mantissa dwords of the next block are loaded while this one decodes
+            const uint32_t man_sel = 0x04040000u + (c & 3u) * 0x01010101u;
+            const uint32_t *mrow = reinterpret_cast<const uint32_t *>(man_half + (c & ~3u));  // + 8 dwords per row
+            uint16_t *o = a.out_bf16 + (size_t)my_row0 * a.N + col0 + c;
+            const uint32_t nblk = half / 8;
+            uint32_t mcur[8], mnext[8];
+#pragma unroll
+            for (int r = 0; r < 8; ++r) mcur[r] = mrow[r * 8];
+            for (uint32_t blk = 0; blk < nblk; ++blk) {
+                const uint32_t *nrow = mrow + (size_t)(blk + 1 < nblk ? blk + 1 : blk) * 64;
+#pragma unroll
+                for (int r = 0; r < 8; ++r) mnext[r] = nrow[r * 8];
+                uint32_t w[4];
+                decode8_weights_asm(st, mcur, man_sel, w);
+#pragma unroll
+                for (int d = 0; d < 4; ++d) {
+                    o[(size_t)(blk * 8 + 2 * d) * a.N] = (uint16_t)w[d];
+                    o[(size_t)(blk * 8 + 2 * d + 1) * a.N] = (uint16_t)(w[d] >> 16);
+                }
+#pragma unroll
+                for (int r = 0; r < 8; ++r) mcur[r] = mnext[r];
+            }
+        } else {
+            const uint64_t ob = reinterpret_cast<uint64_t>(a.out_exp + (size_t)row0 * a.N + col0);
+            // readfirstlane returns a signed int: widen through uint32_t
+            const uint32_t ob_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(ob >> 32));
+            const uint32_t ob_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)ob);
+            decode_tile_asm(st, ((uint64_t)ob_hi << 32) | (uint64_t)ob_lo, hsel * half * a.N + c, a.N, half / 2);
+        }
     } else {
         GlobalBytes src;
         src.init(a.stream + base, depth, 64, lane);
         uint32_t X = state << 3;
-        uint8_t *o = a.out_exp + (size_t)my_row0 * a.N + col0 + c;
+        const size_t o0 = (size_t)my_row0 * a.N + col0 + c;
         for (uint32_t i = 0; i < my_steps; ++i) {
-            o[(size_t)i * a.N] = (uint8_t)(decode_symbol_scaled(X, tab) >> 24);
+            const uint32_t sym = decode_symbol_scaled(X, tab) >> 24;
             src.renorm_scaled(X);
             src.renorm_scaled(X);
+            if (kMerge)
+                a.out_bf16[o0 + (size_t)i * a.N] = (uint16_t)assemble_bf16(sym, man_half[(size_t)i * 32 + c]);
+            else
+                a.out_exp[o0 + (size_t)i * a.N] = (uint8_t)sym;
         }
     }
 }
@@ -154,7 +103,7 @@ __device__ __forceinline__ void decode_one_tile(const DecodeArgs &a, uint32_t ti
 // Wavefront `wave` of workgroup `j` (of the `n_wg` that share this tensor) decodes the tiles
 // (slot * n_wg + j), slot = wave, wave + kWaves, ...: a workgroup's concurrent tiles are n_wg
 // apart, so every workgroup gets the same number of tiles to within one.
-template <int kWaves, uint32_t kStride>
+template <int kWaves, uint32_t kStride, bool kMerge>
 __device__ __forceinline__ void decode_wave_tiles(const DecodeArgs &a, uint32_t j, uint32_t n_wg, const uint2 *tab,
                                                   uint8_t *lds, int wave, int lane) {
     if (wave >= kWaves) return;
@@ -162,7 +111,7 @@ __device__ __forceinline__ void decode_wave_tiles(const DecodeArgs &a, uint32_t 
     for (uint32_t slot = wave;; slot += kWaves) {
         const uint64_t tile = (uint64_t)slot * n_wg + j;
         if (tile >= a.num_tiles) break;
-        decode_one_tile<kStride>(a, (uint32_t)tile, tab, stage, lane);
+        decode_one_tile<kStride, kMerge>(a, (uint32_t)tile, tab, stage, lane);
     }
 }
 
@@ -177,6 +126,7 @@ struct DecodeBatchArgs {
     uint32_t n;
 };
 
+template <bool kMerge>
 __global__ __launch_bounds__(kPersistWaves *kWave) void decode_tiled32_persist_kernel(DecodeBatchArgs b) {
     extern __shared__ __align__(16) uint8_t lds[];
     const uint2 *tab = reinterpret_cast<const uint2 *>(lds);
@@ -188,11 +138,11 @@ __global__ __launch_bounds__(kPersistWaves *kWave) void decode_tiled32_persist_k
 
     const uint32_t cls = persist_prologue(lds, a.tables, a.slot_map, a.tile_max_lens, a.num_tiles, j, n_wg);
     if (cls == 2u)
-        decode_wave_tiles<8, kDepthDeep>(a, j, n_wg, tab, lds, wave, lane);
+        decode_wave_tiles<8, kDepthDeep, kMerge>(a, j, n_wg, tab, lds, wave, lane);
     else if (cls == 1u)
-        decode_wave_tiles<10, kDepthMedium>(a, j, n_wg, tab, lds, wave, lane);
+        decode_wave_tiles<10, kDepthMedium, kMerge>(a, j, n_wg, tab, lds, wave, lane);
     else
-        decode_wave_tiles<kPersistWaves, kDepthShallow>(a, j, n_wg, tab, lds, wave, lane);
+        decode_wave_tiles<kPersistWaves, kDepthShallow, kMerge>(a, j, n_wg, tab, lds, wave, lane);
 }
 
 // Any tile width: one thread per stream, bytes read where they lie.  Used for widths other
@@ -246,7 +196,7 @@ static int cu_count(uint32_t *out) {
 
 // Launch the persistent kernel over the (already checked) tensors of `b`: the device's CUs are
 // divided among the tensors in proportion to their tile counts.
-static int launch_persist(DecodeBatchArgs &b, hipStream_t s) {
+static int launch_persist(DecodeBatchArgs &b, bool merge, hipStream_t s) {
     uint32_t cus = 0;
     if (int rc = cu_count(&cus)) return rc;
     uint64_t total = 0;
@@ -280,11 +230,17 @@ static int launch_persist(DecodeBatchArgs &b, hipStream_t s) {
     b.first_block[b.n] = blocks;
     static bool attr_set = false;  // a per-function attribute; setting it again is harmless
     if (!attr_set) {
-        CI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(decode_tiled32_persist_kernel),
+        CI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(decode_tiled32_persist_kernel<false>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit));
+        CI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(decode_tiled32_persist_kernel<true>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit));
         attr_set = true;
     }
-    hipLaunchKernelGGL(decode_tiled32_persist_kernel, dim3(blocks), dim3(kPersistWaves * kWave), kLdsLimit, s, b);
+    const dim3 grid(blocks), block(kPersistWaves * kWave);
+    if (merge)
+        hipLaunchKernelGGL(decode_tiled32_persist_kernel<true>, grid, block, kLdsLimit, s, b);
+    else
+        hipLaunchKernelGGL(decode_tiled32_persist_kernel<false>, grid, block, kLdsLimit, s, b);
     CI_LAUNCH_CHECK("decode_tiled32_persist_kernel");
     return CI_OK;
 }
@@ -330,11 +286,11 @@ extern "C" int ci_decode_tiled_ilp2_batch(const ci_decode_item *h_items, uint32_
             a.out_exp = it.d_out_exp;
             a.man_tiled = nullptr;
             a.out_bf16 = nullptr;
-            a.stage_bytes = 0;
+            a.man_aligned = 0;
             ++b.n;
         }
         if (b.n == 0) continue;
-        if (int rc = launch_persist(b, s)) return rc;
+        if (int rc = launch_persist(b, false, s)) return rc;
     }
     return CI_OK;
 }
@@ -376,23 +332,13 @@ extern "C" int ci_decode_tiled_ilp2(const uint8_t *d_stream, uint64_t stream_len
     a.out_bf16 = d_out_bf16;
     hipStream_t s = static_cast<hipStream_t>(stream);
 
+    a.man_aligned = merge && aligned(d_man_tiled, 4) ? 1u : 0u;
     if (tile_width == 32 && aligned(d_stream, 16)) {
-        a.stage_bytes = 14336;  // 224 byte rows per tile; deeper tiles read from global memory
-        const uint32_t lds_bytes = kSlotTableBytes + kDecWaves * a.stage_bytes;
-        const dim3 grid(ceil_div(a.num_tiles, kDecWaves)), block(kDecWaves * kWave);
-        if (merge) {
-            CI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(decode_tiled32_kernel<true>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes));
-            hipLaunchKernelGGL(decode_tiled32_kernel<true>, grid, block, lds_bytes, s, a);
-            CI_LAUNCH_CHECK("decode_tiled32_kernel");
-        } else {
-            DecodeBatchArgs b;
-            b.n = 1;
-            b.item[0] = a;
-            if (int rc = launch_persist(b, s)) return rc;
-        }
+        DecodeBatchArgs b;
+        b.n = 1;
+        b.item[0] = a;
+        if (int rc = launch_persist(b, merge, s)) return rc;
     } else {
-        a.stage_bytes = 0;
         const uint64_t streams = (uint64_t)a.num_tiles * 2 * tile_width;
         const dim3 grid((uint32_t)((streams + 255) / 256)), block(256);
         if (merge)
