@@ -251,6 +251,106 @@ __global__ __launch_bounds__(kLinMaxWaves *kWave) void fused_linear32_kernel(Lin
     }
 }
 
+// The same tile work with workgroups resident for the launch (fast_tile.h) and every tile on its
+// own: wavefront w of workgroup j takes tiles j + (w + 11 i) * gridDim.x and writes its 32-column
+// partial product to the fp32 workspace [tiles_k][M][N], which the reduction kernel sums in k order.
+// For weights with more tiles than the chip holds at once (fused gate/up projections): the
+// 8-wavefront workgroups of the kernel above would run in two full rounds.  M <= 32 * MB.
+template <int MB, uint32_t kStride>
+__device__ __forceinline__ void linear_one_tile(const LinearArgs &a, uint32_t tile, const uint2 *tab, uint8_t *stage,
+                                                int lane) {
+    const uint32_t tk = tile / a.tiles_n, tn = tile % a.tiles_n;
+    const uint32_t half = a.th / 2, hsel = lane / 32, c = lane % 32;
+    const uint32_t col0 = tn * 32, k0 = tk * a.th + hsel * half;
+    const uint64_t base = a.tile_offsets[tile];
+    uint32_t depth = a.tile_max_lens[tile];
+    const uint32_t state = a.states[(size_t)tile * 64 + lane];
+    if (base + (uint64_t)depth * 64 > a.stream_len) depth = 0;
+    uint32_t my_steps = 0;
+    if (col0 + c < a.N && k0 < a.K) my_steps = min(half, a.K - k0);
+    const bool full = __builtin_amdgcn_ballot_w64(my_steps != half) == 0;
+    const bool fast = full && a.fast_ok && depth >= 2 && depth < kStride && half % 16 == 0 &&
+                      (uint32_t)(uintptr_t)tab == 0;
+    const uint32_t m = c;  // row of x this lane feeds to the (first) MFMA
+    const bool m_ok = m < a.M, m2_ok = MB == 2 && m + 32 < a.M;
+    f32x16 acc, acc2;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[v] = acc2[v] = 0.f;
+    const uint32_t xrow_elems = (m_ok ? m : 0) * a.x_stride + k0;
+    const uint32_t xrow2_elems = (m2_ok ? m + 32 : 0) * a.x_stride + k0;
+    const size_t man_tile = (size_t)tile * a.th * 32;
+    if (fast) {
+        stage_body<kStride>(stage, a.stream + base, depth, lane);
+        FastLane st;
+        st.init<kStride>(stage, depth, lane, state);
+        const uint64_t mbase = reinterpret_cast<uint64_t>(a.man_tiled + man_tile);
+        // readfirstlane returns a signed int: widen through uint32_t, not by sign extension
+        const uint32_t mb_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(mbase >> 32));
+        const uint32_t mb_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)mbase);
+        const uint64_t mb_u = ((uint64_t)mb_hi << 32) | (uint64_t)mb_lo;
+        const uint32_t moff = hsel * half * 32 + (c & ~3u);
+        const uint32_t man_sel = 0x04040000u + (c & 3u) * 0x01010101u;
+        uint64_t xb = reinterpret_cast<uint64_t>(a.x);
+        uint32_t xo = xrow_elems * 2u, xo2 = xrow2_elems * 2u, xstep = 16;
+        if (a.xf) {
+            const uint32_t kbs = a.K / 8;
+            xb = reinterpret_cast<uint64_t>(a.xf);
+            xo = ((k0 / 8) * 32 + c) * 16;
+            xo2 = xo + kbs * 32 * 16;
+            xstep = 32 * 16;
+        }
+        if (MB == 2)
+            linear_tile_asm2(st, acc, acc2, mb_u, moff, xb, xo, xo2, xstep, man_sel, half / 8);
+        else
+            linear_tile_asm(st, acc, mb_u, moff, xb, xo, xstep, man_sel, half / 8);
+    } else {
+        const uint8_t *man = a.man_tiled + man_tile + (size_t)hsel * half * 32 + c;
+        GlobalBytes src;
+        src.init(a.stream + base, depth, 64, lane);
+        linear_tile_guarded(src, state << 3, tab, a.K, half, my_steps, man, a.x + xrow_elems, m_ok, k0, acc);
+        if (MB == 2) {
+            src.init(a.stream + base, depth, 64, lane);
+            linear_tile_guarded(src, state << 3, tab, a.K, half, my_steps, man, a.x + xrow2_elems, m2_ok, k0, acc2);
+        }
+    }
+    // MFMA 32x32 result layout: register v of lane l is row (v/4)*8 + (l/32)*4 + v%4 (= column of
+    // the tile), column l%32 (= row m of x)
+#pragma unroll
+    for (int g = 0; g < MB; ++g) {
+        const f32x16 &part = g ? acc2 : acc;
+        const uint32_t mg = m + 32 * g;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const uint32_t n = col0 + (v / 4) * 8 + hsel * 4 + (v % 4);
+            if (mg < a.M && n < a.N) a.partial[((size_t)tk * a.M + mg) * a.N + n] = part[v];
+        }
+    }
+}
+
+template <int MB, int kWaves, uint32_t kStride>
+__device__ __forceinline__ void linear_wave_tiles(const LinearArgs &a, const uint2 *tab, uint8_t *lds, int wave, int lane) {
+    if (wave >= kWaves) return;
+    uint8_t *stage = persist_stage<kWaves, kStride>(lds, wave);
+    const uint64_t num_tiles = (uint64_t)a.tiles_k * a.tiles_n;
+    for (uint64_t tile = (uint64_t)wave * gridDim.x + blockIdx.x; tile < num_tiles; tile += (uint64_t)kWaves * gridDim.x)
+        linear_one_tile<MB, kStride>(a, (uint32_t)tile, tab, stage, lane);
+}
+
+template <int MB>
+__global__ __launch_bounds__(kPersistWaves *kWave) void fused_linear32_resident_kernel(LinearArgs a) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    const uint2 *tab = reinterpret_cast<const uint2 *>(lds);
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    const uint32_t cls = persist_prologue(lds, a.tables, a.slot_map, a.tile_max_lens, a.tiles_k * a.tiles_n, blockIdx.x,
+                                          gridDim.x);
+    if (cls == 2u)
+        linear_wave_tiles<MB, 8, kDepthDeep>(a, tab, lds, wave, lane);
+    else if (cls == 1u)
+        linear_wave_tiles<MB, 10, kDepthMedium>(a, tab, lds, wave, lane);
+    else
+        linear_wave_tiles<MB, kPersistWaves, kDepthShallow>(a, tab, lds, wave, lane);
+}
+
 // Any tile width, either tiled layout: one thread per stream, eight rows of x per pass.
 // Partial sums (one per stream, i.e. per (k-tile[, half])) go to the fp32 workspace.
 // grid: (ceil(streams / 256), ceil(M / 8))
@@ -346,16 +446,24 @@ static size_t x_fragment_bytes(uint32_t M, uint32_t K, bool fast_plan) {
 }
 
 struct LinearPlan {
-    bool fast;
+    bool fast, resident;
     uint32_t kw, nw, P;
 };
 
-static LinearPlan plan_linear(uint32_t K, uint32_t th, uint32_t tw, uint32_t tiles_n, bool dense,
+// Tiles from which every tile gets its own wavefront of a resident workgroup: more than a chip of
+// 8-wavefront workgroups holds at once (256 CUs x 8).
+constexpr uint32_t kResidentMinTiles = 2049;
+
+static LinearPlan plan_linear(uint32_t M, uint32_t K, uint32_t th, uint32_t tw, uint32_t tiles_n, bool dense,
                               bool stream_aligned) {
     LinearPlan p;
     const uint32_t tiles_k = ceil_div(K, th);
     p.fast = !dense && tw == 32 && th % 16 == 0 && stream_aligned;
-    if (p.fast) {
+    p.resident = p.fast && M <= 64 && tiles_k >= 2 && (uint64_t)tiles_k * tiles_n >= kResidentMinTiles;
+    if (p.resident) {
+        p.kw = p.nw = 1;
+        p.P = tiles_k;
+    } else if (p.fast) {
         p.P = ceil_div(tiles_k, kLinMaxWaves);
         p.kw = ceil_div(tiles_k, p.P);
         p.nw = kLinMaxWaves / p.kw;
@@ -376,8 +484,8 @@ extern "C" size_t ci_fused_linear_workspace_bytes(uint32_t M, uint32_t K, uint32
                                                   uint32_t tile_width, int dense) {
     if (tile_height == 0 || tile_width == 0) return 0;
     // sized for the slower plan so that the answer does not depend on pointer alignment
-    const LinearPlan fast = plan_linear(K, tile_height, tile_width, ceil_div(N, tile_width), dense != 0, true);
-    const LinearPlan slow = plan_linear(K, tile_height, tile_width, ceil_div(N, tile_width), dense != 0, false);
+    const LinearPlan fast = plan_linear(M, K, tile_height, tile_width, ceil_div(N, tile_width), dense != 0, true);
+    const LinearPlan slow = plan_linear(M, K, tile_height, tile_width, ceil_div(N, tile_width), dense != 0, false);
     const uint32_t P = fast.P > slow.P ? fast.P : slow.P;
     const size_t partial = P > 1 ? (size_t)P * M * N * sizeof(float) : 0;
     return ((partial + 15) & ~(size_t)15) + x_fragment_bytes(M, K, fast.fast);
@@ -423,7 +531,7 @@ static int fused_linear_impl(const uint16_t *d_x, uint32_t M, uint32_t K, uint32
     a.tiles_k = ceil_div(K, th);
     a.fast_ok = aligned(d_x, 16) && x_stride % 8 == 0 && aligned(d_man_tiled, 4) &&
                 (uint64_t)M * x_stride * 2 < (1ull << 31);
-    const LinearPlan p = plan_linear(K, th, tw, a.tiles_n, dense, aligned(d_stream, 16));
+    const LinearPlan p = plan_linear(M, K, th, tw, a.tiles_n, dense, aligned(d_stream, 16));
     a.kw = p.kw;
     a.nw = p.nw;
     a.P = p.P;
@@ -450,7 +558,25 @@ static int fused_linear_impl(const uint16_t *d_x, uint32_t M, uint32_t K, uint32
         }
     }
 
-    if (p.fast) {
+    if (p.resident) {
+        int dev = 0, cus = 0;
+        CI_HIP(hipGetDevice(&dev));
+        CI_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+        static bool res_attr_set = false;
+        if (!res_attr_set) {
+            CI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(fused_linear32_resident_kernel<1>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit));
+            CI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(fused_linear32_resident_kernel<2>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit));
+            res_attr_set = true;
+        }
+        const dim3 grid(cus > 0 ? cus : 1), block(kPersistWaves * kWave);
+        if (M > 32)
+            hipLaunchKernelGGL(fused_linear32_resident_kernel<2>, grid, block, kLdsLimit, s, a);
+        else
+            hipLaunchKernelGGL(fused_linear32_resident_kernel<1>, grid, block, kLdsLimit, s, a);
+        CI_LAUNCH_CHECK("fused_linear32_resident_kernel");
+    } else if (p.fast) {
         const uint32_t waves = p.kw * p.nw;
         const uint32_t lds_bytes = kSlotTableBytes + waves * kFastStageBytes;
         static bool attr_set = false;

@@ -52,6 +52,8 @@ def test_fused_linear_fast_path(oracle, M, K, N, th, tw):
     (1300, 80, 1024, 32, 3),     # ragged K and N
     (1000, 70, 512, 32, 2),
     (9000, 32, 1024, 32, 1),
+    (2048, 32800, 1024, 32, 3),  # more tiles than the chip holds at once: resident workgroups, a partial per k-tile
+    (2048, 32800, 1024, 32, 40),
     (256, 128, 64, 16, 4),       # other tile widths: generic kernel
     (384, 256, 128, 64, 9),
     (256, 256, 256, 128, 1),
