@@ -150,8 +150,34 @@ def cpu_baseline(layer: list[Compressed], budget_s: float = 15.0):
             assert all(np.array_equal(o, c.exp_host) for o, c in zip(outs, layer))
             checked = True
     med = float(np.median(times[1:])) if len(times) > 1 else times[0]
+    # the CPU route to one GEMV on the gate projection: decode, join the planes, torch.matmul (all cores)
+    gate = next(c for c in layer if c.name == "gate")
+    ga = args[[c.name for c in layer].index("gate")]
+    t0 = time.time()
+    e = ro.decode_tiled_ilp2(*ga)
+    t_dec = time.time() - t0
+    man = ci_uninterleave(gate)
+    t0 = time.time()
+    w = torch.from_numpy(ro.merge_bf16(e, man).view(np.int16)).view(torch.bfloat16)
+    t_merge = time.time() - t0
+    x = torch.randn(1, gate.K, generator=torch.Generator("cpu").manual_seed(2)).to(torch.bfloat16)
+    torch.set_num_threads(int(cores))
+    torch.matmul(x, w)
+    t0 = time.time()
+    for _ in range(3):
+        torch.matmul(x, w)
+    t_mm = (time.time() - t0) / 3
     return {"value": round(total / med / 1e9, 3), "unit": "GB/s", "cores": int(cores), "kind": "port",
-            "sample": f"whole layer ({total / 1e6:.0f} M symbols), {len(times)} passes, median, OpenMP over tiles"}
+            "sample": f"whole layer ({total / 1e6:.0f} M symbols), {len(times)} passes, median, OpenMP over tiles",
+            "gate_gemv_M1_ms": {"decode": round(t_dec * 1e3, 2), "merge_planes": round(t_merge * 1e3, 2),
+                                "torch_matmul_bf16": round(t_mm * 1e3, 2)}}
+
+
+def ci_uninterleave(c: "Compressed") -> np.ndarray:
+    """Row-major sign|mantissa plane of a compressed tensor (host)."""
+    import comp_inference_amd as ci
+
+    return ci.uninterleave_mantissas(c.man.cpu(), c.K, c.N, c.th, c.tw).numpy()
 
 
 def main() -> int:

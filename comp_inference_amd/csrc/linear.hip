@@ -145,13 +145,14 @@ __global__ __launch_bounds__(kLinMaxWaves *kWave) void fused_linear32_kernel(Lin
     const uint32_t tile = tk * a.tiles_n + tn;
     const uint32_t half = a.th / 2, hsel = lane / 32, c = lane % 32;
     const uint32_t col0 = tn * 32, k0 = tk * a.th + hsel * half;
-    uint32_t depth = 0, my_steps = 0;
+    uint32_t depth = 0, my_steps = 0, state = 0;
     uint64_t base = 0;
     bool fast = false;
     StageRegs body;
     if (have_tile) {
         base = a.tile_offsets[tile];
         depth = a.tile_max_lens[tile];
+        state = a.states[(size_t)tile * 64 + lane];
         if (base + (uint64_t)depth * 64 > a.stream_len) depth = 0;
         if (col0 + c < a.N && k0 < a.K) my_steps = min(half, a.K - k0);
         const bool full = __builtin_amdgcn_ballot_w64(my_steps != half) == 0;
@@ -183,7 +184,6 @@ __global__ __launch_bounds__(kLinMaxWaves *kWave) void fused_linear32_kernel(Lin
                                                                        // accumulator columns are never stored
         const uint32_t xrow2_elems = (m2_ok ? m + 32 : 0) * a.x_stride + k0;
         const size_t man_tile = (size_t)tile * a.th * 32;
-        const uint32_t state = a.states[(size_t)tile * 64 + lane];
         if (fast) {
             FastLane st;
             st.init(stage, depth, lane, state);
