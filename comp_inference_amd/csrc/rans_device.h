@@ -58,29 +58,6 @@ __device__ __forceinline__ uint32_t decode_symbol_scaled(uint32_t &X, const uint
     return e.x;
 }
 
-// Byte source: a tile body staged in LDS exactly as stored (rows of `row_bytes`, every stream
-// bottom-aligned).  `pos` is the byte offset of the next byte of this lane's stream and `nxt`
-// holds that byte already (read one step ahead so that the LDS latency stays off the state
-// dependency chain).  An exhausted stream walks to negative offsets; LDS reads outside the
-// allocation return zero, and a well-formed stream never asks for those bytes.
-struct LdsBytes {
-    const uint8_t *cur;  // LDS address of the next byte of this lane's stream
-    uint32_t nxt;        // that byte, already read
-    uint32_t row_bytes;
-    __device__ __forceinline__ void init(const uint8_t *b, uint32_t depth, uint32_t rb, uint32_t q) {
-        row_bytes = rb;
-        cur = b + (depth - 1) * rb + q;
-        nxt = depth ? *cur : 0;
-    }
-    __device__ __forceinline__ void renorm(uint32_t &x) {
-        if (x < kRansL) {
-            x = (x << 8) | nxt;
-            cur -= row_bytes;
-            nxt = *cur;
-        }
-    }
-};
-
 // Byte source reading the stream where it lies in global memory, with the reference's
 // "row >= 0" guard (comp_inference/rans_triton.py:108).  Used when a tile body does not fit
 // the LDS staging area.
@@ -123,13 +100,6 @@ struct DenseBytes {
         }
     }
 };
-
-// Copy `nbytes` (a multiple of 16, source 16-byte aligned) into LDS with one wave.
-__device__ __forceinline__ void stage_to_lds(uint8_t *dst, const uint8_t *__restrict__ src,
-                                             uint32_t nbytes, int lane) {
-    for (uint32_t off = (uint32_t)lane * 16; off < nbytes; off += kWave * 16)
-        *reinterpret_cast<u32x4 *>(dst + off) = *reinterpret_cast<const u32x4 *>(src + off);
-}
 
 // bf16 bit pattern from exponent symbol and sign|mantissa byte
 // (comp_inference/rans_triton.py:12-28).
