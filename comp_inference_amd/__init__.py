@@ -23,11 +23,13 @@ from .embedding_hip import (
     fused_rans_embedding_uncoalesced,
 )
 from .linear_hip import (
+    dense_matmul,
     fused_rans_linear,
     fused_rans_linear_triton,
     fused_rans_linear_triton_uncoalesced,
     fused_rans_linear_uncoalesced,
     splitk_reduce,
+    triton_matmul,
 )
 from .rans_hip import (
     rans_decomp_flat,
@@ -52,6 +54,7 @@ from .pytorch_runtime import (
     swap_in_rans_modules,
 )
 from .rans_saving import (
+    load_compressed_model,
     pack_and_save_tensors,
     parse_rans_info,
     rans_tensors_for_module,

@@ -129,3 +129,20 @@ def splitk_reduce(workspace: torch.Tensor, bias=None, out=None):
 # Names under which the reference exports these ops (comp_inference/__init__.py:39-42).
 fused_rans_linear_triton = fused_rans_linear
 fused_rans_linear_triton_uncoalesced = fused_rans_linear_uncoalesced
+
+
+def dense_matmul(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """a[..., K] @ b[K, N] for an uncompressed bf16 weight, bf16 result shaped (*a.shape[:-1], N): the
+    reference's dense helper (`triton_matmul`, comp_inference/triton_gemm.py:324-338, a split-K GEMV for
+    one row and a block GEMM otherwise, fp32 accumulation).  A plain library GEMM: hipBLASLt through
+    torch.matmul, on the GPU only."""
+    _lib.require_device(a)
+    _lib.require_device(b)
+    a2 = a.reshape(-1, a.shape[-1])
+    if a2.dtype != torch.bfloat16:
+        a2 = a2.to(torch.bfloat16)
+    out = torch.matmul(a2, b.to(torch.bfloat16))
+    return out.view(*a.shape[:-1], b.shape[1])
+
+
+triton_matmul = dense_matmul

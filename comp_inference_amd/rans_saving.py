@@ -121,3 +121,67 @@ def save_rans_model_package(model, tokenizer, output_dir: str, fuse: bool = Fals
     path = os.path.join(output_dir, "model.safetensors")
     pack_and_save_tensors(model, path, fuse=fuse, tied_lm_head=tied_lm_head)
     return output_dir
+
+
+def _load_rans_layer(module, prefix: str, f, keys) -> None:
+    """Attributes of one compressed module from its `<prefix>.rans_*` tensors
+    (comp_inference/rans_saving.py:542-656).  Unlike the reference, tensors the writer does not store
+    (`rans_exp_sizes`) are optional, and the tile arrays are loaded whenever the file has them (the
+    reference reads them only into attributes that already exist, :599-613)."""
+    info = parse_rans_info(f.get_tensor(f"{prefix}.rans_info"))
+    module.compressed = "rans_bfloat16"
+    module.expanded_size = info["numel"]
+    module.input_shape = list(info["shape"])
+    module.tile_height = module.exponent_tile_height = info["tile_height"]
+    module.tile_width = module.exponent_tile_width = info["tile_width"]
+    if info["exp_compressed"] <= 0:
+        raise ValueError(f"Corrupt file: {prefix} has no coded exponent plane (a raw one is never written)")
+    module.exponent_compressed_weight = f.get_tensor(f"{prefix}.rans_exp_stream")
+    module.exponent_states = f.get_tensor(f"{prefix}.rans_exp_states")
+    if f"{prefix}.rans_exp_sizes" in keys:
+        module.exponent_output_sizes = f.get_tensor(f"{prefix}.rans_exp_sizes")
+    module.exponent_tables = f.get_tensor(f"{prefix}.rans_exp_tables")
+    module.exponent_slot_map = f.get_tensor(f"{prefix}.rans_exp_slot_map")
+    module.exponent_num_streams = info["exp_streams"]
+    module.exponent_stream_size = module.exponent_total_stream_size = module.exponent_compressed_weight.numel()
+    module.exponent_num_tiles_n, module.exponent_num_tiles_k = info["num_tiles_n"], info["num_tiles_k"]
+    dense = f"{prefix}.rans_exp_stream_offsets" in keys
+    module.exponent_uncoalesced_interleaving = dense
+    if dense:
+        module.exponent_stream_offsets = f.get_tensor(f"{prefix}.rans_exp_stream_offsets")
+    else:
+        module.exponent_tile_offsets = f.get_tensor(f"{prefix}.rans_exp_tile_offsets")
+        module.exponent_tile_max_lens = f.get_tensor(f"{prefix}.rans_exp_tile_max_lens")
+    if f"{prefix}.rans_man_raw" not in keys:
+        raise ValueError(f"Corrupt file: {prefix} marked uncompressed mantissa but raw data missing.")
+    module.mantissa_raw = f.get_tensor(f"{prefix}.rans_man_raw")
+    if f"{prefix}.bias" in keys and getattr(module, "bias", None) is not None:
+        module.bias.data = f.get_tensor(f"{prefix}.bias")
+    if hasattr(module, "weight"):
+        del module.weight  # the skeleton's weight; a forward before decompression must fail loudly
+
+
+def load_compressed_model(model, safetensors_path: str, device="cpu"):
+    """Load a compressed safetensors file into an initialised model skeleton: compressed modules
+    get their `exponent_*` / `mantissa_raw` attributes back (ready for rans_decompress_module_weight
+    or the Rans* runtime modules), everything else its parameters
+    (comp_inference/rans_saving.py:497-539)."""
+    from safetensors import safe_open
+
+    loaded = 0
+    with safe_open(safetensors_path, framework="pt", device=str(device)) as f:
+        keys = set(f.keys())
+        for name, module in model.named_modules():
+            if f"{name}.rans_info" in keys:
+                _load_rans_layer(module, name, f, keys)
+                loaded += 1
+                continue
+            for pname, param in module.named_parameters(recurse=False):
+                full = f"{name}.{pname}" if name else pname
+                if full in keys:
+                    tensor = f.get_tensor(full)
+                    if param.shape != tensor.shape:
+                        print(f"Warning: Shape mismatch for {full}. Expected {param.shape}, got {tensor.shape}")
+                    param.data = tensor
+    print(f"Model loaded. {loaded} layers are compressed.")
+    return model

@@ -122,3 +122,18 @@ def test_splitk_reduce_matches_torch_sum():
     want += bias
     got = splitk_reduce(ws, bias=bias)
     assert torch.equal(got, want)
+
+
+def test_dense_matmul_helper():
+    """The uncompressed helper the reference exports as triton_matmul: shapes and tolerance."""
+    from comp_inference_amd import triton_matmul
+
+    b = make_weight_kn(96, 512, seed=3).cuda()           # [K=512, N=96]
+    for shape in ((512,), (1, 512), (2, 3, 512)):
+        a = make_x(int(np.prod(shape[:-1])) if len(shape) > 1 else 1, 512, seed=len(shape)).view(*shape).cuda()
+        got = triton_matmul(a, b)
+        assert got.dtype == torch.bfloat16 and tuple(got.shape) == (*shape[:-1], 96)
+        want = torch.matmul(a.float().view(-1, 512), b.float()).view(*shape[:-1], 96)
+        assert torch.allclose(got.float(), want, atol=ATOL, rtol=RTOL)
+    with pytest.raises(RuntimeError):
+        triton_matmul(torch.zeros(1, 512, dtype=torch.bfloat16), b)

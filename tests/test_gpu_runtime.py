@@ -123,3 +123,37 @@ def test_modules_from_compressed():
     head.tie_to(re)
     h = torch.randn(2, 64).to(torch.bfloat16)
     assert torch.allclose(head(h.cuda()).float().cpu(), h.float() @ table.float().t(), atol=2e-2, rtol=2e-2)
+
+
+def test_load_compressed_model_into_skeleton(tmp_path):
+    """Package written from compressed modules -> attributes restored on a fresh skeleton ->
+    decompressed weights bit-equal to the originals; uncompressed parameters come back as they were."""
+    import comp_inference_amd as ci
+
+    src = _make()
+    originals = {n: p.detach().clone() for n, p in src.named_parameters()}
+    ci.rans_compress_module_weight(src.embed_tokens, tile_height=256, tile_width=32, transpose_weight=False)
+    ci.rans_compress_module_weight(src.up_proj, tile_height=64, tile_width=32)
+    ci.rans_compress_module_weight(src.down_proj, tile_height=64, tile_width=32, uncoalesced_interleaving=True)
+    path = str(tmp_path / "m.safetensors")
+    ci.pack_and_save_tensors(src, path)
+
+    dst = _make()
+    with torch.no_grad():
+        for p in dst.parameters():
+            p.add_(1.0)  # make sure nothing of the skeleton's own values survives
+    ci.load_compressed_model(dst, path)
+    for name in ("embed_tokens", "up_proj", "down_proj"):
+        mod = getattr(dst, name)
+        assert mod.compressed == "rans_bfloat16" and not hasattr(mod, "weight")
+    assert dst.down_proj.exponent_uncoalesced_interleaving and not dst.up_proj.exponent_uncoalesced_interleaving
+    assert torch.equal(dst.lm_head.weight.detach(), originals["lm_head.weight"])
+    ci.rans_decompress_module_weight(dst.up_proj)
+    ci.rans_decompress_module_weight(dst.down_proj)
+    ci.rans_decompress_module_weight(dst.embed_tokens)
+    assert torch.equal(dst.up_proj.weight.detach().cpu().view(torch.int16),
+                       originals["up_proj.weight"].t().contiguous().view(torch.int16))
+    assert torch.equal(dst.down_proj.weight.detach().cpu().view(torch.int16),
+                       originals["down_proj.weight"].t().contiguous().view(torch.int16))
+    assert torch.equal(dst.embed_tokens.weight.detach().cpu().view(torch.int16),
+                       originals["embed_tokens.weight"].view(torch.int16))
