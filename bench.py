@@ -285,6 +285,7 @@ def main() -> int:
                          "hbm_frac_compressed_bytes": round(nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
                          "effective_weight_GBs": round(2 * gate.K * gate.N / (us * 1e-6) / 1e9, 1),
                          "mfma_TFLOPs": round(2 * M * gate.K * gate.N / (us * 1e-6) / 1e12, 2),
+                         "mfma_util_vs_2500_TFLOPs": round(2 * M * gate.K * gate.N / (us * 1e-6) / 1e12 / 2500.0, 5),
                          "torch_matmul_bf16_us": round(us_ref, 2),
                          "torch_matmul_weight_GBs": round(2 * gate.K * gate.N / (us_ref * 1e-6) / 1e9, 1)})
         out["fused_gemv"] = {"layer": "gate K=4096 N=14336", "bytes_M1": gate.linear_bytes(1), "rows": rows}
