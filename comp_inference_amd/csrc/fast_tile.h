@@ -47,39 +47,52 @@ __device__ __forceinline__ void build_slot_table_x8(uint2 *tab, const uint32_t *
 }
 
 // Stage a tile body (rows of 64 bytes, row r at src + 64 r) into LDS transposed:
-// dst[lane * kFastStride + r] = src[64 r + lane].  Split in two so that all global loads of the
-// body are issued in groups of eight (128 rows) and other work -- the slot-table build -- can
-// run under the first group: stage_fetch issues the loads, stage_commit writes LDS.
+// dst[lane * kStride + r] = src[64 r + lane].  A lane fetches 8 columns of two neighbouring rows per
+// pass and writes the 8 row pairs as 16-bit LDS stores (LDS instructions, not VALU work, bound these
+// kernels: byte stores would be twice as many), so strides are even.  Split in two so that the
+// global loads of a group of eight passes (128 rows) are all issued before the first is needed and
+// other work -- the slot-table build -- can run under them: stage_fetch issues the loads,
+// stage_commit writes LDS.
 constexpr int kStagePasses = 8;                       // 16 rows per pass, 128 rows per group
 constexpr int kStageGroups = (kFastStride + 127) / 128;
 constexpr int stage_groups(uint32_t stride) { return (int)((stride + 127) / 128); }
 struct StageRegs {
-    u32x4 v[kStagePasses];
+    uint2 v[kStagePasses][2];  // [pass][row of the pair]: 8 columns each
 };
 
 // `row0` = first row of the group (a multiple of 128).
 __device__ __forceinline__ void stage_fetch(StageRegs &regs, const uint8_t *__restrict__ src, uint32_t row0,
                                             uint32_t depth, int lane) {
-    const uint32_t g = lane & 3, rr = lane >> 2;
+    const uint32_t g = lane & 7, rp = lane >> 3;
 #pragma unroll
     for (int p = 0; p < kStagePasses; ++p) {
-        const uint32_t r = row0 + p * 16 + rr;
-        regs.v[p] = (u32x4){0, 0, 0, 0};
-        if (r < depth) regs.v[p] = *reinterpret_cast<const u32x4 *>(src + (size_t)r * 64 + g * 16);
+        const uint32_t r = row0 + p * 16 + 2 * rp;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            regs.v[p][h] = make_uint2(0u, 0u);
+            if (r + h < depth) regs.v[p][h] = *reinterpret_cast<const uint2 *>(src + (size_t)(r + h) * 64 + g * 8);
+        }
     }
 }
 
+// `depth` may differ between lanes (two bodies side by side): rows at or past it are not written,
+// except that the odd row of a pair is written with a zero when the even one is the last.
 template <uint32_t kStride = kFastStride>
 __device__ __forceinline__ void stage_commit(const StageRegs &regs, uint8_t *dst, uint32_t row0, uint32_t depth,
                                              int lane) {
-    const uint32_t g = lane & 3, rr = lane >> 2;
+    static_assert(kStride % 2 == 0, "16-bit LDS stores want even column strides");
+    const uint32_t g = lane & 7, rp = lane >> 3;
 #pragma unroll
     for (int p = 0; p < kStagePasses; ++p) {
-        const uint32_t r = row0 + p * 16 + rr;
+        const uint32_t r = row0 + p * 16 + 2 * rp;
         if (r < depth) {
-            uint8_t *d = dst + (g * 16) * kStride + r;
+            uint16_t *d = reinterpret_cast<uint16_t *>(dst + (g * 8) * kStride + r);
 #pragma unroll
-            for (int j = 0; j < 16; ++j) d[j * kStride] = (uint8_t)(regs.v[p][j / 4] >> (8 * (j & 3)));
+            for (int j = 0; j < 8; ++j) {
+                const uint32_t lo = j < 4 ? regs.v[p][0].x : regs.v[p][0].y, hi = j < 4 ? regs.v[p][1].x : regs.v[p][1].y;
+                // byte j&3 of the even row below byte j&3 of the odd row
+                d[j * (kStride / 2)] = (uint16_t)__builtin_amdgcn_perm(hi, lo, 0x0C0C0400u + (j & 3) * 0x0101u);
+            }
         }
     }
 }
@@ -88,9 +101,9 @@ __device__ __forceinline__ void stage_commit(const StageRegs &regs, uint8_t *dst
 // The kernels built on the loops below are bound by wavefronts in flight, not by memory: the whole
 // LDS goes to the slot table plus as many transposed tile bodies as fit, one workgroup per CU, and
 // every wavefront walks a list of tiles.  How many bodies fit depends on the deepest body among the
-// workgroup's tiles: 11 wavefronts x 186 bytes per lane, 10 x 204 or 8 x 255.
+// workgroup's tiles: 11 wavefronts x 186 bytes per lane, 10 x 204 or 8 x 254.
 constexpr int kPersistWaves = 11;
-constexpr uint32_t kDepthShallow = 186, kDepthMedium = 204, kDepthDeep = 255;
+constexpr uint32_t kDepthShallow = 186, kDepthMedium = 204, kDepthDeep = 254;
 
 // Builds the slot table and classifies the workgroup by the deepest tile body it will meet
 // (`deepest` = this thread's maximum over its share of the workgroup's tiles): returns 0 (all below
