@@ -26,30 +26,52 @@ struct DecodeArgs {
     uint32_t man_aligned;  // sign|mantissa plane may be read as dwords
 };
 
-// One tile through the hand-scheduled loops (fast_tile.h): scaled state, tile body staged
-// transposed.  kMerge = false writes the exponent plane; kMerge = true joins it with the tile's
-// sign|mantissa bytes and writes bf16.  Tiles that do not qualify (ragged, odd block counts, body
-// deeper than a lane stride) take the same arithmetic with guarded byte reads from global memory.
+// Work item of the 32-column kernels: one half (top or bottom rows) of two neighbouring column
+// tiles.  Lanes 0..31 own the 32 streams of that half of tile (tk, 2p), lanes 32..63 those of tile
+// (tk, 2p + 1), so every decoded row leaves the wavefront as 64 contiguous bytes (128 as bf16).  With
+// both halves of ONE tile per wavefront every row is a 32-byte piece of a 128-byte line, and the
+// memory side of those partial writes cost a fifth of the kernel's time.
+// item = (tk * pairs + p) * 2 + half.
+//
+// kMerge = false writes the exponent plane; kMerge = true joins it with the tiles' sign|mantissa
+// bytes and writes bf16.  Items that do not qualify for the hand-scheduled loop (ragged, odd block
+// counts, a body deeper than a lane stride) take the same arithmetic with guarded byte reads from
+// global memory.
 template <uint32_t kStride, bool kMerge>
-__device__ __forceinline__ void decode_one_tile(const DecodeArgs &a, uint32_t tile, const uint2 *tab,
+__device__ __forceinline__ void decode_one_item(const DecodeArgs &a, uint32_t item, const uint2 *tab,
                                                 uint8_t *stage, int lane) {
-    const uint32_t tk = tile / a.tiles_n, tn = tile % a.tiles_n;
-    const uint32_t half = a.th / 2, hsel = lane / 32, c = lane % 32;
-    const uint32_t row0 = tk * a.th, col0 = tn * 32, my_row0 = row0 + hsel * half;
-    const uint64_t base = a.tile_offsets[tile];
-    uint32_t depth = a.tile_max_lens[tile];
-    const uint32_t state = a.states[(size_t)tile * 64 + lane];
+    const uint32_t pairs = (a.tiles_n + 1) / 2;
+    const uint32_t hsel = item & 1u, p = (item >> 1) % pairs, tk = (item >> 1) / pairs;
+    const uint32_t half = a.th / 2, side = lane / 32, c = lane % 32;
+    const uint32_t tn = 2 * p + side, col = tn * 32 + c, row_first = tk * a.th + hsel * half;
+    if (row_first >= a.K) return;  // the bottom half of a short last tile row
+    const bool have_b = 2 * p + 1 < a.tiles_n;
+    const uint32_t tile_a = tk * a.tiles_n + 2 * p, tile_b = have_b ? tile_a + 1 : tile_a;
+    uint64_t base_a = a.tile_offsets[tile_a], base_b = a.tile_offsets[tile_b];
+    uint32_t depth_a = a.tile_max_lens[tile_a], depth_b = a.tile_max_lens[tile_b];
     // A body that would run past the stream is treated as empty rather than read.
-    if (base + (uint64_t)depth * 64 > a.stream_len) depth = 0;
-    uint32_t my_steps = 0;
-    if (col0 + c < a.N && my_row0 < a.K) my_steps = min(half, a.K - my_row0);
-    const bool full = __builtin_amdgcn_ballot_w64(my_steps != half) == 0;
-    const bool fast = full && depth >= 2 && depth < kStride && half % (kMerge ? 8 : 2) == 0 && half >= 2 &&
+    if (base_a + (uint64_t)depth_a * 64 > a.stream_len) depth_a = 0;
+    if (base_b + (uint64_t)depth_b * 64 > a.stream_len) depth_b = 0;
+    const uint32_t tile = side ? tile_b : tile_a, depth = side ? depth_b : depth_a;
+    const uint64_t base = side ? base_b : base_a;
+    const uint32_t q = hsel * 32 + c;  // this lane's stream inside its tile
+    const bool col_ok = tn < a.tiles_n && col < a.N;
+    const uint32_t state = a.states[(size_t)tile * 64 + q];
+    const uint32_t steps = min(half, a.K - row_first);  // the same for every lane
+    const bool fast = __builtin_amdgcn_ballot_w64(!col_ok) == 0 && steps == half && depth_a >= 2 && depth_b >= 2 &&
+                      depth_a < kStride && depth_b < kStride && half % (kMerge ? 8 : 2) == 0 && half >= 2 &&
                       (uint64_t)a.K * a.N < (1ull << (kMerge ? 31 : 32)) && (uint32_t)(uintptr_t)tab == 0 &&
                       (!kMerge || a.man_aligned);
     const uint8_t *man_half = kMerge ? a.man_tiled + (size_t)tile * a.th * 32 + (size_t)hsel * half * 32 : nullptr;
     if (fast) {
-        stage_body<kStride>(stage, a.stream + base, depth, lane);
+        StageRegs body;
+        const uint32_t deepest = max(depth_a, depth_b), my_depth = (lane & 4) ? depth_b : depth_a;
+#pragma unroll
+        for (int grp = 0; grp < stage_groups(kStride); ++grp)
+            if ((uint32_t)grp * 128 < deepest) {
+                stage_fetch_pair(body, a.stream + base_a, depth_a, a.stream + base_b, depth_b, hsel, grp * 128, lane);
+                stage_commit<kStride>(body, stage, grp * 128, my_depth, lane);
+            }
         // LDS operations of one wavefront complete in order: the reads below see the writes above
         FastLane st;
         st.init<kStride>(stage, depth, lane, state);
@@ -57,7 +79,7 @@ __device__ __forceinline__ void decode_one_tile(const DecodeArgs &a, uint32_t ti
             // blocks of eight rows: sign|mantissa dwords of the next block are loaded while this one decodes
             const uint32_t man_sel = 0x04040000u + (c & 3u) * 0x01010101u;
             const uint32_t *mrow = reinterpret_cast<const uint32_t *>(man_half + (c & ~3u));  // + 8 dwords per row
-            uint16_t *o = a.out_bf16 + (size_t)my_row0 * a.N + col0 + c;
+            uint16_t *o = a.out_bf16 + (size_t)row_first * a.N + col;
             const uint32_t nblk = half / 8;
             uint32_t mcur[8], mnext[8];
 #pragma unroll
@@ -77,18 +99,18 @@ __device__ __forceinline__ void decode_one_tile(const DecodeArgs &a, uint32_t ti
                 for (int r = 0; r < 8; ++r) mcur[r] = mnext[r];
             }
         } else {
-            const uint64_t ob = reinterpret_cast<uint64_t>(a.out_exp + (size_t)row0 * a.N + col0);
+            const uint64_t ob = reinterpret_cast<uint64_t>(a.out_exp + (size_t)row_first * a.N + 2 * p * 32);
             // readfirstlane returns a signed int: widen through uint32_t
             const uint32_t ob_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(ob >> 32));
             const uint32_t ob_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)ob);
-            decode_tile_asm(st, ((uint64_t)ob_hi << 32) | (uint64_t)ob_lo, hsel * half * a.N + c, a.N, half / 2);
+            decode_tile_asm(st, ((uint64_t)ob_hi << 32) | (uint64_t)ob_lo, lane, a.N, half / 2);
         }
-    } else {
+    } else if (col_ok) {
         GlobalBytes src;
-        src.init(a.stream + base, depth, 64, lane);
+        src.init(a.stream + base, depth, 64, q);
         uint32_t X = state << 3;
-        const size_t o0 = (size_t)my_row0 * a.N + col0 + c;
-        for (uint32_t i = 0; i < my_steps; ++i) {
+        const size_t o0 = (size_t)row_first * a.N + col;
+        for (uint32_t i = 0; i < steps; ++i) {
             const uint32_t sym = decode_symbol_scaled(X, tab) >> 24;
             src.renorm_scaled(X);
             src.renorm_scaled(X);
@@ -100,18 +122,24 @@ __device__ __forceinline__ void decode_one_tile(const DecodeArgs &a, uint32_t ti
     }
 }
 
-// Wavefront `wave` of workgroup `j` (of the `n_wg` that share this tensor) decodes the tiles
-// (slot * n_wg + j), slot = wave, wave + kWaves, ...: a workgroup's concurrent tiles are n_wg
-// apart, so every workgroup gets the same number of tiles to within one.
+__device__ __forceinline__ uint64_t decode_num_pairs(const DecodeArgs &a) {
+    return (uint64_t)(a.num_tiles / a.tiles_n) * ((a.tiles_n + 1) / 2);
+}
+
+// Workgroup `j` (of the `n_wg` that share this tensor) takes the tile pairs j, j + n_wg, ...; its
+// wavefronts take the workgroup's items in turn (slot = wave, wave + kWaves, ...; slot / 2 picks the
+// pair, slot % 2 the half), so the two halves of a pair are staged on the same CU at about the same
+// time and the second reader of a body row finds it in that CU's cache.
 template <int kWaves, uint32_t kStride, bool kMerge>
 __device__ __forceinline__ void decode_wave_tiles(const DecodeArgs &a, uint32_t j, uint32_t n_wg, const uint2 *tab,
                                                   uint8_t *lds, int wave, int lane) {
     if (wave >= kWaves) return;
     uint8_t *stage = persist_stage<kWaves, kStride>(lds, wave);
+    const uint64_t n_pairs = decode_num_pairs(a);
     for (uint32_t slot = wave;; slot += kWaves) {
-        const uint64_t tile = (uint64_t)slot * n_wg + j;
-        if (tile >= a.num_tiles) break;
-        decode_one_tile<kStride, kMerge>(a, (uint32_t)tile, tab, stage, lane);
+        const uint64_t pair = (uint64_t)(slot >> 1) * n_wg + j;
+        if (pair >= n_pairs) break;
+        decode_one_item<kStride, kMerge>(a, (uint32_t)pair * 2 + (slot & 1u), tab, stage, lane);
     }
 }
 
@@ -136,7 +164,18 @@ __global__ __launch_bounds__(kPersistWaves *kWave) void decode_tiled32_persist_k
     const DecodeArgs &a = b.item[i];
     const uint32_t j = blockIdx.x - b.first_block[i], n_wg = b.first_block[i + 1] - b.first_block[i];
 
-    const uint32_t cls = persist_prologue(lds, a.tables, a.slot_map, a.tile_max_lens, a.num_tiles, j, n_wg);
+    uint32_t deepest = 0;
+    {
+        const uint32_t pairs = (a.tiles_n + 1) / 2;
+        const uint64_t n_pairs = decode_num_pairs(a);
+        for (uint64_t pr = (uint64_t)tid * n_wg + j; pr < n_pairs; pr += (uint64_t)kPersistWaves * kWave * n_wg) {
+            const uint32_t p = (uint32_t)(pr % pairs), tk = (uint32_t)(pr / pairs);
+            const uint32_t tile_a = tk * a.tiles_n + 2 * p;
+            deepest = max(deepest, a.tile_max_lens[tile_a]);
+            if (2 * p + 1 < a.tiles_n) deepest = max(deepest, a.tile_max_lens[tile_a + 1]);
+        }
+    }
+    const uint32_t cls = persist_classify(lds, a.tables, a.slot_map, deepest);
     if (cls == 2u)
         decode_wave_tiles<8, kDepthDeep, kMerge>(a, j, n_wg, tab, lds, wave, lane);
     else if (cls == 1u)
@@ -199,26 +238,28 @@ static int cu_count(uint32_t *out) {
 static int launch_persist(DecodeBatchArgs &b, bool merge, hipStream_t s) {
     uint32_t cus = 0;
     if (int rc = cu_count(&cus)) return rc;
-    uint64_t total = 0;
-    for (uint32_t i = 0; i < b.n; ++i) total += b.item[i].num_tiles;
+    // The unit handed to a workgroup is a pair of neighbouring column tiles.
+    uint64_t pairs[kDecBatchMax], total = 0;
+    for (uint32_t i = 0; i < b.n; ++i) {
+        const DecodeArgs &a = b.item[i];
+        pairs[i] = (uint64_t)(a.num_tiles / a.tiles_n) * ((a.tiles_n + 1) / 2);
+        total += pairs[i];
+    }
     // Never more workgroups than CUs (one is resident per CU; a workgroup too many would run alone
     // after all the others): floor of the proportional share, then hand out what is left to the
-    // tensors with the most tiles per workgroup.
+    // tensors with the most pairs per workgroup.
     uint32_t share[kDecBatchMax], used = 0;
     for (uint32_t i = 0; i < b.n; ++i) {
-        const uint64_t tiles = b.item[i].num_tiles;
-        uint64_t sh = tiles * cus / total;  // total >= 1: empty tensors are not in b
+        uint64_t sh = pairs[i] * cus / total;  // total >= 1: empty tensors are not in b
         sh = sh < 1 ? 1 : sh;
-        share[i] = (uint32_t)(sh > tiles ? tiles : sh);
+        share[i] = (uint32_t)(sh > pairs[i] ? pairs[i] : sh);
         used += share[i];
     }
     while (used < cus) {
         int best = -1;
         for (uint32_t i = 0; i < b.n; ++i)
-            if (share[i] < b.item[i].num_tiles &&
-                (best < 0 || (uint64_t)b.item[i].num_tiles * share[best] > (uint64_t)b.item[best].num_tiles * share[i]))
-                best = (int)i;
-        if (best < 0) break;  // every tensor already has one workgroup per tile
+            if (share[i] < pairs[i] && (best < 0 || pairs[i] * share[best] > pairs[best] * share[i])) best = (int)i;
+        if (best < 0) break;  // every tensor already has one workgroup per pair
         ++share[best];
         ++used;
     }

@@ -97,6 +97,27 @@ __device__ __forceinline__ void stage_commit(const StageRegs &regs, uint8_t *dst
     }
 }
 
+// Stage the `hsel` halves (32 columns each) of two tile bodies side by side, transposed: LDS column
+// side * 32 + c holds column hsel * 32 + c of body `side`, one byte per stored row.  Same lane
+// roles as stage_fetch / stage_commit: lane = 8 * (row pair) + (8-column group), groups 0..3 = body
+// A, 4..7 = body B.
+__device__ __forceinline__ void stage_fetch_pair(StageRegs &regs, const uint8_t *__restrict__ src_a, uint32_t depth_a,
+                                                 const uint8_t *__restrict__ src_b, uint32_t depth_b, uint32_t hsel,
+                                                 uint32_t row0, int lane) {
+    const uint32_t g = lane & 7, rp = lane >> 3;
+    const uint8_t *src = (g < 4 ? src_a : src_b) + hsel * 32 + (g & 3) * 8;
+    const uint32_t depth = g < 4 ? depth_a : depth_b;
+#pragma unroll
+    for (int p = 0; p < kStagePasses; ++p) {
+        const uint32_t r = row0 + p * 16 + 2 * rp;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            regs.v[p][h] = make_uint2(0u, 0u);
+            if (r + h < depth) regs.v[p][h] = *reinterpret_cast<const uint2 *>(src + (size_t)(r + h) * 64);
+        }
+    }
+}
+
 // ---- workgroups resident for a whole launch ------------------------------------------------------
 // The kernels built on the loops below are bound by wavefronts in flight, not by memory: the whole
 // LDS goes to the slot table plus as many transposed tile bodies as fit, one workgroup per CU, and
