@@ -30,6 +30,19 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# The binding limit of byte-wise rANS on this chip is not HBM but the rate of dependent decode steps:
+# one step of one wavefront (64 streams) occupies a CU's LDS pipe for about 9.4 ns (one random 8-byte
+# table read and two byte reads; measured with a micro-benchmark, the same from 8 to 16 wavefronts per
+# CU), and a lone wavefront needs about 65 ns per step.  Reported next to every HBM fraction.
+STEP_NS_PER_CU = 9.4
+STEP_NS_LATENCY = 65.0
+NUM_CUS = 256
+
+
+def step_bound_us(wave_steps: int, chain: int) -> dict:
+    """Lower bounds from the step rate: throughput (all CUs busy) and latency (one chain)."""
+    return {"throughput_us": round(wave_steps * STEP_NS_PER_CU / NUM_CUS * 1e-3, 1),
+            "latency_us": round(chain * STEP_NS_LATENCY * 1e-3, 1)}
 # HBM bytes of one batched decode launch on this workload, from rocprofv3 FETCH_SIZE and WRITE_SIZE
 # passes scaled by what the same counters read for a plain copy of known size (profiles/ holds the
 # runs): 45967.4 KiB x 1.9991 fetched + 212992.0 KiB x 1.0 written.
@@ -77,6 +90,10 @@ class Compressed:
     # exponent plane out
     def decode_bytes(self) -> int:
         return self.stream.numel() + 4 * self.n_streams + 8 * self.n_tiles + 1024 + 4096 + self.K * self.N
+
+    # decode steps of 64 streams at a time (one wavefront-step): a tile is th/2 of them
+    def wave_steps(self) -> int:
+        return self.n_tiles * (self.th // 2)
 
     # algorithmic bytes of one fused linear at M rows
     def linear_bytes(self, M: int) -> int:
@@ -255,6 +272,10 @@ def main() -> int:
                 "traffic": MEASURED_TRAFFIC_BYTES, "bytes_per_launch": int(algo_bytes),
                 "launch_us": round(launch_us, 2), "single_tensor_launch_us": per_kernel,
                 "compressed_read_GBs": round(total_stream / (launch_us * 1e-6) / 1e9, 1)}
+    wave_steps = sum(c.wave_steps() for c in layer)
+    sb = step_bound_us(wave_steps, th // 2)
+    roofline["step_rate_bound"] = dict(sb, wavefront_steps=wave_steps, ns_per_wavefront_step_per_cu=STEP_NS_PER_CU,
+                                       frac=round(sb["throughput_us"] / launch_us, 3))
 
     out = {"metric": "decoded GB/s", "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": a.steps,
            "warmup": a.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
@@ -281,7 +302,9 @@ def main() -> int:
             us = batched_time_us(lambda: gate.linear(x), 25, 100)
             us_ref = batched_time_us(lambda: torch.matmul(x, w_dense), 25, 100)
             nbytes = gate.linear_bytes(M)
+            sb = step_bound_us(gate.wave_steps(), gate.th // 2)
             rows.append({"M": M, "us": round(us, 2), "allclose_1e-2": ok,
+                         "step_rate_bound_us": max(sb["throughput_us"], sb["latency_us"]),
                          "hbm_frac_compressed_bytes": round(nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
                          "effective_weight_GBs": round(2 * gate.K * gate.N / (us * 1e-6) / 1e9, 1),
                          "mfma_TFLOPs": round(2 * M * gate.K * gate.N / (us * 1e-6) / 1e12, 2),
