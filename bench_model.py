@@ -1,12 +1,14 @@
 #!/usr/bin/env python3
 """Batch-1 greedy decode of a Llama-3-8B-shaped random-init decoder whose linear and embedding
 weights are rANS-compressed (RansLinear / RansEmbedding / RansLMHead), against the same decoder on
-the decompressed bf16 weights (torch.matmul).
+the decompressed bf16 weights -- once through torch.matmul (hipBLASLt) and once through the fused
+kernels' own contraction order applied to the plain weights (`plain_linear_same_order`), the run
+whose generated ids the compressed model must reproduce exactly.
 
   python bench_model.py [--layers 32] [--prompt 128] [--new 256] [--tile-k 1024] [--gen cpu|cuda]
 
 Prints one JSON object: tokens per second of the compressed model (eager launches and one HIP
-graph replay per token), of the bf16 reference, and how many generated ids agree.
+graph replay per token), of the bf16 reference, and how the generated ids and logits compare.
 
 Shape: hidden 4096, FFN 14336 SwiGLU, 32 query / 8 KV heads of 128, vocabulary 128256, RMSNorm,
 RoPE theta 500000.  Weights bf16 N(0, 0.02) from seed 5 in module order (embedding; per layer q, k, v,
@@ -59,6 +61,19 @@ class Dense:
 
     def __call__(self, x):
         return torch.matmul(x, self.w)
+
+
+class PlainSameOrder:
+    """x @ W for a decompressed [K, N] bf16 weight through the fused kernel's contraction order: what the
+    compressed operator computes if, and only if, it reconstructs every weight bit."""
+
+    def __init__(self, w_kn, tile_k, tile_n):
+        self.w, self.tile_k, self.tile_n = w_kn, tile_k, tile_n
+
+    def __call__(self, x):
+        import comp_inference_amd as ci
+
+        return ci.plain_linear_same_order(x, self.w, tile_k=self.tile_k, tile_n=self.tile_n)
 
 
 class Decoder:
@@ -160,7 +175,7 @@ def teacher_forced(dec: Decoder, prompt, ids):
 
 def build(n_layers, dev, tile_k, tile_n, gen):
     """Draw the weights (seed 5, module order), compress them, and keep a decompressed bf16 copy.
-    Returns (compressed ops, dense ops, byte counts)."""
+    Returns (compressed ops, dense ops through torch.matmul, dense ops in the fused kernels' order, byte counts)."""
     import comp_inference_amd as ci
     from comp_inference_amd.pytorch_runtime import RansEmbedding, RansLinear, RansLMHead
 
@@ -196,15 +211,18 @@ def build(n_layers, dev, tile_k, tile_n, gen):
     def linear(w_out_in):
         w_kn = w_out_in.t().contiguous()
         mod = RansLinear(w_kn.shape[0], w_kn.shape[1], tile_k=tile_k, tile_n=tile_n)
-        return mod, Dense(fill(mod, w_kn))
+        dense = fill(mod, w_kn)
+        return mod, Dense(dense), PlainSameOrder(dense, tile_k, tile_n)
 
     comp = {"qkv": [], "o": [], "gate_up": [], "down": []}
     ref = {"qkv": [], "o": [], "gate_up": [], "down": []}
+    same = {"qkv": [], "o": [], "gate_up": [], "down": []}
     t0 = time.time()
     table = draw(s.vocab, s.hidden)
     emb = RansEmbedding(s.vocab, s.hidden, tile_k=tile_k, tile_n=tile_n)
     table_dense = fill(emb, table)
     comp["embed"], ref["embed"] = emb, (lambda ids, t=table_dense: t.index_select(0, ids))
+    same["embed"] = ref["embed"]
     del table
     for l in range(n_layers):
         q, k, v = draw(s.heads * s.head_dim, s.hidden), draw(s.kv_heads * s.head_dim, s.hidden), \
@@ -214,16 +232,18 @@ def build(n_layers, dev, tile_k, tile_n, gen):
         down = draw(s.hidden, s.ffn)
         for name, w in (("qkv", torch.cat((q, k, v), 0)), ("o", o), ("gate_up", torch.cat((gate, up), 0)),
                         ("down", down)):
-            m, d = linear(w)
+            m, d, p = linear(w)
             comp[name].append(m)
             ref[name].append(d)
+            same[name].append(p)
         if l % 4 == 3 or l == n_layers - 1:
             log(f"  layer {l + 1}/{n_layers} compressed ({time.time() - t0:.0f} s)")
     head_w = draw(s.vocab, s.hidden)                   # [V, H]: the head keeps the table's orientation
     head = RansLMHead(s.hidden, s.vocab, tile_k=tile_k, tile_n=tile_n)
     head_dense = fill(head, head_w)
     comp["head"], ref["head"] = head, (lambda x, w=head_dense: torch.matmul(x, w.t()))
-    return comp, ref, sizes
+    same["head"] = lambda x, w=head_dense: ci.plain_linear_transposed_same_order(x, w, tile_k=tile_k, tile_n=tile_n)
+    return comp, ref, same, sizes
 
 
 def run(n_layers=32, n_prompt=128, n_new=256, tile_k=1024, tile_n=32, gen="cpu"):
@@ -232,13 +252,14 @@ def run(n_layers=32, n_prompt=128, n_new=256, tile_k=1024, tile_n=32, gen="cpu")
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
     log(f"building the {n_layers}-layer decoder (generator: {gen}) ...")
-    comp, ref, sizes = build(n_layers, dev, tile_k, tile_n, gen)
+    comp, ref, same, sizes = build(n_layers, dev, tile_k, tile_n, gen)
     prompt = torch.randint(0, Shape.vocab, (n_prompt,), generator=torch.Generator("cpu").manual_seed(6)).to(dev)
     max_len = n_prompt + n_new + 1
     res = {}
     with torch.no_grad():
         for name, ops, graph in (("reference_bf16", ref, False), ("reference_bf16_graph", ref, True),
-                                 ("compressed_eager", comp, False), ("compressed_graph", comp, True)):
+                                 ("compressed_eager", comp, False), ("compressed_graph", comp, True),
+                                 ("decompressed_same_order", same, False)):
             log(f"decoding: {name} ...")
             dec = Decoder(ops, n_layers, max_len, dev)
             ids, sec = generate(dec, prompt, n_new, graph)
@@ -249,6 +270,9 @@ def run(n_layers=32, n_prompt=128, n_new=256, tile_k=1024, tile_n=32, gen="cpu")
         log("teacher-forced comparison ...")
         lr = teacher_forced(Decoder(ref, n_layers, max_len, dev), prompt, base)
         lc = teacher_forced(Decoder(comp, n_layers, max_len, dev), prompt, base)
+        ls = teacher_forced(Decoder(same, n_layers, max_len, dev), prompt, base)
+    logits_bit_identical = bool(torch.equal(lc, ls))
+    del ls
     forced_same = int((lr.argmax(-1) == lc.argmax(-1)).sum())
     logit_err = float((lr - lc).abs().max())
     top2 = lr.topk(2, dim=-1).values
@@ -270,6 +294,13 @@ def run(n_layers=32, n_prompt=128, n_new=256, tile_k=1024, tile_n=32, gen="cpu")
         "tok_per_s_compressed_eager": round(n_new / res["compressed_eager"][1], 2),
         "tok_per_s_reference_bf16_graph": round(n_new / res["reference_bf16_graph"][1], 2),
         "tok_per_s_reference_bf16_eager": round(n_new / res["reference_bf16"][1], 2),
+        # the run on decompressed weights in the fused kernels' contraction order: equal ids and equal
+        # logit bits mean every weight bit is reconstructed and nothing else differs
+        "ids_equal_to_decompressed_same_order_run": res["compressed_eager"][0] == res["decompressed_same_order"][0],
+        "graph_ids_equal_to_decompressed_same_order_run":
+            res["compressed_graph"][0] == res["decompressed_same_order"][0],
+        "teacher_forced_logits_bit_identical_to_same_order_run": logits_bit_identical,
+        # the run on decompressed weights through hipBLASLt sums in another order
         "ids_equal_to_reference": res["compressed_eager"][0] == base,
         "ids_matching_prefix": agree(res["compressed_eager"][0]),
         "teacher_forced_top1_agreement": f"{forced_same}/{n_new}",

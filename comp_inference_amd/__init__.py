@@ -28,6 +28,7 @@ from .linear_hip import (
     fused_rans_linear_triton,
     fused_rans_linear_triton_uncoalesced,
     fused_rans_linear_uncoalesced,
+    plain_linear_same_order,
     splitk_reduce,
     triton_matmul,
 )
@@ -44,6 +45,7 @@ from .transposed_linear_hip import (
     fused_rans_linear_transposed_triton,
     fused_rans_linear_transposed_triton_uncoalesced,
     fused_rans_linear_transposed_uncoalesced,
+    plain_linear_transposed_same_order,
 )
 from .pytorch_runtime import (
     RansEmbedding,

@@ -50,6 +50,10 @@ struct LinearArgs {
     // x rearranged so that one MFMA operand load reads whole cache lines: fragment (group g of 32 rows,
     // block kb of 8 k, row mm) = 16 bytes at ((g * K/8 + kb) * 32 + mm) * 16, rows >= M zero; or null
     const uint16_t *xf;
+    // Verification aid: when set, the weights are read from this plain bf16 [K, N] matrix instead of
+    // being decoded (every tile takes the guarded path, which issues the same MFMA sequence as the
+    // hand-scheduled one); none of the compressed operands is touched.
+    const uint16_t *dense_w;
 };
 
 // x [M, K] -> the fragment order described at LinearArgs::xf.  In a plain row-major x the 64 lanes of
@@ -95,9 +99,11 @@ __device__ __forceinline__ uint32_t pack_bf16_pair(uint32_t w0, uint32_t w1, uin
 // General path: ragged tiles (rows >= K, columns >= N), unaligned x, odd block counts, or a tile
 // body too deep for the staging area.  Same arithmetic on the scaled state, bytes read where they
 // lie in global memory, every access guarded.
+// wd: null, or this lane's column of a plain bf16 weight at row k0 (row stride wd_stride elements).
 __device__ __forceinline__ void linear_tile_guarded(GlobalBytes &src, uint32_t X, const uint2 *tab, uint32_t K,
                                                     uint32_t half, uint32_t my_steps, const uint8_t *man,
-                                                    const uint16_t *xrow, bool m_ok, uint32_t k0, f32x16 &acc) {
+                                                    const uint16_t *xrow, bool m_ok, uint32_t k0, f32x16 &acc,
+                                                    const uint16_t *wd = nullptr, uint32_t wd_stride = 0) {
     for (uint32_t i = 0; i < half; i += 8) {
         u32x4 xv = (u32x4){0, 0, 0, 0};
         if (m_ok) {
@@ -113,7 +119,7 @@ __device__ __forceinline__ void linear_tile_guarded(GlobalBytes &src, uint32_t X
         for (int j = 0; j < 8; ++j) {
             mb[j] = 0;
             w[j] = 0;
-            if (i + j < my_steps) {
+            if (!wd && i + j < my_steps) {
                 mb[j] = man[(size_t)(i + j) * 32];
                 w[j] = decode_symbol_scaled(X, tab);
                 src.renorm_scaled(X);
@@ -121,8 +127,17 @@ __device__ __forceinline__ void linear_tile_guarded(GlobalBytes &src, uint32_t X
             }
         }
         u32x4 wv;
+        if (wd) {
 #pragma unroll
-        for (int p = 0; p < 4; ++p) wv[p] = pack_bf16_pair(w[2 * p], w[2 * p + 1], mb[2 * p], mb[2 * p + 1]);
+            for (int p = 0; p < 4; ++p) {
+                const uint32_t lo = i + 2 * p < my_steps ? wd[(size_t)(i + 2 * p) * wd_stride] : 0u;
+                const uint32_t hi = i + 2 * p + 1 < my_steps ? wd[(size_t)(i + 2 * p + 1) * wd_stride] : 0u;
+                wv[p] = lo | (hi << 16);
+            }
+        } else {
+#pragma unroll
+            for (int p = 0; p < 4; ++p) wv[p] = pack_bf16_pair(w[2 * p], w[2 * p + 1], mb[2 * p], mb[2 * p + 1]);
+        }
         acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, wv), __builtin_bit_cast(bf16x8, xv),
                                                       acc, 0, 0, 0);
     }
@@ -149,7 +164,9 @@ __global__ __launch_bounds__(kLinMaxWaves *kWave) void fused_linear32_kernel(Lin
     uint64_t base = 0;
     bool fast = false;
     StageRegs body;
-    if (have_tile) {
+    if (have_tile && a.dense_w) {
+        if (col0 + c < a.N && k0 < a.K) my_steps = min(half, a.K - k0);
+    } else if (have_tile) {
         base = a.tile_offsets[tile];
         depth = a.tile_max_lens[tile];
         state = a.states[(size_t)tile * 64 + lane];
@@ -159,10 +176,10 @@ __global__ __launch_bounds__(kLinMaxWaves *kWave) void fused_linear32_kernel(Lin
         // the hand-scheduled loop wants: a full tile, a body that fits one lane stride, an even
         // number of 8-row blocks, 16-byte readable x rows and a dword-aligned sign|mantissa plane
         fast = full && a.fast_ok && depth >= 2 && depth < kFastStride && half % 16 == 0 &&
-               (uint32_t)(uintptr_t)tab == 0;
+               (uint32_t)(uintptr_t)tab == 0;  // (depth is 0 in a plain-weight run)
         if (fast) stage_fetch(body, a.stream + base, 0, depth, lane);
     }
-    build_slot_table_x8(tab, a.tables, a.slot_map, tid, nthreads);  // runs under the body loads
+    if (!a.dense_w) build_slot_table_x8(tab, a.tables, a.slot_map, tid, nthreads);  // runs under the body loads
     if (fast) {
         stage_commit(body, stage, 0, depth, lane);
         for (int grp = 1; grp < kStageGroups; ++grp)
@@ -209,12 +226,16 @@ __global__ __launch_bounds__(kLinMaxWaves *kWave) void fused_linear32_kernel(Lin
                 linear_tile_asm(st, acc, mb_u, moff, xb, xo, xstep, man_sel, half / 8);
         } else {
             const uint8_t *man = a.man_tiled + man_tile + (size_t)hsel * half * 32 + c;
+            // only rows below my_steps are read, and that is 0 for a lane outside the matrix
+            const uint16_t *wd = a.dense_w ? a.dense_w + (size_t)k0 * a.N + col0 + c : nullptr;
             GlobalBytes src;
             src.init(a.stream + base, depth, 64, lane);
-            linear_tile_guarded(src, state << 3, tab, a.K, half, my_steps, man, a.x + xrow_elems, m_ok, k0, acc);
+            linear_tile_guarded(src, state << 3, tab, a.K, half, my_steps, man, a.x + xrow_elems, m_ok, k0, acc,
+                                wd, a.N);
             if (MB == 2) {  // the guarded path simply walks the tile again for the second group of rows
                 src.init(a.stream + base, depth, 64, lane);
-                linear_tile_guarded(src, state << 3, tab, a.K, half, my_steps, man, a.x + xrow2_elems, m2_ok, k0, acc2);
+                linear_tile_guarded(src, state << 3, tab, a.K, half, my_steps, man, a.x + xrow2_elems, m2_ok, k0, acc2,
+                                    wd, a.N);
             }
         }
     }
@@ -262,15 +283,15 @@ __device__ __forceinline__ void linear_one_tile(const LinearArgs &a, uint32_t ti
     const uint32_t tk = tile / a.tiles_n, tn = tile % a.tiles_n;
     const uint32_t half = a.th / 2, hsel = lane / 32, c = lane % 32;
     const uint32_t col0 = tn * 32, k0 = tk * a.th + hsel * half;
-    const uint64_t base = a.tile_offsets[tile];
-    uint32_t depth = a.tile_max_lens[tile];
-    const uint32_t state = a.states[(size_t)tile * 64 + lane];
+    const uint64_t base = a.dense_w ? 0 : a.tile_offsets[tile];
+    uint32_t depth = a.dense_w ? 0 : a.tile_max_lens[tile];
+    const uint32_t state = a.dense_w ? 0 : a.states[(size_t)tile * 64 + lane];
     if (base + (uint64_t)depth * 64 > a.stream_len) depth = 0;
     uint32_t my_steps = 0;
     if (col0 + c < a.N && k0 < a.K) my_steps = min(half, a.K - k0);
     const bool full = __builtin_amdgcn_ballot_w64(my_steps != half) == 0;
     const bool fast = full && a.fast_ok && depth >= 2 && depth < kStride && half % 16 == 0 &&
-                      (uint32_t)(uintptr_t)tab == 0;
+                      (uint32_t)(uintptr_t)tab == 0 && !a.dense_w;
     const uint32_t m = c;  // row of x this lane feeds to the (first) MFMA
     const bool m_ok = m < a.M, m2_ok = MB == 2 && m + 32 < a.M;
     f32x16 acc, acc2;
@@ -305,12 +326,14 @@ __device__ __forceinline__ void linear_one_tile(const LinearArgs &a, uint32_t ti
             linear_tile_asm(st, acc, mb_u, moff, xb, xo, xstep, man_sel, half / 8);
     } else {
         const uint8_t *man = a.man_tiled + man_tile + (size_t)hsel * half * 32 + c;
+        const uint16_t *wd = a.dense_w ? a.dense_w + (size_t)k0 * a.N + col0 + c : nullptr;
         GlobalBytes src;
         src.init(a.stream + base, depth, 64, lane);
-        linear_tile_guarded(src, state << 3, tab, a.K, half, my_steps, man, a.x + xrow_elems, m_ok, k0, acc);
+        linear_tile_guarded(src, state << 3, tab, a.K, half, my_steps, man, a.x + xrow_elems, m_ok, k0, acc, wd, a.N);
         if (MB == 2) {
             src.init(a.stream + base, depth, 64, lane);
-            linear_tile_guarded(src, state << 3, tab, a.K, half, my_steps, man, a.x + xrow2_elems, m2_ok, k0, acc2);
+            linear_tile_guarded(src, state << 3, tab, a.K, half, my_steps, man, a.x + xrow2_elems, m2_ok, k0, acc2, wd,
+                                a.N);
         }
     }
     // MFMA 32x32 result layout: register v of lane l is row (v/4)*8 + (l/32)*4 + v%4 (= column of
@@ -341,8 +364,10 @@ __global__ __launch_bounds__(kPersistWaves *kWave) void fused_linear32_resident_
     extern __shared__ __align__(16) uint8_t lds[];
     const uint2 *tab = reinterpret_cast<const uint2 *>(lds);
     const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
-    const uint32_t cls = persist_prologue(lds, a.tables, a.slot_map, a.tile_max_lens, a.tiles_k * a.tiles_n, blockIdx.x,
-                                          gridDim.x);
+    // (a plain-weight run has no table to build; which wavefront takes which tile does not change a tile's sum)
+    const uint32_t cls = a.dense_w ? 0u
+                                   : persist_prologue(lds, a.tables, a.slot_map, a.tile_max_lens, a.tiles_k * a.tiles_n,
+                                                      blockIdx.x, gridDim.x);
     if (cls == 2u)
         linear_wave_tiles<MB, 8, kDepthDeep>(a, tab, lds, wave, lane);
     else if (cls == 1u)
@@ -496,15 +521,18 @@ static int fused_linear_impl(const uint16_t *d_x, uint32_t M, uint32_t K, uint32
                              const uint32_t *d_tables, const uint8_t *d_slot_map, const uint32_t *d_meta0,
                              const uint32_t *d_meta1, const uint8_t *d_man_tiled, uint32_t th, uint32_t tw,
                              const uint16_t *d_bias, uint16_t *d_out, uint32_t out_stride, void *d_workspace,
-                             size_t workspace_bytes, bool dense, hipStream_t s) {
+                             size_t workspace_bytes, bool dense, hipStream_t s, const uint16_t *d_plain_w = nullptr) {
     if (M == 0 || N == 0) return CI_OK;
     if (K == 0) return fail(CI_ERR_ARG, "fused linear: K is 0");
-    if (!d_x || !d_states || !d_tables || !d_slot_map || !d_meta0 || !d_meta1 || !d_man_tiled || !d_out)
-        return fail(CI_ERR_ARG, "fused linear: null pointer");
-    if (stream_len && !d_stream) return fail(CI_ERR_ARG, "fused linear: null stream");
+    if (!d_x || !d_out) return fail(CI_ERR_ARG, "fused linear: null pointer");
+    if (!d_plain_w) {
+        if (!d_states || !d_tables || !d_slot_map || !d_meta0 || !d_meta1 || !d_man_tiled)
+            return fail(CI_ERR_ARG, "fused linear: null pointer");
+        if (stream_len && !d_stream) return fail(CI_ERR_ARG, "fused linear: null stream");
+        if (!aligned(d_slot_map, 4)) return fail(CI_ERR_ARG, "fused linear: slot_map must be 4-byte aligned");
+    }
     if (th == 0 || tw == 0 || (!dense && (th & 1))) return fail(CI_ERR_ARG, "fused linear: bad tile shape");
     if (x_stride < K || out_stride < N) return fail(CI_ERR_ARG, "fused linear: row stride shorter than the row");
-    if (!aligned(d_slot_map, 4)) return fail(CI_ERR_ARG, "fused linear: slot_map must be 4-byte aligned");
 
     LinearArgs a;
     a.x = d_x;
@@ -522,6 +550,7 @@ static int fused_linear_impl(const uint16_t *d_x, uint32_t M, uint32_t K, uint32
     a.stream_offsets = dense ? d_meta0 : nullptr;
     a.stream_sizes = dense ? d_meta1 : nullptr;
     a.man_tiled = d_man_tiled;
+    a.dense_w = d_plain_w;
     a.bias = d_bias;
     a.out = d_out;
     a.out_stride = out_stride;
@@ -531,7 +560,9 @@ static int fused_linear_impl(const uint16_t *d_x, uint32_t M, uint32_t K, uint32
     a.tiles_k = ceil_div(K, th);
     a.fast_ok = aligned(d_x, 16) && x_stride % 8 == 0 && aligned(d_man_tiled, 4) &&
                 (uint64_t)M * x_stride * 2 < (1ull << 31);
-    const LinearPlan p = plan_linear(M, K, th, tw, a.tiles_n, dense, aligned(d_stream, 16));
+    const LinearPlan p = plan_linear(M, K, th, tw, a.tiles_n, dense, d_plain_w || aligned(d_stream, 16));
+    if (d_plain_w && !p.fast)
+        return fail(CI_ERR_ARG, "plain-weight linear: only the 32-column tiling (tile height a multiple of 16)");
     a.kw = p.kw;
     a.nw = p.nw;
     a.P = p.P;
@@ -545,7 +576,7 @@ static int fused_linear_impl(const uint16_t *d_x, uint32_t M, uint32_t K, uint32
     }
     // the fragment copy of x goes behind the partials when the caller's workspace has room for it
     a.xf = nullptr;
-    const size_t frag_bytes = x_fragment_bytes(M, K, p.fast && a.fast_ok);
+    const size_t frag_bytes = d_plain_w ? 0 : x_fragment_bytes(M, K, p.fast && a.fast_ok);  // (the guarded path reads x in place)
     if (frag_bytes && frag_bytes < (1ull << 31) && d_workspace) {
         uint8_t *at = static_cast<uint8_t *>(d_workspace) + ((partial_bytes + 15) & ~(size_t)15);
         at += (16 - (reinterpret_cast<uintptr_t>(at) & 15)) & 15;
@@ -638,6 +669,16 @@ extern "C" int ci_fused_linear_dense(const uint16_t *d_x, uint32_t M, uint32_t K
     return fused_linear_impl(d_x, M, K, N, x_stride, d_stream, stream_len, d_states, d_tables, d_slot_map,
                              d_stream_offsets, d_stream_sizes, d_man_tiled, tile_height, tile_width, d_bias, d_out,
                              out_stride, d_workspace, workspace_bytes, true, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int ci_plain_linear_same_order(const uint16_t *d_x, uint32_t M, uint32_t K, uint32_t N, uint32_t x_stride,
+                                          const uint16_t *d_w, uint32_t tile_height, uint32_t tile_width,
+                                          const uint16_t *d_bias, uint16_t *d_out, uint32_t out_stride,
+                                          void *d_workspace, size_t workspace_bytes, ci_stream_t stream) {
+    if (!d_w) return fail(CI_ERR_ARG, "plain-weight linear: null weight");
+    return fused_linear_impl(d_x, M, K, N, x_stride, nullptr, 0, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr,
+                             tile_height, tile_width, d_bias, d_out, out_stride, d_workspace, workspace_bytes, false,
+                             static_cast<hipStream_t>(stream), d_w);
 }
 
 extern "C" int ci_splitk_reduce(const void *d_partial, int partial_is_bf16, uint32_t P, uint32_t M, uint32_t N,

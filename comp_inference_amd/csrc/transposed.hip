@@ -35,22 +35,14 @@ struct TransArgs {
     const uint8_t *man_tiled;
     float *partial;  // [P][M][V]
     uint32_t th, tw, tiles_n, tiles_k, num_tiles;
+    // Verification aid: when set, the weights are read from this plain bf16 [V, H] matrix instead of
+    // being decoded (same products, same reduction); none of the compressed operands is touched.
+    const uint16_t *dense_w;
 };
 
 template <int kCtrl>
 __device__ __forceinline__ float dpp_add(float v) {
     const int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(v), kCtrl, 0xF, 0xF, false);
-    return v + __int_as_float(moved);
-}
-
-// Sum over each group of 32 lanes; the total is valid in lane 31 of the group.
-__device__ __forceinline__ float sum32_to_last_lane(float v) {
-    v = dpp_add<0xB1>(v);   // quad_perm [1,0,3,2]
-    v = dpp_add<0x4E>(v);   // quad_perm [2,3,0,1]
-    v = dpp_add<0x141>(v);  // row_half_mirror
-    v = dpp_add<0x140>(v);  // row_mirror: every lane of a 16-lane row holds the row total
-    // row_bcast15: lane 15 of each row is added into the following row (rows 1 and 3 complete a group)
-    const int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x142, 0xA, 0xF, false);
     return v + __int_as_float(moved);
 }
 
@@ -84,22 +76,47 @@ __device__ __forceinline__ float reduce8_over32(const float (&p)[8], bool b8, bo
     return dpp_add<0xB1>(u);  // quad_perm [1,0,3,2]
 }
 
-// One tile: wave walks it once.  Fast path: blocks of eight steps through the hand-scheduled
-// loop, products and the eight-at-once reduction in between; otherwise a guarded step at a time.
+// Eight rows of one tile (w[d] = this lane's weights of rows 2d, 2d + 1 as two bf16) against MB rows
+// of x: products, the eight-at-once reduction, and one store per quad.  `limit` = rows of the block
+// that exist (8 in a full tile).
+template <int MB>
+__device__ __forceinline__ void trans_emit8(const uint32_t (&w)[4], const uint32_t (&xb)[MB], uint32_t M, uint32_t V,
+                                            float *dst_blk, uint32_t limit, int lane) {
+    const bool b8 = (lane & 8) != 0, b4 = (lane & 4) != 0;
+    const uint32_t j = 4u * b4 + 2u * b8 + ((lane >> 4) & 1u);  // which of the 8 rows this quad ends up with
+    const bool writer = (lane & 3) == 0 && j < limit;
+#pragma unroll
+    for (int m = 0; m < MB; ++m) {
+        const float xf = __uint_as_float(xb[m] << 16);
+        float p[8];
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {  // a bf16 x bf16 product is exact in fp32
+            p[2 * d] = __uint_as_float(w[d] << 16) * xf;
+            p[2 * d + 1] = __uint_as_float(w[d] & 0xFFFF0000u) * xf;
+        }
+        const float total = reduce8_over32(p, b8, b4);
+        if (writer && m < (int)M) dst_blk[(size_t)m * V + j] = total;
+    }
+}
+
+// One tile: wave walks it once, eight rows at a time.  Fast path: the eight steps run through the
+// hand-scheduled loop; otherwise guarded steps.  Both feed the same products and the same
+// reduction, so a tile's partial sums do not depend on the path it took.
 template <int MB, uint32_t kStride>
 __device__ __forceinline__ void trans_one_tile(const TransArgs &a, uint32_t tile, const uint2 *tab, uint8_t *stage,
                                                int lane) {
     const uint32_t tk = tile / a.tiles_n, tn = tile % a.tiles_n;
     const uint32_t half = a.th / 2, hsel = lane / 32, c = lane % 32;
     const uint32_t v0 = tk * a.th + hsel * half, h = tn * 32 + c;
-    const uint64_t base = a.tile_offsets[tile];
-    uint32_t depth = a.tile_max_lens[tile];
-    const uint32_t state = a.states[(size_t)tile * 64 + lane];
+    const uint64_t base = a.dense_w ? 0 : a.tile_offsets[tile];
+    uint32_t depth = a.dense_w ? 0 : a.tile_max_lens[tile];
+    const uint32_t state = a.dense_w ? 0 : a.states[(size_t)tile * 64 + lane];
     if (base + (uint64_t)depth * 64 > a.stream_len) depth = 0;
     uint32_t my_steps = 0;
     if (v0 < a.V) my_steps = min(half, a.V - v0);  // rows of this lane's half (same for its 32 lanes)
     const bool full = __builtin_amdgcn_ballot_w64(my_steps != half || h >= a.H) == 0;
-    const bool fast = full && depth >= 2 && depth < kStride && half % 8 == 0 && (uint32_t)(uintptr_t)tab == 0;
+    const bool fast = full && depth >= 2 && depth < kStride && half % 8 == 0 && (uint32_t)(uintptr_t)tab == 0 &&
+                      !a.dense_w;
 
     uint32_t xb[MB];  // bf16 bits of x[m, h]
 #pragma unroll
@@ -113,9 +130,6 @@ __device__ __forceinline__ void trans_one_tile(const TransArgs &a, uint32_t tile
         st.init<kStride>(stage, depth, lane, state);
         const uint32_t man_sel = 0x04040000u + (c & 3u) * 0x01010101u;
         const uint32_t *mrow = reinterpret_cast<const uint32_t *>(man_tile + (c & ~3u));  // + 8 dwords per row
-        const bool b8 = (lane & 8) != 0, b4 = (lane & 4) != 0;
-        const uint32_t j = 4u * b4 + 2u * b8 + ((lane >> 4) & 1u);  // which of the 8 rows this quad ends up with
-        const bool writer = (lane & 3) == 0;
         const uint32_t nblk = half / 8;
         uint32_t mcur[8], mnext[8];
 #pragma unroll
@@ -127,18 +141,7 @@ __device__ __forceinline__ void trans_one_tile(const TransArgs &a, uint32_t tile
             for (int r = 0; r < 8; ++r) mnext[r] = nrow[r * 8];
             uint32_t w[4];
             decode8_weights_asm(st, mcur, man_sel, w);
-#pragma unroll
-            for (int m = 0; m < MB; ++m) {
-                const float xf = __uint_as_float(xb[m] << 16);
-                float p[8];
-#pragma unroll
-                for (int d = 0; d < 4; ++d) {  // a bf16 x bf16 product is exact in fp32
-                    p[2 * d] = __uint_as_float(w[d] << 16) * xf;
-                    p[2 * d + 1] = __uint_as_float(w[d] & 0xFFFF0000u) * xf;
-                }
-                const float total = reduce8_over32(p, b8, b4);
-                if (writer && m < (int)a.M) dst[(size_t)m * a.V + blk * 8 + j] = total;
-            }
+            trans_emit8<MB>(w, xb, a.M, a.V, dst + blk * 8, 8u, lane);
 #pragma unroll
             for (int r = 0; r < 8; ++r) mcur[r] = mnext[r];
         }
@@ -148,24 +151,31 @@ __device__ __forceinline__ void trans_one_tile(const TransArgs &a, uint32_t tile
     // In the last k-tile the bottom half has fewer rows than the top half: the wave runs to the
     // top half's count, lanes past their own count (or past the last column) contribute zero.
     const uint32_t n_wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)my_steps);
-    const bool writer = c == 31, col_ok = h < a.H;
+    const bool col_ok = h < a.H;
     const uint8_t *man = man_tile + c;
+    const uint16_t *wd = a.dense_w ? a.dense_w + (size_t)v0 * a.H + h : nullptr;  // read below my_steps only
     GlobalBytes src;
     src.init(a.stream + base, depth, 64, lane);
     uint32_t X = state << 3;
-    for (uint32_t i = 0; i < n_wave; ++i) {
-        float w = 0.f;
-        if (col_ok && i < my_steps) {
-            const uint32_t sym = decode_symbol_scaled(X, tab) >> 24;
-            src.renorm_scaled(X);
-            src.renorm_scaled(X);
-            w = weight_f32(sym, man[(size_t)i * 32]);
-        }
+    for (uint32_t i0 = 0; i0 < n_wave; i0 += 8) {
+        uint32_t w[4] = {0u, 0u, 0u, 0u};
 #pragma unroll
-        for (int m = 0; m < MB; ++m) {
-            const float s = sum32_to_last_lane(w * __uint_as_float(xb[m] << 16));
-            if (writer && m < (int)a.M && i < my_steps) dst[(size_t)m * a.V + i] = s;
+        for (int r = 0; r < 8; ++r) {
+            const uint32_t i = i0 + r;
+            uint32_t bits = 0;
+            if (col_ok && i < my_steps) {
+                if (wd) {
+                    bits = wd[(size_t)i * a.H];
+                } else {
+                    const uint32_t sym = decode_symbol_scaled(X, tab) >> 24;
+                    src.renorm_scaled(X);
+                    src.renorm_scaled(X);
+                    bits = assemble_bf16(sym, man[(size_t)i * 32]);
+                }
+            }
+            w[r / 2] |= bits << (16 * (r & 1));
         }
+        trans_emit8<MB>(w, xb, a.M, a.V, dst + i0, my_steps > i0 ? my_steps - i0 : 0u, lane);
     }
 }
 
@@ -184,7 +194,10 @@ __global__ __launch_bounds__(kPersistWaves *kWave) void trans32_kernel(TransArgs
     extern __shared__ __align__(16) uint8_t lds[];
     const uint2 *tab = reinterpret_cast<const uint2 *>(lds);
     const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
-    const uint32_t cls = persist_prologue(lds, a.tables, a.slot_map, a.tile_max_lens, a.num_tiles, blockIdx.x, gridDim.x);
+    // (a plain-weight run has no table to build; which wavefront takes which tile does not change a tile's sums)
+    const uint32_t cls = a.dense_w ? 0u
+                                   : persist_prologue(lds, a.tables, a.slot_map, a.tile_max_lens, a.num_tiles,
+                                                      blockIdx.x, gridDim.x);
     if (cls == 2u)
         trans_wave_tiles<MB, 8, kDepthDeep>(a, tab, lds, wave, lane);
     else if (cls == 1u)
@@ -265,15 +278,19 @@ static int transposed_impl(const uint16_t *d_x, uint32_t M, uint32_t H, uint32_t
                            const uint32_t *d_tables, const uint8_t *d_slot_map, const uint32_t *d_meta0,
                            const uint32_t *d_meta1, const uint8_t *d_man_tiled, uint32_t th, uint32_t tw,
                            const uint16_t *d_bias, uint16_t *d_out, uint32_t out_stride, void *d_workspace,
-                           size_t workspace_bytes, bool dense, ci_stream_t stream) {
+                           size_t workspace_bytes, bool dense, ci_stream_t stream,
+                           const uint16_t *d_plain_w = nullptr) {
     if (M == 0 || V == 0) return CI_OK;
     if (H == 0) return fail(CI_ERR_ARG, "transposed linear: hidden size is 0");
-    if (!d_x || !d_states || !d_tables || !d_slot_map || !d_meta0 || !d_meta1 || !d_man_tiled || !d_out)
-        return fail(CI_ERR_ARG, "transposed linear: null pointer");
-    if (stream_len && !d_stream) return fail(CI_ERR_ARG, "transposed linear: null stream");
+    if (!d_x || !d_out) return fail(CI_ERR_ARG, "transposed linear: null pointer");
+    if (!d_plain_w) {
+        if (!d_states || !d_tables || !d_slot_map || !d_meta0 || !d_meta1 || !d_man_tiled)
+            return fail(CI_ERR_ARG, "transposed linear: null pointer");
+        if (stream_len && !d_stream) return fail(CI_ERR_ARG, "transposed linear: null stream");
+        if (!aligned(d_slot_map, 4)) return fail(CI_ERR_ARG, "transposed linear: slot_map must be 4-byte aligned");
+    }
     if (th == 0 || tw == 0 || (!dense && (th & 1))) return fail(CI_ERR_ARG, "transposed linear: bad tile shape");
     if (x_stride < H || out_stride < V) return fail(CI_ERR_ARG, "transposed linear: row stride shorter than the row");
-    if (!aligned(d_slot_map, 4)) return fail(CI_ERR_ARG, "transposed linear: slot_map must be 4-byte aligned");
     const size_t need = ci_fused_linear_transposed_workspace_bytes(M, H, V, tw);
     if (!d_workspace || workspace_bytes < need)
         return fail(CI_ERR_CAPACITY, "transposed linear: workspace needs %zu bytes, got %zu", need, workspace_bytes);
@@ -293,6 +310,7 @@ static int transposed_impl(const uint16_t *d_x, uint32_t M, uint32_t H, uint32_t
     a.stream_offsets = dense ? d_meta0 : nullptr;
     a.stream_sizes = dense ? d_meta1 : nullptr;
     a.man_tiled = d_man_tiled;
+    a.dense_w = d_plain_w;
     a.partial = static_cast<float *>(d_workspace);
     a.th = th;
     a.tw = tw;
@@ -300,7 +318,8 @@ static int transposed_impl(const uint16_t *d_x, uint32_t M, uint32_t H, uint32_t
     a.tiles_k = ceil_div(V, th);
     a.num_tiles = a.tiles_n * a.tiles_k;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const bool fast = !dense && tw == 32 && aligned(d_stream, 16) && aligned(d_man_tiled, 4);
+    const bool fast = !dense && tw == 32 && (d_plain_w || (aligned(d_stream, 16) && aligned(d_man_tiled, 4)));
+    if (d_plain_w && !fast) return fail(CI_ERR_ARG, "plain-weight transposed linear: only the 32-column tiling");
     uint32_t cus = 1;
     if (fast) {
         int dev = 0, n = 0;
@@ -367,4 +386,15 @@ extern "C" int ci_fused_linear_transposed_dense(const uint16_t *d_x, uint32_t M,
     return transposed_impl(d_x, M, H, V, x_stride, d_stream, stream_len, d_states, d_tables, d_slot_map,
                            d_stream_offsets, d_stream_sizes, d_man_tiled, tile_height, tile_width, d_bias, d_out,
                            out_stride, d_workspace, workspace_bytes, true, stream);
+}
+
+extern "C" int ci_plain_linear_transposed_same_order(const uint16_t *d_x, uint32_t M, uint32_t H, uint32_t V,
+                                                     uint32_t x_stride, const uint16_t *d_w, uint32_t tile_height,
+                                                     uint32_t tile_width, const uint16_t *d_bias, uint16_t *d_out,
+                                                     uint32_t out_stride, void *d_workspace, size_t workspace_bytes,
+                                                     ci_stream_t stream) {
+    if (!d_w) return fail(CI_ERR_ARG, "plain-weight transposed linear: null weight");
+    return transposed_impl(d_x, M, H, V, x_stride, nullptr, 0, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr,
+                           tile_height, tile_width, d_bias, d_out, out_stride, d_workspace, workspace_bytes, false,
+                           stream, d_w);
 }

@@ -126,6 +126,32 @@ def splitk_reduce(workspace: torch.Tensor, bias=None, out=None):
     return result
 
 
+def plain_linear_same_order(x, weight_kn, tile_k=1024, tile_n=32, bias=None, workspace=None):
+    """x[..., K] @ weight_kn[K, N] (+ bias) for an uncompressed bf16 weight, through the fused kernel's
+    own contraction: same tiling, same matrix instructions in the same order, same partial sums.  The
+    result is bit-identical to `fused_rans_linear` on the compressed form of `weight_kn` (tile
+    `tile_k` x 32), which `torch.matmul` is not (other summation order).  A verification aid without
+    a counterpart in the reference; slow.  `workspace` as for `fused_rans_linear`: when the contraction is
+    split over K, the fp32 partial sums [P, M, N] are left at its start."""
+    _lib.require_device(x)
+    _lib.require_device(weight_kn)
+    if weight_kn.dtype != torch.bfloat16 or weight_kn.dim() != 2:
+        raise RuntimeError("weight_kn must be a 2-D bfloat16 tensor [K, N]")
+    dev = x.device
+    w = weight_kn.contiguous()
+    K, N = w.shape
+    x2 = _prep_x(x, K)
+    M = x2.shape[0]
+    result = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+    need = lib().ci_fused_linear_workspace_bytes(M, K, N, int(tile_k), int(tile_n), 0)
+    ws, ws_bytes = _pick_workspace(workspace, need, dev)
+    b = bias.to(device=dev, dtype=torch.bfloat16).contiguous() if bias is not None else None
+    check(lib().ci_plain_linear_same_order(ptr(x2), M, K, N, x2.stride(0), ptr(w), int(tile_k), int(tile_n), ptr(b),
+                                           ptr(result), result.stride(0), ptr(ws), C.c_size_t(ws_bytes),
+                                           _lib.stream_handle(dev)))
+    return result.view(*x.shape[:-1], N)
+
+
 # Names under which the reference exports these ops (comp_inference/__init__.py:39-42).
 fused_rans_linear_triton = fused_rans_linear
 fused_rans_linear_triton_uncoalesced = fused_rans_linear_uncoalesced

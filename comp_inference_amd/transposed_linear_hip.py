@@ -67,6 +67,30 @@ def fused_rans_linear_transposed_uncoalesced(x, compressed_data, initial_states,
                 tile_k, tile_n, mantissas, bias, out, dense=True)
 
 
+def plain_linear_transposed_same_order(x, weight_vh, tile_k=1024, tile_n=32, bias=None):
+    """x[..., H] @ weight_vh[V, H]^T (+ bias) for an uncompressed bf16 weight, through the fused
+    kernel's own products and reductions: bit-identical to `fused_rans_linear_transposed` on the
+    compressed form of `weight_vh` (tile `tile_k` x 32).  A verification aid without a counterpart in
+    the reference; slow."""
+    _lib.require_device(x)
+    _lib.require_device(weight_vh)
+    if weight_vh.dtype != torch.bfloat16 or weight_vh.dim() != 2:
+        raise RuntimeError("weight_vh must be a 2-D bfloat16 tensor [V, H]")
+    dev = x.device
+    w = weight_vh.contiguous()
+    V, H = w.shape
+    x2 = _prep_x(x, H)
+    M = x2.shape[0]
+    result = torch.empty((M, V), dtype=torch.bfloat16, device=dev)
+    need = lib().ci_fused_linear_transposed_workspace_bytes(M, H, V, int(tile_n))
+    ws = _Scratch.get(need, ("lmhead", dev))
+    b = bias.to(device=dev, dtype=torch.bfloat16).contiguous() if bias is not None else None
+    check(lib().ci_plain_linear_transposed_same_order(ptr(x2), M, H, V, x2.stride(0), ptr(w), int(tile_k), int(tile_n),
+                                                      ptr(b), ptr(result), result.stride(0), ptr(ws),
+                                                      C.c_size_t(ws.numel()), _lib.stream_handle(dev)))
+    return result.view(*x.shape[:-1], V)
+
+
 # Names under which the reference exports these ops (comp_inference/__init__.py:44-47).
 fused_rans_linear_transposed_triton = fused_rans_linear_transposed
 fused_rans_linear_transposed_triton_uncoalesced = fused_rans_linear_transposed_uncoalesced

@@ -292,6 +292,32 @@ typedef struct ci_decode_item {
 
 int ci_decode_tiled_ilp2_batch(const ci_decode_item *h_items, uint32_t n_items, ci_stream_t stream);
 
+/* ---------------------------------------------------------------------------------------
+ * Verification aids: the contraction of the fused kernels applied to a plain (uncompressed) bf16
+ * weight.  No counterpart in the reference, whose tests compare the fused kernels with
+ * torch.matmul within allclose(1e-2, 1e-2) (tests/test_mat_mul.py:220, :238) -- a bar that a wrong
+ * low mantissa bit passes.  These run the same kernels with the same tiling, the same sequence of
+ * matrix instructions, partial sums and reductions as ci_fused_linear_ilp2 /
+ * ci_fused_linear_transposed_ilp2 for the same (M, K, N, tile shape), but read the weights from
+ * d_w instead of decoding them; their output is therefore bit-identical to the fused kernels' on
+ * the compressed form of d_w, and a run of a whole model on decompressed weights can be compared
+ * token by token.  Slow (no staging, guarded loads); 32-column tiles only.
+ *   ci_plain_linear_same_order:             d_w = bf16 [K, N] row-major; workspace as
+ *                                           ci_fused_linear_workspace_bytes(M, K, N, th, tw, 0)
+ *   ci_plain_linear_transposed_same_order:  d_w = bf16 [V, H] row-major; workspace as
+ *                                           ci_fused_linear_transposed_workspace_bytes(M, H, V, tw)
+ * ------------------------------------------------------------------------------------- */
+int ci_plain_linear_same_order(const uint16_t *d_x, uint32_t M, uint32_t K, uint32_t N, uint32_t x_stride,
+                               const uint16_t *d_w, uint32_t tile_height, uint32_t tile_width,
+                               const uint16_t *d_bias, uint16_t *d_out, uint32_t out_stride,
+                               void *d_workspace, size_t workspace_bytes, ci_stream_t stream);
+
+int ci_plain_linear_transposed_same_order(const uint16_t *d_x, uint32_t M, uint32_t H, uint32_t V,
+                                          uint32_t x_stride, const uint16_t *d_w, uint32_t tile_height,
+                                          uint32_t tile_width, const uint16_t *d_bias, uint16_t *d_out,
+                                          uint32_t out_stride, void *d_workspace, size_t workspace_bytes,
+                                          ci_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

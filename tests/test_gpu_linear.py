@@ -137,3 +137,75 @@ def test_dense_matmul_helper():
         assert torch.allclose(got.float(), want, atol=ATOL, rtol=RTOL)
     with pytest.raises(RuntimeError):
         triton_matmul(torch.zeros(1, 512, dtype=torch.bfloat16), b)
+
+
+@pytest.mark.parametrize("K,N,th,M", [
+    (4096, 256, 1024, 1), (4096, 256, 1024, 16), (4096, 256, 1024, 17), (4096, 256, 1024, 64),
+    (4096, 256, 1024, 100),      # more than 64 rows: one pass per 64
+    (3072, 128, 512, 4),
+    (14336, 64, 1024, 1),        # two partial sums per output + reduction kernel
+    (14336, 64, 1024, 40),
+    (1300, 80, 1024, 3),         # ragged K and N: guarded path in both runs
+    (1300, 80, 1024, 50),
+    (2048, 32800, 1024, 3),      # resident workgroups, one partial per k-tile
+    (2048, 32800, 1024, 40),
+])
+def test_fused_linear_bit_identical_to_plain_weight_contraction(oracle, K, N, th, M):
+    """The fused kernel on the compressed weight and the same contraction on the plain bf16 weight give
+    the same bits: every weight bit, sign and low mantissa bits included, reaches the matrix unit
+    as the encoder saw it -- which the 1e-2 tolerance against torch.matmul cannot show."""
+    from comp_inference_amd import plain_linear_same_order
+
+    w = make_weight_kn(N, K, seed=K + N + 1)
+    enc, man, wdec = _compress(oracle, w, th, 32)
+    x = make_x(M, K, seed=M + 7)
+    bias = make_x(1, N, seed=3).view(N) if M == 3 else None
+    got = _call(enc, man, x, K, N, th, 32, bias=bias)
+    same = plain_linear_same_order(x.cuda(), wdec.cuda(), tile_k=th, tile_n=32,
+                                   bias=None if bias is None else bias.cuda())
+    assert same.shape == got.shape and same.dtype == torch.bfloat16
+    assert torch.equal(got.view(torch.int16), same.view(torch.int16))
+    want = torch.matmul(x.float(), wdec.float()) + (0 if bias is None else bias.float())
+    assert torch.allclose(same.float().cpu(), want, atol=ATOL, rtol=RTOL)
+
+
+@pytest.mark.parametrize("K,N,M,P", [(14336, 64, 1, 2), (14336, 64, 40, 2), (2048, 32800, 3, 2)])
+def test_fp32_partial_sums_bit_identical_and_sharp(oracle, K, N, M, P):
+    """Where the contraction is split over K the fp32 partial sums stay in the caller's workspace: they
+    too are equal bit for bit, and one flipped low mantissa bit of one weight changes exactly the
+    partial sums of its column -- an error far below what the bf16 output or a 1e-2 tolerance shows."""
+    from comp_inference_amd import plain_linear_same_order
+
+    th = 1024
+    w = make_weight_kn(N, K, seed=K + N + 2)
+    enc, man, wdec = _compress(oracle, w, th, 32)
+    x = make_x(M, K, seed=M + 30)
+    nbytes = P * M * N * 4 + (1 << 22)
+    ws_a = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+    ws_b = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+    got = _call(enc, man, x, K, N, th, 32, workspace=ws_a)
+    same = plain_linear_same_order(x.cuda(), wdec.cuda(), tile_k=th, tile_n=32, workspace=ws_b)
+    pa = ws_a[:P * M * N * 4].view(torch.int32).view(P, M, N)
+    pb = ws_b[:P * M * N * 4].view(torch.int32).view(P, M, N)
+    assert torch.equal(got.view(torch.int16), same.view(torch.int16))
+    assert torch.equal(pa, pb)
+    assert int((pa != 0).sum()) > P * M * N // 2       # (the workspace really holds the partial sums)
+
+    bits = wdec.view(torch.int16).clone()
+    k = int(x[0].float().abs().argmax())               # a row of the weight that certainly contributes
+    bits[k, 5] ^= 1
+    plain_linear_same_order(x.cuda(), bits.view(torch.bfloat16).cuda(), tile_k=th, tile_n=32, workspace=ws_b)
+    torch.cuda.synchronize()
+    diff = (pa != pb).nonzero()
+    assert diff.numel() > 0 and set(diff[:, 2].tolist()) == {5}
+
+
+def test_plain_weight_contraction_rejects_other_tilings():
+    from comp_inference_amd import plain_linear_same_order
+
+    x = torch.zeros(1, 256, dtype=torch.bfloat16, device="cuda")
+    w = torch.zeros(256, 128, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(RuntimeError):
+        plain_linear_same_order(x, w, tile_k=64, tile_n=16)
+    with pytest.raises(RuntimeError):
+        plain_linear_same_order(x.cpu(), w)

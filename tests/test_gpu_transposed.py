@@ -56,3 +56,51 @@ def test_transposed_linear_dense_layout(oracle):
         th, tw, torch.from_numpy(man).to(dev), workspace=None)
     want = torch.matmul(x.float(), w.float().t())
     assert torch.allclose(got.float().cpu(), want, atol=ATOL, rtol=RTOL)
+
+
+@pytest.mark.parametrize("V,H,th,M", [
+    (2048, 128, 1024, 1), (2048, 128, 1024, 4), (2048, 128, 1024, 6),
+    (1300, 96, 1024, 1),    # short last tile row: the bottom half has fewer rows than the top half
+    (1300, 96, 1024, 3),
+    (2048, 64, 512, 2),
+    (700, 100, 256, 2),     # ragged columns: guarded steps in both runs
+])
+def test_transposed_linear_bit_identical_to_plain_weight_contraction(oracle, V, H, th, M):
+    """Fused kernel on the compressed [V, H] weight == the same products and reductions on the plain bf16
+    weight, bit for bit (sharper than the tolerance against torch.matmul)."""
+    from comp_inference_amd import fused_rans_linear_transposed_triton, plain_linear_transposed_same_order
+
+    w = make_weight_kn(H, V, seed=V + H + 1)  # [V, H]
+    enc, man = oracle.compress_bf16(bf16_bits(w), th, 32)
+    x = make_x(M, H, seed=M + 20)
+    dev = "cuda"
+    got = fused_rans_linear_transposed_triton(
+        x.to(dev), torch.from_numpy(enc.stream).to(dev), _t32(enc.states).to(dev), _t32(enc.tables).to(dev),
+        torch.from_numpy(enc.slot_map).to(dev), (V, H), _t32(enc.tile_offsets).to(dev),
+        _t32(enc.tile_max_lens).to(dev), th, 32, torch.from_numpy(man).to(dev), workspace=None)
+    same = plain_linear_transposed_same_order(x.to(dev), w.to(dev), tile_k=th, tile_n=32)
+    assert torch.equal(got.view(torch.int16), same.view(torch.int16))
+    want = torch.matmul(x.float(), w.float().t())
+    assert torch.allclose(same.float().cpu(), want, atol=ATOL, rtol=RTOL)
+
+
+def test_transposed_guarded_and_fast_tiles_sum_alike(oracle):
+    """A tile's partial sums do not depend on the path it took: bodies too deep for the staging area
+    (nearly incompressible exponents) take guarded steps, and still match the plain-weight contraction."""
+    from comp_inference_amd import fused_rans_linear_transposed_triton, plain_linear_transposed_same_order
+
+    V, H, th, M = 2048, 64, 1024, 2
+    rng = np.random.default_rng(5)
+    bits = rng.integers(0, 1 << 16, size=(V, H), dtype=np.uint16)
+    bits = (bits & 0x807F) | (rng.integers(100, 140, size=(V, H)).astype(np.uint16) << 7)  # 40 exponents, finite
+    w = torch.from_numpy(bits.view(np.int16)).view(torch.bfloat16)
+    enc, man = oracle.compress_bf16(bits, th, 32)
+    assert int(enc.tile_max_lens.max()) >= 254      # deeper than the largest lane stride
+    x = make_x(M, H, seed=9)
+    dev = "cuda"
+    got = fused_rans_linear_transposed_triton(
+        x.to(dev), torch.from_numpy(enc.stream).to(dev), _t32(enc.states).to(dev), _t32(enc.tables).to(dev),
+        torch.from_numpy(enc.slot_map).to(dev), (V, H), _t32(enc.tile_offsets).to(dev),
+        _t32(enc.tile_max_lens).to(dev), th, 32, torch.from_numpy(man).to(dev), workspace=None)
+    same = plain_linear_transposed_same_order(x.to(dev), w.to(dev), tile_k=th, tile_n=32)
+    assert torch.equal(got.view(torch.int16), same.view(torch.int16))
