@@ -32,6 +32,27 @@ class _Scratch:
         return b
 
 
+# Rows of x above which the fused linear decodes the weight ONCE into a bf16 scratch and multiplies with
+# a library GEMM (hipBLASLt through torch.matmul), instead of decoding it inside the product once per
+# 64 rows: with hundreds of prompt tokens the decode, not the product, would otherwise be repeated
+# (gate projection 4096 x 14336: 121 us fused against 96 us at 96 rows, 1497 against 264 at 2048).
+# None switches the policy off.  The reference always fuses, one decode per 16 rows
+# (comp_inference/linear_triton.py:250-266).
+DECODE_ONCE_ABOVE_ROWS = 64
+
+
+def _decode_once_weight(dev, compressed_data, initial_states, tables, slot_map, shape, tile_offsets, tile_max_lens,
+                        tile_k, tile_n, mantissas, tag):
+    """The bf16 weight, decoded into a grow-only scratch of its own (valid until the next such call)."""
+    from .rans_hip import rans_decomp_tiled
+
+    rows, cols = shape
+    buf = _Scratch.get(rows * cols * 2, (tag, dev))
+    w = buf[:rows * cols * 2].view(torch.bfloat16).view(rows, cols)
+    return rans_decomp_tiled(compressed_data, initial_states, tables, slot_map, (rows, cols), tile_offsets,
+                             tile_max_lens, tile_k=tile_k, tile_n=tile_n, mantissas=mantissas, out=w)
+
+
 def _prep_x(x: torch.Tensor, K: int):
     if x.dtype != torch.bfloat16:
         x = x.to(torch.bfloat16)  # the kernel computes on bf16 (comp_inference/linear_triton.py:431-436)
@@ -68,6 +89,16 @@ def _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, met
         result = out.view(M, N) if out.is_contiguous() else out
         if result.stride(-1) != 1:
             raise RuntimeError("out must have unit stride in its last dimension")
+    if not dense and DECODE_ONCE_ABOVE_ROWS is not None and M > DECODE_ONCE_ABOVE_ROWS:
+        w = _decode_once_weight(dev, compressed_data, initial_states, tables, slot_map, (K, N), meta0, meta1,
+                                int(tile_k), int(tile_n), mantissas, "weight_kn")
+        if result.is_contiguous():
+            torch.matmul(x2.detach(), w, out=result)  # (like the fused kernels: inference only)
+        else:
+            result.copy_(torch.matmul(x2.detach(), w))
+        if bias is not None:  # the reference's `out += bias` on the bf16 result
+            result += bias.to(device=dev, dtype=torch.bfloat16)
+        return out if out is not None else result.view(*x.shape[:-1], N)
     stream_t = _lib.as_u8(compressed_data, dev)
     man = _lib.as_u8(mantissas, dev).view(-1)
     need_man = (-(-K // tile_k)) * (-(-N // tile_n)) * tile_k * tile_n
@@ -131,7 +162,8 @@ def plain_linear_same_order(x, weight_kn, tile_k=1024, tile_n=32, bias=None, wor
     own contraction: same tiling, same matrix instructions in the same order, same partial sums.  The
     result is bit-identical to `fused_rans_linear` on the compressed form of `weight_kn` (tile
     `tile_k` x 32), which `torch.matmul` is not (other summation order).  A verification aid without
-    a counterpart in the reference; slow.  `workspace` as for `fused_rans_linear`: when the contraction is
+    a counterpart in the reference; slow.  Above DECODE_ONCE_ABOVE_ROWS rows it does what
+    `fused_rans_linear` does there, a library GEMM.  `workspace` as for `fused_rans_linear`: when the contraction is
     split over K, the fp32 partial sums [P, M, N] are left at its start."""
     _lib.require_device(x)
     _lib.require_device(weight_kn)
@@ -142,6 +174,12 @@ def plain_linear_same_order(x, weight_kn, tile_k=1024, tile_n=32, bias=None, wor
     K, N = w.shape
     x2 = _prep_x(x, K)
     M = x2.shape[0]
+    if DECODE_ONCE_ABOVE_ROWS is not None and M > DECODE_ONCE_ABOVE_ROWS:
+        # what fused_rans_linear computes for this many rows: a library GEMM on the decoded weight
+        result = torch.matmul(x2, w)
+        if bias is not None:
+            result += bias.to(device=dev, dtype=torch.bfloat16)
+        return result.view(*x.shape[:-1], N)
     result = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
     need = lib().ci_fused_linear_workspace_bytes(M, K, N, int(tile_k), int(tile_n), 0)
     ws, ws_bytes = _pick_workspace(workspace, need, dev)

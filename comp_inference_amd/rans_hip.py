@@ -19,10 +19,11 @@ def _tiles(K: int, N: int, tile_k: int, tile_n: int):
 
 
 def rans_decomp_tiled(compressed_streams, initial_states, tables, slot_map, output_shape,
-                      tile_offsets, tile_max_lens, tile_k=1024, tile_n=32, mantissas=None):
+                      tile_offsets, tile_max_lens, tile_k=1024, tile_n=32, mantissas=None, out=None):
     """Decode the tiled two-streams-per-column format into the exponent plane u8[K,N]
     (comp_inference/rans_triton.py:122-168).  With `mantissas` (the tile-interleaved sign|mantissa
-    plane) the bf16 weight [K,N] is returned instead, merged in the same kernel."""
+    plane) the bf16 weight [K,N] is returned instead, merged in the same kernel.  `out`: a contiguous
+    GPU tensor of that shape and dtype to decode into (not in the reference's signature)."""
     K, N = int(output_shape[0]), int(output_shape[1])
     num_tiles_n, num_tiles_k = _tiles(K, N, tile_k, tile_n)
     expected_streams = num_tiles_n * num_tiles_k * tile_n * 2
@@ -38,10 +39,13 @@ def rans_decomp_tiled(compressed_streams, initial_states, tables, slot_map, outp
         need = num_tiles_k * num_tiles_n * tile_k * tile_n
         if man.numel() < need:  # a truncated tail reads as zero padding (comp_inference.py:76-83)
             man = torch.nn.functional.pad(man, (0, need - man.numel()))
-        out = torch.empty((K, N), device=dev, dtype=torch.bfloat16)
     else:
         man = None
-        out = torch.empty((K, N), device=dev, dtype=torch.uint8)
+    want = torch.bfloat16 if merge else torch.uint8
+    if out is None:
+        out = torch.empty((K, N), device=dev, dtype=want)
+    elif out.dtype != want or tuple(out.shape) != (K, N) or out.device != dev or not out.is_contiguous():
+        raise RuntimeError(f"out must be a contiguous {want} tensor of shape ({K}, {N}) on {dev}")
     # device copies must stay referenced until the launch has been enqueued
     st, tb, sm = _lib.as_u32(initial_states, dev), _lib.as_u32(tables, dev), _lib.as_u8(slot_map, dev)
     to, tl = _lib.as_u32(tile_offsets, dev), _lib.as_u32(tile_max_lens, dev)

@@ -11,7 +11,13 @@ import torch
 
 from . import _lib
 from ._lib import check, lib, ptr
+from . import linear_hip
 from .linear_hip import _Scratch, _prep_x
+
+# Rows of x above which the weight is decoded once into a bf16 scratch and multiplied with a library
+# GEMM; the fused kernel walks the whole table once per 4 rows (128256 x 4096 table: 1286 us fused against
+# 791 us at 5 rows, 23 ms against 0.83 ms at 128).  None switches the policy off.
+DECODE_ONCE_ABOVE_ROWS = 4
 
 
 def _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, meta0, meta1, tile_k, tile_n,
@@ -27,6 +33,16 @@ def _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, met
         if out.dtype != torch.bfloat16 or not out.is_cuda:
             raise RuntimeError("out must be a bfloat16 GPU tensor")
         result = out.view(M, V)
+    if not dense and DECODE_ONCE_ABOVE_ROWS is not None and M > DECODE_ONCE_ABOVE_ROWS:
+        w = linear_hip._decode_once_weight(dev, compressed_data, initial_states, tables, slot_map, (V, H), meta0, meta1,
+                                           int(tile_k), int(tile_n), mantissas, "weight_vh")
+        if result.is_contiguous():
+            torch.matmul(x2.detach(), w.t(), out=result)  # (like the fused kernels: inference only)
+        else:
+            result.copy_(torch.matmul(x2.detach(), w.t()))
+        if bias is not None:
+            result += bias.to(device=dev, dtype=torch.bfloat16)
+        return out if out is not None else result.view(*x.shape[:-1], V)
     stream_t = _lib.as_u8(compressed_data, dev)
     man = _lib.as_u8(mantissas, dev).view(-1)
     need_man = (-(-V // tile_k)) * (-(-H // tile_n)) * tile_k * tile_n
@@ -81,6 +97,12 @@ def plain_linear_transposed_same_order(x, weight_vh, tile_k=1024, tile_n=32, bia
     V, H = w.shape
     x2 = _prep_x(x, H)
     M = x2.shape[0]
+    if DECODE_ONCE_ABOVE_ROWS is not None and M > DECODE_ONCE_ABOVE_ROWS:
+        # what fused_rans_linear_transposed computes for this many rows: a library GEMM on the decoded weight
+        result = torch.matmul(x2, w.t())
+        if bias is not None:
+            result += bias.to(device=dev, dtype=torch.bfloat16)
+        return result.view(*x.shape[:-1], V)
     result = torch.empty((M, V), dtype=torch.bfloat16, device=dev)
     need = lib().ci_fused_linear_transposed_workspace_bytes(M, H, V, int(tile_n))
     ws = _Scratch.get(need, ("lmhead", dev))

@@ -18,3 +18,13 @@ def oracle():
 
     rans_oracle.build()
     return rans_oracle
+
+
+@pytest.fixture
+def always_fused(monkeypatch):
+    """Many-row inputs normally decode the weight once and call a library GEMM; with this fixture they stay
+    on the fused kernels (one decode per pass of rows)."""
+    from comp_inference_amd import linear_hip, transposed_linear_hip
+
+    monkeypatch.setattr(linear_hip, "DECODE_ONCE_ABOVE_ROWS", None)
+    monkeypatch.setattr(transposed_linear_hip, "DECODE_ONCE_ABOVE_ROWS", None)

@@ -189,3 +189,27 @@ def test_flat_encode_decode(oracle, K, N):
     assert np.array_equal(flat.cpu().numpy(), want)
     if K <= 512:
         assert np.array_equal(want.reshape(K, N), sym)
+
+
+def test_tiled_decode_into_caller_tensor(oracle):
+    """`out=`: decode in place into a tensor of the caller (exponent plane or merged bf16)."""
+    from comp_inference_amd import rans_decomp_tiled
+
+    K, N, th, tw = 1300, 80, 1024, 32
+    w = make_weight_kn(N, K, seed=31)
+    bits = bf16_bits(w)
+    enc, man = oracle.compress_bf16(bits, th, tw)
+    dev = "cuda"
+    args = (torch.from_numpy(enc.stream).to(dev), _t32(enc.states).to(dev), _t32(enc.tables).to(dev),
+            torch.from_numpy(enc.slot_map).to(dev), (K, N), _t32(enc.tile_offsets).to(dev),
+            _t32(enc.tile_max_lens).to(dev))
+    e = torch.empty(K, N, dtype=torch.uint8, device=dev)
+    assert rans_decomp_tiled(*args, tile_k=th, tile_n=tw, out=e) is e
+    assert np.array_equal(e.cpu().numpy(), (bits >> 7).astype(np.uint8))
+    b = torch.empty(K, N, dtype=torch.bfloat16, device=dev)
+    assert rans_decomp_tiled(*args, tile_k=th, tile_n=tw, mantissas=torch.from_numpy(man).to(dev), out=b) is b
+    assert torch.equal(b.cpu().view(torch.int16), w.view(torch.int16))
+    with pytest.raises(RuntimeError):
+        rans_decomp_tiled(*args, tile_k=th, tile_n=tw, out=b)            # wrong dtype for the exponent plane
+    with pytest.raises(RuntimeError):
+        rans_decomp_tiled(*args, tile_k=th, tile_n=tw, out=e[:, :40])    # wrong shape

@@ -209,3 +209,45 @@ def test_plain_weight_contraction_rejects_other_tilings():
         plain_linear_same_order(x, w, tile_k=64, tile_n=16)
     with pytest.raises(RuntimeError):
         plain_linear_same_order(x.cpu(), w)
+
+
+def test_many_rows_decode_the_weight_once(oracle):
+    """Above DECODE_ONCE_ABOVE_ROWS rows the weight is decoded once and a library GEMM does the product:
+    the result is torch.matmul on the decoded weight, bit for bit, with bias and a strided `out`."""
+    from comp_inference_amd import linear_hip
+
+    K, N, th, M = 2048, 160, 1024, 200
+    assert M > linear_hip.DECODE_ONCE_ABOVE_ROWS
+    w = make_weight_kn(N, K, seed=21)
+    enc, man, wdec = _compress(oracle, w, th, 32)
+    x = make_x(M, K, seed=22).cuda()
+    bias = make_x(1, N, seed=23).view(N).cuda()
+    want = torch.matmul(x, wdec.cuda())
+    want += bias
+    got = _call(enc, man, x, K, N, th, 32, bias=bias)
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    big = torch.zeros(M, N + 32, dtype=torch.bfloat16, device="cuda")
+    ret = _call(enc, man, x, K, N, th, 32, bias=bias, out=big[:, :N])
+    assert ret.data_ptr() == big.data_ptr()
+    assert torch.equal(big[:, :N].view(torch.int16), want.view(torch.int16)) and not big[:, N:].any()
+    # 3-D input keeps its leading shape
+    got3 = _call(enc, man, x.view(2, 100, K), K, N, th, 32)
+    assert tuple(got3.shape) == (2, 100, N)
+
+
+@pytest.mark.parametrize("K,N,th,M", [(4096, 256, 1024, 100), (3072, 128, 512, 150), (1300, 80, 1024, 70)])
+def test_fused_kernels_above_64_rows(oracle, always_fused, K, N, th, M):
+    """With the decode-once policy off, more than 64 rows run the fused kernel in passes of 64: within
+    tolerance of torch.matmul and bit-identical to the same contraction on the plain weight."""
+    from comp_inference_amd import plain_linear_same_order
+
+    w = make_weight_kn(N, K, seed=K + M)
+    enc, man, wdec = _compress(oracle, w, th, 32)
+    x = make_x(M, K, seed=M)
+    got = _call(enc, man, x, K, N, th, 32)
+    want = torch.matmul(x.float(), wdec.float())
+    assert torch.allclose(got.float().cpu(), want, atol=ATOL, rtol=RTOL), (got.float().cpu() - want).abs().max()
+    same = plain_linear_same_order(x.cuda(), wdec.cuda(), tile_k=th, tile_n=32)
+    assert torch.equal(got.view(torch.int16), same.view(torch.int16))
+    # and it is not the library GEMM's summation order
+    assert not torch.equal(got.view(torch.int16), torch.matmul(x.cuda(), wdec.cuda()).view(torch.int16))

@@ -104,3 +104,39 @@ def test_transposed_guarded_and_fast_tiles_sum_alike(oracle):
         _t32(enc.tile_max_lens).to(dev), th, 32, torch.from_numpy(man).to(dev), workspace=None)
     same = plain_linear_transposed_same_order(x.to(dev), w.to(dev), tile_k=th, tile_n=32)
     assert torch.equal(got.view(torch.int16), same.view(torch.int16))
+
+
+@pytest.mark.parametrize("V,H,th,M", [(2048, 128, 1024, 6), (1300, 96, 1024, 9), (2048, 64, 512, 5)])
+def test_transposed_fused_kernel_above_4_rows(oracle, always_fused, V, H, th, M):
+    """With the decode-once policy off, more than 4 rows run the fused kernel in passes of 4."""
+    from comp_inference_amd import fused_rans_linear_transposed_triton, plain_linear_transposed_same_order
+
+    w = make_weight_kn(H, V, seed=V + M)
+    enc, man = oracle.compress_bf16(bf16_bits(w), th, 32)
+    x = make_x(M, H, seed=M + 40)
+    dev = "cuda"
+    got = fused_rans_linear_transposed_triton(
+        x.to(dev), torch.from_numpy(enc.stream).to(dev), _t32(enc.states).to(dev), _t32(enc.tables).to(dev),
+        torch.from_numpy(enc.slot_map).to(dev), (V, H), _t32(enc.tile_offsets).to(dev),
+        _t32(enc.tile_max_lens).to(dev), th, 32, torch.from_numpy(man).to(dev), workspace=None)
+    want = torch.matmul(x.float(), w.float().t())
+    assert torch.allclose(got.float().cpu(), want, atol=ATOL, rtol=RTOL)
+    same = plain_linear_transposed_same_order(x.to(dev), w.to(dev), tile_k=th, tile_n=32)
+    assert torch.equal(got.view(torch.int16), same.view(torch.int16))
+
+
+def test_transposed_many_rows_decode_the_weight_once(oracle):
+    """Above DECODE_ONCE_ABOVE_ROWS rows: torch.matmul on the weight decoded once, bit for bit."""
+    from comp_inference_amd import fused_rans_linear_transposed_triton
+
+    V, H, th, M = 1300, 96, 1024, 20
+    w = make_weight_kn(H, V, seed=51)
+    enc, man = oracle.compress_bf16(bf16_bits(w), th, 32)
+    x = make_x(M, H, seed=52).cuda()
+    dev = "cuda"
+    got = fused_rans_linear_transposed_triton(
+        x, torch.from_numpy(enc.stream).to(dev), _t32(enc.states).to(dev), _t32(enc.tables).to(dev),
+        torch.from_numpy(enc.slot_map).to(dev), (V, H), _t32(enc.tile_offsets).to(dev),
+        _t32(enc.tile_max_lens).to(dev), th, 32, torch.from_numpy(man).to(dev), workspace=None)
+    want = torch.matmul(x, w.cuda().t())
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
