@@ -213,3 +213,31 @@ def test_tiled_decode_into_caller_tensor(oracle):
         rans_decomp_tiled(*args, tile_k=th, tile_n=tw, out=b)            # wrong dtype for the exponent plane
     with pytest.raises(RuntimeError):
         rans_decomp_tiled(*args, tile_k=th, tile_n=tw, out=e[:, :40])    # wrong shape
+
+
+def test_flat_one_column_as_the_reference_script_drives_it(oracle):
+    """tests/test_rans.py:55-131 of the reference: numpy bytes of one column through RansManager.compress
+    and decompress_into with pinned buffers.  With more than one 512-row segment the extension's strided
+    decoder returns the segments transposed (the reference's encoder and decoder disagree,
+    src/cuda/rans_kernels.cuh:470-471 against :659-680); the segment-aware decoder returns the data."""
+    from comp_inference_amd import ccore, rans_decomp_triton
+
+    size = 4 << 20
+    data = zipf_bytes(size, 4.0, 17)
+    f, c = oracle.get_lut(data)
+    pinned_input, pinned_output = ccore.allocate_pinned_memory(size), ccore.allocate_pinned_memory(size)
+    np.copyto(pinned_input, data)
+    manager = ccore.RansManager(size)
+    res = manager.compress(pinned_input, f, c, 512)
+    S = res.num_streams
+    assert S == size // 512 and res.stream.size == int(res.output_sizes.max()) * S
+    ms = manager.decompress_into(res.stream, res.states, res.output_sizes, S, f, c, pinned_output)
+    assert ms > 0
+    assert np.array_equal(pinned_output.reshape(512, S), data.reshape(S, 512).T)
+    out, _ = manager.decompress(res.stream, res.states, res.output_sizes, S, size, f, c)
+    assert np.array_equal(out, pinned_output)
+    dev = "cuda"
+    tables, slot_map = oracle.build_tables(f, c)
+    seg = rans_decomp_triton(torch.from_numpy(res.stream).to(dev), _t32(res.states).to(dev), _t32(tables).to(dev),
+                             torch.from_numpy(slot_map).to(dev), _t32(res.output_sizes).to(dev), (size, 1))
+    assert np.array_equal(seg.cpu().numpy().reshape(-1), data)
