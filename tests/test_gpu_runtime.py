@@ -157,3 +157,60 @@ def test_load_compressed_model_into_skeleton(tmp_path):
                        originals["down_proj.weight"].t().contiguous().view(torch.int16))
     assert torch.equal(dst.embed_tokens.weight.detach().cpu().view(torch.int16),
                        originals["embed_tokens.weight"].view(torch.int16))
+
+
+def _fused_forward(proj, x):
+    import comp_inference_amd as ci
+
+    K, N = proj.input_shape
+    return ci.fused_rans_linear_triton(
+        x=x, compressed_data=proj.exponent_compressed_weight.cuda(), initial_states=proj.exponent_states.cuda(),
+        tables=proj.exponent_tables.cuda(), slot_map=proj.exponent_slot_map.cuda(), weight_shape=(K, N),
+        tile_offsets=proj.exponent_tile_offsets.cuda(), tile_max_lens=proj.exponent_tile_max_lens.cuda(),
+        tile_k=proj.exponent_tile_height, tile_n=proj.exponent_tile_width, mantissas=proj.mantissa_raw.cuda())
+
+
+def test_fused_qkv_and_gate_up_compression():
+    """comp_inference/comp_inference.py:242-341: q/k/v (and gate/up) concatenated along the outputs and
+    compressed as one weight under the first projection's name; the reference's own check feeds real
+    activations through the fused QKV and compares with torch.matmul (tests/test_fused_model.py:66-95,
+    8 rows, K = 1024, N = 4096, max difference below 0.1)."""
+    import comp_inference_amd as ci
+
+    torch.manual_seed(3)
+    K, Nq, Nkv, F = 1024, 2048, 1024, 3072
+
+    class Attn(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.q_proj, self.k_proj, self.v_proj = (nn.Linear(K, Nq, bias=False), nn.Linear(K, Nkv, bias=False),
+                                                     nn.Linear(K, Nkv, bias=False))
+
+    class Mlp(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.gate_proj, self.up_proj = nn.Linear(K, F, bias=False), nn.Linear(K, F, bias=False)
+
+    attn, mlp = Attn().to(torch.bfloat16), Mlp().to(torch.bfloat16)
+    x = torch.randn(8, K).to(torch.bfloat16).cuda()
+    qkv_w = torch.cat([attn.q_proj.weight, attn.k_proj.weight, attn.v_proj.weight], 0).detach().clone()
+    gu_w = torch.cat([mlp.gate_proj.weight, mlp.up_proj.weight], 0).detach().clone()
+
+    ci.rans_compress_qkv_fused(attn)
+    assert attn.qkv_fused and not hasattr(attn, "k_proj") and not hasattr(attn, "v_proj")
+    assert attn.q_proj.input_shape == [K, Nq + 2 * Nkv] and attn.q_proj.compressed == "rans_bfloat16"
+    got = _fused_forward(attn.q_proj, x)
+    want = torch.matmul(x, qkv_w.cuda().t())
+    assert got.shape == (8, Nq + 2 * Nkv) and float((got.float() - want.float()).abs().max()) < 0.1
+    assert torch.allclose(got.float(), want.float(), atol=1e-2, rtol=1e-2)
+    ci.rans_decompress_module_weight(attn.q_proj)
+    assert torch.equal(attn.q_proj.weight.detach().cpu().view(torch.int16), qkv_w.t().contiguous().view(torch.int16))
+
+    ci.rans_compress_gate_up_fused(mlp, tile_height=512, tile_width=32)
+    assert mlp.gate_up_fused and not hasattr(mlp, "up_proj")
+    assert mlp.gate_proj.input_shape == [K, 2 * F] and mlp.gate_proj.exponent_tile_height == 512
+    got = _fused_forward(mlp.gate_proj, x)
+    want = torch.matmul(x, gu_w.cuda().t())
+    assert torch.allclose(got.float(), want.float(), atol=1e-2, rtol=1e-2)
+    ci.rans_decompress_module_weight(mlp.gate_proj)
+    assert torch.equal(mlp.gate_proj.weight.detach().cpu().view(torch.int16), gu_w.t().contiguous().view(torch.int16))
