@@ -2,6 +2,7 @@
 // error message, and launch checking.  gfx950 only.
 #pragma once
 #include <hip/hip_runtime.h>
+#include <atomic>
 #include <stdarg.h>
 #include <stdint.h>
 #include <stdio.h>
@@ -43,5 +44,32 @@ inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_
 
 // Largest LDS allocation a workgroup may ask for on gfx950 (160 KB per CU).
 constexpr uint32_t kLdsLimit = 160 * 1024;
+
+// CUs of the current device.
+inline int cu_count(uint32_t *out) {
+    int dev = 0, n = 0;
+    CI_HIP(hipGetDevice(&dev));
+    CI_HIP(hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev));
+    *out = n > 0 ? (uint32_t)n : 1u;
+    return CI_OK;
+}
+
+// Lets kernel `fn` ask for the whole LDS.  The attribute belongs to (function, device): `done` is the
+// call site's record of the devices it has been set on (bit = device index), safe to share between
+// threads -- two threads setting it at once set the same value.
+inline int allow_full_lds(const void *fn, std::atomic<uint64_t> &done) {
+    int dev = 0;
+    CI_HIP(hipGetDevice(&dev));
+    const uint64_t bit = 1ull << (dev & 63);
+    if (done.load(std::memory_order_acquire) & bit) return CI_OK;
+    CI_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit));
+    done.fetch_or(bit, std::memory_order_release);
+    return CI_OK;
+}
+#define CI_ALLOW_FULL_LDS(kernel)                                                             \
+    do {                                                                                      \
+        static std::atomic<uint64_t> done_{0};                                                \
+        if (int rc_ = ci::allow_full_lds(reinterpret_cast<const void *>(kernel), done_)) return rc_; \
+    } while (0)
 
 }  // namespace ci

@@ -224,15 +224,6 @@ __global__ __launch_bounds__(256) void decode_tiled_generic_kernel(DecodeArgs a)
 
 using namespace ci;
 
-// Number of CUs of the current device (one resident workgroup each for the persistent kernel).
-static int cu_count(uint32_t *out) {
-    int dev = 0, n = 0;
-    CI_HIP(hipGetDevice(&dev));
-    CI_HIP(hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev));
-    *out = n > 0 ? (uint32_t)n : 1u;
-    return CI_OK;
-}
-
 // Launch the persistent kernel over the (already checked) tensors of `b`: the device's CUs are
 // divided among the tensors in proportion to their tile counts.
 static int launch_persist(DecodeBatchArgs &b, bool merge, hipStream_t s) {
@@ -269,14 +260,8 @@ static int launch_persist(DecodeBatchArgs &b, bool merge, hipStream_t s) {
         blocks += share[i];
     }
     b.first_block[b.n] = blocks;
-    static bool attr_set = false;  // a per-function attribute; setting it again is harmless
-    if (!attr_set) {
-        CI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(decode_tiled32_persist_kernel<false>),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit));
-        CI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(decode_tiled32_persist_kernel<true>),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit));
-        attr_set = true;
-    }
+    CI_ALLOW_FULL_LDS(decode_tiled32_persist_kernel<false>);
+    CI_ALLOW_FULL_LDS(decode_tiled32_persist_kernel<true>);
     const dim3 grid(blocks), block(kPersistWaves * kWave);
     if (merge)
         hipLaunchKernelGGL(decode_tiled32_persist_kernel<true>, grid, block, kLdsLimit, s, b);

@@ -398,17 +398,10 @@ static int embedding_impl(const int64_t *d_ids, uint32_t n_ids, const uint8_t *d
     a.keys = static_cast<uint32_t *>(d_workspace);
     a.pos = a.keys + chunk_cap;
     a.chunk_start = a.pos + chunk_cap + 1;  // one word in front holds the count
-    static bool attr_set = false;
-    if (!attr_set) {
-        CI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(embed_gather32_kernel),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit));
-        CI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(embed_sort_kernel),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit));
-        attr_set = true;
-    }
-    int dev = 0, cus = 0;
-    CI_HIP(hipGetDevice(&dev));
-    CI_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    CI_ALLOW_FULL_LDS(embed_gather32_kernel);
+    CI_ALLOW_FULL_LDS(embed_sort_kernel);
+    uint32_t cus = 0;
+    if (int rc = cu_count(&cus)) return rc;
     // as many work items as chunks x pairs of column tiles; the chunk count is known on the device only
     // chunks run one after another on the stream and reuse the workspace
     for (uint32_t first = 0; first < n_ids; first += kEmbChunk) {
@@ -419,7 +412,7 @@ static int embedding_impl(const int64_t *d_ids, uint32_t n_ids, const uint8_t *d
         hipLaunchKernelGGL(embed_sort_kernel, dim3(1), dim3(1024), a.n_pad * 8 + 4096, s, a);
         CI_LAUNCH_CHECK("embed_sort_kernel");
         const uint64_t most = (uint64_t)emb_max_chunks(a.n_ids, a.n_buckets) * ceil_div(a.tiles_n, 2u);
-        const uint32_t gather_grid = (uint32_t)(most < (uint64_t)(cus > 0 ? cus : 1) ? most : (uint64_t)(cus > 0 ? cus : 1));
+        const uint32_t gather_grid = (uint32_t)(most < (uint64_t)cus ? most : (uint64_t)cus);
         hipLaunchKernelGGL(embed_gather32_kernel, dim3(gather_grid), dim3(kPersistWaves * kWave), kLdsLimit, s, a);
         CI_LAUNCH_CHECK("embed_gather32_kernel");
     }

@@ -590,18 +590,11 @@ static int fused_linear_impl(const uint16_t *d_x, uint32_t M, uint32_t K, uint32
     }
 
     if (p.resident) {
-        int dev = 0, cus = 0;
-        CI_HIP(hipGetDevice(&dev));
-        CI_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-        static bool res_attr_set = false;
-        if (!res_attr_set) {
-            CI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(fused_linear32_resident_kernel<1>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit));
-            CI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(fused_linear32_resident_kernel<2>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit));
-            res_attr_set = true;
-        }
-        const dim3 grid(cus > 0 ? cus : 1), block(kPersistWaves * kWave);
+        uint32_t cus = 0;
+        if (int rc = cu_count(&cus)) return rc;
+        CI_ALLOW_FULL_LDS(fused_linear32_resident_kernel<1>);
+        CI_ALLOW_FULL_LDS(fused_linear32_resident_kernel<2>);
+        const dim3 grid(cus), block(kPersistWaves * kWave);
         if (M > 32)
             hipLaunchKernelGGL(fused_linear32_resident_kernel<2>, grid, block, kLdsLimit, s, a);
         else
@@ -610,14 +603,8 @@ static int fused_linear_impl(const uint16_t *d_x, uint32_t M, uint32_t K, uint32
     } else if (p.fast) {
         const uint32_t waves = p.kw * p.nw;
         const uint32_t lds_bytes = kSlotTableBytes + waves * kFastStageBytes;
-        static bool attr_set = false;
-        if (!attr_set) {
-            CI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(fused_linear32_kernel<1>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit));
-            CI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(fused_linear32_kernel<2>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit));
-            attr_set = true;
-        }
+        CI_ALLOW_FULL_LDS(fused_linear32_kernel<1>);
+        CI_ALLOW_FULL_LDS(fused_linear32_kernel<2>);
         const dim3 block(waves * kWave);
         if (M > 32)
             hipLaunchKernelGGL(fused_linear32_kernel<2>, dim3(ceil_div(a.tiles_n, p.nw), p.P, ceil_div(M, 64)), block,

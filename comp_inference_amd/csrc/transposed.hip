@@ -322,18 +322,9 @@ static int transposed_impl(const uint16_t *d_x, uint32_t M, uint32_t H, uint32_t
     if (d_plain_w && !fast) return fail(CI_ERR_ARG, "plain-weight transposed linear: only the 32-column tiling");
     uint32_t cus = 1;
     if (fast) {
-        int dev = 0, n = 0;
-        CI_HIP(hipGetDevice(&dev));
-        CI_HIP(hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev));
-        cus = n > 0 ? (uint32_t)n : 1u;
-    }
-    static bool attr_set = false;
-    if (fast && !attr_set) {
-        CI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(trans32_kernel<1>),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit));
-        CI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(trans32_kernel<kTrRows>),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit));
-        attr_set = true;
+        if (int rc = cu_count(&cus)) return rc;
+        CI_ALLOW_FULL_LDS(trans32_kernel<1>);
+        CI_ALLOW_FULL_LDS(trans32_kernel<kTrRows>);
     }
     // passes of kTrRows rows of x reuse the workspace one after another on the stream
     for (uint32_t m0 = 0; m0 < M; m0 += kTrRows) {
