@@ -45,8 +45,8 @@ def step_bound_us(wave_steps: int, chain: int) -> dict:
             "latency_us": round(chain * STEP_NS_LATENCY * 1e-3, 1)}
 # HBM bytes of one batched decode launch on this workload, from rocprofv3 FETCH_SIZE and WRITE_SIZE
 # passes scaled by what the same counters read for a plain copy of known size (profiles/ holds the
-# runs): 45967.4 KiB x 1.9991 fetched + 212992.0 KiB x 1.0 written.
-MEASURED_TRAFFIC_BYTES = 312_205_369
+# runs): 38115.2 KiB x 1.9991 fetched + 212992.0 KiB x 1.0 written.
+MEASURED_TRAFFIC_BYTES = 296_130_080
 LAYER = [("q", 4096, 4096), ("k", 1024, 4096), ("v", 1024, 4096), ("o", 4096, 4096),
          ("gate", 14336, 4096), ("up", 14336, 4096), ("down", 4096, 14336)]  # (name, out, in)
 

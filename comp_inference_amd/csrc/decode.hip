@@ -175,13 +175,13 @@ __global__ __launch_bounds__(kPersistWaves *kWave) void decode_tiled32_persist_k
             if (2 * p + 1 < a.tiles_n) deepest = max(deepest, a.tile_max_lens[tile_a + 1]);
         }
     }
+    // (this kernel measures a little faster on 10 wavefronts with 204-byte lane strides -- 51 dwords, odd, so
+    // the lanes' bytes spread over the banks -- than on 11 with 186: the shallow class is not used)
     const uint32_t cls = persist_classify(lds, a.tables, a.slot_map, deepest);
     if (cls == 2u)
         decode_wave_tiles<8, kDepthDeep, kMerge>(a, j, n_wg, tab, lds, wave, lane);
-    else if (cls == 1u)
-        decode_wave_tiles<10, kDepthMedium, kMerge>(a, j, n_wg, tab, lds, wave, lane);
     else
-        decode_wave_tiles<kPersistWaves, kDepthShallow, kMerge>(a, j, n_wg, tab, lds, wave, lane);
+        decode_wave_tiles<10, kDepthMedium, kMerge>(a, j, n_wg, tab, lds, wave, lane);
 }
 
 // Any tile width: one thread per stream, bytes read where they lie.  Used for widths other

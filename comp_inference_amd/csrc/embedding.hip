@@ -268,13 +268,13 @@ __global__ __launch_bounds__(kPersistWaves *kWave) void embed_gather32_kernel(Em
         deepest = max(deepest, a.tile_max_lens[tile_a]);
         if (pair * 2 + 1 < a.tiles_n) deepest = max(deepest, a.tile_max_lens[tile_a + 1]);
     }
+    // (this kernel measures a little faster on 10 wavefronts with 204-byte lane strides -- 51 dwords, odd, so
+    // the lanes' bytes spread over the banks -- than on 11 with 186: the shallow class is not used)
     const uint32_t cls = persist_classify(lds, a.tables, a.slot_map, deepest);
     if (cls == 2u)
         embed_wave_items<8, kDepthDeep>(a, tab, lds, wave, lane);
-    else if (cls == 1u)
-        embed_wave_items<10, kDepthMedium>(a, tab, lds, wave, lane);
     else
-        embed_wave_items<kPersistWaves, kDepthShallow>(a, tab, lds, wave, lane);
+        embed_wave_items<10, kDepthMedium>(a, tab, lds, wave, lane);
 }
 
 // Any tile width and the dense layout: one thread per (token, column), discarding the rows above
