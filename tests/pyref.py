@@ -45,7 +45,10 @@ def decode_tiled(stream, states, tables, slot_map, tile_offsets, tile_max_lens, 
             x = np.where(live, nx, x)
             for _ in range(2):
                 need = live & (x < L) & (r >= 0)
-                b = stream[np.clip(base + r * spt + lane, 0, len(stream) - 1)].astype(np.int64)
+                if len(stream):
+                    b = stream[np.clip(base + r * spt + lane, 0, len(stream) - 1)].astype(np.int64)
+                else:  # nothing was emitted (a constant plane): no lane can need a byte
+                    b = np.zeros(spt, np.int64)
                 x = np.where(need, (x << 8) | b, x)
                 r = r - need
     return out
