@@ -241,3 +241,26 @@ def test_flat_one_column_as_the_reference_script_drives_it(oracle):
     seg = rans_decomp_triton(torch.from_numpy(res.stream).to(dev), _t32(res.states).to(dev), _t32(tables).to(dev),
                              torch.from_numpy(slot_map).to(dev), _t32(res.output_sizes).to(dev), (size, 1))
     assert np.array_equal(seg.cpu().numpy().reshape(-1), data)
+
+
+def test_tiled_decode_random_shapes(oracle):
+    """Forty seeded random shapes through the 32-column kernels (odd and even numbers of column tiles,
+    short last rows and columns, several tile heights): exponent plane and merged bf16 against the oracle."""
+    from comp_inference_amd import rans_decomp_tiled
+
+    rng = np.random.default_rng(2024)
+    dev = "cuda"
+    for case in range(40):
+        th = int(rng.choice([64, 256, 1024]))
+        K = int(rng.integers(1, 3 * th + 1))
+        N = int(rng.integers(1, 200))
+        w = make_weight_kn(N, K, seed=1000 + case)
+        bits = bf16_bits(w)
+        enc, man = oracle.compress_bf16(bits, th, 32)
+        args = (torch.from_numpy(enc.stream).to(dev), _t32(enc.states).to(dev), _t32(enc.tables).to(dev),
+                torch.from_numpy(enc.slot_map).to(dev), (K, N), _t32(enc.tile_offsets).to(dev),
+                _t32(enc.tile_max_lens).to(dev))
+        e = rans_decomp_tiled(*args, tile_k=th, tile_n=32)
+        assert np.array_equal(e.cpu().numpy(), (bits >> 7).astype(np.uint8)), (case, K, N, th)
+        b = rans_decomp_tiled(*args, tile_k=th, tile_n=32, mantissas=torch.from_numpy(man).to(dev))
+        assert torch.equal(b.cpu().view(torch.int16), w.view(torch.int16)), (case, K, N, th)
