@@ -106,3 +106,28 @@ def test_embedding_dense_layout(oracle):
         torch.from_numpy(enc.slot_map).to(dev), (K, N), _t32(enc.stream_offsets).to(dev), _t32(enc.sizes).to(dev),
         th, tw, torch.from_numpy(man).to(dev))
     assert torch.equal(got.cpu().view(torch.int16), _expected(table, ids).view(torch.int16))
+
+
+def test_embedding_random_shapes(oracle):
+    """Twenty seeded random tables and id lists (duplicates, invalid ids, ragged shapes, three tile heights)."""
+    from comp_inference_amd import fused_rans_embedding_triton
+
+    rng = np.random.default_rng(99)
+    dev = "cuda"
+    for case in range(20):
+        th = int(rng.choice([64, 256, 1024]))
+        K = int(rng.integers(1, 3 * th + 1))
+        N = int(rng.integers(8, 200))   # (fewer real columns than 8 of 32 overrun the reference's stream capacity)
+        T = int(rng.integers(1, 300))
+        table = make_weight_kn(K, N, seed=4000 + case).t().contiguous()  # [K rows, N columns]
+        assert tuple(table.shape) == (K, N)
+        enc, man = oracle.compress_bf16(bf16_bits(table), th, 32)
+        ids = rng.integers(-2, K + 2, T)
+        got = fused_rans_embedding_triton(
+            torch.from_numpy(ids).to(dev), torch.from_numpy(enc.stream).to(dev), _t32(enc.states).to(dev),
+            _t32(enc.tables).to(dev), torch.from_numpy(enc.slot_map).to(dev), (K, N), _t32(enc.tile_offsets).to(dev),
+            _t32(enc.tile_max_lens).to(dev), th, 32, torch.from_numpy(man).to(dev))
+        want = torch.zeros(T, N, dtype=torch.bfloat16)
+        ok = (ids >= 0) & (ids < K)
+        want[torch.from_numpy(ok)] = table[torch.from_numpy(ids[ok])]
+        assert torch.equal(got.cpu().view(torch.int16), want.view(torch.int16)), (case, K, N, T, th)

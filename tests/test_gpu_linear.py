@@ -251,3 +251,24 @@ def test_fused_kernels_above_64_rows(oracle, always_fused, K, N, th, M):
     assert torch.equal(got.view(torch.int16), same.view(torch.int16))
     # and it is not the library GEMM's summation order
     assert not torch.equal(got.view(torch.int16), torch.matmul(x.cuda(), wdec.cuda()).view(torch.int16))
+
+
+def test_fused_linear_random_shapes(oracle, always_fused):
+    """Thirty seeded random shapes (ragged K and N, 1 to 70 rows of x, three tile heights) on the fused
+    kernels: within tolerance of torch.matmul and bit-identical to the plain-weight contraction."""
+    from comp_inference_amd import plain_linear_same_order
+
+    rng = np.random.default_rng(77)
+    for case in range(30):
+        th = int(rng.choice([64, 256, 1024]))
+        K = int(rng.integers(1, 3 * th + 1))
+        N = int(rng.integers(8, 200))   # (fewer real columns than 8 of 32 overrun the reference's stream capacity)
+        M = int(rng.integers(1, 71))
+        w = make_weight_kn(N, K, seed=2000 + case)
+        enc, man, wdec = _compress(oracle, w, th, 32)
+        x = make_x(M, K, seed=3000 + case)
+        got = _call(enc, man, x, K, N, th, 32)
+        want = torch.matmul(x.float(), wdec.float())
+        assert torch.allclose(got.float().cpu(), want, atol=ATOL, rtol=RTOL), (case, K, N, M, th)
+        same = plain_linear_same_order(x.cuda(), wdec.cuda(), tile_k=th, tile_n=32)
+        assert torch.equal(got.view(torch.int16), same.view(torch.int16)), (case, K, N, M, th)
