@@ -264,3 +264,36 @@ def test_tiled_decode_random_shapes(oracle):
         assert np.array_equal(e.cpu().numpy(), (bits >> 7).astype(np.uint8)), (case, K, N, th)
         b = rans_decomp_tiled(*args, tile_k=th, tile_n=32, mantissas=torch.from_numpy(man).to(dev))
         assert torch.equal(b.cpu().view(torch.int16), w.view(torch.int16)), (case, K, N, th)
+
+
+def test_encoder_random_shapes(oracle):
+    """Thirty seeded random planes (shape, tile, skew) through the HIP encoder and packer: every output
+    array equals the oracle's, so the stream is the reference's byte for byte."""
+    rng = np.random.default_rng(31337)
+    overflowed = 0
+    for case in range(30):
+        th = int(rng.choice([32, 64, 256, 1024]))
+        tw = int(rng.choice([16, 32, 32, 64]))
+        K = int(rng.integers(1, 3 * th + 1))
+        N = int(rng.integers(max(1, tw // 4), 5 * tw))
+        sym = zipf_bytes(K * N, float(rng.choice([1.0, 2.0, 4.0])), 5000 + case).reshape(K, N)
+        try:
+            ref, got = _encode_both(oracle, sym, th, tw)
+        except RuntimeError as e:
+            # a ragged plane of poorly compressible symbols can outgrow the reference's per-stream
+            # capacity (src/cuda/rans_host.cuh:470-471): then both encoders must say so
+            assert "capacity" in str(e), (case, K, N, th, tw, str(e))
+            from comp_inference_amd import ccore, get_rans_lut
+
+            ft, ct = get_rans_lut(torch.from_numpy(sym))
+            with pytest.raises(RuntimeError):
+                ccore.RansManager(sym.size).compress_tiled(torch.from_numpy(sym), ft, ct, th, tw)
+            overflowed += 1
+            continue
+        assert got.success and got.num_streams == ref.num_streams, (case, K, N, th, tw)
+        assert np.array_equal(_np32(got.states), ref.states), (case, K, N, th, tw)
+        assert np.array_equal(_np32(got.output_sizes), ref.sizes), (case, K, N, th, tw)
+        assert np.array_equal(_np32(got.tile_offsets), ref.tile_offsets), (case, K, N, th, tw)
+        assert np.array_equal(_np32(got.tile_max_lens), ref.tile_max_lens), (case, K, N, th, tw)
+        assert np.array_equal(got.stream.numpy(), ref.stream), (case, K, N, th, tw)
+    assert overflowed < 10

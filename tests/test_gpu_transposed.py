@@ -140,3 +140,28 @@ def test_transposed_many_rows_decode_the_weight_once(oracle):
         _t32(enc.tile_max_lens).to(dev), th, 32, torch.from_numpy(man).to(dev), workspace=None)
     want = torch.matmul(x, w.cuda().t())
     assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+
+
+def test_transposed_random_shapes(oracle, always_fused):
+    """Twenty seeded random [V, H] weights (ragged, 1 to 9 rows of x, three tile heights) on the fused kernel:
+    within tolerance of torch.matmul and bit-identical to the plain-weight contraction."""
+    from comp_inference_amd import fused_rans_linear_transposed_triton, plain_linear_transposed_same_order
+
+    rng = np.random.default_rng(55)
+    dev = "cuda"
+    for case in range(20):
+        th = int(rng.choice([64, 256, 1024]))
+        V = int(rng.integers(1, 3 * th + 1))
+        H = int(rng.integers(8, 200))
+        M = int(rng.integers(1, 10))
+        w = make_weight_kn(H, V, seed=6000 + case)  # [V, H]
+        enc, man = oracle.compress_bf16(bf16_bits(w), th, 32)
+        x = make_x(M, H, seed=7000 + case)
+        got = fused_rans_linear_transposed_triton(
+            x.to(dev), torch.from_numpy(enc.stream).to(dev), _t32(enc.states).to(dev), _t32(enc.tables).to(dev),
+            torch.from_numpy(enc.slot_map).to(dev), (V, H), _t32(enc.tile_offsets).to(dev),
+            _t32(enc.tile_max_lens).to(dev), th, 32, torch.from_numpy(man).to(dev), workspace=None)
+        want = torch.matmul(x.float(), w.float().t())
+        assert torch.allclose(got.float().cpu(), want, atol=ATOL, rtol=RTOL), (case, V, H, M, th)
+        same = plain_linear_transposed_same_order(x.to(dev), w.to(dev), tile_k=th, tile_n=32)
+        assert torch.equal(got.view(torch.int16), same.view(torch.int16)), (case, V, H, M, th)
