@@ -68,12 +68,17 @@ class PlainSameOrder:
     compressed operator computes if, and only if, it reconstructs every weight bit."""
 
     def __init__(self, w_kn, tile_k, tile_n):
+        import comp_inference_amd as ci
+
         self.w, self.tile_k, self.tile_n = w_kn, tile_k, tile_n
+        # the compressed operator splits every stream into this many segments (decoder checkpoints),
+        # which is also how its contraction is split into partial sums
+        self.segments = ci.suggest_segments(tuple(w_kn.shape), tile_k, tile_n)
 
     def __call__(self, x):
         import comp_inference_amd as ci
 
-        return ci.plain_linear_same_order(x, self.w, tile_k=self.tile_k, tile_n=self.tile_n)
+        return ci.plain_linear_same_order(x, self.w, tile_k=self.tile_k, tile_n=self.tile_n, segments=self.segments)
 
 
 class Decoder:

@@ -33,12 +33,14 @@ from .linear_hip import (
     triton_matmul,
 )
 from .rans_hip import (
+    build_checkpoints,
     rans_decomp_flat,
     rans_decomp_tiled,
     rans_decomp_tiled_batch,
     rans_decomp_tiled_uncoalesced,
     rans_decomp_triton,
     rans_decomp_triton_tiled,
+    suggest_segments,
 )
 from .transposed_linear_hip import (
     fused_rans_linear_transposed,

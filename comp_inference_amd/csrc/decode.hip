@@ -220,9 +220,91 @@ __global__ __launch_bounds__(256) void decode_tiled_generic_kernel(DecodeArgs a)
     }
 }
 
+// Decoder checkpoints.  A stream is a chain of th/2 dependent steps; with the decoder's state and
+// byte position recorded at `segs` evenly spaced rows, the segments of a stream can be decoded by
+// different wavefronts at the same time.  The checkpoints are derived from the stream (an index kept
+// beside it), the stream itself is untouched.  One thread per stream walks it once:
+// ckpt[(tile * (segs - 1) + j - 1) * 2 tw + q] = {state, row of the next unread byte (-1: none left)}
+// at the first row of segment j = 1 .. segs - 1 of stream q.  The reference keeps such checkpoints for
+// its flat format only (src/cuda/rans_kernels.cuh:454-465).
+__global__ __launch_bounds__(256) void checkpoints_kernel(DecodeArgs a, uint32_t segs, uint2 *__restrict__ ckpt) {
+    __shared__ uint2 tab[kProbScale];
+    build_slot_table(tab, a.tables, a.slot_map, threadIdx.x, 256);
+    __syncthreads();
+    const uint32_t spt = 2 * a.tw;
+    const uint64_t sid = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (sid >= (uint64_t)a.num_tiles * spt) return;
+    const uint32_t tile = (uint32_t)(sid / spt), q = (uint32_t)(sid % spt);
+    const uint32_t tk = tile / a.tiles_n, tn = tile % a.tiles_n;
+    const uint32_t half = a.th / 2, seglen = half / segs, hsel = q / a.tw, c = q % a.tw;
+    const uint32_t col = tn * a.tw + c, my_row0 = tk * a.th + hsel * half;
+    const uint32_t my_steps = (col < a.N && my_row0 < a.K) ? min(half, a.K - my_row0) : 0u;
+    uint64_t base = a.tile_offsets[tile];
+    uint32_t depth = a.tile_max_lens[tile];
+    if (base + (uint64_t)depth * spt > a.stream_len) depth = 0;
+    GlobalBytes src;
+    src.init(a.stream + base, depth, spt, q);
+    uint32_t x = a.states[sid];
+    uint2 *mine = ckpt + (size_t)tile * (segs - 1) * spt + q;
+    uint32_t next = 1;
+    for (uint32_t i = 0; i < my_steps; ++i) {
+        if (next < segs && i == next * seglen) {
+            mine[(size_t)(next - 1) * spt] = make_uint2(x, (uint32_t)src.row);
+            ++next;
+        }
+        decode_symbol(x, tab);
+        src.renorm(x);
+        src.renorm(x);
+    }
+    for (; next < segs; ++next) mine[(size_t)(next - 1) * spt] = make_uint2(x, (uint32_t)src.row);  // short streams
+}
+
 }  // namespace ci
 
 using namespace ci;
+
+extern "C" size_t ci_checkpoint_bytes(uint32_t K, uint32_t N, uint32_t tile_height, uint32_t tile_width,
+                                      uint32_t segments) {
+    if (tile_height == 0 || tile_width == 0 || segments < 2) return 0;
+    return (size_t)ceil_div(K, tile_height) * ceil_div(N, tile_width) * (segments - 1) * 2 * tile_width * sizeof(uint2);
+}
+
+extern "C" int ci_build_checkpoints_ilp2(const uint8_t *d_stream, uint64_t stream_len, const uint32_t *d_states,
+                                         const uint32_t *d_tables, const uint8_t *d_slot_map,
+                                         const uint32_t *d_tile_offsets, const uint32_t *d_tile_max_lens, uint32_t K,
+                                         uint32_t N, uint32_t tile_height, uint32_t tile_width, uint32_t segments,
+                                         void *d_checkpoints, size_t checkpoint_bytes, ci_stream_t stream) {
+    if (K == 0 || N == 0 || segments < 2) return CI_OK;
+    if (!d_states || !d_tables || !d_slot_map || !d_tile_offsets || !d_tile_max_lens || !d_checkpoints)
+        return fail(CI_ERR_ARG, "ci_build_checkpoints_ilp2: null pointer");
+    if (stream_len && !d_stream) return fail(CI_ERR_ARG, "ci_build_checkpoints_ilp2: null stream");
+    if (tile_height == 0 || tile_width == 0 || (tile_height & 1) || (tile_height / 2) % segments)
+        return fail(CI_ERR_ARG, "ci_build_checkpoints_ilp2: half the tile height must be a multiple of the segment count");
+    if (!aligned(d_slot_map, 4) || !aligned(d_checkpoints, 8))
+        return fail(CI_ERR_ARG, "ci_build_checkpoints_ilp2: slot_map must be 4-byte, checkpoints 8-byte aligned");
+    const size_t need = ci_checkpoint_bytes(K, N, tile_height, tile_width, segments);
+    if (checkpoint_bytes < need)
+        return fail(CI_ERR_CAPACITY, "ci_build_checkpoints_ilp2: checkpoints need %zu bytes, got %zu", need, checkpoint_bytes);
+    DecodeArgs a = {};
+    a.stream = d_stream;
+    a.stream_len = stream_len;
+    a.states = d_states;
+    a.tables = d_tables;
+    a.slot_map = d_slot_map;
+    a.tile_offsets = d_tile_offsets;
+    a.tile_max_lens = d_tile_max_lens;
+    a.K = K;
+    a.N = N;
+    a.th = tile_height;
+    a.tw = tile_width;
+    a.tiles_n = ceil_div(N, tile_width);
+    a.num_tiles = ceil_div(K, tile_height) * a.tiles_n;
+    const uint64_t streams = (uint64_t)a.num_tiles * 2 * tile_width;
+    hipLaunchKernelGGL(checkpoints_kernel, dim3((uint32_t)((streams + 255) / 256)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), a, segments, static_cast<uint2 *>(d_checkpoints));
+    CI_LAUNCH_CHECK("checkpoints_kernel");
+    return CI_OK;
+}
 
 // Launch the persistent kernel over the (already checked) tensors of `b`: the device's CUs are
 // divided among the tensors in proportion to their tile counts.

@@ -118,6 +118,18 @@ __device__ __forceinline__ void stage_fetch_pair(StageRegs &regs, const uint8_t 
     }
 }
 
+// Maximum of a signed value over the 64 lanes of the wavefront (every lane must be active): four DPP
+// steps inside each row of 16 lanes, then the four row results.
+__device__ __forceinline__ int32_t wave_max_i32(int32_t v) {
+    v = max(v, __builtin_amdgcn_update_dpp(v, v, 0xB1, 0xF, 0xF, false));   // quad_perm [1,0,3,2]
+    v = max(v, __builtin_amdgcn_update_dpp(v, v, 0x4E, 0xF, 0xF, false));   // quad_perm [2,3,0,1]
+    v = max(v, __builtin_amdgcn_update_dpp(v, v, 0x141, 0xF, 0xF, false));  // row_half_mirror
+    v = max(v, __builtin_amdgcn_update_dpp(v, v, 0x140, 0xF, 0xF, false));  // row_mirror
+    return max(max(__builtin_amdgcn_readlane(v, 0), __builtin_amdgcn_readlane(v, 16)),
+               max(__builtin_amdgcn_readlane(v, 32), __builtin_amdgcn_readlane(v, 48)));
+}
+__device__ __forceinline__ int32_t wave_min_i32(int32_t v) { return -wave_max_i32(-v); }
+
 // ---- workgroups resident for a whole launch ------------------------------------------------------
 // The kernels built on the loops below are bound by wavefronts in flight, not by memory: the whole
 // LDS goes to the slot table plus as many transposed tile bodies as fit, one workgroup per CU, and
@@ -298,11 +310,18 @@ struct FastLane {
     // kStride = bytes of LDS per lane in the staging area (must exceed the tile's depth).
     template <uint32_t kStride = kFastStride>
     __device__ __forceinline__ void init(const uint8_t *stage, uint32_t depth, uint32_t q_lane, uint32_t state) {
+        init_at<kStride>(stage, (int32_t)depth, q_lane, state);
+    }
+    // The same for a lane that starts in the middle of its stream: `have` = staged bytes of this lane's
+    // column from its first row up to and including the next unread byte (<= 0: none left; the bytes such
+    // a lane prefetches are never used).
+    template <uint32_t kStride = kFastStride>
+    __device__ __forceinline__ void init_at(const uint8_t *stage, int32_t have, uint32_t q_lane, uint32_t state) {
         X = state << 3;
         const uint8_t *col = stage + q_lane * kStride;
-        q = (uint32_t)(uintptr_t)col + depth - 2;  // low 32 bits of an LDS pointer are its LDS address
-        n1 = depth >= 1 ? col[depth - 1] : 0;
-        n2 = depth >= 2 ? col[depth - 2] : 0;
+        q = (uint32_t)(uintptr_t)col + (uint32_t)have - 2;  // low 32 bits of an LDS pointer are its LDS address
+        n1 = have >= 1 ? col[have - 1] : 0;
+        n2 = have >= 2 ? col[have - 2] : 0;
     }
 };
 

@@ -54,6 +54,10 @@ struct LinearArgs {
     // being decoded (every tile takes the guarded path, which issues the same MFMA sequence as the
     // hand-scheduled one); none of the compressed operands is touched.
     const uint16_t *dense_w;
+    // Decoder checkpoints (ci_build_checkpoints_ilp2) and the number of segments per stream they cut, or
+    // null / 1: with them the resident kernel gives every (tile, segment) its own wavefront.
+    const uint2 *ckpt;
+    uint32_t segs;
 };
 
 // x [M, K] -> the fragment order described at LinearArgs::xf.  In a plain row-major x the 64 lanes of
@@ -272,25 +276,48 @@ __global__ __launch_bounds__(kLinMaxWaves *kWave) void fused_linear32_kernel(Lin
     }
 }
 
-// The same tile work with workgroups resident for the launch (fast_tile.h) and every tile on its
-// own: wavefront w of workgroup j takes tiles j + (w + 11 i) * gridDim.x and writes its 32-column
-// partial product to the fp32 workspace [tiles_k][M][N], which the reduction kernel sums in k order.
-// For weights with more tiles than the chip holds at once (fused gate/up projections): the
-// 8-wavefront workgroups of the kernel above would run in two full rounds.  M <= 32 * MB.
+// The same tile work with workgroups resident for the launch (fast_tile.h): wavefront w of workgroup j
+// takes the items j + (w + n i) * gridDim.x and writes its 32-column partial product to the fp32 workspace
+// [tiles_k * segs][M][N], which the reduction kernel sums in k order.  For weights with more tiles than
+// the chip holds at once (fused gate/up projections), where the 8-wavefront workgroups of the kernel
+// above would run in two full rounds -- and for weights with so few tiles that their th/2-step chains,
+// not the chip, bound the time: with decoder checkpoints every stream is cut into `segs` segments
+// and an item is one segment of the 64 streams of a tile.  M <= 32 * MB.
+//
+// Item vk * tiles_n + tn, vk = tk * segs + seg: rows [seg, seg + 1) * th / (2 segs) of both halves of tile
+// (tk, tn).  A segment's bytes are the rows between its own checkpoint and the next one's, about
+// depth / segs of them per lane plus the spread between lanes; only that window of the body is staged.
 template <int MB, uint32_t kStride>
-__device__ __forceinline__ void linear_one_tile(const LinearArgs &a, uint32_t tile, const uint2 *tab, uint8_t *stage,
-                                                int lane) {
-    const uint32_t tk = tile / a.tiles_n, tn = tile % a.tiles_n;
-    const uint32_t half = a.th / 2, hsel = lane / 32, c = lane % 32;
-    const uint32_t col0 = tn * 32, k0 = tk * a.th + hsel * half;
+__device__ __forceinline__ void linear_one_item(const LinearArgs &a, uint32_t vk, uint32_t tn, const uint2 *tab,
+                                                uint8_t *stage, int lane) {
+    const uint32_t tk = vk / a.segs, seg = vk % a.segs, tile = tk * a.tiles_n + tn;
+    const uint32_t half = a.th / 2, seglen = half / a.segs, hsel = lane / 32, c = lane % 32;
+    const uint32_t col0 = tn * 32, k0 = tk * a.th + hsel * half + seg * seglen;
     const uint64_t base = a.dense_w ? 0 : a.tile_offsets[tile];
     uint32_t depth = a.dense_w ? 0 : a.tile_max_lens[tile];
-    const uint32_t state = a.dense_w ? 0 : a.states[(size_t)tile * 64 + lane];
     if (base + (uint64_t)depth * 64 > a.stream_len) depth = 0;
+    // decoder state and row of the next unread byte at the first row of the segment, and at its end
+    uint32_t state = 0;
+    int32_t row = (int32_t)depth - 1, row_end = -1;
+    if (!a.dense_w) {
+        const uint2 *ck = a.ckpt + ((size_t)tile * (a.segs - 1)) * 64 + lane;  // (only read when segs > 1)
+        if (seg == 0) {
+            state = a.states[(size_t)tile * 64 + lane];
+        } else {
+            const uint2 v = ck[(size_t)(seg - 1) * 64];
+            state = v.x;
+            row = min((int32_t)v.y, (int32_t)depth - 1);
+        }
+        if (seg + 1 < a.segs) row_end = min((int32_t)ck[(size_t)seg * 64].y, row);
+    }
     uint32_t my_steps = 0;
-    if (col0 + c < a.N && k0 < a.K) my_steps = min(half, a.K - k0);
-    const bool full = __builtin_amdgcn_ballot_w64(my_steps != half) == 0;
-    const bool fast = full && a.fast_ok && depth >= 2 && depth < kStride && half % 16 == 0 &&
+    if (col0 + c < a.N && k0 < a.K) my_steps = min(seglen, a.K - k0);
+    const bool full = __builtin_amdgcn_ballot_w64(my_steps != seglen) == 0;
+    // rows of the body this item can touch: from the lowest end row (less the two prefetched bytes) to the
+    // highest start row
+    const int32_t lo = max(wave_min_i32(row_end) - 1, 0), hi = wave_max_i32(row);
+    const uint32_t window = hi >= lo ? (uint32_t)(hi - lo + 1) : 0u;
+    const bool fast = full && a.fast_ok && window >= 2 && window < kStride && seglen % 16 == 0 &&
                       (uint32_t)(uintptr_t)tab == 0 && !a.dense_w;
     const uint32_t m = c;  // row of x this lane feeds to the (first) MFMA
     const bool m_ok = m < a.M, m2_ok = MB == 2 && m + 32 < a.M;
@@ -301,15 +328,15 @@ __device__ __forceinline__ void linear_one_tile(const LinearArgs &a, uint32_t ti
     const uint32_t xrow2_elems = (m2_ok ? m + 32 : 0) * a.x_stride + k0;
     const size_t man_tile = (size_t)tile * a.th * 32;
     if (fast) {
-        stage_body<kStride>(stage, a.stream + base, depth, lane);
+        stage_body<kStride>(stage, a.stream + base + (size_t)lo * 64, window, lane);
         FastLane st;
-        st.init<kStride>(stage, depth, lane, state);
+        st.init_at<kStride>(stage, row - lo + 1, lane, state);
         const uint64_t mbase = reinterpret_cast<uint64_t>(a.man_tiled + man_tile);
         // readfirstlane returns a signed int: widen through uint32_t, not by sign extension
         const uint32_t mb_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(mbase >> 32));
         const uint32_t mb_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)mbase);
         const uint64_t mb_u = ((uint64_t)mb_hi << 32) | (uint64_t)mb_lo;
-        const uint32_t moff = hsel * half * 32 + (c & ~3u);
+        const uint32_t moff = (hsel * half + seg * seglen) * 32 + (c & ~3u);
         const uint32_t man_sel = 0x04040000u + (c & 3u) * 0x01010101u;
         uint64_t xb = reinterpret_cast<uint64_t>(a.x);
         uint32_t xo = xrow_elems * 2u, xo2 = xrow2_elems * 2u, xstep = 16;
@@ -321,18 +348,18 @@ __device__ __forceinline__ void linear_one_tile(const LinearArgs &a, uint32_t ti
             xstep = 32 * 16;
         }
         if (MB == 2)
-            linear_tile_asm2(st, acc, acc2, mb_u, moff, xb, xo, xo2, xstep, man_sel, half / 8);
+            linear_tile_asm2(st, acc, acc2, mb_u, moff, xb, xo, xo2, xstep, man_sel, seglen / 8);
         else
-            linear_tile_asm(st, acc, mb_u, moff, xb, xo, xstep, man_sel, half / 8);
+            linear_tile_asm(st, acc, mb_u, moff, xb, xo, xstep, man_sel, seglen / 8);
     } else {
-        const uint8_t *man = a.man_tiled + man_tile + (size_t)hsel * half * 32 + c;
+        const uint8_t *man = a.man_tiled + man_tile + (size_t)(hsel * half + seg * seglen) * 32 + c;
         const uint16_t *wd = a.dense_w ? a.dense_w + (size_t)k0 * a.N + col0 + c : nullptr;
         GlobalBytes src;
-        src.init(a.stream + base, depth, 64, lane);
-        linear_tile_guarded(src, state << 3, tab, a.K, half, my_steps, man, a.x + xrow_elems, m_ok, k0, acc, wd, a.N);
+        src.init(a.stream + base, (uint32_t)(row + 1), 64, lane);
+        linear_tile_guarded(src, state << 3, tab, a.K, seglen, my_steps, man, a.x + xrow_elems, m_ok, k0, acc, wd, a.N);
         if (MB == 2) {
-            src.init(a.stream + base, depth, 64, lane);
-            linear_tile_guarded(src, state << 3, tab, a.K, half, my_steps, man, a.x + xrow2_elems, m2_ok, k0, acc2, wd,
+            src.init(a.stream + base, (uint32_t)(row + 1), 64, lane);
+            linear_tile_guarded(src, state << 3, tab, a.K, seglen, my_steps, man, a.x + xrow2_elems, m2_ok, k0, acc2, wd,
                                 a.N);
         }
     }
@@ -345,18 +372,24 @@ __device__ __forceinline__ void linear_one_tile(const LinearArgs &a, uint32_t ti
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             const uint32_t n = col0 + (v / 4) * 8 + hsel * 4 + (v % 4);
-            if (mg < a.M && n < a.N) a.partial[((size_t)tk * a.M + mg) * a.N + n] = part[v];
+            if (mg < a.M && n < a.N) a.partial[((size_t)vk * a.M + mg) * a.N + n] = part[v];
         }
     }
 }
 
 template <int MB, int kWaves, uint32_t kStride>
 __device__ __forceinline__ void linear_wave_tiles(const LinearArgs &a, const uint2 *tab, uint8_t *lds, int wave, int lane) {
-    if (wave >= kWaves) return;
+    const uint64_t num_items = (uint64_t)a.tiles_k * a.segs * a.tiles_n;
+    // Items of this workgroup, the rounds they take on kWaves wavefronts, and the fewest wavefronts that do
+    // them in as many rounds: 12 items run as 6 + 6, not 11 + 1 (a round lasts as long as a full one however
+    // few wavefronts take part, and fewer wavefronts at a time step faster).
+    const uint32_t mine = blockIdx.x < num_items ? (uint32_t)((num_items - blockIdx.x + gridDim.x - 1) / gridDim.x) : 0u;
+    const uint32_t rounds = (mine + kWaves - 1) / kWaves;
+    const uint32_t active = rounds ? (mine + rounds - 1) / rounds : 0u;
+    if ((uint32_t)wave >= active) return;
     uint8_t *stage = persist_stage<kWaves, kStride>(lds, wave);
-    const uint64_t num_tiles = (uint64_t)a.tiles_k * a.tiles_n;
-    for (uint64_t tile = (uint64_t)wave * gridDim.x + blockIdx.x; tile < num_tiles; tile += (uint64_t)kWaves * gridDim.x)
-        linear_one_tile<MB, kStride>(a, (uint32_t)tile, tab, stage, lane);
+    for (uint64_t item = (uint64_t)wave * gridDim.x + blockIdx.x; item < num_items; item += (uint64_t)active * gridDim.x)
+        linear_one_item<MB, kStride>(a, (uint32_t)(item / a.tiles_n), (uint32_t)(item % a.tiles_n), tab, stage, lane);
 }
 
 template <int MB>
@@ -365,9 +398,17 @@ __global__ __launch_bounds__(kPersistWaves *kWave) void fused_linear32_resident_
     const uint2 *tab = reinterpret_cast<const uint2 *>(lds);
     const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
     // (a plain-weight run has no table to build; which wavefront takes which tile does not change a tile's sum)
-    const uint32_t cls = a.dense_w ? 0u
-                                   : persist_prologue(lds, a.tables, a.slot_map, a.tile_max_lens, a.tiles_k * a.tiles_n,
-                                                      blockIdx.x, gridDim.x);
+    uint32_t cls = 0;
+    if (!a.dense_w && a.segs <= 1) {
+        cls = persist_prologue(lds, a.tables, a.slot_map, a.tile_max_lens, a.tiles_k * a.tiles_n, blockIdx.x, gridDim.x);
+    } else if (!a.dense_w) {
+        // a segment's window is about its share of the body plus the spread between the lanes; an item
+        // whose window turns out larger than the class allows takes the guarded path
+        uint32_t deepest = 0;
+        for (uint32_t t = threadIdx.x; t < a.tiles_k * a.tiles_n; t += kPersistWaves * kWave)
+            deepest = max(deepest, a.tile_max_lens[t]);
+        cls = persist_classify(lds, a.tables, a.slot_map, deepest / a.segs + 40);
+    }
     if (cls == 2u)
         linear_wave_tiles<MB, 8, kDepthDeep>(a, tab, lds, wave, lane);
     else if (cls == 1u)
@@ -472,22 +513,27 @@ static size_t x_fragment_bytes(uint32_t M, uint32_t K, bool fast_plan) {
 
 struct LinearPlan {
     bool fast, resident;
-    uint32_t kw, nw, P;
+    uint32_t kw, nw, P, segs;
 };
 
 // Tiles from which every tile gets its own wavefront of a resident workgroup: more than a chip of
 // 8-wavefront workgroups holds at once (256 CUs x 8).
 constexpr uint32_t kResidentMinTiles = 2049;
+constexpr uint32_t kPlanCus = 256;  // CUs assumed when segments are suggested
 
+// segments: 1, or the number of segments the caller's checkpoints cut every stream into.
 static LinearPlan plan_linear(uint32_t M, uint32_t K, uint32_t th, uint32_t tw, uint32_t tiles_n, bool dense,
-                              bool stream_aligned) {
+                              bool stream_aligned, uint32_t segments = 1) {
     LinearPlan p;
     const uint32_t tiles_k = ceil_div(K, th);
     p.fast = !dense && tw == 32 && th % 16 == 0 && stream_aligned;
-    p.resident = p.fast && M <= 64 && tiles_k >= 2 && (uint64_t)tiles_k * tiles_n >= kResidentMinTiles;
+    p.segs = 1;
+    if (p.fast && M <= 64 && segments > 1 && (th / 2) % (16 * segments) == 0) p.segs = segments;
+    p.resident = p.fast && M <= 64 &&
+                 (p.segs > 1 || (tiles_k >= 2 && (uint64_t)tiles_k * tiles_n >= kResidentMinTiles));
     if (p.resident) {
         p.kw = p.nw = 1;
-        p.P = tiles_k;
+        p.P = tiles_k * p.segs;
     } else if (p.fast) {
         p.P = ceil_div(tiles_k, kLinMaxWaves);
         p.kw = ceil_div(tiles_k, p.P);
@@ -505,15 +551,37 @@ static LinearPlan plan_linear(uint32_t M, uint32_t K, uint32_t th, uint32_t tw, 
 
 using namespace ci;
 
-extern "C" size_t ci_fused_linear_workspace_bytes(uint32_t M, uint32_t K, uint32_t N, uint32_t tile_height,
-                                                  uint32_t tile_width, int dense) {
+extern "C" size_t ci_fused_linear_workspace_bytes_segmented(uint32_t M, uint32_t K, uint32_t N, uint32_t tile_height,
+                                                            uint32_t tile_width, int dense, uint32_t segments) {
     if (tile_height == 0 || tile_width == 0) return 0;
     // sized for the slower plan so that the answer does not depend on pointer alignment
-    const LinearPlan fast = plan_linear(M, K, tile_height, tile_width, ceil_div(N, tile_width), dense != 0, true);
-    const LinearPlan slow = plan_linear(M, K, tile_height, tile_width, ceil_div(N, tile_width), dense != 0, false);
+    const uint32_t tiles_n = ceil_div(N, tile_width);
+    const LinearPlan fast = plan_linear(M, K, tile_height, tile_width, tiles_n, dense != 0, true, segments);
+    const LinearPlan slow = plan_linear(M, K, tile_height, tile_width, tiles_n, dense != 0, false, segments);
     const uint32_t P = fast.P > slow.P ? fast.P : slow.P;
     const size_t partial = P > 1 ? (size_t)P * M * N * sizeof(float) : 0;
     return ((partial + 15) & ~(size_t)15) + x_fragment_bytes(M, K, fast.fast);
+}
+
+extern "C" size_t ci_fused_linear_workspace_bytes(uint32_t M, uint32_t K, uint32_t N, uint32_t tile_height,
+                                                  uint32_t tile_width, int dense) {
+    return ci_fused_linear_workspace_bytes_segmented(M, K, N, tile_height, tile_width, dense, 1);
+}
+
+// Segments per stream for a weight of this shape, from measurements on 256 CUs x 11 wavefronts: as many
+// (2, 4 or 8) as still give every (tile, segment) a wavefront of its own in one round -- the time is
+// then one chain of th / (2 segments) steps instead of th / 2 -- and 2 for weights that take several
+// rounds anyway (shorter items fill the last round better); 1 in between, where the chip is busy with
+// whole tiles.
+extern "C" uint32_t ci_suggest_segments(uint32_t K, uint32_t N, uint32_t tile_height, uint32_t tile_width) {
+    if (tile_height == 0 || tile_width != 32 || tile_height % 16) return 1;
+    const uint64_t tiles = (uint64_t)ceil_div(K, tile_height) * ceil_div(N, tile_width);
+    const uint64_t one_round = (uint64_t)kPlanCus * kPersistWaves;
+    auto fits = [&](uint32_t segs) { return (tile_height / 2) % (16 * segs) == 0; };
+    for (uint32_t segs = 8; segs >= 2; segs /= 2)
+        if (tiles * segs <= one_round && fits(segs)) return segs;
+    if (tiles >= kResidentMinTiles && fits(2)) return 2;
+    return 1;
 }
 
 static int fused_linear_impl(const uint16_t *d_x, uint32_t M, uint32_t K, uint32_t N, uint32_t x_stride,
@@ -521,7 +589,8 @@ static int fused_linear_impl(const uint16_t *d_x, uint32_t M, uint32_t K, uint32
                              const uint32_t *d_tables, const uint8_t *d_slot_map, const uint32_t *d_meta0,
                              const uint32_t *d_meta1, const uint8_t *d_man_tiled, uint32_t th, uint32_t tw,
                              const uint16_t *d_bias, uint16_t *d_out, uint32_t out_stride, void *d_workspace,
-                             size_t workspace_bytes, bool dense, hipStream_t s, const uint16_t *d_plain_w = nullptr) {
+                             size_t workspace_bytes, bool dense, hipStream_t s, const uint16_t *d_plain_w = nullptr,
+                             const void *d_checkpoints = nullptr, uint32_t segments = 1) {
     if (M == 0 || N == 0) return CI_OK;
     if (K == 0) return fail(CI_ERR_ARG, "fused linear: K is 0");
     if (!d_x || !d_out) return fail(CI_ERR_ARG, "fused linear: null pointer");
@@ -560,9 +629,19 @@ static int fused_linear_impl(const uint16_t *d_x, uint32_t M, uint32_t K, uint32
     a.tiles_k = ceil_div(K, th);
     a.fast_ok = aligned(d_x, 16) && x_stride % 8 == 0 && aligned(d_man_tiled, 4) &&
                 (uint64_t)M * x_stride * 2 < (1ull << 31);
-    const LinearPlan p = plan_linear(M, K, th, tw, a.tiles_n, dense, d_plain_w || aligned(d_stream, 16));
+    if (segments == 0) segments = 1;
+    if (segments > 1) {
+        if (dense || tw != 32 || th % 16 || (th / 2) % (16 * segments))
+            return fail(CI_ERR_ARG, "fused linear: %u segments need 32-column tiles whose half height is a multiple of %u",
+                        segments, 16 * segments);
+        if (!d_plain_w && (!d_checkpoints || !aligned(d_checkpoints, 8)))
+            return fail(CI_ERR_ARG, "fused linear: segments without (8-byte aligned) checkpoints");
+    }
+    const LinearPlan p = plan_linear(M, K, th, tw, a.tiles_n, dense, d_plain_w || aligned(d_stream, 16), segments);
     if (d_plain_w && !p.fast)
         return fail(CI_ERR_ARG, "plain-weight linear: only the 32-column tiling (tile height a multiple of 16)");
+    a.ckpt = static_cast<const uint2 *>(d_checkpoints);
+    a.segs = p.segs;
     a.kw = p.kw;
     a.nw = p.nw;
     a.P = p.P;
@@ -658,14 +737,29 @@ extern "C" int ci_fused_linear_dense(const uint16_t *d_x, uint32_t M, uint32_t K
                              out_stride, d_workspace, workspace_bytes, true, static_cast<hipStream_t>(stream));
 }
 
+extern "C" int ci_fused_linear_ilp2_segmented(const uint16_t *d_x, uint32_t M, uint32_t K, uint32_t N, uint32_t x_stride,
+                                              const uint8_t *d_stream, uint64_t stream_len, const uint32_t *d_states,
+                                              const uint32_t *d_tables, const uint8_t *d_slot_map,
+                                              const uint32_t *d_tile_offsets, const uint32_t *d_tile_max_lens,
+                                              const uint8_t *d_man_tiled, uint32_t tile_height, uint32_t tile_width,
+                                              const void *d_checkpoints, uint32_t segments, const uint16_t *d_bias,
+                                              uint16_t *d_out, uint32_t out_stride, void *d_workspace,
+                                              size_t workspace_bytes, ci_stream_t stream) {
+    return fused_linear_impl(d_x, M, K, N, x_stride, d_stream, stream_len, d_states, d_tables, d_slot_map,
+                             d_tile_offsets, d_tile_max_lens, d_man_tiled, tile_height, tile_width, d_bias, d_out,
+                             out_stride, d_workspace, workspace_bytes, false, static_cast<hipStream_t>(stream), nullptr,
+                             d_checkpoints, segments);
+}
+
 extern "C" int ci_plain_linear_same_order(const uint16_t *d_x, uint32_t M, uint32_t K, uint32_t N, uint32_t x_stride,
                                           const uint16_t *d_w, uint32_t tile_height, uint32_t tile_width,
-                                          const uint16_t *d_bias, uint16_t *d_out, uint32_t out_stride,
-                                          void *d_workspace, size_t workspace_bytes, ci_stream_t stream) {
+                                          uint32_t segments, const uint16_t *d_bias, uint16_t *d_out,
+                                          uint32_t out_stride, void *d_workspace, size_t workspace_bytes,
+                                          ci_stream_t stream) {
     if (!d_w) return fail(CI_ERR_ARG, "plain-weight linear: null weight");
     return fused_linear_impl(d_x, M, K, N, x_stride, nullptr, 0, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr,
                              tile_height, tile_width, d_bias, d_out, out_stride, d_workspace, workspace_bytes, false,
-                             static_cast<hipStream_t>(stream), d_w);
+                             static_cast<hipStream_t>(stream), d_w, nullptr, segments);
 }
 
 extern "C" int ci_splitk_reduce(const void *d_partial, int partial_is_bf16, uint32_t P, uint32_t M, uint32_t N,

@@ -75,7 +75,7 @@ def _pick_workspace(workspace, need: int, dev):
 
 
 def _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, meta0, meta1, tile_k,
-         tile_n, mantissas, bias, out, workspace, dense: bool):
+         tile_n, mantissas, bias, out, workspace, dense: bool, checkpoints=None, segments: int = 1):
     K, N = int(weight_shape[0]), int(weight_shape[1])
     _lib.require_device(x)
     dev = x.device
@@ -104,18 +104,28 @@ def _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, met
     need_man = (-(-K // tile_k)) * (-(-N // tile_n)) * tile_k * tile_n
     if man.numel() < need_man:
         man = torch.nn.functional.pad(man, (0, need_man - man.numel()))
-    need = lib().ci_fused_linear_workspace_bytes(M, K, N, int(tile_k), int(tile_n), int(dense))
+    segments = int(segments) if checkpoints is not None and not dense else 1
+    need = lib().ci_fused_linear_workspace_bytes_segmented(M, K, N, int(tile_k), int(tile_n), int(dense), segments)
     ws, ws_bytes = _pick_workspace(workspace, need, dev)
     b = None
     if bias is not None:
         b = bias.to(device=dev, dtype=torch.bfloat16).contiguous()
-    fn = lib().ci_fused_linear_dense if dense else lib().ci_fused_linear_ilp2
     # device copies must stay referenced until the launch has been enqueued
     st, tb, sm = _lib.as_u32(initial_states, dev), _lib.as_u32(tables, dev), _lib.as_u8(slot_map, dev)
     m0, m1 = _lib.as_u32(meta0, dev), _lib.as_u32(meta1, dev)
-    check(fn(ptr(x2), M, K, N, x2.stride(0), ptr(stream_t), C.c_uint64(stream_t.numel()),
-             ptr(st), ptr(tb), ptr(sm), ptr(m0), ptr(m1), ptr(man), int(tile_k), int(tile_n), ptr(b), ptr(result), result.stride(0), ptr(ws),
-             C.c_size_t(ws_bytes), _lib.stream_handle(dev)))
+    if segments > 1:
+        ck = checkpoints.to(dev).contiguous()
+        if ck.dtype != torch.int64 or ck.numel() * 8 != lib().ci_checkpoint_bytes(K, N, int(tile_k), int(tile_n), segments):
+            raise RuntimeError("checkpoints do not belong to this weight shape, tiling and segment count")
+        check(lib().ci_fused_linear_ilp2_segmented(
+            ptr(x2), M, K, N, x2.stride(0), ptr(stream_t), C.c_uint64(stream_t.numel()), ptr(st), ptr(tb), ptr(sm),
+            ptr(m0), ptr(m1), ptr(man), int(tile_k), int(tile_n), ptr(ck), segments, ptr(b), ptr(result),
+            result.stride(0), ptr(ws), C.c_size_t(ws_bytes), _lib.stream_handle(dev)))
+    else:
+        fn = lib().ci_fused_linear_dense if dense else lib().ci_fused_linear_ilp2
+        check(fn(ptr(x2), M, K, N, x2.stride(0), ptr(stream_t), C.c_uint64(stream_t.numel()),
+                 ptr(st), ptr(tb), ptr(sm), ptr(m0), ptr(m1), ptr(man), int(tile_k), int(tile_n), ptr(b), ptr(result),
+                 result.stride(0), ptr(ws), C.c_size_t(ws_bytes), _lib.stream_handle(dev)))
     if out is not None:
         return out
     return result.view(*x.shape[:-1], N)
@@ -123,13 +133,16 @@ def _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, met
 
 def fused_rans_linear(x, compressed_data, initial_states, tables, slot_map, weight_shape, tile_offsets,
                       tile_max_lens, tile_k, tile_n, mantissas, accum_block_size=32, bias=None, out=None,
-                      SPLIT_K=8, workspace=None):
+                      SPLIT_K=8, workspace=None, checkpoints=None, segments=1):
     """x[..., K] @ W[K, N] (+ bias) with W in the tiled two-streams-per-column format
     (comp_inference/linear_triton.py:229-315).  `accum_block_size` and `SPLIT_K` are accepted for
     signature compatibility: the kernel always gives every tile its own wavefront and sums the
-    per-tile partials in a fixed order, which is the finest split the format allows."""
+    per-tile partials in a fixed order, which is the finest split the format allows.
+    `checkpoints`, `segments` (not in the reference): the index made by `build_checkpoints`, with which
+    every segment of every tile gets a wavefront of its own -- for weights with few tiles."""
     return _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, tile_offsets,
-                tile_max_lens, tile_k, tile_n, mantissas, bias, out, workspace, dense=False)
+                tile_max_lens, tile_k, tile_n, mantissas, bias, out, workspace, dense=False,
+                checkpoints=checkpoints, segments=segments)
 
 
 def fused_rans_linear_uncoalesced(x, compressed_data, initial_states, tables, slot_map, weight_shape,
@@ -157,12 +170,13 @@ def splitk_reduce(workspace: torch.Tensor, bias=None, out=None):
     return result
 
 
-def plain_linear_same_order(x, weight_kn, tile_k=1024, tile_n=32, bias=None, workspace=None):
+def plain_linear_same_order(x, weight_kn, tile_k=1024, tile_n=32, bias=None, workspace=None, segments=1):
     """x[..., K] @ weight_kn[K, N] (+ bias) for an uncompressed bf16 weight, through the fused kernel's
     own contraction: same tiling, same matrix instructions in the same order, same partial sums.  The
     result is bit-identical to `fused_rans_linear` on the compressed form of `weight_kn` (tile
     `tile_k` x 32), which `torch.matmul` is not (other summation order).  A verification aid without
-    a counterpart in the reference; slow.  Above DECODE_ONCE_ABOVE_ROWS rows it does what
+    a counterpart in the reference; slow.  `segments` as given to `fused_rans_linear` (it changes how the
+    contraction is split into partial sums).  Above DECODE_ONCE_ABOVE_ROWS rows it does what
     `fused_rans_linear` does there, a library GEMM.  `workspace` as for `fused_rans_linear`: when the contraction is
     split over K, the fp32 partial sums [P, M, N] are left at its start."""
     _lib.require_device(x)
@@ -181,12 +195,12 @@ def plain_linear_same_order(x, weight_kn, tile_k=1024, tile_n=32, bias=None, wor
             result += bias.to(device=dev, dtype=torch.bfloat16)
         return result.view(*x.shape[:-1], N)
     result = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
-    need = lib().ci_fused_linear_workspace_bytes(M, K, N, int(tile_k), int(tile_n), 0)
+    need = lib().ci_fused_linear_workspace_bytes_segmented(M, K, N, int(tile_k), int(tile_n), 0, int(segments))
     ws, ws_bytes = _pick_workspace(workspace, need, dev)
     b = bias.to(device=dev, dtype=torch.bfloat16).contiguous() if bias is not None else None
-    check(lib().ci_plain_linear_same_order(ptr(x2), M, K, N, x2.stride(0), ptr(w), int(tile_k), int(tile_n), ptr(b),
-                                           ptr(result), result.stride(0), ptr(ws), C.c_size_t(ws_bytes),
-                                           _lib.stream_handle(dev)))
+    check(lib().ci_plain_linear_same_order(ptr(x2), M, K, N, x2.stride(0), ptr(w), int(tile_k), int(tile_n),
+                                           int(segments), ptr(b), ptr(result), result.stride(0), ptr(ws),
+                                           C.c_size_t(ws_bytes), _lib.stream_handle(dev)))
     return result.view(*x.shape[:-1], N)
 
 

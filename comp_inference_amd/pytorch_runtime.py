@@ -13,6 +13,7 @@ import torch.nn as nn
 
 from .embedding_hip import fused_rans_embedding
 from .linear_hip import fused_rans_linear
+from .rans_hip import build_checkpoints, suggest_segments
 from .transposed_linear_hip import fused_rans_linear_transposed
 
 
@@ -78,10 +79,35 @@ class RansLinear(nn.Module):
             mod.bias = bias.detach().to(torch.bfloat16).clone()
         return mod
 
+    # Weights with few tiles are bound by the length of one stream's decode chain; decoder checkpoints cut
+    # every stream into segments that decode side by side.  `auto`: as many segments as the library
+    # suggests for the shape; an int fixes them; 1 switches the index off.
+    segments = "auto"
+
+    def _checkpoints(self, device):
+        """(checkpoints, segments) for the weight as it lies on `device`: built on first use from the
+        compressed stream (one pass of the decoder) and kept beside it; not part of the saved state."""
+        key = (str(device), self.rans_exp_stream.data_ptr(), self.rans_exp_stream.numel())
+        cached = getattr(self, "_ckpt_cache", None)
+        if cached is not None and cached[0] == key:
+            return cached[1], cached[2]
+        shape = (self.in_features, self.out_features)
+        segs = suggest_segments(shape, self.tile_k, self.tile_n) if self.segments == "auto" else int(self.segments)
+        ck = None
+        if segs > 1:
+            ck = build_checkpoints(self.rans_exp_stream.to(device), self.rans_exp_states.to(device),
+                                   self.rans_exp_tables.to(device), self.rans_exp_slot_map.to(device), shape,
+                                   self.rans_exp_tile_offsets.to(device), self.rans_exp_tile_max_lens.to(device),
+                                   self.tile_k, self.tile_n, segs)
+        self._ckpt_cache = (key, ck, segs if ck is not None else 1)
+        return self._ckpt_cache[1], self._ckpt_cache[2]
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         device = x.device
+        checkpoints, segments = self._checkpoints(device)
         return fused_rans_linear(
             x=x,
+            checkpoints=checkpoints, segments=segments,
             compressed_data=self.rans_exp_stream.to(device, non_blocking=True),
             initial_states=self.rans_exp_states.to(device, non_blocking=True),
             tables=self.rans_exp_tables.to(device, non_blocking=True),

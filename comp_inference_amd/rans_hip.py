@@ -56,6 +56,37 @@ def rans_decomp_tiled(compressed_streams, initial_states, tables, slot_map, outp
     return out
 
 
+def suggest_segments(weight_shape, tile_k=1024, tile_n=32) -> int:
+    """Segments per stream (1, 2, 4 or 8) with which a weight of this shape fills the chip in the fused
+    linear: 1 for weights with enough tiles of their own.  See `build_checkpoints`."""
+    K, N = int(weight_shape[0]), int(weight_shape[1])
+    return int(lib().ci_suggest_segments(K, N, int(tile_k), int(tile_n)))
+
+
+def build_checkpoints(compressed_streams, initial_states, tables, slot_map, weight_shape, tile_offsets,
+                      tile_max_lens, tile_k=1024, tile_n=32, segments=4):
+    """Decoder checkpoints of a tiled-format tensor: state and byte position of every stream at `segments`
+    evenly spaced rows, as an int64 tensor [tiles, segments - 1, 2 * tile_n] (low half state, high half
+    row of the next unread byte), or None for segments <= 1.  An index kept beside the compressed
+    tensor -- the stream is not changed -- which lets `fused_rans_linear(..., checkpoints=, segments=)`
+    decode the segments of a stream at the same time instead of one after the other.  Not in the
+    reference, whose tiled format has no checkpoints."""
+    if segments <= 1:
+        return None
+    K, N = int(weight_shape[0]), int(weight_shape[1])
+    _lib.require_device(compressed_streams)
+    dev = compressed_streams.device
+    tiles_n, tiles_k = _tiles(K, N, tile_k, tile_n)
+    out = torch.empty((tiles_k * tiles_n, segments - 1, 2 * tile_n), dtype=torch.int64, device=dev)
+    stream_t = _lib.as_u8(compressed_streams, dev)
+    st, tb, sm = _lib.as_u32(initial_states, dev), _lib.as_u32(tables, dev), _lib.as_u8(slot_map, dev)
+    to, tl = _lib.as_u32(tile_offsets, dev), _lib.as_u32(tile_max_lens, dev)
+    check(lib().ci_build_checkpoints_ilp2(
+        ptr(stream_t), C.c_uint64(stream_t.numel()), ptr(st), ptr(tb), ptr(sm), ptr(to), ptr(tl), K, N,
+        int(tile_k), int(tile_n), int(segments), ptr(out), C.c_size_t(out.numel() * 8), _lib.stream_handle(dev)))
+    return out
+
+
 class _DecodeItem(C.Structure):
     _fields_ = [("d_stream", C.c_void_p), ("stream_len", C.c_uint64), ("d_states", C.c_void_p),
                 ("d_tables", C.c_void_p), ("d_slot_map", C.c_void_p), ("d_tile_offsets", C.c_void_p),

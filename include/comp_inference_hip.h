@@ -293,6 +293,41 @@ typedef struct ci_decode_item {
 int ci_decode_tiled_ilp2_batch(const ci_decode_item *h_items, uint32_t n_items, ci_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------
+ * Decoder checkpoints and the fused linear that uses them.  No counterpart in the reference for the
+ * tiled format (its flat format records a checkpoint every 128 symbols, src/cuda/rans_kernels.cuh:454-465).
+ * A stream of the tiled format is a chain of tile_height / 2 dependent decode steps, and a weight
+ * with few tiles (a 4096 x 4096 projection has two per CU) is bound by the length of that chain, not
+ * by the chip.  ci_build_checkpoints_ilp2 walks every stream once and records, at `segments` evenly
+ * spaced rows, the decoder's state and byte position: an index kept beside the compressed weight
+ * (ci_checkpoint_bytes bytes, 8 per stream and checkpoint; the stream is untouched, so the weight stays
+ * readable by the reference).  ci_fused_linear_ilp2_segmented then gives every segment of every
+ * tile its own wavefront.  tile_width must be 32 and tile_height / 2 a multiple of 16 * segments;
+ * ci_suggest_segments returns 1, 2, 4 or 8 for a weight's shape (1: enough tiles of its own).
+ * M above 64, or segments == 1, behaves as ci_fused_linear_ilp2.
+ * ------------------------------------------------------------------------------------- */
+size_t ci_checkpoint_bytes(uint32_t K, uint32_t N, uint32_t tile_height, uint32_t tile_width, uint32_t segments);
+
+uint32_t ci_suggest_segments(uint32_t K, uint32_t N, uint32_t tile_height, uint32_t tile_width);
+
+int ci_build_checkpoints_ilp2(const uint8_t *d_stream, uint64_t stream_len, const uint32_t *d_states,
+                              const uint32_t *d_tables, const uint8_t *d_slot_map,
+                              const uint32_t *d_tile_offsets, const uint32_t *d_tile_max_lens, uint32_t K,
+                              uint32_t N, uint32_t tile_height, uint32_t tile_width, uint32_t segments,
+                              void *d_checkpoints, size_t checkpoint_bytes, ci_stream_t stream);
+
+size_t ci_fused_linear_workspace_bytes_segmented(uint32_t M, uint32_t K, uint32_t N, uint32_t tile_height,
+                                                 uint32_t tile_width, int dense, uint32_t segments);
+
+int ci_fused_linear_ilp2_segmented(const uint16_t *d_x, uint32_t M, uint32_t K, uint32_t N, uint32_t x_stride,
+                                   const uint8_t *d_stream, uint64_t stream_len, const uint32_t *d_states,
+                                   const uint32_t *d_tables, const uint8_t *d_slot_map,
+                                   const uint32_t *d_tile_offsets, const uint32_t *d_tile_max_lens,
+                                   const uint8_t *d_man_tiled, uint32_t tile_height, uint32_t tile_width,
+                                   const void *d_checkpoints, uint32_t segments, const uint16_t *d_bias,
+                                   uint16_t *d_out, uint32_t out_stride, void *d_workspace,
+                                   size_t workspace_bytes, ci_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------
  * Verification aids: the contraction of the fused kernels applied to a plain (uncompressed) bf16
  * weight.  No counterpart in the reference, whose tests compare the fused kernels with
  * torch.matmul within allclose(1e-2, 1e-2) (tests/test_mat_mul.py:220, :238) -- a bar that a wrong
@@ -302,15 +337,17 @@ int ci_decode_tiled_ilp2_batch(const ci_decode_item *h_items, uint32_t n_items, 
  * d_w instead of decoding them; their output is therefore bit-identical to the fused kernels' on
  * the compressed form of d_w, and a run of a whole model on decompressed weights can be compared
  * token by token.  Slow (no staging, guarded loads); 32-column tiles only.
- *   ci_plain_linear_same_order:             d_w = bf16 [K, N] row-major; workspace as
- *                                           ci_fused_linear_workspace_bytes(M, K, N, th, tw, 0)
+ *   ci_plain_linear_same_order:             d_w = bf16 [K, N] row-major; segments as given to
+ *                                           ci_fused_linear_ilp2_segmented (1 for ci_fused_linear_ilp2);
+ *                                           workspace as ci_fused_linear_workspace_bytes_segmented
  *   ci_plain_linear_transposed_same_order:  d_w = bf16 [V, H] row-major; workspace as
  *                                           ci_fused_linear_transposed_workspace_bytes(M, H, V, tw)
  * ------------------------------------------------------------------------------------- */
 int ci_plain_linear_same_order(const uint16_t *d_x, uint32_t M, uint32_t K, uint32_t N, uint32_t x_stride,
                                const uint16_t *d_w, uint32_t tile_height, uint32_t tile_width,
-                               const uint16_t *d_bias, uint16_t *d_out, uint32_t out_stride,
-                               void *d_workspace, size_t workspace_bytes, ci_stream_t stream);
+                               uint32_t segments, const uint16_t *d_bias, uint16_t *d_out,
+                               uint32_t out_stride, void *d_workspace, size_t workspace_bytes,
+                               ci_stream_t stream);
 
 int ci_plain_linear_transposed_same_order(const uint16_t *d_x, uint32_t M, uint32_t H, uint32_t V,
                                           uint32_t x_stride, const uint16_t *d_w, uint32_t tile_height,

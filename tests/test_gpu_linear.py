@@ -272,3 +272,103 @@ def test_fused_linear_random_shapes(oracle, always_fused):
         assert torch.allclose(got.float().cpu(), want, atol=ATOL, rtol=RTOL), (case, K, N, M, th)
         same = plain_linear_same_order(x.cuda(), wdec.cuda(), tile_k=th, tile_n=32)
         assert torch.equal(got.view(torch.int16), same.view(torch.int16)), (case, K, N, M, th)
+
+
+def _pyref_resume(enc, ck, tile, q, seg, seglen, th):
+    """Symbols of segment `seg` of stream q of `tile`, decoded from its checkpoint with plain integers."""
+    spt = 64
+    tables, slot_map = enc.tables, enc.slot_map
+    x, row = (int(enc.states[tile * spt + q]), int(enc.tile_max_lens[tile]) - 1) if seg == 0 else \
+        (int(ck[tile, seg - 1, q]) & 0xFFFFFFFF, ((int(ck[tile, seg - 1, q]) >> 32) + (1 << 31)) % (1 << 32) - (1 << 31))
+    base, out = int(enc.tile_offsets[tile]), []
+    for _ in range(seglen):
+        slot = x & 4095
+        s = int(slot_map[slot])
+        out.append(s)
+        f, c = int(tables[s]) & 0xFFFF, int(tables[s]) >> 16
+        x = f * (x >> 12) + slot - c
+        for _ in range(2):
+            if x < (1 << 16) and row >= 0:
+                x = (x << 8) | int(enc.stream[base + row * spt + q])
+                row -= 1
+    return out, x, row
+
+
+@pytest.mark.parametrize("segments", [2, 4, 8])
+def test_checkpoints_resume_the_decoder(oracle, segments):
+    """A checkpoint is the decoder's state and byte position at the first row of a segment: decoding on from
+    it gives that segment's symbols and arrives exactly at the next checkpoint."""
+    from comp_inference_amd import build_checkpoints
+
+    K, N, th = 2048, 64, 1024
+    w = make_weight_kn(N, K, seed=61)
+    enc, man, wdec = _compress(oracle, w, th, 32)
+    exp_plane = (bf16_bits(wdec) >> 7).astype(np.uint8)
+    dev = "cuda"
+    ck = build_checkpoints(torch.from_numpy(enc.stream).to(dev), _t32(enc.states).to(dev), _t32(enc.tables).to(dev),
+                           torch.from_numpy(enc.slot_map).to(dev), (K, N), _t32(enc.tile_offsets).to(dev),
+                           _t32(enc.tile_max_lens).to(dev), th, 32, segments).cpu().numpy()
+    assert ck.shape == (4, segments - 1, 64)
+    half, seglen = th // 2, th // 2 // segments
+    for tile, q in ((0, 0), (1, 37), (3, 63), (2, 5)):
+        tk, tn = divmod(tile, 2)
+        col, r0 = tn * 32 + q % 32, tk * th + (q // 32) * half
+        for seg in range(segments):
+            syms, x, row = _pyref_resume(enc, ck, tile, q, seg, seglen, th)
+            assert syms == exp_plane[r0 + seg * seglen: r0 + (seg + 1) * seglen, col].tolist(), (tile, q, seg)
+            if seg + 1 < segments:
+                nxt = int(ck[tile, seg, q])
+                assert (x, row) == (nxt & 0xFFFFFFFF, ((nxt >> 32) + (1 << 31)) % (1 << 32) - (1 << 31))
+            else:
+                assert x == 1 << 16  # the stream ends where the encoder began
+
+
+@pytest.mark.parametrize("K,N,th,M,segments", [
+    (4096, 256, 1024, 1, 2), (4096, 256, 1024, 1, 4), (4096, 256, 1024, 1, 8), (4096, 256, 1024, 16, 4),
+    (4096, 256, 1024, 17, 4), (4096, 256, 1024, 64, 2),
+    (3072, 128, 512, 4, 4),
+    (1300, 80, 1024, 3, 4),     # ragged: short last tile row, 80 columns
+    (1300, 80, 1024, 50, 2),
+    (2048, 32800, 1024, 3, 2),  # many tiles and segments
+])
+def test_segmented_fused_linear(oracle, K, N, th, M, segments):
+    """With decoder checkpoints every (tile, segment) is decoded by a wavefront of its own: same result
+    within tolerance, and bit-identical to the plain-weight contraction split the same way."""
+    from comp_inference_amd import build_checkpoints, plain_linear_same_order
+
+    w = make_weight_kn(N, K, seed=K + N + segments)
+    enc, man, wdec = _compress(oracle, w, th, 32)
+    x = make_x(M, K, seed=M + segments)
+    dev = "cuda"
+    ck = build_checkpoints(torch.from_numpy(enc.stream).to(dev), _t32(enc.states).to(dev), _t32(enc.tables).to(dev),
+                           torch.from_numpy(enc.slot_map).to(dev), (K, N), _t32(enc.tile_offsets).to(dev),
+                           _t32(enc.tile_max_lens).to(dev), th, 32, segments)
+    bias = make_x(1, N, seed=5).view(N) if M == 3 else None
+    got = _call(enc, man, x, K, N, th, 32, checkpoints=ck, segments=segments, bias=bias)
+    want = torch.matmul(x.float(), wdec.float()) + (0 if bias is None else bias.float())
+    assert torch.allclose(got.float().cpu(), want, atol=ATOL, rtol=RTOL), (got.float().cpu() - want).abs().max()
+    same = plain_linear_same_order(x.cuda(), wdec.cuda(), tile_k=th, tile_n=32, segments=segments,
+                                   bias=None if bias is None else bias.cuda())
+    assert torch.equal(got.view(torch.int16), same.view(torch.int16))
+    again = _call(enc, man, x, K, N, th, 32, checkpoints=ck, segments=segments, bias=bias)
+    assert torch.equal(got, again)
+
+
+def test_segment_arguments_are_checked(oracle):
+    from comp_inference_amd import build_checkpoints, suggest_segments
+
+    assert suggest_segments((4096, 4096)) == 4 and suggest_segments((4096, 14336)) == 1
+    assert suggest_segments((4096, 28672)) == 2 and suggest_segments((4096, 4096), 1024, 64) == 1
+    K, N, th = 1024, 64, 1024
+    w = make_weight_kn(N, K, seed=71)
+    enc, man, wdec = _compress(oracle, w, th, 32)
+    dev = "cuda"
+    args = (torch.from_numpy(enc.stream).to(dev), _t32(enc.states).to(dev), _t32(enc.tables).to(dev),
+            torch.from_numpy(enc.slot_map).to(dev), (K, N), _t32(enc.tile_offsets).to(dev), _t32(enc.tile_max_lens).to(dev))
+    assert build_checkpoints(*args, th, 32, 1) is None
+    with pytest.raises(RuntimeError):
+        build_checkpoints(*args, th, 32, 3)            # 512 rows do not split into 3 equal segments
+    ck = build_checkpoints(*args, th, 32, 4)
+    x = make_x(2, K, seed=1)
+    with pytest.raises(RuntimeError):
+        _call(enc, man, x, K, N, th, 32, checkpoints=ck, segments=2)   # index made for 4 segments
