@@ -112,6 +112,20 @@ class Compressed:
         return ci.fused_rans_linear(x, self.stream, self.states, self.tables, self.slot_map, (self.K, self.N),
                                     self.tile_offsets, self.tile_max_lens, self.th, self.tw, self.man)
 
+    def linear_segmented(self, x):
+        """The fused linear with decoder checkpoints, as many segments as the library suggests for the shape
+        (built once, on first use, like RansLinear does)."""
+        import comp_inference_amd as ci
+
+        if not hasattr(self, "segments"):
+            self.segments = ci.suggest_segments((self.K, self.N), self.th, self.tw)
+            self.checkpoints = ci.build_checkpoints(self.stream, self.states, self.tables, self.slot_map,
+                                                    (self.K, self.N), self.tile_offsets, self.tile_max_lens,
+                                                    self.th, self.tw, self.segments)
+        return ci.fused_rans_linear(x, self.stream, self.states, self.tables, self.slot_map, (self.K, self.N),
+                                    self.tile_offsets, self.tile_max_lens, self.th, self.tw, self.man,
+                                    checkpoints=self.checkpoints, segments=self.segments)
+
 
 def event_times_us(fn, warmup: int, iters: int):
     """Per-call GPU time with events on the stream the kernels are launched on."""
@@ -312,6 +326,32 @@ def main() -> int:
                          "torch_matmul_bf16_us": round(us_ref, 2),
                          "torch_matmul_weight_GBs": round(2 * gate.K * gate.N / (us_ref * 1e-6) / 1e9, 1)})
         out["fused_gemv"] = {"layer": "gate K=4096 N=14336", "bytes_M1": gate.linear_bytes(1), "rows": rows}
+
+    # --- the four GEMVs of a decoder layer at M = 1 (q/k/v and gate/up fused along the outputs, as the
+    # runtime modules hold them), with decoder checkpoints where the library suggests them
+    if not a.no_gemv:
+        by = {n: w for n, w in make_layer(1)}
+        shapes = [("qkv", torch.cat((by["q"], by["k"], by["v"]), 0)), ("o", by["o"]),
+                  ("gate_up", torch.cat((by["gate"], by["up"]), 0)), ("down", by["down"])]
+        g = torch.Generator("cpu").manual_seed(2)
+        rows, total, total_ref = [], 0.0, 0.0
+        for name, w in shapes:
+            c = Compressed(name, w, dev)
+            x = torch.randn(1, c.K, generator=g, dtype=torch.float32).to(torch.bfloat16).to(dev)
+            w_dense = w.t().contiguous().to(dev)
+            ok = bool(torch.allclose(c.linear_segmented(x).float(), torch.matmul(x, w_dense).float(), atol=1e-2, rtol=1e-2))
+            us = batched_time_us(lambda: c.linear_segmented(x), 25, 100)
+            us_plain = batched_time_us(lambda: c.linear(x), 25, 100)
+            us_ref = batched_time_us(lambda: torch.matmul(x, w_dense), 25, 100)
+            total, total_ref = total + us, total_ref + us_ref
+            rows.append({"layer": f"{name} K={c.K} N={c.N}", "segments": int(c.segments), "us": round(us, 2),
+                         "us_without_checkpoints": round(us_plain, 2), "allclose_1e-2": ok,
+                         "checkpoint_bytes": 0 if c.checkpoints is None else int(c.checkpoints.numel() * 8),
+                         "compressed_bytes": int(c.linear_bytes(1)),
+                         "effective_weight_GBs": round(2 * c.K * c.N / (us * 1e-6) / 1e9, 1),
+                         "torch_matmul_bf16_us": round(us_ref, 2)})
+            del c, w_dense
+        out["fused_gemv_layer_M1"] = {"rows": rows, "sum_us": round(total, 1), "sum_torch_matmul_bf16_us": round(total_ref, 1)}
 
     # --- fused decompress-gather on a 128256 x 4096 table, 2048 Zipf(1.1) ids
     if not a.no_embedding:

@@ -87,10 +87,10 @@ class RansLinear(nn.Module):
     def _checkpoints(self, device):
         """(checkpoints, segments) for the weight as it lies on `device`: built on first use from the
         compressed stream (one pass of the decoder) and kept beside it; not part of the saved state."""
-        key = (str(device), self.rans_exp_stream.data_ptr(), self.rans_exp_stream.numel())
         cached = getattr(self, "_ckpt_cache", None)
-        if cached is not None and cached[0] == key:
+        if cached is not None and cached[0][0] is self.rans_exp_stream and cached[0][1] == device:
             return cached[1], cached[2]
+        key = (self.rans_exp_stream, device)
         shape = (self.in_features, self.out_features)
         segs = suggest_segments(shape, self.tile_k, self.tile_n) if self.segments == "auto" else int(self.segments)
         ck = None

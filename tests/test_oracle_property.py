@@ -32,7 +32,18 @@ def planes(draw):
     return sym.astype(np.uint8), th, tw
 
 
-@settings(max_examples=250, deadline=None)
+def _encode(fn, *args):
+    """The encoders refuse a stream that outgrows the reference's per-stream capacity (1.25 x the mean
+    stream length + 64 bytes, src/cuda/rans_host.cuh:470-471), which ragged planes of poorly compressible
+    symbols can do: such a case has nothing to round-trip."""
+    try:
+        return fn(*args)
+    except RuntimeError as e:
+        assert "capacity" in str(e)
+        return None
+
+
+@settings(max_examples=250, deadline=None, derandomize=True)
 @given(planes())
 def test_every_layout_round_trips(oracle, case):
     sym, th, tw = case
@@ -40,7 +51,11 @@ def test_every_layout_round_trips(oracle, case):
     f, c = oracle.get_lut(sym)
     assert int(f.astype(np.int64).sum()) == 4096 and int(f.min()) >= 1
 
-    enc = oracle.encode_tiled_ilp2(sym, f, c, th, tw)
+    enc = _encode(oracle.encode_tiled_ilp2, sym, f, c, th, tw)
+    den = _encode(oracle.encode_tiled_dense, sym, f, c, th, tw)
+    flat = _encode(oracle.encode_flat, sym, f, c, 512)
+    if enc is None or den is None or flat is None:
+        return
     spt = 2 * tw
     assert (enc.states >= L).all() and (enc.states < (1 << 24)).all()
     lens = enc.tile_max_lens.astype(np.int64) * spt
@@ -55,17 +70,15 @@ def test_every_layout_round_trips(oracle, case):
         assert np.array_equal(pyref.decode_tiled(enc.stream, enc.states, enc.tables, enc.slot_map, enc.tile_offsets,
                                                  enc.tile_max_lens, K, N, th, tw), sym)
 
-    den = oracle.encode_tiled_dense(sym, f, c, th, tw)
     assert np.array_equal(oracle.decode_tiled_dense(den.stream, den.states, den.tables, den.slot_map,
                                                     den.stream_offsets, den.sizes, K, N, th, tw), sym)
     assert den.stream.size == int(den.sizes.astype(np.int64).sum())
 
-    flat = oracle.encode_flat(sym, f, c, 512)
     assert np.array_equal(oracle.decode_flat_segmented(flat.stream, flat.states, flat.sizes, flat.tables,
                                                        flat.slot_map, K, N), sym)
 
 
-@settings(max_examples=150, deadline=None)
+@settings(max_examples=150, deadline=None, derandomize=True)
 @given(st.lists(st.integers(0, 255), min_size=1, max_size=96), st.integers(0, 2 ** 31 - 1))
 def test_one_stream_equals_the_plain_integer_encoder(oracle, symbols, seed):
     """One column, one tile: the C encoder's state and bytes against the Python-integer encoder, with a
