@@ -364,21 +364,31 @@ def main() -> int:
         ids_np = np.random.default_rng(4).choice(V, T, p=p / p.sum())
         ids = torch.from_numpy(ids_np).to(dev)
 
-        def gather():
-            return ci.fused_rans_embedding(ids, emb.stream, emb.states, emb.tables, emb.slot_map, (V, H),
-                                           emb.tile_offsets, emb.tile_max_lens, emb.th, emb.tw, emb.man)
+        emb_segments = 8  # decoder checkpoints every 64 rows, as RansEmbedding keeps them
+        ck = ci.build_checkpoints(emb.stream, emb.states, emb.tables, emb.slot_map, (V, H), emb.tile_offsets,
+                                  emb.tile_max_lens, emb.th, emb.tw, emb_segments)
 
-        exact = bool(torch.equal(gather().cpu().view(torch.int16), table[torch.from_numpy(ids_np)].view(torch.int16)))
+        def gather(use_ck=True):
+            return ci.fused_rans_embedding(ids, emb.stream, emb.states, emb.tables, emb.slot_map, (V, H),
+                                           emb.tile_offsets, emb.tile_max_lens, emb.th, emb.tw, emb.man,
+                                           checkpoints=ck if use_ck else None, segments=emb_segments if use_ck else 1)
+
+        want_rows = table[torch.from_numpy(ids_np)].view(torch.int16)
+        exact = bool(torch.equal(gather().cpu().view(torch.int16), want_rows)) and \
+            bool(torch.equal(gather(False).cpu().view(torch.int16), want_rows))
         us = batched_time_us(gather, 10, 50)
+        us_no_ck = batched_time_us(lambda: gather(False), 10, 50)
         table_dev = table.to(dev)
         us_ref = batched_time_us(lambda: table_dev[ids], 10, 50)
         out["fused_embedding"] = {"table": f"{V}x{H} bf16 N(0,0.02) seed 3", "ids": f"{T} Zipf(1.1) seed 4",
                                   "distinct_ids": int(np.unique(ids_np).size), "bit_exact": exact, "us": round(us, 1),
+                                  "segments": emb_segments, "checkpoint_bytes": int(ck.numel() * 8),
+                                  "us_without_checkpoints": round(us_no_ck, 1),
                                   "rows_per_s": round(T / (us * 1e-6), 1),
                                   "gathered_GBs": round(T * H * 2 / (us * 1e-6) / 1e9, 2),
                                   "compressed_table_bytes": int(emb.stream.numel() + emb.man.numel()),
                                   "torch_index_bf16_us": round(us_ref, 1)}
-        del emb, table_dev, table
+        del emb, table_dev, table, ck
 
     if not a.no_cpu_baseline:
         log("timing the CPU oracle ...")

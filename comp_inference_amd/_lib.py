@@ -38,6 +38,7 @@ def lib() -> C.CDLL:
         _lib.ci_fused_linear_transposed_workspace_bytes.restype = C.c_size_t
         _lib.ci_fused_linear_workspace_bytes_segmented.restype = C.c_size_t
         _lib.ci_checkpoint_bytes.restype = C.c_size_t
+        _lib.ci_fused_embedding_workspace_bytes_segmented.restype = C.c_size_t
         _lib.ci_suggest_segments.restype = C.c_uint32
     return _lib
 

@@ -11,6 +11,9 @@
 // neighbouring column tiles (32 + 32 lanes, all on the same half): a wavefront walks the two half
 // tiles once up to the deepest requested row and writes every requested row on the way as one
 // 128-byte store.  Items of buckets nobody asked for are skipped before touching the stream.
+// With decoder checkpoints (ci_build_checkpoints_ilp2) a bucket is one *segment* of a half tile: the
+// walk starts at the segment's checkpoint instead of the top of the stream, so a requested row costs at
+// most th / (2 segments) decode steps instead of th / 2.
 #include "ci_common.h"
 #include "rans_device.h"
 #include "fast_tile.h"
@@ -39,6 +42,9 @@ struct EmbedArgs {
     const uint32_t *stream_sizes;    // dense layout
     const uint8_t *man_tiled;
     uint32_t K, N, th, tw, tiles_n, n_buckets;
+    const uint2 *ckpt;     // decoder checkpoints, or null
+    uint32_t segs;         // segments per stream (1 without checkpoints)
+    uint32_t bucket_rows;  // rows of a bucket: th / (2 segs)
     uint16_t *out;
     uint32_t out_stride;
     uint32_t *keys;          // workspace: sorted row ids (invalid = 0xFFFFFFFF, sorted last)
@@ -53,7 +59,7 @@ __global__ __launch_bounds__(1024) void embed_sort_kernel(EmbedArgs a) {
     extern __shared__ __align__(16) uint8_t lds[];
     uint32_t *key = reinterpret_cast<uint32_t *>(lds);
     uint32_t *val = key + a.n_pad;
-    const uint32_t tid = threadIdx.x, half = a.th / 2;
+    const uint32_t tid = threadIdx.x, half = a.bucket_rows;  // rows of a bucket
     for (uint32_t i = tid; i < a.n_pad; i += 1024) {
         uint32_t k = 0xFFFFFFFFu;
         if (i < a.n_ids) {
@@ -135,7 +141,7 @@ __device__ __forceinline__ void embed_one_item(const EmbedArgs &a, uint32_t chun
     const uint32_t lo = a.chunk_start[chunk], hi = a.chunk_start[chunk + 1];
     if (lo >= hi || hi > a.n_ids) return;
     const uint32_t key0 = a.keys[lo];
-    const uint32_t b = key0 == 0xFFFFFFFFu ? a.n_buckets : min(key0 / (a.th / 2), a.n_buckets - 1);
+    const uint32_t b = key0 == 0xFFFFFFFFu ? a.n_buckets : min(key0 / a.bucket_rows, a.n_buckets - 1);
     const uint32_t c = lane % 32, side = lane / 32;
     const uint32_t tn = pair * 2 + side, col = tn * 32 + c;
     const bool col_ok = tn < a.tiles_n && col < a.N;
@@ -144,7 +150,9 @@ __device__ __forceinline__ void embed_one_item(const EmbedArgs &a, uint32_t chun
             if (col_ok) a.out[(size_t)a.pos[j] * a.out_stride + col] = 0;
         return;
     }
-    const uint32_t half = a.th / 2, tk = b / 2, hsel = b & 1;
+    // bucket b = rows [b, b + 1) * bucket_rows: segment b % segs of half (b / segs) % 2 of k-tile b / (2 segs)
+    const uint32_t half = a.th / 2, rows_b = a.bucket_rows, seg = b % a.segs, hsel = (b / a.segs) & 1,
+                   tk = b / (2 * a.segs);
     const uint32_t tile_a = tk * a.tiles_n + pair * 2;
     const bool have_b = pair * 2 + 1 < a.tiles_n;
     const uint32_t tile_b = have_b ? tile_a + 1 : tile_a;
@@ -155,23 +163,42 @@ __device__ __forceinline__ void embed_one_item(const EmbedArgs &a, uint32_t chun
     const uint32_t tile = side ? tile_b : tile_a, depth = side ? depth_b : depth_a;
     const uint64_t base = side ? base_b : base_a;
     const uint32_t q = hsel * 32 + c;  // this lane's stream inside its tile
-    const uint32_t state = a.states[(size_t)tile * 64 + q];
-    const uint32_t bucket_row0 = b * half;
-    const uint8_t *man = a.man_tiled + (size_t)tile * a.th * 32 + (size_t)hsel * half * 32 + c;
-    const bool fast = __builtin_amdgcn_ballot_w64(!col_ok) == 0 && depth_a >= 2 && depth_b >= 2 &&
-                      depth_a < kStride && depth_b < kStride && (uint32_t)(uintptr_t)tab == 0;
+    // decoder state and row of the next unread byte at the first row of the bucket, and the row the
+    // stream has reached at the bucket's end
+    uint32_t state;
+    int32_t row = (int32_t)depth - 1, row_end = -1;
+    {
+        const uint2 *ck = a.ckpt + ((size_t)tile * (a.segs - 1)) * 64 + q;  // (only read when segs > 1)
+        if (seg == 0) {
+            state = a.states[(size_t)tile * 64 + q];
+        } else {
+            const uint2 v = ck[(size_t)(seg - 1) * 64];
+            state = v.x;
+            row = min((int32_t)v.y, (int32_t)depth - 1);
+        }
+        if (seg + 1 < a.segs) row_end = min((int32_t)ck[(size_t)seg * 64].y, row);
+    }
+    const uint32_t bucket_row0 = b * rows_b;
+    const uint8_t *man = a.man_tiled + (size_t)tile * a.th * 32 + (size_t)(hsel * half + seg * rows_b) * 32 + c;
+    // rows of the two bodies this item can touch (one window for both: neighbouring tiles lie alike)
+    const int32_t w_lo = max(wave_min_i32(row_end) - 1, 0), w_hi = wave_max_i32(row);
+    const uint32_t win_a = (uint32_t)max(min(w_hi + 1, (int32_t)depth_a) - w_lo, 0),
+                   win_b = (uint32_t)max(min(w_hi + 1, (int32_t)depth_b) - w_lo, 0);
+    const bool fast = __builtin_amdgcn_ballot_w64(!col_ok) == 0 && win_a >= 2 && win_b >= 2 && win_a < kStride &&
+                      win_b < kStride && (uint32_t)(uintptr_t)tab == 0;
     uint32_t j = lo;
     if (fast) {
         StageRegs body;
-        const uint32_t deepest = max(depth_a, depth_b), my_depth = (lane & 4) ? depth_b : depth_a;
+        const uint32_t deepest = max(win_a, win_b), my_depth = (lane & 4) ? win_b : win_a;
+        const uint8_t *src_a = a.stream + base_a + (size_t)w_lo * 64, *src_b = a.stream + base_b + (size_t)w_lo * 64;
 #pragma unroll
         for (int grp = 0; grp < stage_groups(kStride); ++grp)
             if ((uint32_t)grp * 128 < deepest) {
-                stage_fetch_pair(body, a.stream + base_a, depth_a, a.stream + base_b, depth_b, hsel, grp * 128, lane);
+                stage_fetch_pair(body, src_a, win_a, src_b, win_b, hsel, grp * 128, lane);
                 stage_commit<kStride>(body, stage, grp * 128, my_depth, lane);
             }
         FastLane st;
-        st.init<kStride>(stage, depth, lane, state);
+        st.init_at<kStride>(stage, row - w_lo + 1, lane, state);
         // Requests are taken 64 at a time (one sorted key and output row per lane, read back with
         // readlane) and their sign|mantissa bytes eight at a time, one group ahead of the decoding,
         // so that no load sits on the chain of decode steps.
@@ -187,7 +214,7 @@ __device__ __forceinline__ void embed_one_item(const EmbedArgs &a, uint32_t chun
 #pragma unroll
                 for (int u = 0; u < kG; ++u) {
                     const uint32_t idx = min(first + u, nb - 1);  // wave uniform
-                    rows[u] = min((uint32_t)__builtin_amdgcn_readlane((int)my_row, (int)idx), half - 1);
+                    rows[u] = min((uint32_t)__builtin_amdgcn_readlane((int)my_row, (int)idx), rows_b - 1);
                     mans[u] = man[(size_t)rows[u] * 32];
                 }
             };
@@ -215,7 +242,7 @@ __device__ __forceinline__ void embed_one_item(const EmbedArgs &a, uint32_t chun
         return;
     }
     GlobalBytes src;
-    src.init(a.stream + base, depth, 64, q);
+    src.init(a.stream + base, (uint32_t)(row + 1), 64, q);
     uint32_t X = state << 3;
     const uint32_t last_row = a.keys[hi - 1] - bucket_row0;  // deepest requested row of the bucket
     uint32_t want = a.keys[j] - bucket_row0;
@@ -263,11 +290,14 @@ __global__ __launch_bounds__(kPersistWaves *kWave) void embed_gather32_kernel(Em
         if (lo >= a.n_ids) continue;
         const uint32_t key0 = a.keys[lo];
         if (key0 == 0xFFFFFFFFu) continue;  // the chunks of invalid ids touch no tile
-        const uint32_t b = min(key0 / (a.th / 2), a.n_buckets - 1);
-        const uint32_t tile_a = (b / 2) * a.tiles_n + pair * 2;
+        const uint32_t b = min(key0 / a.bucket_rows, a.n_buckets - 1);
+        const uint32_t tile_a = (b / (2 * a.segs)) * a.tiles_n + pair * 2;
         deepest = max(deepest, a.tile_max_lens[tile_a]);
         if (pair * 2 + 1 < a.tiles_n) deepest = max(deepest, a.tile_max_lens[tile_a + 1]);
     }
+    // a segment's window is about its share of the body plus the spread between the lanes; an item whose
+    // window turns out larger than the class allows takes the guarded path
+    if (a.segs > 1) deepest = deepest / a.segs + 40;
     // (this kernel measures a little faster on 10 wavefronts with 204-byte lane strides -- 51 dwords, odd, so
     // the lanes' bytes spread over the banks -- than on 11 with 186: the shallow class is not used)
     const uint32_t cls = persist_classify(lds, a.tables, a.slot_map, deepest);
@@ -336,19 +366,33 @@ static uint32_t next_pow2(uint32_t v) {
     return p;
 }
 
-extern "C" size_t ci_fused_embedding_workspace_bytes(uint32_t n_ids, uint32_t K, uint32_t tile_height) {
-    if (tile_height < 2) return 0;
+extern "C" size_t ci_fused_embedding_workspace_bytes_segmented(uint32_t n_ids, uint32_t K, uint32_t tile_height,
+                                                               uint32_t segments) {
+    if (segments == 0) segments = 1;
+    if (tile_height < 2 || (tile_height / 2) % segments) return 0;
     const uint32_t chunk = n_ids < kEmbChunk ? n_ids : kEmbChunk;
-    const uint32_t n_buckets = ceil_div(K, tile_height / 2);
+    const uint32_t n_buckets = ceil_div(K, tile_height / 2 / segments);
     return (size_t)chunk * 8 + (size_t)(emb_max_chunks(chunk, n_buckets) + 2) * 4;
+}
+
+extern "C" size_t ci_fused_embedding_workspace_bytes(uint32_t n_ids, uint32_t K, uint32_t tile_height) {
+    return ci_fused_embedding_workspace_bytes_segmented(n_ids, K, tile_height, 1);
 }
 
 static int embedding_impl(const int64_t *d_ids, uint32_t n_ids, const uint8_t *d_stream, uint64_t stream_len,
                           const uint32_t *d_states, const uint32_t *d_tables, const uint8_t *d_slot_map,
                           const uint32_t *d_meta0, const uint32_t *d_meta1, const uint8_t *d_man_tiled, uint32_t K,
                           uint32_t N, uint32_t th, uint32_t tw, uint16_t *d_out, uint32_t out_stride,
-                          void *d_workspace, size_t workspace_bytes, bool dense, hipStream_t s) {
+                          void *d_workspace, size_t workspace_bytes, bool dense, hipStream_t s,
+                          const void *d_checkpoints = nullptr, uint32_t segments = 1) {
     if (n_ids == 0 || N == 0) return CI_OK;
+    if (segments == 0) segments = 1;
+    if (segments > 1) {
+        if (dense || tw != 32 || (th & 1) || (th / 2) % segments)
+            return fail(CI_ERR_ARG, "fused embedding: %u segments need 32-column tiles whose half height they divide", segments);
+        if (!d_checkpoints || !aligned(d_checkpoints, 8))
+            return fail(CI_ERR_ARG, "fused embedding: segments without (8-byte aligned) checkpoints");
+    }
     if (!d_ids || !d_states || !d_tables || !d_slot_map || !d_meta0 || !d_meta1 || !d_man_tiled || !d_out)
         return fail(CI_ERR_ARG, "fused embedding: null pointer");
     if (stream_len && !d_stream) return fail(CI_ERR_ARG, "fused embedding: null stream");
@@ -373,6 +417,9 @@ static int embedding_impl(const int64_t *d_ids, uint32_t n_ids, const uint8_t *d
     a.tw = tw;
     a.tiles_n = ceil_div(N, tw);
     a.out_stride = out_stride;
+    a.ckpt = static_cast<const uint2 *>(d_checkpoints);
+    a.segs = 1;
+    a.bucket_rows = th / 2;
 
     const bool fast = !dense && tw == 32 && aligned(d_stream, 16);
     if (!fast) {
@@ -389,8 +436,10 @@ static int embedding_impl(const int64_t *d_ids, uint32_t n_ids, const uint8_t *d
         return CI_OK;
     }
 
-    a.n_buckets = ceil_div(K, th / 2);
-    const size_t need = ci_fused_embedding_workspace_bytes(n_ids, K, th);
+    a.segs = segments;
+    a.bucket_rows = th / 2 / segments;
+    a.n_buckets = ceil_div(K, a.bucket_rows);
+    const size_t need = ci_fused_embedding_workspace_bytes_segmented(n_ids, K, th, segments);
     if (!d_workspace || workspace_bytes < need)
         return fail(CI_ERR_CAPACITY, "fused embedding: workspace needs %zu bytes, got %zu", need, workspace_bytes);
     if (!aligned(d_workspace, 4)) return fail(CI_ERR_ARG, "fused embedding: workspace must be 4-byte aligned");
@@ -429,6 +478,21 @@ extern "C" int ci_fused_embedding_ilp2(const int64_t *d_ids, uint32_t n_ids, con
     return embedding_impl(d_ids, n_ids, d_stream, stream_len, d_states, d_tables, d_slot_map, d_tile_offsets,
                           d_tile_max_lens, d_man_tiled, K, N, tile_height, tile_width, d_out, out_stride,
                           d_workspace, workspace_bytes, false, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int ci_fused_embedding_ilp2_segmented(const int64_t *d_ids, uint32_t n_ids, const uint8_t *d_stream,
+                                                 uint64_t stream_len, const uint32_t *d_states,
+                                                 const uint32_t *d_tables, const uint8_t *d_slot_map,
+                                                 const uint32_t *d_tile_offsets, const uint32_t *d_tile_max_lens,
+                                                 const uint8_t *d_man_tiled, uint32_t K, uint32_t N,
+                                                 uint32_t tile_height, uint32_t tile_width,
+                                                 const void *d_checkpoints, uint32_t segments, uint16_t *d_out,
+                                                 uint32_t out_stride, void *d_workspace, size_t workspace_bytes,
+                                                 ci_stream_t stream) {
+    return embedding_impl(d_ids, n_ids, d_stream, stream_len, d_states, d_tables, d_slot_map, d_tile_offsets,
+                          d_tile_max_lens, d_man_tiled, K, N, tile_height, tile_width, d_out, out_stride,
+                          d_workspace, workspace_bytes, false, static_cast<hipStream_t>(stream), d_checkpoints,
+                          segments);
 }
 
 extern "C" int ci_fused_embedding_dense(const int64_t *d_ids, uint32_t n_ids, const uint8_t *d_stream,

@@ -15,7 +15,7 @@ from .linear_hip import _Scratch
 
 
 def _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, meta0, meta1, tile_k, tile_n,
-         mantissas, out, dense: bool):
+         mantissas, out, dense: bool, checkpoints=None, segments: int = 1):
     K, N = int(weight_shape[0]), int(weight_shape[1])  # K = vocabulary, N = hidden
     _lib.require_device(x)
     dev = x.device
@@ -42,6 +42,17 @@ def _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, met
         check(lib().ci_fused_embedding_dense(
             ptr(ids), n, ptr(stream_t), C.c_uint64(stream_t.numel()), ptr(st), ptr(tb), ptr(sm), ptr(m0), ptr(m1),
             ptr(man), K, N, int(tile_k), int(tile_n), ptr(result), result.stride(0), _lib.stream_handle(dev)))
+    elif checkpoints is not None and int(segments) > 1:
+        segments = int(segments)
+        ck = checkpoints.to(dev).contiguous()
+        if ck.dtype != torch.int64 or ck.numel() * 8 != lib().ci_checkpoint_bytes(K, N, int(tile_k), int(tile_n), segments):
+            raise RuntimeError("checkpoints do not belong to this table shape, tiling and segment count")
+        need = lib().ci_fused_embedding_workspace_bytes_segmented(n, K, int(tile_k), segments)
+        ws = _Scratch.get(need, ("emb", dev))
+        check(lib().ci_fused_embedding_ilp2_segmented(
+            ptr(ids), n, ptr(stream_t), C.c_uint64(stream_t.numel()), ptr(st), ptr(tb), ptr(sm), ptr(m0), ptr(m1),
+            ptr(man), K, N, int(tile_k), int(tile_n), ptr(ck), segments, ptr(result), result.stride(0), ptr(ws),
+            C.c_size_t(ws.numel() if ws is not None else 0), _lib.stream_handle(dev)))
     else:
         need = lib().ci_fused_embedding_workspace_bytes(n, K, int(tile_k))
         ws = _Scratch.get(need, ("emb", dev))
@@ -55,11 +66,13 @@ def _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, met
 
 
 def fused_rans_embedding(x, compressed_data, initial_states, tables, slot_map, weight_shape, tile_offsets,
-                         tile_max_lens, tile_k, tile_n, mantissas, out=None):
+                         tile_max_lens, tile_k, tile_n, mantissas, out=None, checkpoints=None, segments=1):
     """table[x] for a table in the tiled two-streams-per-column format; ids outside the table give
-    zero rows (comp_inference/embedding_triton.py:204-210, :278-330)."""
+    zero rows (comp_inference/embedding_triton.py:204-210, :278-330).  `checkpoints`, `segments` (not in
+    the reference): the index made by `rans_hip.build_checkpoints`; a row then costs at most
+    tile_k / (2 segments) decode steps instead of tile_k / 2."""
     return _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, tile_offsets, tile_max_lens,
-                tile_k, tile_n, mantissas, out, dense=False)
+                tile_k, tile_n, mantissas, out, dense=False, checkpoints=checkpoints, segments=segments)
 
 
 def fused_rans_embedding_uncoalesced(x, compressed_data, initial_states, tables, slot_map, weight_shape,

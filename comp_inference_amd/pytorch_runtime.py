@@ -56,6 +56,23 @@ def _load_from_compressed(mod: nn.Module, src: nn.Module) -> None:
     mod.tile_k, mod.tile_n = int(src.exponent_tile_height), int(src.exponent_tile_width)
 
 
+def _cached_checkpoints(mod: nn.Module, device, shape, segments: int):
+    """(checkpoints, segments) of `mod`'s compressed weight as it lies on `device`: built on first use from
+    the stream (one pass of the decoder) and kept beside it; derived data, not part of the saved state."""
+    cached = getattr(mod, "_ckpt_cache", None)
+    if cached is not None and cached[0][0] is mod.rans_exp_stream and cached[0][1] == device \
+            and cached[0][2] == segments:
+        return cached[1], cached[2]
+    ck = None
+    if segments > 1:
+        ck = build_checkpoints(mod.rans_exp_stream.to(device), mod.rans_exp_states.to(device),
+                               mod.rans_exp_tables.to(device), mod.rans_exp_slot_map.to(device), shape,
+                               mod.rans_exp_tile_offsets.to(device), mod.rans_exp_tile_max_lens.to(device),
+                               mod.tile_k, mod.tile_n, segments)
+    mod._ckpt_cache = ((mod.rans_exp_stream, device, segments), ck, segments if ck is not None else 1)
+    return mod._ckpt_cache[1], mod._ckpt_cache[2]
+
+
 class RansLinear(nn.Module):
     """comp_inference/pytorch_runtime.py:397-459.  Weight stored as [K=in, N=out]."""
 
@@ -85,22 +102,9 @@ class RansLinear(nn.Module):
     segments = "auto"
 
     def _checkpoints(self, device):
-        """(checkpoints, segments) for the weight as it lies on `device`: built on first use from the
-        compressed stream (one pass of the decoder) and kept beside it; not part of the saved state."""
-        cached = getattr(self, "_ckpt_cache", None)
-        if cached is not None and cached[0][0] is self.rans_exp_stream and cached[0][1] == device:
-            return cached[1], cached[2]
-        key = (self.rans_exp_stream, device)
         shape = (self.in_features, self.out_features)
         segs = suggest_segments(shape, self.tile_k, self.tile_n) if self.segments == "auto" else int(self.segments)
-        ck = None
-        if segs > 1:
-            ck = build_checkpoints(self.rans_exp_stream.to(device), self.rans_exp_states.to(device),
-                                   self.rans_exp_tables.to(device), self.rans_exp_slot_map.to(device), shape,
-                                   self.rans_exp_tile_offsets.to(device), self.rans_exp_tile_max_lens.to(device),
-                                   self.tile_k, self.tile_n, segs)
-        self._ckpt_cache = (key, ck, segs if ck is not None else 1)
-        return self._ckpt_cache[1], self._ckpt_cache[2]
+        return _cached_checkpoints(self, device, shape, segs)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         device = x.device
@@ -176,10 +180,22 @@ class RansEmbedding(nn.Module):
         _load_from_compressed(mod, src)
         return mod
 
+    # Decoder checkpoints every 64 rows (8 segments of a 512-row stream): a looked-up row then costs at most
+    # 64 decode steps instead of 512, for an index of 8 % of the compressed table.  1 switches it off.
+    segments = "auto"
+
+    def _checkpoints(self, device):
+        half = self.tile_k // 2
+        segs = int(self.segments) if self.segments != "auto" else \
+            (max(1, half // 64) if self.tile_n == 32 and half % 64 == 0 else 1)
+        return _cached_checkpoints(self, device, (self.num_embeddings, self.embedding_dim), segs)
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         device = x.device
+        checkpoints, segments = self._checkpoints(device)
         return fused_rans_embedding(
             x=x,
+            checkpoints=checkpoints, segments=segments,
             compressed_data=self.rans_exp_stream.to(device, non_blocking=True),
             initial_states=self.rans_exp_states.to(device, non_blocking=True),
             tables=self.rans_exp_tables.to(device, non_blocking=True),

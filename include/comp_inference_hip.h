@@ -301,7 +301,8 @@ int ci_decode_tiled_ilp2_batch(const ci_decode_item *h_items, uint32_t n_items, 
  * spaced rows, the decoder's state and byte position: an index kept beside the compressed weight
  * (ci_checkpoint_bytes bytes, 8 per stream and checkpoint; the stream is untouched, so the weight stays
  * readable by the reference).  ci_fused_linear_ilp2_segmented then gives every segment of every
- * tile its own wavefront.  tile_width must be 32 and tile_height / 2 a multiple of 16 * segments;
+ * tile its own wavefront.  tile_width must be 32 and tile_height / 2 a multiple of 16 * segments
+ * (for ci_build_checkpoints_ilp2 itself any segment count that divides tile_height / 2 will do);
  * ci_suggest_segments returns 1, 2, 4 or 8 for a weight's shape (1: enough tiles of its own).
  * M above 64, or segments == 1, behaves as ci_fused_linear_ilp2.
  * ------------------------------------------------------------------------------------- */
@@ -326,6 +327,20 @@ int ci_fused_linear_ilp2_segmented(const uint16_t *d_x, uint32_t M, uint32_t K, 
                                    const void *d_checkpoints, uint32_t segments, const uint16_t *d_bias,
                                    uint16_t *d_out, uint32_t out_stride, void *d_workspace,
                                    size_t workspace_bytes, ci_stream_t stream);
+
+/* The gather with decoder checkpoints (any segment count that divides tile_height / 2): a requested row
+ * costs at most tile_height / (2 segments) decode steps instead of tile_height / 2. */
+size_t ci_fused_embedding_workspace_bytes_segmented(uint32_t n_ids, uint32_t K, uint32_t tile_height,
+                                                    uint32_t segments);
+
+int ci_fused_embedding_ilp2_segmented(const int64_t *d_ids, uint32_t n_ids, const uint8_t *d_stream,
+                                      uint64_t stream_len, const uint32_t *d_states, const uint32_t *d_tables,
+                                      const uint8_t *d_slot_map, const uint32_t *d_tile_offsets,
+                                      const uint32_t *d_tile_max_lens, const uint8_t *d_man_tiled, uint32_t K,
+                                      uint32_t N, uint32_t tile_height, uint32_t tile_width,
+                                      const void *d_checkpoints, uint32_t segments, uint16_t *d_out,
+                                      uint32_t out_stride, void *d_workspace, size_t workspace_bytes,
+                                      ci_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------
  * Verification aids: the contraction of the fused kernels applied to a plain (uncompressed) bf16

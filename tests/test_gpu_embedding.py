@@ -131,3 +131,26 @@ def test_embedding_random_shapes(oracle):
         ok = (ids >= 0) & (ids < K)
         want[torch.from_numpy(ok)] = table[torch.from_numpy(ids[ok])]
         assert torch.equal(got.cpu().view(torch.int16), want.view(torch.int16)), (case, K, N, T, th)
+
+
+@pytest.mark.parametrize("K,N,th,segments", [(1300, 128, 1024, 8), (2048, 96, 1024, 4), (2048, 96, 1024, 16),
+                                             (700, 64, 256, 2), (3000, 160, 1024, 8)])
+def test_embedding_with_checkpoints(oracle, K, N, th, segments):
+    """With decoder checkpoints the gather starts every walk at a segment boundary: same rows, bit for bit
+    (ragged shapes, duplicates, invalid ids, hot segments with more than 64 requests)."""
+    from comp_inference_amd import build_checkpoints
+
+    table = make_weight_kn(K, N, seed=K + segments).t().contiguous()
+    enc, man = oracle.compress_bf16(bf16_bits(table), th, 32)
+    rng = np.random.default_rng(K + N)
+    ids = np.concatenate([rng.integers(0, K, 400), np.full(150, min(K - 1, 70)), [0, K - 1, K, -1, th // 2 - 1,
+                          th // 2, min(K - 1, th), min(K - 1, th // 2 // segments)], rng.integers(60, 70, 100)])
+    ids = torch.from_numpy(ids)
+    dev = "cuda"
+    ck = build_checkpoints(torch.from_numpy(enc.stream).to(dev), _t32(enc.states).to(dev), _t32(enc.tables).to(dev),
+                           torch.from_numpy(enc.slot_map).to(dev), (K, N), _t32(enc.tile_offsets).to(dev),
+                           _t32(enc.tile_max_lens).to(dev), th, 32, segments)
+    got = _gather(enc, man, ids, K, N, th, 32, checkpoints=ck, segments=segments)
+    assert torch.equal(got.cpu().view(torch.int16), _expected(table, ids).view(torch.int16))
+    plain = _gather(enc, man, ids, K, N, th, 32)
+    assert torch.equal(got, plain)
