@@ -270,6 +270,13 @@ def run(n_layers=32, n_prompt=128, n_new=256, tile_k=1024, tile_n=32, gen="cpu")
             ids, sec = generate(dec, prompt, n_new, graph)
             res[name] = (ids, sec)
             del dec
+    # the decoder-checkpoint indexes the compressed modules built for themselves on first use
+    index_bytes = 0
+    for mods in ([comp["embed"], comp["head"]], comp["qkv"], comp["o"], comp["gate_up"], comp["down"]):
+        for m in mods:
+            ck = getattr(m, "_ckpt_cache", None)
+            if ck is not None and ck[1] is not None:
+                index_bytes += ck[1].numel() * 8
     base = res["reference_bf16"][0]
     with torch.no_grad():
         log("teacher-forced comparison ...")
@@ -295,6 +302,7 @@ def run(n_layers=32, n_prompt=128, n_new=256, tile_k=1024, tile_n=32, gen="cpu")
         "model": f"Llama-3-8B shape, {n_layers} layers, random init seed 5 ({gen} generator), tile {tile_k}x{tile_n}",
         "prompt_tokens": n_prompt, "new_tokens": n_new,
         "weight_bytes_compressed": sizes["compressed"], "weight_bytes_bf16": sizes["bf16"],
+        "checkpoint_index_bytes": int(index_bytes),
         "tok_per_s_compressed_graph": round(n_new / res["compressed_graph"][1], 2),
         "tok_per_s_compressed_eager": round(n_new / res["compressed_eager"][1], 2),
         "tok_per_s_reference_bf16_graph": round(n_new / res["reference_bf16_graph"][1], 2),
