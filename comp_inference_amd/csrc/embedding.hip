@@ -303,6 +303,8 @@ __global__ __launch_bounds__(kPersistWaves *kWave) void embed_gather32_kernel(Em
     const uint32_t cls = persist_classify(lds, a.tables, a.slot_map, deepest);
     if (cls == 2u)
         embed_wave_items<8, kDepthDeep>(a, tab, lds, wave, lane);
+    else if (cls == 3u)
+        embed_wave_items<12, kDepthTiny>(a, tab, lds, wave, lane);
     else
         embed_wave_items<10, kDepthMedium>(a, tab, lds, wave, lane);
 }

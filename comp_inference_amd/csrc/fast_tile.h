@@ -134,28 +134,31 @@ __device__ __forceinline__ int32_t wave_min_i32(int32_t v) { return -wave_max_i3
 // The kernels built on the loops below are bound by wavefronts in flight, not by memory: the whole
 // LDS goes to the slot table plus as many transposed tile bodies as fit, one workgroup per CU, and
 // every wavefront walks a list of tiles.  How many bodies fit depends on the deepest body among the
-// workgroup's tiles: 11 wavefronts x 186 bytes per lane, 10 x 204 or 8 x 254.
-constexpr int kPersistWaves = 11;
-constexpr uint32_t kDepthShallow = 186, kDepthMedium = 204, kDepthDeep = 254;
+// workgroup's tiles: 12 wavefronts x 164 bytes per lane (segments of streams, shallow bodies), 11 x 186,
+// 10 x 204 or 8 x 254.  Twelve is also the most the register file allows (three wavefronts per SIMD
+// at 168 VGPRs).
+constexpr int kPersistWaves = 12;
+constexpr uint32_t kDepthTiny = 164, kDepthShallow = 186, kDepthMedium = 204, kDepthDeep = 254;
 
 // Builds the slot table and classifies the workgroup by the deepest tile body it will meet
-// (`deepest` = this thread's maximum over its share of the workgroup's tiles): returns 0 (all below
-// kDepthShallow), 1 (all below kDepthMedium) or 2.  Contains the only workgroup barrier of such a
-// kernel; blockDim.x must be kPersistWaves * 64.
+// (`deepest` = this thread's maximum over its share of the workgroup's tiles): returns 3 (all below
+// kDepthTiny), 0 (all below kDepthShallow), 1 (all below kDepthMedium) or 2.  Contains the only workgroup
+// barrier of such a kernel; blockDim.x must be kPersistWaves * 64.
 __device__ __forceinline__ uint32_t persist_classify(uint8_t *lds, const uint32_t *__restrict__ tables,
                                                      const uint8_t *__restrict__ slot_map, uint32_t deepest) {
     const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
     uint32_t *flags = reinterpret_cast<uint32_t *>(lds + kLdsLimit - 64);  // beyond every staging area
     build_slot_table_x8(reinterpret_cast<uint2 *>(lds), tables, slot_map, tid, kPersistWaves * 64);
     const uint32_t mine = (__builtin_amdgcn_ballot_w64(deepest >= kDepthShallow) ? 1u : 0u) |
-                          (__builtin_amdgcn_ballot_w64(deepest >= kDepthMedium) ? 2u : 0u);
+                          (__builtin_amdgcn_ballot_w64(deepest >= kDepthMedium) ? 2u : 0u) |
+                          (__builtin_amdgcn_ballot_w64(deepest >= kDepthTiny) ? 4u : 0u);
     if (lane == 0) flags[wave] = mine;
     __syncthreads();
     uint32_t any = 0;
 #pragma unroll
     for (int w = 0; w < kPersistWaves; ++w) any |= flags[w];
     any = (uint32_t)__builtin_amdgcn_readfirstlane((int)any);
-    return (any & 2u) ? 2u : (any & 1u);
+    return (any & 2u) ? 2u : (any & 1u) ? 1u : (any & 4u) ? 0u : 3u;
 }
 
 // The same for a workgroup that takes the tiles j, j + n_wg, ... of one tensor.

@@ -413,8 +413,10 @@ __global__ __launch_bounds__(kPersistWaves *kWave) void fused_linear32_resident_
         linear_wave_tiles<MB, 8, kDepthDeep>(a, tab, lds, wave, lane);
     else if (cls == 1u)
         linear_wave_tiles<MB, 10, kDepthMedium>(a, tab, lds, wave, lane);
+    else if (cls == 0u)
+        linear_wave_tiles<MB, 11, kDepthShallow>(a, tab, lds, wave, lane);
     else
-        linear_wave_tiles<MB, kPersistWaves, kDepthShallow>(a, tab, lds, wave, lane);
+        linear_wave_tiles<MB, 12, kDepthTiny>(a, tab, lds, wave, lane);
 }
 
 // Any tile width, either tiled layout: one thread per stream, eight rows of x per pass.

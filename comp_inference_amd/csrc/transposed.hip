@@ -203,7 +203,7 @@ __global__ __launch_bounds__(kPersistWaves *kWave) void trans32_kernel(TransArgs
     else if (cls == 1u)
         trans_wave_tiles<MB, 10, kDepthMedium>(a, tab, lds, wave, lane);
     else
-        trans_wave_tiles<MB, kPersistWaves, kDepthShallow>(a, tab, lds, wave, lane);
+        trans_wave_tiles<MB, 11, kDepthShallow>(a, tab, lds, wave, lane);
 }
 
 // Any tile width and the dense layout: one thread per (tile, half): it decodes the tile's columns
