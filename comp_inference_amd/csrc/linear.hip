@@ -487,8 +487,19 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *partial
     const uint64_t e = (uint64_t)blockIdx.x * 256 + threadIdx.x;
     if (e >= (uint64_t)M * N) return;
     const uint32_t m = (uint32_t)(e / N), n = (uint32_t)(e % N);
+    const size_t plane = (size_t)M * N;
     float s = 0.f;
-    for (uint32_t p = 0; p < P; ++p) s += partial[(size_t)p * M * N + e];
+    uint32_t p = 0;
+    // eight loads in flight at a time (the sum keeps its order): one load per iteration would make the
+    // kernel a chain of P memory latencies
+    for (; p + 8 <= P; p += 8) {
+        float v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = partial[(size_t)(p + j) * plane + e];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) s += v[j];
+    }
+    for (; p < P; ++p) s += partial[(size_t)p * plane + e];
     out[(size_t)m * out_stride + n] = finish_bf16(s, bias, n);
 }
 
