@@ -490,14 +490,21 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *partial
     const size_t plane = (size_t)M * N;
     float s = 0.f;
     uint32_t p = 0;
-    // eight loads in flight at a time (the sum keeps its order): one load per iteration would make the
-    // kernel a chain of P memory latencies
-    for (; p + 8 <= P; p += 8) {
-        float v[8];
+    // sixteen, then four loads in flight at a time (the sum keeps its order): one load per iteration would
+    // make the kernel a chain of P memory latencies
+    for (; p + 16 <= P; p += 16) {
+        float v[16];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) v[j] = partial[(size_t)(p + j) * plane + e];
+        for (int j = 0; j < 16; ++j) v[j] = partial[(size_t)(p + j) * plane + e];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) s += v[j];
+        for (int j = 0; j < 16; ++j) s += v[j];
+    }
+    for (; p + 4 <= P; p += 4) {
+        float v[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] = partial[(size_t)(p + j) * plane + e];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) s += v[j];
     }
     for (; p < P; ++p) s += partial[(size_t)p * plane + e];
     out[(size_t)m * out_stride + n] = finish_bf16(s, bias, n);
