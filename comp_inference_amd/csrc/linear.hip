@@ -588,7 +588,7 @@ extern "C" size_t ci_fused_linear_workspace_bytes(uint32_t M, uint32_t K, uint32
     return ci_fused_linear_workspace_bytes_segmented(M, K, N, tile_height, tile_width, dense, 1);
 }
 
-// Segments per stream for a weight of this shape, from measurements on 256 CUs x 11 wavefronts: as many
+// Segments per stream for a weight of this shape, from measurements on 256 CUs x 12 wavefronts: as many
 // (2, 4 or 8) as still give every (tile, segment) a wavefront of its own in one round -- the time is
 // then one chain of th / (2 segments) steps instead of th / 2 -- and 2 for weights that take several
 // rounds anyway (shorter items fill the last round better); 1 in between, where the chip is busy with
