@@ -193,46 +193,46 @@ __device__ __forceinline__ void stage_body(uint8_t *stage, const uint8_t *__rest
 
 // ---- assembly building blocks ----------------------------------------------------------------
 // Fixed temporaries (declared as clobbers by every user):
-//   v[96:97], v[98:99]  slot-table entries of the even / odd step of a pair
-//   v100 address, v101 quotient, v102 n1 << 3, v103 n2 << 3, v104 t, v105 t<<8|n1, v106 ..<<8|n2
+//   v[72:73], v[74:75]  slot-table entries of the even / odd step of a pair
+//   v76 address, v77 quotient, v78 n1 << 3, v79 n2 << 3, v80 t, v81 t<<8|n1, v82 ..<<8|n2
 //   s[20:21] second compare
 // Operands by name: X q n1 n2 (lane state), L8 B8 (scaled 2^16 and 2^8 in SGPRs).
 
 // Issue the table read and prepare everything that does not depend on it.
 #define CI_STEP_ISSUE(E)                       \
-    "v_and_b32 v100, 0x7ff8, %[X]\n"           \
-    "ds_read_b64 " E ", v100\n"                \
-    "v_lshrrev_b32 v101, 15, %[X]\n"           \
+    "v_and_b32 v76, 0x7ff8, %[X]\n"           \
+    "ds_read_b64 " E ", v76\n"                \
+    "v_lshrrev_b32 v77, 15, %[X]\n"           \
     "s_waitcnt lgkmcnt(1)\n"                   \
-    "v_lshlrev_b32 v102, 3, %[n1]\n"           \
-    "v_lshlrev_b32 v103, 3, %[n2]\n"
+    "v_lshlrev_b32 v78, 3, %[n1]\n"           \
+    "v_lshlrev_b32 v79, 3, %[n2]\n"
 
 // Consume the table entry (ELO/EHI = its two dwords): new state, pointer, next two bytes.
 #define CI_STEP_FINISH(ELO, EHI)                        \
     "s_waitcnt lgkmcnt(0)\n"                            \
-    "v_mad_u32_u24 v104, " ELO ", v101, " EHI "\n"      \
-    "v_cmp_gt_u32 vcc, %[L8], v104\n"                   \
-    "v_cmp_gt_u32 s[20:21], %[B8], v104\n"              \
-    "v_lshl_or_b32 v105, v104, 8, v102\n"               \
-    "v_lshl_or_b32 v106, v105, 8, v103\n"               \
-    "v_cndmask_b32 %[X], v104, v105, vcc\n"             \
+    "v_mad_u32_u24 v80, " ELO ", v77, " EHI "\n"      \
+    "v_cmp_gt_u32 vcc, %[L8], v80\n"                   \
+    "v_cmp_gt_u32 s[20:21], %[B8], v80\n"              \
+    "v_lshl_or_b32 v81, v80, 8, v78\n"               \
+    "v_lshl_or_b32 v82, v81, 8, v79\n"               \
+    "v_cndmask_b32 %[X], v80, v81, vcc\n"             \
     "v_subbrev_co_u32 %[q], vcc, 0, %[q], vcc\n"        \
-    "v_cndmask_b32 %[X], %[X], v106, s[20:21]\n"        \
+    "v_cndmask_b32 %[X], %[X], v82, s[20:21]\n"        \
     "v_subbrev_co_u32 %[q], vcc, 0, %[q], s[20:21]\n"   \
     "ds_read_u8 %[n1], %[q] offset:1\n"                 \
     "ds_read_u8 %[n2], %[q]\n"
 
 #define CI_STEP_CLOBBERS                                                                                  \
-    "vcc", "s20", "s21", "v96", "v97", "v98", "v99", "v100", "v101", "v102", "v103", "v104", "v105", "v106", \
+    "vcc", "s20", "s21", "v72", "v73", "v74", "v75", "v76", "v77", "v78", "v79", "v80", "v81", "v82", \
         "memory"
 
 // Two decoded symbols (top bytes of ELO0, ELO1) and their sign|mantissa bytes (byte %[msel] of the
-// dwords M0, M1) -> one dword holding two bf16 (first row in the low half).  v107/v136 temporaries.
+// dwords M0, M1) -> one dword holding two bf16 (first row in the low half).  v83/v112 temporaries.
 #define CI_PACK(ELO0, ELO1, M0, M1, WV)                       \
-    "v_perm_b32 v107, " ELO1 ", " ELO0 ", %[selE]\n"          \
-    "v_lshrrev_b32 v107, 1, v107\n"                           \
-    "v_perm_b32 v136, " M1 ", " M0 ", %[msel]\n"              \
-    "v_and_or_b32 " WV ", v136, %[mask], v107\n"
+    "v_perm_b32 v83, " ELO1 ", " ELO0 ", %[selE]\n"          \
+    "v_lshrrev_b32 v83, 1, v83\n"                           \
+    "v_perm_b32 v112, " M1 ", " M0 ", %[msel]\n"              \
+    "v_and_or_b32 " WV ", v112, %[mask], v83\n"
 
 // Advance the per-lane load offsets to the block after the current one (wrapping to block 0
 // after the last, so the loads stay inside the tile) -- s23 counts the blocks requested so far.
@@ -267,43 +267,43 @@ __device__ __forceinline__ void stage_body(uint8_t *stage, const uint8_t *__rest
 // pack of the previous block and its MFMA.
 // EXTRA_OFFS / EXTRA_LOAD: nothing, or the offset step and load of a second x fragment.
 #define CI_BLOCK(TAIL, EXTRA_OFFS, EXTRA_LOAD, C0, C1, C2, C3, C4, C5, C6, C7, N0, N1, N2, N3, N4, N5, N6, N7, NX) \
-    CI_STEP_ISSUE("v[96:97]") TAIL CI_STEP_FINISH("v96", "v97")                                  \
-    CI_STEP_ISSUE("v[98:99]") CI_NEXT_BLOCK_OFFSETS EXTRA_OFFS CI_LOAD_LO(N0, N1, N2, N3, N4)    \
-    CI_STEP_FINISH("v98", "v99")                                                                 \
-    CI_STEP_ISSUE("v[140:141]") "s_waitcnt vmcnt(5)\n" CI_PACK("v96", "v98", C0, C1, "v132")     \
-    CI_STEP_FINISH("v140", "v141")                                                               \
-    CI_STEP_ISSUE("v[142:143]") CI_LOAD_HI(N5, N6, N7, NX) EXTRA_LOAD CI_STEP_FINISH("v142", "v143") \
-    CI_STEP_ISSUE("v[96:97]") CI_PACK("v140", "v142", C2, C3, "v133") CI_STEP_FINISH("v96", "v97") \
-    CI_STEP_ISSUE("v[98:99]") CI_STEP_FINISH("v98", "v99")                                       \
-    CI_STEP_ISSUE("v[140:141]") CI_PACK("v96", "v98", C4, C5, "v134") CI_STEP_FINISH("v140", "v141") \
-    CI_STEP_ISSUE("v[142:143]") CI_STEP_FINISH("v142", "v143")
+    CI_STEP_ISSUE("v[72:73]") TAIL CI_STEP_FINISH("v72", "v73")                                  \
+    CI_STEP_ISSUE("v[74:75]") CI_NEXT_BLOCK_OFFSETS EXTRA_OFFS CI_LOAD_LO(N0, N1, N2, N3, N4)    \
+    CI_STEP_FINISH("v74", "v75")                                                                 \
+    CI_STEP_ISSUE("v[116:117]") "s_waitcnt vmcnt(5)\n" CI_PACK("v72", "v74", C0, C1, "v108")     \
+    CI_STEP_FINISH("v116", "v117")                                                               \
+    CI_STEP_ISSUE("v[118:119]") CI_LOAD_HI(N5, N6, N7, NX) EXTRA_LOAD CI_STEP_FINISH("v118", "v119") \
+    CI_STEP_ISSUE("v[72:73]") CI_PACK("v116", "v118", C2, C3, "v109") CI_STEP_FINISH("v72", "v73") \
+    CI_STEP_ISSUE("v[74:75]") CI_STEP_FINISH("v74", "v75")                                       \
+    CI_STEP_ISSUE("v[116:117]") CI_PACK("v72", "v74", C4, C5, "v110") CI_STEP_FINISH("v116", "v117") \
+    CI_STEP_ISSUE("v[118:119]") CI_STEP_FINISH("v118", "v119")
 
 // Last pack of a block whose buffer is (.., M6, M7, XR) and the block's MFMA.
 #define CI_TAIL(M6, M7, XR)                                             \
-    CI_PACK("v140", "v142", M6, M7, "v135")                             \
+    CI_PACK("v116", "v118", M6, M7, "v111")                             \
     "s_nop 1\n"                                                         \
-    "v_mfma_f32_32x32x16_bf16 %[acc], v[132:135], " XR ", %[acc]\n"
+    "v_mfma_f32_32x32x16_bf16 %[acc], v[108:111], " XR ", %[acc]\n"
 // ... and a second MFMA of the same weights with the x fragment of rows 32..63
 #define CI_TAIL2(M6, M7, XR, XR2) \
-    CI_TAIL(M6, M7, XR) "v_mfma_f32_32x32x16_bf16 %[acc2], v[132:135], " XR2 ", %[acc2]\n"
+    CI_TAIL(M6, M7, XR) "v_mfma_f32_32x32x16_bf16 %[acc2], v[108:111], " XR2 ", %[acc2]\n"
 
 // (argument lists are expanded before CI_BLOCK counts them)
 #define CI_BLOCK_X(...) CI_BLOCK(__VA_ARGS__)
-#define CI_BUF_A "v108", "v109", "v110", "v111", "v112", "v113", "v114", "v115"
-#define CI_BUF_B "v116", "v117", "v118", "v119", "v120", "v121", "v122", "v123"
+#define CI_BUF_A "v84", "v85", "v86", "v87", "v88", "v89", "v90", "v91"
+#define CI_BUF_B "v92", "v93", "v94", "v95", "v96", "v97", "v98", "v99"
 
 // Eight decode steps whose weights leave the statement: W0..W3 = four dwords of two bf16 each
 // (rows 0/1, 2/3, 4/5, 6/7 of the block), from the sign|mantissa dwords M0..M7 of those rows.
 #define CI_BLOCK8_OUT                                                                                      \
-    CI_STEP_ISSUE("v[96:97]") CI_STEP_FINISH("v96", "v97")                                                 \
-    CI_STEP_ISSUE("v[98:99]") CI_STEP_FINISH("v98", "v99")                                                 \
-    CI_STEP_ISSUE("v[140:141]") CI_PACK("v96", "v98", "%[m0]", "%[m1]", "%[w0]") CI_STEP_FINISH("v140", "v141") \
-    CI_STEP_ISSUE("v[142:143]") CI_STEP_FINISH("v142", "v143")                                             \
-    CI_STEP_ISSUE("v[96:97]") CI_PACK("v140", "v142", "%[m2]", "%[m3]", "%[w1]") CI_STEP_FINISH("v96", "v97")  \
-    CI_STEP_ISSUE("v[98:99]") CI_STEP_FINISH("v98", "v99")                                                 \
-    CI_STEP_ISSUE("v[140:141]") CI_PACK("v96", "v98", "%[m4]", "%[m5]", "%[w2]") CI_STEP_FINISH("v140", "v141") \
-    CI_STEP_ISSUE("v[142:143]") CI_STEP_FINISH("v142", "v143")                                             \
-    CI_PACK("v140", "v142", "%[m6]", "%[m7]", "%[w3]")                                                     \
+    CI_STEP_ISSUE("v[72:73]") CI_STEP_FINISH("v72", "v73")                                                 \
+    CI_STEP_ISSUE("v[74:75]") CI_STEP_FINISH("v74", "v75")                                                 \
+    CI_STEP_ISSUE("v[116:117]") CI_PACK("v72", "v74", "%[m0]", "%[m1]", "%[w0]") CI_STEP_FINISH("v116", "v117") \
+    CI_STEP_ISSUE("v[118:119]") CI_STEP_FINISH("v118", "v119")                                             \
+    CI_STEP_ISSUE("v[72:73]") CI_PACK("v116", "v118", "%[m2]", "%[m3]", "%[w1]") CI_STEP_FINISH("v72", "v73")  \
+    CI_STEP_ISSUE("v[74:75]") CI_STEP_FINISH("v74", "v75")                                                 \
+    CI_STEP_ISSUE("v[116:117]") CI_PACK("v72", "v74", "%[m4]", "%[m5]", "%[w2]") CI_STEP_FINISH("v116", "v117") \
+    CI_STEP_ISSUE("v[118:119]") CI_STEP_FINISH("v118", "v119")                                             \
+    CI_PACK("v116", "v118", "%[m6]", "%[m7]", "%[w3]")                                                     \
     "s_waitcnt lgkmcnt(0)\n"
 
 // Per-lane decoder state of the hand-scheduled loops.
@@ -344,20 +344,20 @@ __device__ __forceinline__ void linear_tile_asm(FastLane &st, f32x16_t &acc, uin
         "s_lshr_b32 s22, %[nblk], 1\n"
         "s_sub_u32 s22, s22, 1\n"
         // block 0 into buffer A
-        CI_LOAD_LO("v108", "v109", "v110", "v111", "v112")
-        CI_LOAD_HI("v113", "v114", "v115", "v[124:127]")
-        CI_BLOCK_X("", "", "", CI_BUF_A, CI_BUF_B, "v[128:131]")
-        CI_BLOCK_X(CI_TAIL("v114", "v115", "v[124:127]"), "", "", CI_BUF_B, CI_BUF_A, "v[124:127]")
+        CI_LOAD_LO("v84", "v85", "v86", "v87", "v88")
+        CI_LOAD_HI("v89", "v90", "v91", "v[100:103]")
+        CI_BLOCK_X("", "", "", CI_BUF_A, CI_BUF_B, "v[104:107]")
+        CI_BLOCK_X(CI_TAIL("v90", "v91", "v[100:103]"), "", "", CI_BUF_B, CI_BUF_A, "v[100:103]")
         "ci_lin_loop%=:\n"
         "s_cmp_eq_u32 s22, 0\n"
         "s_cbranch_scc1 ci_lin_done%=\n"
-        CI_BLOCK_X(CI_TAIL("v122", "v123", "v[128:131]"), "", "", CI_BUF_A, CI_BUF_B, "v[128:131]")
-        CI_BLOCK_X(CI_TAIL("v114", "v115", "v[124:127]"), "", "", CI_BUF_B, CI_BUF_A, "v[124:127]")
+        CI_BLOCK_X(CI_TAIL("v98", "v99", "v[104:107]"), "", "", CI_BUF_A, CI_BUF_B, "v[104:107]")
+        CI_BLOCK_X(CI_TAIL("v90", "v91", "v[100:103]"), "", "", CI_BUF_B, CI_BUF_A, "v[100:103]")
         "s_sub_u32 s22, s22, 1\n"
         "s_branch ci_lin_loop%=\n"
         "ci_lin_done%=:\n"
         "s_waitcnt vmcnt(0) lgkmcnt(0)\n"
-        CI_TAIL("v122", "v123", "v[128:131]")
+        CI_TAIL("v98", "v99", "v[104:107]")
         "s_nop 15\n"
         "s_nop 15\n"
         : [X] "+v"(st.X), [q] "+v"(st.q), [n1] "+v"(st.n1), [n2] "+v"(st.n2), [acc] "+v"(acc), [moff] "+v"(moff),
@@ -365,14 +365,14 @@ __device__ __forceinline__ void linear_tile_asm(FastLane &st, f32x16_t &acc, uin
         : [L8] "s"(kRansL << 3), [B8] "s"(256u << 3), [selE] "s"(0x070C030Cu), [mask] "s"(0x807F807Fu),
           [msel] "v"(man_sel), [mbase] "s"(mbase), [xbase] "s"(xbase), [nblk] "s"(nblocks), [wrapM] "s"(wrap_m),
           [wrapX] "s"(wrap_x), [xstep] "s"(xstep)
-        : CI_STEP_CLOBBERS, "scc", "s22", "s23", "s24", "s25", "v107", "v108", "v109", "v110", "v111", "v112",
-          "v113", "v114", "v115", "v116", "v117", "v118", "v119", "v120", "v121", "v122", "v123", "v124", "v125",
-          "v126", "v127", "v128", "v129", "v130", "v131", "v132", "v133", "v134", "v135", "v136", "v140", "v141",
-          "v142", "v143");
+        : CI_STEP_CLOBBERS, "scc", "s22", "s23", "s24", "s25", "v83", "v84", "v85", "v86", "v87", "v88",
+          "v89", "v90", "v91", "v92", "v93", "v94", "v95", "v96", "v97", "v98", "v99", "v100", "v101",
+          "v102", "v103", "v104", "v105", "v106", "v107", "v108", "v109", "v110", "v111", "v112", "v116", "v117",
+          "v118", "v119");
 }
 
 // The same loop for up to 64 rows of x: a second x fragment (rows 32..63, per-lane offset xoff2,
-// buffers v[144:147] / v[148:151]) and a second accumulator fed with the same decoded weights.
+// buffers v[120:123] / v[124:127]) and a second accumulator fed with the same decoded weights.
 __device__ __forceinline__ void linear_tile_asm2(FastLane &st, f32x16_t &acc, f32x16_t &acc2, uint64_t mbase,
                                                  uint32_t moff, uint64_t xbase, uint32_t xoff, uint32_t xoff2,
                                                  uint32_t xstep, uint32_t man_sel, uint32_t nblocks) {
@@ -382,23 +382,23 @@ __device__ __forceinline__ void linear_tile_asm2(FastLane &st, f32x16_t &acc, f3
         "s_lshr_b32 s22, %[nblk], 1\n"
         "s_sub_u32 s22, s22, 1\n"
         // block 0 into buffer A
-        CI_LOAD_LO("v108", "v109", "v110", "v111", "v112")
-        CI_LOAD_HI("v113", "v114", "v115", "v[124:127]") CI_LOAD_X2("v[144:147]")
-        CI_BLOCK_X("", CI_NEXT_BLOCK_OFFSETS2, CI_LOAD_X2("v[148:151]"), CI_BUF_A, CI_BUF_B, "v[128:131]")
-        CI_BLOCK_X(CI_TAIL2("v114", "v115", "v[124:127]", "v[144:147]"), CI_NEXT_BLOCK_OFFSETS2,
-                   CI_LOAD_X2("v[144:147]"), CI_BUF_B, CI_BUF_A, "v[124:127]")
+        CI_LOAD_LO("v84", "v85", "v86", "v87", "v88")
+        CI_LOAD_HI("v89", "v90", "v91", "v[100:103]") CI_LOAD_X2("v[120:123]")
+        CI_BLOCK_X("", CI_NEXT_BLOCK_OFFSETS2, CI_LOAD_X2("v[124:127]"), CI_BUF_A, CI_BUF_B, "v[104:107]")
+        CI_BLOCK_X(CI_TAIL2("v90", "v91", "v[100:103]", "v[120:123]"), CI_NEXT_BLOCK_OFFSETS2,
+                   CI_LOAD_X2("v[120:123]"), CI_BUF_B, CI_BUF_A, "v[100:103]")
         "ci_lin2_loop%=:\n"
         "s_cmp_eq_u32 s22, 0\n"
         "s_cbranch_scc1 ci_lin2_done%=\n"
-        CI_BLOCK_X(CI_TAIL2("v122", "v123", "v[128:131]", "v[148:151]"), CI_NEXT_BLOCK_OFFSETS2,
-                   CI_LOAD_X2("v[148:151]"), CI_BUF_A, CI_BUF_B, "v[128:131]")
-        CI_BLOCK_X(CI_TAIL2("v114", "v115", "v[124:127]", "v[144:147]"), CI_NEXT_BLOCK_OFFSETS2,
-                   CI_LOAD_X2("v[144:147]"), CI_BUF_B, CI_BUF_A, "v[124:127]")
+        CI_BLOCK_X(CI_TAIL2("v98", "v99", "v[104:107]", "v[124:127]"), CI_NEXT_BLOCK_OFFSETS2,
+                   CI_LOAD_X2("v[124:127]"), CI_BUF_A, CI_BUF_B, "v[104:107]")
+        CI_BLOCK_X(CI_TAIL2("v90", "v91", "v[100:103]", "v[120:123]"), CI_NEXT_BLOCK_OFFSETS2,
+                   CI_LOAD_X2("v[120:123]"), CI_BUF_B, CI_BUF_A, "v[100:103]")
         "s_sub_u32 s22, s22, 1\n"
         "s_branch ci_lin2_loop%=\n"
         "ci_lin2_done%=:\n"
         "s_waitcnt vmcnt(0) lgkmcnt(0)\n"
-        CI_TAIL2("v122", "v123", "v[128:131]", "v[148:151]")
+        CI_TAIL2("v98", "v99", "v[104:107]", "v[124:127]")
         "s_nop 15\n"
         "s_nop 15\n"
         : [X] "+v"(st.X), [q] "+v"(st.q), [n1] "+v"(st.n1), [n2] "+v"(st.n2), [acc] "+v"(acc), [acc2] "+v"(acc2),
@@ -406,16 +406,16 @@ __device__ __forceinline__ void linear_tile_asm2(FastLane &st, f32x16_t &acc, f3
         : [L8] "s"(kRansL << 3), [B8] "s"(256u << 3), [selE] "s"(0x070C030Cu), [mask] "s"(0x807F807Fu),
           [msel] "v"(man_sel), [mbase] "s"(mbase), [xbase] "s"(xbase), [nblk] "s"(nblocks), [wrapM] "s"(wrap_m),
           [wrapX] "s"(wrap_x), [xstep] "s"(xstep)
-        : CI_STEP_CLOBBERS, "scc", "s22", "s23", "s24", "s25", "v107", "v108", "v109", "v110", "v111", "v112",
-          "v113", "v114", "v115", "v116", "v117", "v118", "v119", "v120", "v121", "v122", "v123", "v124", "v125",
-          "v126", "v127", "v128", "v129", "v130", "v131", "v132", "v133", "v134", "v135", "v136", "v140", "v141",
-          "v142", "v143", "v144", "v145", "v146", "v147", "v148", "v149", "v150", "v151");
+        : CI_STEP_CLOBBERS, "scc", "s22", "s23", "s24", "s25", "v83", "v84", "v85", "v86", "v87", "v88",
+          "v89", "v90", "v91", "v92", "v93", "v94", "v95", "v96", "v97", "v98", "v99", "v100", "v101",
+          "v102", "v103", "v104", "v105", "v106", "v107", "v108", "v109", "v110", "v111", "v112", "v116", "v117",
+          "v118", "v119", "v120", "v121", "v122", "v123", "v124", "v125", "v126", "v127");
 }
 
 // Symbol of the step that used table entry ELO -> one byte at obase + off; off advances a row.
 #define CI_STORE_SYM(ELO)                                  \
-    "v_lshrrev_b32 v107, 24, " ELO "\n"                    \
-    "global_store_byte %[off], v107, %[obase]\n"           \
+    "v_lshrrev_b32 v83, 24, " ELO "\n"                    \
+    "global_store_byte %[off], v83, %[obase]\n"           \
     "v_add_u32 %[off], %[stride], %[off]\n"
 
 // Stand-alone decode of one half tile per lane: `npairs` >= 1 pairs of steps, symbol i stored at
@@ -424,21 +424,21 @@ __device__ __forceinline__ void decode_tile_asm(FastLane &st, uint64_t obase, ui
                                                 uint32_t npairs) {
     asm volatile(
         "s_sub_u32 s22, %[npairs], 1\n"
-        CI_STEP_ISSUE("v[96:97]") CI_STEP_FINISH("v96", "v97")
+        CI_STEP_ISSUE("v[72:73]") CI_STEP_FINISH("v72", "v73")
         "ci_dec_loop%=:\n"
         "s_cmp_eq_u32 s22, 0\n"
         "s_cbranch_scc1 ci_dec_done%=\n"
-        CI_STEP_ISSUE("v[98:99]") CI_STORE_SYM("v96") CI_STEP_FINISH("v98", "v99")
-        CI_STEP_ISSUE("v[96:97]") CI_STORE_SYM("v98") CI_STEP_FINISH("v96", "v97")
+        CI_STEP_ISSUE("v[74:75]") CI_STORE_SYM("v72") CI_STEP_FINISH("v74", "v75")
+        CI_STEP_ISSUE("v[72:73]") CI_STORE_SYM("v74") CI_STEP_FINISH("v72", "v73")
         "s_sub_u32 s22, s22, 1\n"
         "s_branch ci_dec_loop%=\n"
         "ci_dec_done%=:\n"
-        CI_STEP_ISSUE("v[98:99]") CI_STORE_SYM("v96") CI_STEP_FINISH("v98", "v99")
-        CI_STORE_SYM("v98")
+        CI_STEP_ISSUE("v[74:75]") CI_STORE_SYM("v72") CI_STEP_FINISH("v74", "v75")
+        CI_STORE_SYM("v74")
         "s_waitcnt vmcnt(0) lgkmcnt(0)\n"
         : [X] "+v"(st.X), [q] "+v"(st.q), [n1] "+v"(st.n1), [n2] "+v"(st.n2), [off] "+v"(off)
         : [L8] "s"(kRansL << 3), [B8] "s"(256u << 3), [obase] "s"(obase), [stride] "s"(stride), [npairs] "s"(npairs)
-        : CI_STEP_CLOBBERS, "scc", "s22", "v107");
+        : CI_STEP_CLOBBERS, "scc", "s22", "v83");
 }
 
 // Eight symbols of this lane's stream as bf16 weights: w[d] = rows 2d (low half) and 2d + 1 of the
@@ -452,7 +452,7 @@ __device__ __forceinline__ void decode8_weights_asm(FastLane &st, const uint32_t
                  : [L8] "s"(kRansL << 3), [B8] "s"(256u << 3), [selE] "s"(0x070C030Cu), [mask] "s"(0x807F807Fu),
                    [msel] "v"(man_sel), [m0] "v"(m[0]), [m1] "v"(m[1]), [m2] "v"(m[2]), [m3] "v"(m[3]), [m4] "v"(m[4]),
                    [m5] "v"(m[5]), [m6] "v"(m[6]), [m7] "v"(m[7])
-                 : CI_STEP_CLOBBERS, "v107", "v136", "v140", "v141", "v142", "v143");
+                 : CI_STEP_CLOBBERS, "v83", "v112", "v116", "v117", "v118", "v119");
 }
 
 // Advance the lane's stream by n >= 1 symbols; returns the table word (symbol in the top byte) of
@@ -463,12 +463,12 @@ __device__ __forceinline__ uint32_t advance_asm(FastLane &st, uint32_t n) {
     asm volatile(
         "s_mov_b32 s22, %[n]\n"
         "ci_adv_loop%=:\n"
-        CI_STEP_ISSUE("v[96:97]") CI_STEP_FINISH("v96", "v97")
+        CI_STEP_ISSUE("v[72:73]") CI_STEP_FINISH("v72", "v73")
         "s_sub_u32 s22, s22, 1\n"
         "s_cmp_lg_u32 s22, 0\n"
         "s_cbranch_scc1 ci_adv_loop%=\n"
         "s_waitcnt lgkmcnt(0)\n"
-        "v_mov_b32 %[e], v96\n"
+        "v_mov_b32 %[e], v72\n"
         : [X] "+v"(st.X), [q] "+v"(st.q), [n1] "+v"(st.n1), [n2] "+v"(st.n2), [e] "=&v"(e)
         : [L8] "s"(kRansL << 3), [B8] "s"(256u << 3), [n] "s"(n)
         : CI_STEP_CLOBBERS, "scc", "s22");
