@@ -15,8 +15,10 @@ from ._lib import check, lib, ptr
 
 
 class _Scratch:
-    """Grow-only fp32 scratch for split-K partials, one per device
-    (the reference keeps a class-level buffer too, comp_inference/pytorch_runtime.py:386-394)."""
+    """Grow-only scratch areas (split-K partials, decoded weights, sort keys), one per device and purpose
+    (the reference keeps a class-level buffer too, comp_inference/pytorch_runtime.py:386-394).  Calls that
+    follow each other on one stream share them safely; calls that run at the same time on different
+    streams of one device would overwrite each other's scratch -- pass `workspace=` of your own there."""
     _buf: dict = {}
 
     @classmethod
