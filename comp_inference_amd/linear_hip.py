@@ -133,6 +133,65 @@ def _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, met
     return result.view(*x.shape[:-1], N)
 
 
+class PreparedLinear:
+    """One compressed weight with everything a call needs converted once: device tensors, their
+    pointers, the checkpoint index, the workspace size per row count.  `RansLinear` keeps one per device; a
+    call then costs one output allocation and one library call instead of a dozen tensor conversions.
+    Same kernels, same results as `fused_rans_linear`."""
+
+    def __init__(self, dev, compressed_data, initial_states, tables, slot_map, weight_shape, tile_offsets,
+                 tile_max_lens, tile_k, tile_n, mantissas, bias=None, checkpoints=None, segments=1):
+        self.dev = dev
+        self.K, self.N = int(weight_shape[0]), int(weight_shape[1])
+        self.tile_k, self.tile_n = int(tile_k), int(tile_n)
+        man = _lib.as_u8(mantissas, dev).view(-1)
+        need_man = (-(-self.K // self.tile_k)) * (-(-self.N // self.tile_n)) * self.tile_k * self.tile_n
+        if man.numel() < need_man:
+            man = torch.nn.functional.pad(man, (0, need_man - man.numel()))
+        self.segments = int(segments) if checkpoints is not None else 1
+        ck = None
+        if self.segments > 1:
+            ck = checkpoints.to(dev).contiguous()
+            if ck.dtype != torch.int64 or \
+                    ck.numel() * 8 != lib().ci_checkpoint_bytes(self.K, self.N, self.tile_k, self.tile_n, self.segments):
+                raise RuntimeError("checkpoints do not belong to this weight shape, tiling and segment count")
+        # the tensors stay referenced here for as long as their pointers are in use
+        self.keep = (_lib.as_u8(compressed_data, dev), _lib.as_u32(initial_states, dev), _lib.as_u32(tables, dev),
+                     _lib.as_u8(slot_map, dev), _lib.as_u32(tile_offsets, dev), _lib.as_u32(tile_max_lens, dev), man,
+                     None if bias is None else bias.to(device=dev, dtype=torch.bfloat16).contiguous(), ck)
+        self.p = [ptr(t) for t in self.keep]
+        self.stream_len = C.c_uint64(self.keep[0].numel())
+        self.need = {}
+
+    def __call__(self, x: torch.Tensor) -> torch.Tensor:
+        if x.device != self.dev:
+            raise RuntimeError(f"x is on {x.device}, the prepared weight on {self.dev}")
+        x2 = _prep_x(x, self.K)
+        M = x2.shape[0]
+        if DECODE_ONCE_ABOVE_ROWS is not None and M > DECODE_ONCE_ABOVE_ROWS:
+            o = self.keep
+            return _run(x, o[0], o[1], o[2], o[3], (self.K, self.N), o[4], o[5], self.tile_k, self.tile_n, o[6],
+                        o[7], None, None, dense=False)
+        result = torch.empty((M, self.N), dtype=torch.bfloat16, device=self.dev)
+        need = self.need.get(M)
+        if need is None:
+            need = self.need[M] = lib().ci_fused_linear_workspace_bytes_segmented(M, self.K, self.N, self.tile_k,
+                                                                                   self.tile_n, 0, self.segments)
+        ws, ws_bytes = _pick_workspace(None, need, self.dev)
+        p = self.p
+        if self.segments > 1:
+            check(lib().ci_fused_linear_ilp2_segmented(
+                ptr(x2), M, self.K, self.N, x2.stride(0), p[0], self.stream_len, p[1], p[2], p[3], p[4], p[5], p[6],
+                self.tile_k, self.tile_n, p[8], self.segments, p[7], ptr(result), self.N, ptr(ws),
+                C.c_size_t(ws_bytes), _lib.stream_handle(self.dev)))
+        else:
+            check(lib().ci_fused_linear_ilp2(
+                ptr(x2), M, self.K, self.N, x2.stride(0), p[0], self.stream_len, p[1], p[2], p[3], p[4], p[5], p[6],
+                self.tile_k, self.tile_n, p[7], ptr(result), self.N, ptr(ws), C.c_size_t(ws_bytes),
+                _lib.stream_handle(self.dev)))
+        return result.view(*x.shape[:-1], self.N)
+
+
 def fused_rans_linear(x, compressed_data, initial_states, tables, slot_map, weight_shape, tile_offsets,
                       tile_max_lens, tile_k, tile_n, mantissas, accum_block_size=32, bias=None, out=None,
                       SPLIT_K=8, workspace=None, checkpoints=None, segments=1):

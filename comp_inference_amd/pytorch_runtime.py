@@ -12,7 +12,7 @@ import torch
 import torch.nn as nn
 
 from .embedding_hip import fused_rans_embedding
-from .linear_hip import fused_rans_linear
+from .linear_hip import PreparedLinear, fused_rans_linear
 from .rans_hip import build_checkpoints, suggest_segments
 from .transposed_linear_hip import fused_rans_linear_transposed
 
@@ -108,21 +108,19 @@ class RansLinear(nn.Module):
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         device = x.device
-        checkpoints, segments = self._checkpoints(device)
-        return fused_rans_linear(
-            x=x,
-            checkpoints=checkpoints, segments=segments,
-            compressed_data=self.rans_exp_stream.to(device, non_blocking=True),
-            initial_states=self.rans_exp_states.to(device, non_blocking=True),
-            tables=self.rans_exp_tables.to(device, non_blocking=True),
-            slot_map=self.rans_exp_slot_map.to(device, non_blocking=True),
-            weight_shape=(self.in_features, self.out_features),
-            tile_offsets=self.rans_exp_tile_offsets.to(device, non_blocking=True),
-            tile_max_lens=self.rans_exp_tile_max_lens.to(device, non_blocking=True),
-            tile_k=self.tile_k, tile_n=self.tile_n,
-            mantissas=self.rans_man_raw.to(device, non_blocking=True),
-            SPLIT_K=self.split_k,
-            bias=self.bias.to(device, non_blocking=True) if self.bias is not None else None)
+        prepared = getattr(self, "_prepared", None)
+        if prepared is None or prepared[0] is not self.rans_exp_stream or prepared[1] != device \
+                or prepared[2] is not self.bias or prepared[3] != self.segments:
+            from . import _lib
+
+            _lib.require_device(x)
+            checkpoints, segments = self._checkpoints(device)
+            call = PreparedLinear(device, self.rans_exp_stream, self.rans_exp_states, self.rans_exp_tables,
+                                  self.rans_exp_slot_map, (self.in_features, self.out_features),
+                                  self.rans_exp_tile_offsets, self.rans_exp_tile_max_lens, self.tile_k, self.tile_n,
+                                  self.rans_man_raw, self.bias, checkpoints, segments)
+            prepared = self._prepared = (self.rans_exp_stream, device, self.bias, self.segments, call)
+        return prepared[4](x)
 
 
 class RansLMHead(nn.Module):

@@ -214,3 +214,53 @@ def test_fused_qkv_and_gate_up_compression():
     assert torch.allclose(got.float(), want.float(), atol=1e-2, rtol=1e-2)
     ci.rans_decompress_module_weight(mlp.gate_proj)
     assert torch.equal(mlp.gate_proj.weight.detach().cpu().view(torch.int16), gu_w.t().contiguous().view(torch.int16))
+
+
+def test_rans_linear_prepares_once_and_follows_its_buffers():
+    """RansLinear converts its buffers once per device and then reuses the pointers: repeated calls, calls
+    with other row counts (also above the decode-once threshold), a module moved to the device, a replaced
+    bias and a changed segment count all give what the entry point gives on the same arguments."""
+    import comp_inference_amd as ci
+
+    torch.manual_seed(11)
+    K, N = 2048, 160
+    lin = nn.Linear(K, N, bias=True).to(torch.bfloat16)
+    bias = lin.bias.detach().clone()
+    ci.rans_compress_module_weight(lin)
+    rl = ci.RansLinear.from_compressed(lin, bias=bias)
+
+    def entry(x, b, segments):
+        ck = None
+        if segments > 1:
+            ck = ci.build_checkpoints(rl.rans_exp_stream.cuda(), rl.rans_exp_states.cuda(), rl.rans_exp_tables.cuda(),
+                                      rl.rans_exp_slot_map.cuda(), (K, N), rl.rans_exp_tile_offsets.cuda(),
+                                      rl.rans_exp_tile_max_lens.cuda(), rl.tile_k, rl.tile_n, segments)
+        return ci.fused_rans_linear_triton(
+            x=x, compressed_data=rl.rans_exp_stream.cuda(), initial_states=rl.rans_exp_states.cuda(),
+            tables=rl.rans_exp_tables.cuda(), slot_map=rl.rans_exp_slot_map.cuda(), weight_shape=(K, N),
+            tile_offsets=rl.rans_exp_tile_offsets.cuda(), tile_max_lens=rl.rans_exp_tile_max_lens.cuda(),
+            tile_k=rl.tile_k, tile_n=rl.tile_n, mantissas=rl.rans_man_raw.cuda(), bias=b.cuda(),
+            checkpoints=ck, segments=segments)
+
+    def same(a, b):
+        return torch.equal(a.view(torch.int16), b.view(torch.int16))
+
+    segs = rl._checkpoints(torch.device("cuda", 0))[1]
+    xs = {M: torch.randn(M, K).to(torch.bfloat16).cuda() for M in (1, 5, 64, 70)}
+    for M in (1, 5, 1, 64, 70, 5):                       # buffers on the host: device copies are kept
+        assert same(rl(xs[M]), entry(xs[M], bias, segs)), M
+    first = rl._prepared[4]
+    assert rl(xs[1][None]).shape == (1, 1, N) and rl._prepared[4] is first
+
+    rl = rl.cuda()                                       # the buffers are new tensors now
+    assert same(rl(xs[5]), entry(xs[5], bias, segs)) and rl._prepared[4] is not first
+    assert rl._prepared[4].keep[0].data_ptr() == rl.rans_exp_stream.data_ptr()      # no second copy
+
+    rl.bias = (bias.float() + 1).to(torch.bfloat16).cuda()
+    assert same(rl(xs[5]), entry(xs[5], rl.bias, segs))
+    rl.segments = 1 if segs > 1 else 2
+    assert same(rl(xs[5]), entry(xs[5], rl.bias, rl.segments))
+    with pytest.raises(RuntimeError):
+        rl(xs[5].cpu())
+    with pytest.raises(RuntimeError):
+        rl._prepared[4](xs[5].cpu())
