@@ -64,3 +64,4 @@ from .rans_saving import (
     rans_tensors_for_module,
     save_rans_model_package,
 )
+from .rans_gguf import save_rans_model_gguf

@@ -264,3 +264,82 @@ def test_rans_linear_prepares_once_and_follows_its_buffers():
         rl(xs[5].cpu())
     with pytest.raises(RuntimeError):
         rl._prepared[4](xs[5].cpu())
+
+
+def test_gguf_export_holds_the_weights(tmp_path):
+    """comp_inference/rans_gguf.py:111-238 stores states, sizes, freqs and cdf but neither tables nor tile
+    offsets: all of them follow from what is stored (tables = freq | cdf << 16, a tile's length = its longest
+    stream, offsets = running sum).  Rebuilt that way from the file alone, every weight decodes to its
+    original bits."""
+    import sys
+    import types
+
+    sys.path.insert(0, os.path.dirname(__file__))
+    from gguf_parse import parse_gguf
+
+    import comp_inference_amd as ci
+    from comp_inference_amd.rans_gguf import save_rans_model_gguf
+
+    class Block(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.mlp = nn.Module()
+            self.mlp.up_proj = nn.Linear(1100, 200, bias=True)
+            self.mlp.down_proj = nn.Linear(200, 1100, bias=False)
+
+    class Net(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.model = nn.Module()
+            self.model.embed_tokens = nn.Embedding(1300, 96)
+            self.model.layers = nn.ModuleList([Block()])
+            self.config = types.SimpleNamespace(num_hidden_layers=1, hidden_size=96, intermediate_size=200,
+                                                num_attention_heads=4)
+
+    torch.manual_seed(21)
+    net = Net().to(torch.bfloat16)
+    up, down, emb = net.model.layers[0].mlp.up_proj, net.model.layers[0].mlp.down_proj, net.model.embed_tokens
+    want = {"blk.0.ffn_up": up.weight.detach().t().contiguous(), "blk.0.ffn_down": down.weight.detach().t().contiguous(),
+            "token_embd": emb.weight.detach().clone()}
+    ci.rans_compress_module_weight(up)
+    ci.rans_compress_module_weight(down, tile_height=64, tile_width=32)
+    ci.rans_compress_module_weight(emb, transpose_weight=False)
+    tiles = {"blk.0.ffn_up": (1024, 32), "blk.0.ffn_down": (64, 32), "token_embd": (1024, 32)}
+
+    class Tok:
+        bos_token_id = eos_token_id = pad_token_id = None
+        all_special_ids = []
+        backend_tokenizer = types.SimpleNamespace(model=types.SimpleNamespace(get_merges=lambda: ["a b"]))
+
+        def get_vocab(self):
+            return {"a": 0, "b": 1, "ab": 2}
+
+    path = tmp_path / "net.gguf"
+    save_rans_model_gguf(net, Tok(), str(path))
+    _, _, tensors, _, _ = parse_gguf(path)
+
+    def u(name, dtype):
+        return torch.from_numpy(tensors[name][0].copy()).view(dtype)
+
+    for base, w in want.items():
+        info = tensors[f"{base}.rans_info"][0].tolist()
+        K, N = info[7:9]
+        th, tw = tiles[base]
+        assert info[:7] == [1, K * N, 1, -(-K // th) * -(-N // tw) * 2 * tw, 0, 0, 2] and (K, N) == tuple(w.shape)
+        freqs, cdf = u(f"{base}.rans_exp_freqs", torch.uint16), u(f"{base}.rans_exp_cdf", torch.uint16)
+        f64, c64 = freqs.to(torch.int64), cdf.to(torch.int64)
+        tables = (f64 | (c64 << 16)).to(torch.uint32)
+        slot_map = torch.repeat_interleave(torch.arange(256), f64).to(torch.uint8)
+        assert slot_map.numel() == 4096
+        sizes = u(f"{base}.rans_exp_sizes", torch.uint32).to(torch.int64).view(-1, 2 * tw)
+        max_lens = sizes.max(dim=1).values
+        offsets = torch.cumsum(max_lens * 2 * tw, 0) - max_lens * 2 * tw
+        stream = u(f"{base}.rans_exp_stream", torch.uint8)
+        assert stream.numel() == int((max_lens * 2 * tw).sum())
+        exp = ci.rans_decomp_triton_tiled(stream.cuda(), u(f"{base}.rans_exp_states", torch.uint32).cuda(),
+                                          tables.cuda(), slot_map.cuda(), (K, N), offsets.to(torch.uint32).cuda(),
+                                          max_lens.to(torch.uint32).cuda(), tile_k=th, tile_n=tw)
+        man = ci.uninterleave_mantissas(u(f"{base}.rans_man_raw", torch.uint8), K, N, TILE_K=th, TILE_N=tw)
+        got = ci.reconstruct_from_exp_and_mantissa(exp.cpu(), man)
+        assert torch.equal(got.view(torch.int16), w.view(torch.int16)), base
+    assert torch.equal(u("blk.0.ffn_up.bias", torch.float32), up.bias.detach().float())
