@@ -159,9 +159,23 @@ class PreparedLinear:
         self.keep = (_lib.as_u8(compressed_data, dev), _lib.as_u32(initial_states, dev), _lib.as_u32(tables, dev),
                      _lib.as_u8(slot_map, dev), _lib.as_u32(tile_offsets, dev), _lib.as_u32(tile_max_lens, dev), man,
                      None if bias is None else bias.to(device=dev, dtype=torch.bfloat16).contiguous(), ck)
+        self.need = {}
+        self._bind()
+
+    def _bind(self) -> None:
         self.p = [ptr(t) for t in self.keep]
         self.stream_len = C.c_uint64(self.keep[0].numel())
-        self.need = {}
+
+    # A copy (copy.deepcopy of the owning module, pickling) gets its own tensors: the pointers are taken
+    # again from them instead of travelling as numbers.
+    def __getstate__(self):
+        state = dict(self.__dict__)
+        del state["p"], state["stream_len"]
+        return state
+
+    def __setstate__(self, state):
+        self.__dict__.update(state)
+        self._bind()
 
     def __call__(self, x: torch.Tensor) -> torch.Tensor:
         if x.device != self.dev:

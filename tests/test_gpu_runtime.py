@@ -265,6 +265,16 @@ def test_rans_linear_prepares_once_and_follows_its_buffers():
     with pytest.raises(RuntimeError):
         rl._prepared[4](xs[5].cpu())
 
+    import copy                                          # a copy of the module points at its own tensors
+    want = rl(xs[5])
+    twin = copy.deepcopy(rl)
+    call = twin._prepared[4]
+    assert call is not rl._prepared[4] and call.keep[0] is twin.rans_exp_stream
+    assert call.keep[0].data_ptr() != rl.rans_exp_stream.data_ptr()
+    assert call.p[0].value == call.keep[0].data_ptr() and call.p[6].value == call.keep[6].data_ptr()
+    del rl
+    assert same(twin(xs[5]), want)
+
 
 def test_gguf_export_holds_the_weights(tmp_path):
     """comp_inference/rans_gguf.py:111-238 stores states, sizes, freqs and cdf but neither tables nor tile
