@@ -281,10 +281,8 @@ def test_gguf_export_holds_the_weights(tmp_path):
     offsets: all of them follow from what is stored (tables = freq | cdf << 16, a tile's length = its longest
     stream, offsets = running sum).  Rebuilt that way from the file alone, every weight decodes to its
     original bits."""
-    import sys
     import types
 
-    sys.path.insert(0, os.path.dirname(__file__))
     from gguf_parse import parse_gguf
 
     import comp_inference_amd as ci
