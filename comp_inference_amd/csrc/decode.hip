@@ -24,6 +24,10 @@ struct DecodeArgs {
     const uint8_t *man_tiled;
     uint16_t *out_bf16;
     uint32_t man_aligned;  // sign|mantissa plane may be read as dwords
+    // Decoder checkpoints (see checkpoints_kernel): with segs > 1 every stream is cut into segs segments
+    // that are decoded as work items of their own.
+    const uint2 *ckpt;
+    uint32_t segs;
 };
 
 // Work item of the 32-column kernels: one half (top or bottom rows) of two neighbouring column
@@ -31,20 +35,25 @@ struct DecodeArgs {
 // (tk, 2p + 1), so every decoded row leaves the wavefront as 64 contiguous bytes (128 as bf16).  With
 // both halves of ONE tile per wavefront every row is a 32-byte piece of a 128-byte line, and the
 // memory side of those partial writes cost a fifth of the kernel's time.
-// item = (tk * pairs + p) * 2 + half.
+// item = ((tk * pairs + p) * segs + segment) * 2 + half.
+//
+// With decoder checkpoints an item is one segment of those streams: it starts from the recorded state
+// and byte position, stages only the rows of the two bodies its lanes can touch (from the lowest row any
+// lane reaches by the segment's end to the highest any lane starts at) and decodes th / (2 segs) rows.
 //
 // kMerge = false writes the exponent plane; kMerge = true joins it with the tiles' sign|mantissa
 // bytes and writes bf16.  Items that do not qualify for the hand-scheduled loop (ragged, odd block
-// counts, a body deeper than a lane stride) take the same arithmetic with guarded byte reads from
+// counts, a window deeper than a lane stride) take the same arithmetic with guarded byte reads from
 // global memory.
 template <uint32_t kStride, bool kMerge>
 __device__ __forceinline__ void decode_one_item(const DecodeArgs &a, uint32_t item, const uint2 *tab,
                                                 uint8_t *stage, int lane) {
     const uint32_t pairs = (a.tiles_n + 1) / 2;
-    const uint32_t hsel = item & 1u, p = (item >> 1) % pairs, tk = (item >> 1) / pairs;
-    const uint32_t half = a.th / 2, side = lane / 32, c = lane % 32;
-    const uint32_t tn = 2 * p + side, col = tn * 32 + c, row_first = tk * a.th + hsel * half;
-    if (row_first >= a.K) return;  // the bottom half of a short last tile row
+    const uint32_t hsel = item & 1u, seg = (item >> 1) % a.segs, pr = (item >> 1) / a.segs;
+    const uint32_t p = pr % pairs, tk = pr / pairs;
+    const uint32_t half = a.th / 2, seglen = half / a.segs, side = lane / 32, c = lane % 32;
+    const uint32_t tn = 2 * p + side, col = tn * 32 + c, row_first = tk * a.th + hsel * half + seg * seglen;
+    if (row_first >= a.K) return;  // past the end of a short last tile row
     const bool have_b = 2 * p + 1 < a.tiles_n;
     const uint32_t tile_a = tk * a.tiles_n + 2 * p, tile_b = have_b ? tile_a + 1 : tile_a;
     uint64_t base_a = a.tile_offsets[tile_a], base_b = a.tile_offsets[tile_b];
@@ -56,31 +65,51 @@ __device__ __forceinline__ void decode_one_item(const DecodeArgs &a, uint32_t it
     const uint64_t base = side ? base_b : base_a;
     const uint32_t q = hsel * 32 + c;  // this lane's stream inside its tile
     const bool col_ok = tn < a.tiles_n && col < a.N;
-    const uint32_t state = a.states[(size_t)tile * 64 + q];
-    const uint32_t steps = min(half, a.K - row_first);  // the same for every lane
-    const bool fast = __builtin_amdgcn_ballot_w64(!col_ok) == 0 && steps == half && depth_a >= 2 && depth_b >= 2 &&
-                      depth_a < kStride && depth_b < kStride && half % (kMerge ? 8 : 2) == 0 && half >= 2 &&
+    // decoder state and row of the next unread byte at the segment's first row, and the row the stream
+    // has reached at the segment's end
+    uint32_t state;
+    int32_t row = (int32_t)depth - 1, row_end = -1;
+    {
+        const uint2 *ck = a.ckpt + ((size_t)tile * (a.segs - 1)) * 64 + q;  // (only read when segs > 1)
+        if (seg == 0) {
+            state = a.states[(size_t)tile * 64 + q];
+        } else {
+            const uint2 v = ck[(size_t)(seg - 1) * 64];
+            state = v.x;
+            row = min((int32_t)v.y, (int32_t)depth - 1);
+        }
+        if (seg + 1 < a.segs) row_end = min((int32_t)ck[(size_t)seg * 64].y, row);
+    }
+    const uint32_t steps = min(seglen, a.K - row_first);  // the same for every lane
+    // rows of the two bodies this item can touch (one window for both: neighbouring tiles lie alike)
+    const int32_t w_lo = max(wave_min_i32(row_end) - 1, 0), w_hi = wave_max_i32(row);
+    const uint32_t win_a = (uint32_t)max(min(w_hi + 1, (int32_t)depth_a) - w_lo, 0),
+                   win_b = (uint32_t)max(min(w_hi + 1, (int32_t)depth_b) - w_lo, 0);
+    const bool fast = __builtin_amdgcn_ballot_w64(!col_ok) == 0 && steps == seglen && win_a >= 2 && win_b >= 2 &&
+                      win_a < kStride && win_b < kStride && seglen % (kMerge ? 8 : 2) == 0 && seglen >= 2 &&
                       (uint64_t)a.K * a.N < (1ull << (kMerge ? 31 : 32)) && (uint32_t)(uintptr_t)tab == 0 &&
                       (!kMerge || a.man_aligned);
-    const uint8_t *man_half = kMerge ? a.man_tiled + (size_t)tile * a.th * 32 + (size_t)hsel * half * 32 : nullptr;
+    const uint8_t *man_seg =
+        kMerge ? a.man_tiled + (size_t)tile * a.th * 32 + (size_t)(hsel * half + seg * seglen) * 32 : nullptr;
     if (fast) {
         StageRegs body;
-        const uint32_t deepest = max(depth_a, depth_b), my_depth = (lane & 4) ? depth_b : depth_a;
+        const uint32_t deepest = max(win_a, win_b), my_depth = (lane & 4) ? win_b : win_a;
+        const uint8_t *src_a = a.stream + base_a + (size_t)w_lo * 64, *src_b = a.stream + base_b + (size_t)w_lo * 64;
 #pragma unroll
         for (int grp = 0; grp < stage_groups(kStride); ++grp)
             if ((uint32_t)grp * 128 < deepest) {
-                stage_fetch_pair(body, a.stream + base_a, depth_a, a.stream + base_b, depth_b, hsel, grp * 128, lane);
+                stage_fetch_pair(body, src_a, win_a, src_b, win_b, hsel, grp * 128, lane);
                 stage_commit<kStride>(body, stage, grp * 128, my_depth, lane);
             }
         // LDS operations of one wavefront complete in order: the reads below see the writes above
         FastLane st;
-        st.init<kStride>(stage, depth, lane, state);
+        st.init_at<kStride>(stage, row - w_lo + 1, lane, state);
         if (kMerge) {
             // blocks of eight rows: sign|mantissa dwords of the next block are loaded while this one decodes
             const uint32_t man_sel = 0x04040000u + (c & 3u) * 0x01010101u;
-            const uint32_t *mrow = reinterpret_cast<const uint32_t *>(man_half + (c & ~3u));  // + 8 dwords per row
+            const uint32_t *mrow = reinterpret_cast<const uint32_t *>(man_seg + (c & ~3u));  // + 8 dwords per row
             uint16_t *o = a.out_bf16 + (size_t)row_first * a.N + col;
-            const uint32_t nblk = half / 8;
+            const uint32_t nblk = seglen / 8;
             uint32_t mcur[8], mnext[8];
 #pragma unroll
             for (int r = 0; r < 8; ++r) mcur[r] = mrow[r * 8];
@@ -103,11 +132,11 @@ __device__ __forceinline__ void decode_one_item(const DecodeArgs &a, uint32_t it
             // readfirstlane returns a signed int: widen through uint32_t
             const uint32_t ob_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(ob >> 32));
             const uint32_t ob_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)ob);
-            decode_tile_asm(st, ((uint64_t)ob_hi << 32) | (uint64_t)ob_lo, lane, a.N, half / 2);
+            decode_tile_asm(st, ((uint64_t)ob_hi << 32) | (uint64_t)ob_lo, lane, a.N, seglen / 2);
         }
     } else if (col_ok) {
         GlobalBytes src;
-        src.init(a.stream + base, depth, 64, q);
+        src.init(a.stream + base, (uint32_t)(row + 1), 64, q);
         uint32_t X = state << 3;
         const size_t o0 = (size_t)row_first * a.N + col;
         for (uint32_t i = 0; i < steps; ++i) {
@@ -115,7 +144,7 @@ __device__ __forceinline__ void decode_one_item(const DecodeArgs &a, uint32_t it
             src.renorm_scaled(X);
             src.renorm_scaled(X);
             if (kMerge)
-                a.out_bf16[o0 + (size_t)i * a.N] = (uint16_t)assemble_bf16(sym, man_half[(size_t)i * 32 + c]);
+                a.out_bf16[o0 + (size_t)i * a.N] = (uint16_t)assemble_bf16(sym, man_seg[(size_t)i * 32 + c]);
             else
                 a.out_exp[o0 + (size_t)i * a.N] = (uint8_t)sym;
         }
@@ -126,20 +155,20 @@ __device__ __forceinline__ uint64_t decode_num_pairs(const DecodeArgs &a) {
     return (uint64_t)(a.num_tiles / a.tiles_n) * ((a.tiles_n + 1) / 2);
 }
 
-// Workgroup `j` (of the `n_wg` that share this tensor) takes the tile pairs j, j + n_wg, ...; its
-// wavefronts take the workgroup's items in turn (slot = wave, wave + kWaves, ...; slot / 2 picks the
-// pair, slot % 2 the half), so the two halves of a pair are staged on the same CU at about the same
-// time and the second reader of a body row finds it in that CU's cache.
+// Workgroup `j` (of the `n_wg` that share this tensor) takes the units j, j + n_wg, ... (a unit = a tile
+// pair, or one segment of it); its wavefronts take the workgroup's items in turn (slot = wave,
+// wave + kWaves, ...; slot / 2 picks the unit, slot % 2 the half), so the two halves of a unit are staged
+// on the same CU at about the same time and the second reader of a body row finds it in that CU's cache.
 template <int kWaves, uint32_t kStride, bool kMerge>
 __device__ __forceinline__ void decode_wave_tiles(const DecodeArgs &a, uint32_t j, uint32_t n_wg, const uint2 *tab,
                                                   uint8_t *lds, int wave, int lane) {
     if (wave >= kWaves) return;
     uint8_t *stage = persist_stage<kWaves, kStride>(lds, wave);
-    const uint64_t n_pairs = decode_num_pairs(a);
+    const uint64_t n_units = decode_num_pairs(a) * a.segs;  // unit = one segment of a pair, both halves
     for (uint32_t slot = wave;; slot += kWaves) {
-        const uint64_t pair = (uint64_t)(slot >> 1) * n_wg + j;
-        if (pair >= n_pairs) break;
-        decode_one_item<kStride, kMerge>(a, (uint32_t)pair * 2 + (slot & 1u), tab, stage, lane);
+        const uint64_t unit = (uint64_t)(slot >> 1) * n_wg + j;
+        if (unit >= n_units) break;
+        decode_one_item<kStride, kMerge>(a, (uint32_t)unit * 2 + (slot & 1u), tab, stage, lane);
     }
 }
 
@@ -165,7 +194,12 @@ __global__ __launch_bounds__(kPersistWaves *kWave) void decode_tiled32_persist_k
     const uint32_t j = blockIdx.x - b.first_block[i], n_wg = b.first_block[i + 1] - b.first_block[i];
 
     uint32_t deepest = 0;
-    {
+    if (a.segs > 1) {
+        // a segment's window is about its share of the body plus the spread between the lanes; an item whose
+        // window turns out larger than the class allows takes the guarded path
+        for (uint32_t t = tid; t < a.num_tiles; t += kPersistWaves * kWave) deepest = max(deepest, a.tile_max_lens[t]);
+        deepest = deepest / a.segs + 40;
+    } else {
         const uint32_t pairs = (a.tiles_n + 1) / 2;
         const uint64_t n_pairs = decode_num_pairs(a);
         for (uint64_t pr = (uint64_t)tid * n_wg + j; pr < n_pairs; pr += (uint64_t)kPersistWaves * kWave * n_wg) {
@@ -306,16 +340,26 @@ extern "C" int ci_build_checkpoints_ilp2(const uint8_t *d_stream, uint64_t strea
     return CI_OK;
 }
 
+// Segmented decode: 32-column tiles whose half height splits into `segments` runs of whole 16-row blocks.
+static int check_segments(const char *who, uint32_t tile_height, uint32_t segments, const void *d_checkpoints) {
+    if (tile_height % 2 || (tile_height / 2) % (16 * segments))
+        return fail(CI_ERR_ARG, "%s: %u segments need a tile half height that is a multiple of %u", who, segments,
+                    16 * segments);
+    if (!d_checkpoints || !aligned(d_checkpoints, 8))
+        return fail(CI_ERR_ARG, "%s: segments without (8-byte aligned) checkpoints", who);
+    return CI_OK;
+}
+
 // Launch the persistent kernel over the (already checked) tensors of `b`: the device's CUs are
 // divided among the tensors in proportion to their tile counts.
 static int launch_persist(DecodeBatchArgs &b, bool merge, hipStream_t s) {
     uint32_t cus = 0;
     if (int rc = cu_count(&cus)) return rc;
-    // The unit handed to a workgroup is a pair of neighbouring column tiles.
+    // The unit handed to a workgroup is a pair of neighbouring column tiles, or one segment of it.
     uint64_t pairs[kDecBatchMax], total = 0;
     for (uint32_t i = 0; i < b.n; ++i) {
         const DecodeArgs &a = b.item[i];
-        pairs[i] = (uint64_t)(a.num_tiles / a.tiles_n) * ((a.tiles_n + 1) / 2);
+        pairs[i] = (uint64_t)(a.num_tiles / a.tiles_n) * ((a.tiles_n + 1) / 2) * a.segs;
         total += pairs[i];
     }
     // Never more workgroups than CUs (one is resident per CU; a workgroup too many would run alone
@@ -395,6 +439,14 @@ extern "C" int ci_decode_tiled_ilp2_batch(const ci_decode_item *h_items, uint32_
             a.man_tiled = nullptr;
             a.out_bf16 = nullptr;
             a.man_aligned = 0;
+            a.ckpt = nullptr;
+            a.segs = 1;
+            if (it.segments > 1) {
+                if (int rc = check_segments("ci_decode_tiled_ilp2_batch", it.tile_height, it.segments, it.d_checkpoints))
+                    return rc;
+                a.ckpt = static_cast<const uint2 *>(it.d_checkpoints);
+                a.segs = it.segments;
+            }
             ++b.n;
         }
         if (b.n == 0) continue;
@@ -410,6 +462,19 @@ extern "C" int ci_decode_tiled_ilp2(const uint8_t *d_stream, uint64_t stream_len
                                     uint32_t tile_height, uint32_t tile_width, uint8_t *d_out_exp,
                                     const uint8_t *d_man_tiled, uint16_t *d_out_bf16,
                                     ci_stream_t stream) {
+    return ci_decode_tiled_ilp2_segmented(d_stream, stream_len, d_states, d_tables, d_slot_map, d_tile_offsets,
+                                          d_tile_max_lens, K, N, tile_height, tile_width, nullptr, 1, d_out_exp,
+                                          d_man_tiled, d_out_bf16, stream);
+}
+
+extern "C" int ci_decode_tiled_ilp2_segmented(const uint8_t *d_stream, uint64_t stream_len,
+                                              const uint32_t *d_states, const uint32_t *d_tables,
+                                              const uint8_t *d_slot_map, const uint32_t *d_tile_offsets,
+                                              const uint32_t *d_tile_max_lens, uint32_t K, uint32_t N,
+                                              uint32_t tile_height, uint32_t tile_width,
+                                              const void *d_checkpoints, uint32_t segments, uint8_t *d_out_exp,
+                                              const uint8_t *d_man_tiled, uint16_t *d_out_bf16,
+                                              ci_stream_t stream) {
     if (K == 0 || N == 0) return CI_OK;
     if (!d_states || !d_tables || !d_slot_map || !d_tile_offsets || !d_tile_max_lens)
         return fail(CI_ERR_ARG, "ci_decode_tiled_ilp2: null table or metadata pointer");
@@ -441,6 +506,13 @@ extern "C" int ci_decode_tiled_ilp2(const uint8_t *d_stream, uint64_t stream_len
     hipStream_t s = static_cast<hipStream_t>(stream);
 
     a.man_aligned = merge && aligned(d_man_tiled, 4) ? 1u : 0u;
+    a.ckpt = nullptr;
+    a.segs = 1;
+    if (segments > 1 && tile_width == 32) {  // (other widths decode one thread per stream: nothing to split)
+        if (int rc = check_segments("ci_decode_tiled_ilp2_segmented", tile_height, segments, d_checkpoints)) return rc;
+        a.ckpt = static_cast<const uint2 *>(d_checkpoints);
+        a.segs = segments;
+    }
     if (tile_width == 32 && aligned(d_stream, 16)) {
         DecodeBatchArgs b;
         b.n = 1;

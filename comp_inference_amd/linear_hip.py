@@ -44,15 +44,18 @@ DECODE_ONCE_ABOVE_ROWS = 64
 
 
 def _decode_once_weight(dev, compressed_data, initial_states, tables, slot_map, shape, tile_offsets, tile_max_lens,
-                        tile_k, tile_n, mantissas, tag):
-    """The bf16 weight, decoded into a grow-only scratch of its own (valid until the next such call)."""
+                        tile_k, tile_n, mantissas, tag, checkpoints=None, segments=1):
+    """The bf16 weight, decoded into a grow-only scratch of its own (valid until the next such call).  With
+    the weight's decoder checkpoints the segments of a stream are decoded side by side (a 4096 x 4096
+    weight: 53 -> 30 us)."""
     from .rans_hip import rans_decomp_tiled
 
     rows, cols = shape
     buf = _Scratch.get(rows * cols * 2, (tag, dev))
     w = buf[:rows * cols * 2].view(torch.bfloat16).view(rows, cols)
     return rans_decomp_tiled(compressed_data, initial_states, tables, slot_map, (rows, cols), tile_offsets,
-                             tile_max_lens, tile_k=tile_k, tile_n=tile_n, mantissas=mantissas, out=w)
+                             tile_max_lens, tile_k=tile_k, tile_n=tile_n, mantissas=mantissas, out=w,
+                             checkpoints=checkpoints, segments=segments)
 
 
 def _prep_x(x: torch.Tensor, K: int):
@@ -93,7 +96,7 @@ def _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, met
             raise RuntimeError("out must have unit stride in its last dimension")
     if not dense and DECODE_ONCE_ABOVE_ROWS is not None and M > DECODE_ONCE_ABOVE_ROWS:
         w = _decode_once_weight(dev, compressed_data, initial_states, tables, slot_map, (K, N), meta0, meta1,
-                                int(tile_k), int(tile_n), mantissas, "weight_kn")
+                                int(tile_k), int(tile_n), mantissas, "weight_kn", checkpoints, segments)
         if result.is_contiguous():
             torch.matmul(x2.detach(), w, out=result)  # (like the fused kernels: inference only)
         else:
@@ -185,7 +188,7 @@ class PreparedLinear:
         if DECODE_ONCE_ABOVE_ROWS is not None and M > DECODE_ONCE_ABOVE_ROWS:
             o = self.keep
             return _run(x, o[0], o[1], o[2], o[3], (self.K, self.N), o[4], o[5], self.tile_k, self.tile_n, o[6],
-                        o[7], None, None, dense=False)
+                        o[7], None, None, dense=False, checkpoints=o[8], segments=self.segments)
         result = torch.empty((M, self.N), dtype=torch.bfloat16, device=self.dev)
         need = self.need.get(M)
         if need is None:

@@ -18,12 +18,26 @@ def _tiles(K: int, N: int, tile_k: int, tile_n: int):
     return (N + tile_n - 1) // tile_n, (K + tile_k - 1) // tile_k
 
 
+def _checked_checkpoints(checkpoints, segments, K, N, tile_k, tile_n, dev):
+    """-> (device tensor or None, segment count) for the segmented entry points."""
+    segments = int(segments) if checkpoints is not None else 1
+    if segments <= 1:
+        return None, 1
+    ck = checkpoints.to(dev).contiguous()
+    if ck.dtype != torch.int64 or ck.numel() * 8 != lib().ci_checkpoint_bytes(K, N, int(tile_k), int(tile_n), segments):
+        raise RuntimeError("checkpoints do not belong to this shape, tiling and segment count")
+    return ck, segments
+
+
 def rans_decomp_tiled(compressed_streams, initial_states, tables, slot_map, output_shape,
-                      tile_offsets, tile_max_lens, tile_k=1024, tile_n=32, mantissas=None, out=None):
+                      tile_offsets, tile_max_lens, tile_k=1024, tile_n=32, mantissas=None, out=None,
+                      checkpoints=None, segments=1):
     """Decode the tiled two-streams-per-column format into the exponent plane u8[K,N]
     (comp_inference/rans_triton.py:122-168).  With `mantissas` (the tile-interleaved sign|mantissa
     plane) the bf16 weight [K,N] is returned instead, merged in the same kernel.  `out`: a contiguous
-    GPU tensor of that shape and dtype to decode into (not in the reference's signature)."""
+    GPU tensor of that shape and dtype to decode into (not in the reference's signature).
+    `checkpoints`, `segments` (not in the reference either): the index made by `build_checkpoints`; the
+    segments of every stream are then decoded side by side -- same bytes out, a shorter chain of steps."""
     K, N = int(output_shape[0]), int(output_shape[1])
     num_tiles_n, num_tiles_k = _tiles(K, N, tile_k, tile_n)
     expected_streams = num_tiles_n * num_tiles_k * tile_n * 2
@@ -49,9 +63,10 @@ def rans_decomp_tiled(compressed_streams, initial_states, tables, slot_map, outp
     # device copies must stay referenced until the launch has been enqueued
     st, tb, sm = _lib.as_u32(initial_states, dev), _lib.as_u32(tables, dev), _lib.as_u8(slot_map, dev)
     to, tl = _lib.as_u32(tile_offsets, dev), _lib.as_u32(tile_max_lens, dev)
-    check(lib().ci_decode_tiled_ilp2(
+    ck, segments = _checked_checkpoints(checkpoints, segments, K, N, tile_k, tile_n, dev)
+    check(lib().ci_decode_tiled_ilp2_segmented(
         ptr(stream_t), C.c_uint64(stream_t.numel()), ptr(st), ptr(tb), ptr(sm), ptr(to), ptr(tl),
-        K, N, int(tile_k), int(tile_n), None if merge else ptr(out), ptr(man) if merge else None,
+        K, N, int(tile_k), int(tile_n), ptr(ck), segments, None if merge else ptr(out), ptr(man) if merge else None,
         ptr(out) if merge else None, _lib.stream_handle(dev)))
     return out
 
@@ -91,15 +106,17 @@ class _DecodeItem(C.Structure):
     _fields_ = [("d_stream", C.c_void_p), ("stream_len", C.c_uint64), ("d_states", C.c_void_p),
                 ("d_tables", C.c_void_p), ("d_slot_map", C.c_void_p), ("d_tile_offsets", C.c_void_p),
                 ("d_tile_max_lens", C.c_void_p), ("K", C.c_uint32), ("N", C.c_uint32),
-                ("tile_height", C.c_uint32), ("tile_width", C.c_uint32), ("d_out_exp", C.c_void_p)]
+                ("tile_height", C.c_uint32), ("tile_width", C.c_uint32), ("d_out_exp", C.c_void_p),
+                ("d_checkpoints", C.c_void_p), ("segments", C.c_uint32)]
 
 
 def rans_decomp_tiled_batch(items, tile_k=1024, tile_n=32):
     """Decode several tensors with one launch.  `items` is a sequence of tuples
     (compressed_streams, initial_states, tables, slot_map, output_shape, tile_offsets, tile_max_lens)
-    -- the positional arguments of rans_decomp_tiled -- all on the same GPU; returns the list of
-    exponent planes.  A stand-alone decode takes tile_k / 2 dependent steps per wavefront whatever
-    the tensor's size, so decoding a layer's tensors together keeps the whole chip busy."""
+    -- the positional arguments of rans_decomp_tiled, optionally followed by (checkpoints, segments) --
+    all on the same GPU; returns the list of exponent planes.  A stand-alone decode takes tile_k / 2
+    dependent steps per wavefront whatever the tensor's size, so decoding a layer's tensors together
+    keeps the whole chip busy."""
     items = list(items)
     if not items:
         return []
@@ -107,19 +124,21 @@ def rans_decomp_tiled_batch(items, tile_k=1024, tile_n=32):
     dev = items[0][0].device
     arr = (_DecodeItem * len(items))()
     keep, outs = [], []
-    for i, (cs, st, tb, sm, shape, to, tl) in enumerate(items):
+    for i, item in enumerate(items):
+        cs, st, tb, sm, shape, to, tl = item[:7]
         K, N = int(shape[0]), int(shape[1])
+        ck, segs = _checked_checkpoints(*(item[7:9] if len(item) >= 9 else (None, 1)), K, N, tile_k, tile_n, dev)
         expected = (-(-N // tile_n)) * (-(-K // tile_k)) * tile_n * 2
         if st.numel() != expected:
             raise ValueError(f"Initial states size mismatch. Expected {expected}")
         t = (_lib.as_u8(cs, dev), _lib.as_u32(st, dev), _lib.as_u32(tb, dev), _lib.as_u8(sm, dev),
              _lib.as_u32(to, dev), _lib.as_u32(tl, dev))
         out = torch.empty((K, N), device=dev, dtype=torch.uint8)
-        keep.append(t)
+        keep.append((t, ck))
         outs.append(out)
         arr[i] = _DecodeItem(t[0].data_ptr() if t[0].numel() else None, t[0].numel(), t[1].data_ptr(),
                              t[2].data_ptr(), t[3].data_ptr(), t[4].data_ptr(), t[5].data_ptr(), K, N,
-                             int(tile_k), int(tile_n), out.data_ptr())
+                             int(tile_k), int(tile_n), out.data_ptr(), None if ck is None else ck.data_ptr(), segs)
     check(lib().ci_decode_tiled_ilp2_batch(arr, len(items), _lib.stream_handle(dev)))
     return outs
 

@@ -288,6 +288,8 @@ typedef struct ci_decode_item {
     const uint32_t *d_tile_max_lens;
     uint32_t K, N, tile_height, tile_width;
     uint8_t *d_out_exp;
+    const void *d_checkpoints; /* NULL, or the index made by ci_build_checkpoints_ilp2 for `segments` */
+    uint32_t segments;         /* 0 or 1: whole streams */
 } ci_decode_item;
 
 int ci_decode_tiled_ilp2_batch(const ci_decode_item *h_items, uint32_t n_items, ci_stream_t stream);
@@ -341,6 +343,18 @@ int ci_fused_embedding_ilp2_segmented(const int64_t *d_ids, uint32_t n_ids, cons
                                       const void *d_checkpoints, uint32_t segments, uint16_t *d_out,
                                       uint32_t out_stride, void *d_workspace, size_t workspace_bytes,
                                       ci_stream_t stream);
+
+/* The stand-alone decode with decoder checkpoints (tile_width 32, tile_height / 2 a multiple of
+ * 16 * segments): every segment of every stream is a work item of its own, so a tensor with few tiles
+ * is no longer a chain of tile_height / 2 steps per wavefront, and a batch of tensors ends on short
+ * items instead of long ones.  Same output as ci_decode_tiled_ilp2, byte for byte.  Other tile widths
+ * ignore the checkpoints.  In a batch, set d_checkpoints / segments per item (ci_decode_item). */
+int ci_decode_tiled_ilp2_segmented(const uint8_t *d_stream, uint64_t stream_len, const uint32_t *d_states,
+                                   const uint32_t *d_tables, const uint8_t *d_slot_map,
+                                   const uint32_t *d_tile_offsets, const uint32_t *d_tile_max_lens, uint32_t K,
+                                   uint32_t N, uint32_t tile_height, uint32_t tile_width,
+                                   const void *d_checkpoints, uint32_t segments, uint8_t *d_out_exp,
+                                   const uint8_t *d_man_tiled, uint16_t *d_out_bf16, ci_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------
  * Verification aids: the contraction of the fused kernels applied to a plain (uncompressed) bf16

@@ -297,3 +297,51 @@ def test_encoder_random_shapes(oracle):
         assert np.array_equal(_np32(got.tile_max_lens), ref.tile_max_lens), (case, K, N, th, tw)
         assert np.array_equal(got.stream.numpy(), ref.stream), (case, K, N, th, tw)
     assert overflowed < 10
+
+
+@pytest.mark.parametrize("K,N,th", [(4096, 256, 1024), (1300, 80, 1024), (2048, 96, 256), (1024, 33, 1024), (700, 64, 64)])
+def test_segmented_decode_is_the_same_decode(oracle, K, N, th):
+    """Decoder checkpoints only change which wavefront decodes which rows: exponent plane, merged bf16,
+    single tensor and batch give the bytes of the unsegmented decode (and of the oracle) for every
+    segment count the tile height allows, ragged edges included."""
+    from comp_inference_amd import build_checkpoints, rans_decomp_tiled, rans_decomp_tiled_batch
+
+    w = make_weight_kn(N, K, seed=K + N + th)
+    e, m = oracle.split_bf16(bf16_bits(w))
+    f, c = oracle.get_lut(e)
+    enc = oracle.encode_tiled_ilp2(e, f, c, th, 32)
+    man = torch.from_numpy(oracle.interleave_plane(m, th, 32)).cuda()
+    args = (torch.from_numpy(enc.stream).cuda(), _t32(enc.states).cuda(), _t32(enc.tables).cuda(),
+            torch.from_numpy(enc.slot_map).cuda(), (K, N), _t32(enc.tile_offsets).cuda(), _t32(enc.tile_max_lens).cuda())
+    plain = rans_decomp_tiled(*args, tile_k=th, tile_n=32)
+    assert np.array_equal(plain.cpu().numpy(), e)
+    for segs in [s for s in (2, 4, 8) if (th // 2) % (16 * s) == 0]:
+        ck = build_checkpoints(*args, tile_k=th, tile_n=32, segments=segs)
+        got = rans_decomp_tiled(*args, tile_k=th, tile_n=32, checkpoints=ck, segments=segs)
+        assert torch.equal(got, plain), segs
+        merged = rans_decomp_tiled(*args, tile_k=th, tile_n=32, mantissas=man, checkpoints=ck, segments=segs)
+        assert np.array_equal(bf16_bits(merged), bf16_bits(w)), segs
+        a, b = rans_decomp_tiled_batch([args + (ck, segs), args], tile_k=th, tile_n=32)
+        assert torch.equal(a, plain) and torch.equal(b, plain), segs
+    with pytest.raises(RuntimeError, match="checkpoints"):
+        rans_decomp_tiled(*args, tile_k=th, tile_n=32, checkpoints=torch.zeros(3, dtype=torch.int64), segments=2)
+
+
+def test_segmented_decode_depth_classes(oracle):
+    """Shallow, medium and deep bodies (and ones deeper than any staging area) through the segmented
+    decode: windows of every class, and items that fall back to guarded reads."""
+    from comp_inference_amd import build_checkpoints, rans_decomp_tiled
+
+    for n_sym in (4, 6, 9, 40, 256):
+        rng = np.random.default_rng(n_sym)
+        K, N = 3072, 96
+        e = rng.integers(0 if n_sym == 256 else 100, 256 if n_sym == 256 else 100 + n_sym, size=(K, N), dtype=np.uint8)
+        e[:1024] = np.where(rng.random((1024, N)) < 0.95, 120, e[:1024]).astype(np.uint8)
+        f, c = oracle.get_lut(e)
+        enc = oracle.encode_tiled_ilp2(e, f, c, 1024, 32)
+        args = (torch.from_numpy(enc.stream).cuda(), _t32(enc.states).cuda(), _t32(enc.tables).cuda(),
+                torch.from_numpy(enc.slot_map).cuda(), (K, N), _t32(enc.tile_offsets).cuda(), _t32(enc.tile_max_lens).cuda())
+        for segs in (2, 8):
+            ck = build_checkpoints(*args, tile_k=1024, tile_n=32, segments=segs)
+            got = rans_decomp_tiled(*args, tile_k=1024, tile_n=32, checkpoints=ck, segments=segs)
+            assert np.array_equal(got.cpu().numpy(), e), (n_sym, segs)

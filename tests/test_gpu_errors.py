@@ -71,6 +71,11 @@ def test_null_and_misshapen_arguments_are_rejected(oracle):
     assert lib.ci_decode_tiled_ilp2(*args(out=None)) == CI_ERR_ARG
     assert lib.ci_decode_tiled_ilp2(*args(th=1023)) == CI_ERR_ARG  # odd tile height
     assert lib.ci_last_error() != b""
+    seg = lambda ck, segs: args()[:11] + (_p(ck), segs) + args()[11:]  # noqa: E731
+    ck = torch.zeros(lib.ci_checkpoint_bytes(K, N, 1024, 32, 4) // 8, dtype=torch.int64, device="cuda")
+    assert lib.ci_decode_tiled_ilp2_segmented(*seg(None, 4)) == CI_ERR_ARG     # segments without checkpoints
+    assert lib.ci_decode_tiled_ilp2_segmented(*seg(ck, 3)) == CI_ERR_ARG       # 512 rows do not split in 3 x 16 n
+    assert lib.ci_decode_tiled_ilp2_segmented(*seg(None, 1)) == 0
     x = make_x(1, K, seed=1).cuda()
     o = torch.empty((1, N), dtype=torch.bfloat16, device="cuda")
     rc = lib.ci_fused_linear_ilp2(_p(x), 1, K, N, K - 8, _p(e["stream"]), C.c_uint64(e["stream"].numel()),

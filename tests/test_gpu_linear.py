@@ -233,6 +233,14 @@ def test_many_rows_decode_the_weight_once(oracle):
     # 3-D input keeps its leading shape
     got3 = _call(enc, man, x.view(2, 100, K), K, N, th, 32)
     assert tuple(got3.shape) == (2, 100, N)
+    # with decoder checkpoints the one decode runs segmented: same weight, same product
+    from comp_inference_amd import build_checkpoints
+
+    ck = build_checkpoints(torch.from_numpy(enc.stream).cuda(), _t32(enc.states).cuda(), _t32(enc.tables).cuda(),
+                           torch.from_numpy(enc.slot_map).cuda(), (K, N), _t32(enc.tile_offsets).cuda(),
+                           _t32(enc.tile_max_lens).cuda(), th, 32, 4)
+    got4 = _call(enc, man, x, K, N, th, 32, bias=bias, checkpoints=ck, segments=4)
+    assert torch.equal(got4.view(torch.int16), want.view(torch.int16))
 
 
 @pytest.mark.parametrize("K,N,th,M", [(4096, 256, 1024, 100), (3072, 128, 512, 150), (1300, 80, 1024, 70)])

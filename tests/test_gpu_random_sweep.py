@@ -144,13 +144,14 @@ def _one_case(ci, rng, big):
     else:
         K = max(th, rng.choice([th, rng.randrange(1, 4 * th), rng.randrange(th, 20 * th)]))
         N = max(32, rng.choice([1, 31, 32, 33, 64, rng.randrange(1, 900)]))
-        what = f"decode K={K} N={N} th={th} {kind}"
+        what = f"decode K={K} N={N} th={th} {kind} segs={segs}"
         w = _weight(K, N, kind, g)
         a = _compress(ci, w, th, True)
         if a is None:
             return None
         exp = ci.rans_decomp_tiled(a["compressed_data"], a["initial_states"], a["tables"], a["slot_map"], (K, N),
-                                   a["tile_offsets"], a["tile_max_lens"], th, 32)
+                                   a["tile_offsets"], a["tile_max_lens"], th, 32, checkpoints=_checkpoints(ci, a, segs),
+                                   segments=segs)
         assert torch.equal(exp.cpu(), ((w.view(torch.int16).to(torch.int32) >> 7) & 0xFF).to(torch.uint8)), what
     return op
 
