@@ -510,6 +510,40 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *partial
     out[(size_t)m * out_stride + n] = finish_bf16(s, bias, n);
 }
 
+// The same sums, four neighbouring outputs per thread (16-byte loads): for large outputs, where the kernel
+// is a stream of P planes and request count matters.  N % 4 == 0, partial 16-byte aligned.  Every output
+// is still summed in index order, so both kernels give the same bits.
+__global__ __launch_bounds__(64) void splitk_reduce4_kernel(const float *partial, uint32_t P, uint32_t M, uint32_t N,
+                                                            const uint16_t *bias, uint16_t *out, uint32_t out_stride) {
+    const uint64_t e = ((uint64_t)blockIdx.x * 64 + threadIdx.x) * 4;
+    if (e >= (uint64_t)M * N) return;
+    const uint32_t m = (uint32_t)(e / N), n = (uint32_t)(e % N);
+    const size_t plane = (size_t)M * N;
+    float s[4] = {0.f, 0.f, 0.f, 0.f};
+    uint32_t p = 0;
+    for (; p + 8 <= P; p += 8) {
+        float4 v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = *reinterpret_cast<const float4 *>(partial + (size_t)(p + j) * plane + e);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            s[0] += v[j].x;
+            s[1] += v[j].y;
+            s[2] += v[j].z;
+            s[3] += v[j].w;
+        }
+    }
+    for (; p < P; ++p) {
+        const float4 v = *reinterpret_cast<const float4 *>(partial + (size_t)p * plane + e);
+        s[0] += v.x;
+        s[1] += v.y;
+        s[2] += v.z;
+        s[3] += v.w;
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) out[(size_t)m * out_stride + n + j] = finish_bf16(s[j], bias, n + j);
+}
+
 // Same reduction over a bf16 workspace [P][M][N], the layout the reference's own kernels leave
 // behind (comp_inference/linear_triton.py:257-264, :303-314).
 __global__ __launch_bounds__(256) void splitk_reduce_bf16_kernel(const uint16_t *partial, uint32_t P,
@@ -526,6 +560,21 @@ __global__ __launch_bounds__(256) void splitk_reduce_bf16_kernel(const uint16_t 
 // Rows of x from which the fragment copy pays (below, the lanes past M re-read row 0 and one operand
 // load touches only M + 1 cache lines), and its size.
 constexpr uint32_t kFragMinRows = 17;
+// Outputs from which the four-per-thread reduction is used (below, one output per thread keeps more
+// wavefronts in flight).
+constexpr uint64_t kReduce4MinOutputs = 65536;
+static void launch_splitk_reduce(const float *partial, uint32_t P, uint32_t M, uint32_t N, const uint16_t *bias,
+                                 uint16_t *out, uint32_t out_stride, hipStream_t s) {
+    const uint64_t n = (uint64_t)M * N;
+    if (n >= kReduce4MinOutputs && N % 4 == 0 && aligned(partial, 16)) {
+        hipLaunchKernelGGL(splitk_reduce4_kernel, dim3((uint32_t)((n / 4 + 63) / 64)), dim3(64), 0, s, partial, P, M, N,
+                           bias, out, out_stride);
+    } else {
+        hipLaunchKernelGGL(splitk_reduce_kernel, dim3((uint32_t)((n + 255) / 256)), dim3(256), 0, s, partial, P, M, N, bias,
+                           out, out_stride);
+    }
+}
+
 static size_t x_fragment_bytes(uint32_t M, uint32_t K, bool fast_plan) {
     if (!fast_plan || M < kFragMinRows || K % 8) return 0;
     return (size_t)ceil_div(M, 32u) * 32 * K * 2;
@@ -725,9 +774,7 @@ static int fused_linear_impl(const uint16_t *d_x, uint32_t M, uint32_t K, uint32
         CI_LAUNCH_CHECK("fused_linear_generic_kernel");
     }
     if (p.P > 1) {
-        const uint64_t n = (uint64_t)M * N;
-        hipLaunchKernelGGL(splitk_reduce_kernel, dim3((uint32_t)((n + 255) / 256)), dim3(256), 0, s, a.partial, p.P,
-                           M, N, d_bias, d_out, out_stride);
+        launch_splitk_reduce(a.partial, p.P, M, N, d_bias, d_out, out_stride, s);
         CI_LAUNCH_CHECK("splitk_reduce_kernel");
     }
     return CI_OK;
@@ -795,8 +842,7 @@ extern "C" int ci_splitk_reduce(const void *d_partial, int partial_is_bf16, uint
         hipLaunchKernelGGL(splitk_reduce_bf16_kernel, grid, block, 0, s, static_cast<const uint16_t *>(d_partial), P,
                            M, N, d_bias, d_out, out_stride);
     else
-        hipLaunchKernelGGL(splitk_reduce_kernel, grid, block, 0, s, static_cast<const float *>(d_partial), P, M, N,
-                           d_bias, d_out, out_stride);
+        launch_splitk_reduce(static_cast<const float *>(d_partial), P, M, N, d_bias, d_out, out_stride, s);
     CI_LAUNCH_CHECK("splitk_reduce_kernel");
     return CI_OK;
 }

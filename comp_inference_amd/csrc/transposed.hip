@@ -99,6 +99,31 @@ __device__ __forceinline__ void trans_emit8(const uint32_t (&w)[4], const uint32
     }
 }
 
+// The fast path's variant: the same products and reduction, but the eight sums of a block stay in
+// registers -- block b of a group of four in lane b of every quad -- and one store per four blocks writes
+// 32 consecutive rows from the 32 lanes of a half: whole 128-byte lines instead of 32-byte pieces.
+// `keep` carries the sums between the calls of a group; blk = index of the block in the half tile.
+template <int MB>
+__device__ __forceinline__ void trans_emit8_lines(const uint32_t (&w)[4], const uint32_t (&xb)[MB], uint32_t M, uint32_t V,
+                                                  float *dst, uint32_t blk, float (&keep)[MB], int lane) {
+    const bool b8 = (lane & 8) != 0, b4 = (lane & 4) != 0;
+    const uint32_t j = 4u * b4 + 2u * b8 + ((lane >> 4) & 1u);  // which of the 8 rows this quad ends up with
+    const bool mine = (uint32_t)(lane & 3) == (blk & 3u);
+#pragma unroll
+    for (int m = 0; m < MB; ++m) {
+        const float xf = __uint_as_float(xb[m] << 16);
+        float p[8];
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {  // a bf16 x bf16 product is exact in fp32
+            p[2 * d] = __uint_as_float(w[d] << 16) * xf;
+            p[2 * d + 1] = __uint_as_float(w[d] & 0xFFFF0000u) * xf;
+        }
+        const float total = reduce8_over32(p, b8, b4);
+        keep[m] = mine ? total : keep[m];
+        if ((blk & 3u) == 3u && m < (int)M) dst[(size_t)m * V + (blk - 3u) * 8u + 8u * (uint32_t)(lane & 3) + j] = keep[m];
+    }
+}
+
 // One tile: wave walks it once, eight rows at a time.  Fast path: the eight steps run through the
 // hand-scheduled loop; otherwise guarded steps.  Both feed the same products and the same
 // reduction, so a tile's partial sums do not depend on the path it took.
@@ -115,7 +140,8 @@ __device__ __forceinline__ void trans_one_tile(const TransArgs &a, uint32_t tile
     uint32_t my_steps = 0;
     if (v0 < a.V) my_steps = min(half, a.V - v0);  // rows of this lane's half (same for its 32 lanes)
     const bool full = __builtin_amdgcn_ballot_w64(my_steps != half || h >= a.H) == 0;
-    const bool fast = full && depth >= 2 && depth < kStride && half % 8 == 0 && (uint32_t)(uintptr_t)tab == 0 &&
+    // (half % 32: the fast path stores groups of four eight-row blocks)
+    const bool fast = full && depth >= 2 && depth < kStride && half % 32 == 0 && (uint32_t)(uintptr_t)tab == 0 &&
                       !a.dense_w;
 
     uint32_t xb[MB];  // bf16 bits of x[m, h]
@@ -132,6 +158,9 @@ __device__ __forceinline__ void trans_one_tile(const TransArgs &a, uint32_t tile
         const uint32_t *mrow = reinterpret_cast<const uint32_t *>(man_tile + (c & ~3u));  // + 8 dwords per row
         const uint32_t nblk = half / 8;
         uint32_t mcur[8], mnext[8];
+        float keep[MB];
+#pragma unroll
+        for (int m = 0; m < MB; ++m) keep[m] = 0.f;
 #pragma unroll
         for (int r = 0; r < 8; ++r) mcur[r] = mrow[r * 8];
         for (uint32_t blk = 0; blk < nblk; ++blk) {
@@ -141,7 +170,7 @@ __device__ __forceinline__ void trans_one_tile(const TransArgs &a, uint32_t tile
             for (int r = 0; r < 8; ++r) mnext[r] = nrow[r * 8];
             uint32_t w[4];
             decode8_weights_asm(st, mcur, man_sel, w);
-            trans_emit8<MB>(w, xb, a.M, a.V, dst + blk * 8, 8u, lane);
+            trans_emit8_lines<MB>(w, xb, a.M, a.V, dst, blk, keep, lane);
 #pragma unroll
             for (int r = 0; r < 8; ++r) mcur[r] = mnext[r];
         }

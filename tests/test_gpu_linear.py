@@ -124,6 +124,41 @@ def test_splitk_reduce_matches_torch_sum():
     assert torch.equal(got, want)
 
 
+@pytest.mark.parametrize("P,M,N", [(128, 1, 128256), (14, 3, 40000), (5, 2, 32772), (9, 1, 70001)])
+def test_splitk_reduce_fp32_both_kernels_sum_in_index_order(P, M, N):
+    """fp32 partials (the library's own workspace layout): large outputs take the four-per-thread kernel,
+    a workspace that is not 16-byte aligned (or a row length that is no multiple of 4) the one-per-thread
+    kernel.  Both add plane after plane in index order, so they agree bit for bit with each other and
+    with that loop written in torch."""
+    import ctypes as C
+
+    from comp_inference_amd import _lib
+
+    g = torch.Generator("cpu").manual_seed(P + N)
+    flat = torch.zeros(P * M * N + 4, dtype=torch.float32, device="cuda")
+    data = torch.randn(P, M, N, generator=g).cuda()
+    bias = torch.randn(N, generator=g).to(torch.bfloat16).cuda()
+    want = torch.zeros(M, N, dtype=torch.float32, device="cuda")
+    for p in range(P):
+        want += data[p]
+    want = want.to(torch.bfloat16)                       # rounded once, then the reference's bf16 `out += bias`
+    want += bias
+
+    def run(offset):
+        part = flat[offset:offset + P * M * N]
+        part.copy_(data.view(-1))
+        assert part.data_ptr() % 16 == (0 if offset % 4 == 0 else 4 * (offset % 4))
+        out = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+        rc = _lib.lib().ci_splitk_reduce(C.c_void_p(part.data_ptr()), 0, P, M, N, C.c_void_p(bias.data_ptr()),
+                                         C.c_void_p(out.data_ptr()), N, _lib.stream_handle(out.device))
+        assert rc == 0
+        return out
+
+    a, b = run(0), run(1)
+    assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+    assert torch.equal(a.view(torch.int16), want.view(torch.int16))
+
+
 def test_dense_matmul_helper():
     """The uncompressed helper the reference exports as triton_matmul: shapes and tolerance."""
     from comp_inference_amd import triton_matmul
