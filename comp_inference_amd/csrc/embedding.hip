@@ -49,8 +49,9 @@ struct EmbedArgs {
     uint32_t out_stride;
     uint32_t *keys;          // workspace: sorted row ids (invalid = 0xFFFFFFFF, sorted last)
     uint32_t *pos;           // workspace: output row of each sorted id
-    uint32_t *chunk_start;   // workspace: first sorted request of every chunk, then n_ids; [-1] = chunk count
-                             // (bucket n_buckets collects the invalid ids)
+    uint2 *chunk_rec;        // workspace: per chunk {first sorted request, its key}, then {n_ids, -}; the word at
+                             // chunk_count holds the number of chunks (bucket n_buckets collects the invalid ids)
+    uint32_t *chunk_count;
     uint32_t n_pad;          // n_ids rounded up to a power of two
 };
 
@@ -137,11 +138,11 @@ __global__ __launch_bounds__(1024) void embed_sort_kernel(EmbedArgs a) {
     uint32_t at = before + incl - mine;
     for (uint32_t u = 0; u < per; ++u) {
         const uint32_t i = tid * per + u;
-        if (opens(i)) a.chunk_start[at++] = i;
+        if (opens(i)) a.chunk_rec[at++] = make_uint2(i, key[i]);
     }
     if (tid == 0) {
-        a.chunk_start[total] = a.n_ids;  // end marker
-        a.chunk_start[-1] = total;       // number of chunks
+        a.chunk_rec[total] = make_uint2(a.n_ids, 0xFFFFFFFFu);  // end marker
+        *a.chunk_count = total;
     }
 }
 
@@ -149,12 +150,13 @@ __global__ __launch_bounds__(1024) void embed_sort_kernel(EmbedArgs a) {
 // lanes 0..31 the first tile's 32 streams of that half, lanes 32..63 the second tile's.  Walks the
 // streams once, to the chunk's deepest row, and writes every requested row on the way as one
 // 128-byte store.
+// rec = the chunk's record {first request, its key}, hi = the first request of the next chunk.
 template <uint32_t kStride>
-__device__ __forceinline__ void embed_one_item(const EmbedArgs &a, uint32_t chunk, uint32_t pair, const uint2 *tab,
-                                               uint8_t *stage, int lane) {
-    const uint32_t lo = a.chunk_start[chunk], hi = a.chunk_start[chunk + 1];
+__device__ __forceinline__ void embed_one_item(const EmbedArgs &a, uint2 rec, uint32_t hi, uint32_t pair,
+                                               const uint2 *tab, uint8_t *stage, int lane) {
+    const uint32_t lo = rec.x;
     if (lo >= hi || hi > a.n_ids) return;
-    const uint32_t key0 = a.keys[lo];
+    const uint32_t key0 = rec.y;
     const uint32_t b = key0 == 0xFFFFFFFFu ? a.n_buckets : min(key0 / a.bucket_rows, a.n_buckets - 1);
     const uint32_t c = lane % 32, side = lane / 32;
     const uint32_t tn = pair * 2 + side, col = tn * 32 + c;
@@ -283,9 +285,28 @@ __device__ __forceinline__ void embed_wave_items(const EmbedArgs &a, const uint2
     if (wave >= kWaves) return;
     uint8_t *stage = persist_stage<kWaves, kStride>(lds, wave);
     const uint32_t pairs = (a.tiles_n + 1) / 2;
-    const uint64_t n_items = (uint64_t)min(a.chunk_start[-1], emb_max_chunks(a.n_ids, a.n_buckets)) * pairs;
-    for (uint64_t item = (uint64_t)wave * gridDim.x + blockIdx.x; item < n_items; item += (uint64_t)kWaves * gridDim.x)
-        embed_one_item<kStride>(a, (uint32_t)(item / pairs), (uint32_t)(item % pairs), tab, stage, lane);
+    const uint64_t n_items = (uint64_t)min(*a.chunk_count, emb_max_chunks(a.n_ids, a.n_buckets)) * pairs;
+    // An item's walk starts three dependent loads after its first one (chunk record -> tile offsets and
+    // checkpoints -> body rows), and with checkpoints an item is short: the record of the next item is
+    // fetched while this one runs.
+    const uint64_t step = (uint64_t)kWaves * gridDim.x;
+    auto record = [&](uint64_t item, uint2 &rec, uint32_t &hi) {
+        const uint32_t chunk = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(item / pairs));
+        rec = a.chunk_rec[chunk];
+        hi = a.chunk_rec[chunk + 1].x;
+    };
+    uint64_t item = (uint64_t)wave * gridDim.x + blockIdx.x;
+    uint2 rec = make_uint2(0u, 0u), next_rec = make_uint2(0u, 0u);
+    uint32_t hi = 0, next_hi = 0;
+    if (item < n_items) record(item, rec, hi);
+    while (item < n_items) {
+        if (item + step < n_items) record(item + step, next_rec, next_hi);
+        embed_one_item<kStride>(a, rec, hi, (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(item % pairs)), tab,
+                                stage, lane);
+        rec = next_rec;
+        hi = next_hi;
+        item += step;
+    }
 }
 
 // grid: at most one workgroup per CU, resident for the whole launch (fast_tile.h).  Work items are
@@ -296,13 +317,13 @@ __global__ __launch_bounds__(kPersistWaves *kWave) void embed_gather32_kernel(Em
     const uint2 *tab = reinterpret_cast<const uint2 *>(lds);
     const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
     const uint32_t pairs = (a.tiles_n + 1) / 2;
-    const uint64_t n_items = (uint64_t)min(a.chunk_start[-1], emb_max_chunks(a.n_ids, a.n_buckets)) * pairs;
+    const uint64_t n_items = (uint64_t)min(*a.chunk_count, emb_max_chunks(a.n_ids, a.n_buckets)) * pairs;
     uint32_t deepest = 0;
     for (uint64_t item = (uint64_t)threadIdx.x * gridDim.x + blockIdx.x; item < n_items;
          item += (uint64_t)kPersistWaves * kWave * gridDim.x) {
-        const uint32_t lo = a.chunk_start[item / pairs], pair = (uint32_t)(item % pairs);
-        if (lo >= a.n_ids) continue;
-        const uint32_t key0 = a.keys[lo];
+        const uint2 rec = a.chunk_rec[item / pairs];
+        const uint32_t pair = (uint32_t)(item % pairs), key0 = rec.y;
+        if (rec.x >= a.n_ids) continue;
         if (key0 == 0xFFFFFFFFu) continue;  // the chunks of invalid ids touch no tile
         const uint32_t b = min(key0 / a.bucket_rows, a.n_buckets - 1);
         const uint32_t tile_a = (b / (2 * a.segs)) * a.tiles_n + pair * 2;
@@ -388,7 +409,8 @@ extern "C" size_t ci_fused_embedding_workspace_bytes_segmented(uint32_t n_ids, u
     if (tile_height < 2 || (tile_height / 2) % segments) return 0;
     const uint32_t chunk = n_ids < kEmbChunk ? n_ids : kEmbChunk;
     const uint32_t n_buckets = ceil_div(K, tile_height / 2 / segments);
-    return (size_t)chunk * 8 + (size_t)(emb_max_chunks(chunk, n_buckets) + 2) * 4;
+    // sorted keys and positions, the chunk count, (8-byte aligned) one record per chunk and an end marker
+    return (size_t)chunk * 8 + 4 + 8 + (size_t)(emb_max_chunks(chunk, n_buckets) + 1) * 8;
 }
 
 extern "C" size_t ci_fused_embedding_workspace_bytes(uint32_t n_ids, uint32_t K, uint32_t tile_height) {
@@ -462,7 +484,11 @@ static int embedding_impl(const int64_t *d_ids, uint32_t n_ids, const uint8_t *d
     const uint32_t chunk_cap = n_ids < kEmbChunk ? n_ids : kEmbChunk;
     a.keys = static_cast<uint32_t *>(d_workspace);
     a.pos = a.keys + chunk_cap;
-    a.chunk_start = a.pos + chunk_cap + 1;  // one word in front holds the count
+    a.chunk_count = a.pos + chunk_cap;
+    {   // the records behind the count, at the next 8-byte boundary
+        uintptr_t at = reinterpret_cast<uintptr_t>(a.chunk_count + 1);
+        a.chunk_rec = reinterpret_cast<uint2 *>((at + 7) & ~(uintptr_t)7);
+    }
     CI_ALLOW_FULL_LDS(embed_gather32_kernel);
     CI_ALLOW_FULL_LDS(embed_sort_kernel);
     uint32_t cus = 0;
