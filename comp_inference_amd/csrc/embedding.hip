@@ -55,20 +55,28 @@ struct EmbedArgs {
     uint32_t n_pad;          // n_ids rounded up to a power of two
 };
 
-// One workgroup: sort (id, position) by id, then list the chunks of requests.
+// Keys below this many rows and positions below kEmbChunk fit one word.
+constexpr uint32_t kEmbPosBits = 13, kEmbPackedInvalid = (1u << (32 - kEmbPosBits)) - 1;
+static_assert((1u << kEmbPosBits) == kEmbChunk, "a position inside a pass must fit its bit field");
+
+// One workgroup: sort (id, position) by id, then list the chunks of requests.  kPacked: while the row
+// ids fit 19 bits an element of the sort is one word, id << 13 | position (the same order as the pair,
+// ties included), which halves the LDS traffic and the instructions of a compare-exchange -- and one CU
+// does all of this work.
+template <bool kPacked>
 __global__ __launch_bounds__(1024) void embed_sort_kernel(EmbedArgs a) {
     extern __shared__ __align__(16) uint8_t lds[];
     uint32_t *key = reinterpret_cast<uint32_t *>(lds);
     uint32_t *val = key + a.n_pad;
     const uint32_t tid = threadIdx.x, half = a.bucket_rows;  // rows of a bucket
     for (uint32_t i = tid; i < a.n_pad; i += 1024) {
-        uint32_t k = 0xFFFFFFFFu;
+        uint32_t k = kPacked ? kEmbPackedInvalid : 0xFFFFFFFFu;  // invalid ids sort last
         if (i < a.n_ids) {
             const int64_t id = a.ids[i];
             if (id >= 0 && id < (int64_t)a.K) k = (uint32_t)id;
         }
-        key[i] = k;
-        val[i] = i;
+        key[i] = kPacked ? (k << kEmbPosBits) | i : k;
+        if (!kPacked) val[i] = i;
     }
     __syncthreads();
     // Compare-exchange t works on elements inside the aligned block of 2 * stride elements around 2 t.  For
@@ -81,14 +89,22 @@ __global__ __launch_bounds__(1024) void embed_sort_kernel(EmbedArgs a) {
             for (uint32_t t = tid; t < a.n_pad / 2; t += 1024) {
                 const uint32_t lo = 2 * t - (t & (stride - 1)), hi = lo + stride;
                 const bool up = (lo & size) == 0;
-                const uint32_t ka = key[lo], kb = key[hi], va = val[lo], vb = val[hi];
-                // ties are ordered by position so that the result does not depend on the network
-                const bool gt = ka > kb || (ka == kb && va > vb);
-                if (gt == up) {
-                    key[lo] = kb;
-                    key[hi] = ka;
-                    val[lo] = vb;
-                    val[hi] = va;
+                const uint32_t ka = key[lo], kb = key[hi];
+                if (kPacked) {
+                    if ((ka > kb) == up) {
+                        key[lo] = kb;
+                        key[hi] = ka;
+                    }
+                } else {
+                    const uint32_t va = val[lo], vb = val[hi];
+                    // ties are ordered by position so that the result does not depend on the network
+                    const bool gt = ka > kb || (ka == kb && va > vb);
+                    if (gt == up) {
+                        key[lo] = kb;
+                        key[hi] = ka;
+                        val[lo] = vb;
+                        val[hi] = va;
+                    }
                 }
             }
             // the stage that follows: stride / 2, or size (the first of the next size) after stride 1
@@ -102,6 +118,21 @@ __global__ __launch_bounds__(1024) void embed_sort_kernel(EmbedArgs a) {
             }
         }
     __syncthreads();
+    if (kPacked) {  // back to (id, position) for what follows
+        uint32_t e[kEmbChunk / 1024];
+#pragma unroll
+        for (uint32_t r = 0; r < kEmbChunk / 1024; ++r) e[r] = tid + 1024 * r < a.n_pad ? key[tid + 1024 * r] : 0u;
+#pragma unroll
+        for (uint32_t r = 0; r < kEmbChunk / 1024; ++r) {
+            const uint32_t i = tid + 1024 * r;
+            if (i < a.n_pad) {
+                const uint32_t id = e[r] >> kEmbPosBits;
+                key[i] = id == kEmbPackedInvalid ? 0xFFFFFFFFu : id;
+                val[i] = e[r] & (kEmbChunk - 1);
+            }
+        }
+        __syncthreads();
+    }
     for (uint32_t i = tid; i < a.n_ids; i += 1024) {
         a.keys[i] = key[i];
         a.pos[i] = val[i];
@@ -490,7 +521,8 @@ static int embedding_impl(const int64_t *d_ids, uint32_t n_ids, const uint8_t *d
         a.chunk_rec = reinterpret_cast<uint2 *>((at + 7) & ~(uintptr_t)7);
     }
     CI_ALLOW_FULL_LDS(embed_gather32_kernel);
-    CI_ALLOW_FULL_LDS(embed_sort_kernel);
+    CI_ALLOW_FULL_LDS(embed_sort_kernel<true>);
+    CI_ALLOW_FULL_LDS(embed_sort_kernel<false>);
     uint32_t cus = 0;
     if (int rc = cu_count(&cus)) return rc;
     // as many work items as chunks x pairs of column tiles; the chunk count is known on the device only
@@ -500,7 +532,10 @@ static int embedding_impl(const int64_t *d_ids, uint32_t n_ids, const uint8_t *d
         a.n_ids = n_ids - first < kEmbChunk ? n_ids - first : kEmbChunk;
         a.out = d_out + (size_t)first * out_stride;
         a.n_pad = next_pow2(a.n_ids);
-        hipLaunchKernelGGL(embed_sort_kernel, dim3(1), dim3(1024), a.n_pad * 8 + 4096, s, a);
+        if (K < kEmbPackedInvalid)
+            hipLaunchKernelGGL(embed_sort_kernel<true>, dim3(1), dim3(1024), a.n_pad * 8 + 4096, s, a);
+        else
+            hipLaunchKernelGGL(embed_sort_kernel<false>, dim3(1), dim3(1024), a.n_pad * 8 + 4096, s, a);
         CI_LAUNCH_CHECK("embed_sort_kernel");
         const uint64_t most = (uint64_t)emb_max_chunks(a.n_ids, a.n_buckets) * ceil_div(a.tiles_n, 2u);
         const uint32_t gather_grid = (uint32_t)(most < (uint64_t)cus ? most : (uint64_t)cus);

@@ -154,3 +154,25 @@ def test_embedding_with_checkpoints(oracle, K, N, th, segments):
     assert torch.equal(got.cpu().view(torch.int16), _expected(table, ids).view(torch.int16))
     plain = _gather(enc, man, ids, K, N, th, 32)
     assert torch.equal(got, plain)
+
+
+def test_table_with_more_rows_than_a_one_word_sort_key_holds():
+    """The ids of a pass are sorted as (row << 13 | position) in one word while rows fit 19 bits, and as
+    (row, position) pairs beyond: a table of 530,000 rows takes the second form.  Both orders are the same
+    total order; duplicates, the last row, invalid ids and more ids than one sorting pass holds."""
+    import torch.nn as nn
+
+    import comp_inference_amd as ci
+
+    K, N = 530000, 32
+    g = torch.Generator().manual_seed(8)
+    table = (torch.randn(K, N, generator=g) * 0.02).to(torch.bfloat16)
+    emb = nn.Embedding(K, N).to(torch.bfloat16)
+    emb.weight.data = table.clone()
+    ci.rans_compress_module_weight(emb, transpose_weight=False)
+    mod = ci.RansEmbedding.from_compressed(emb).cuda()
+    ids = torch.cat([torch.randint(0, K, (9000,), generator=g), torch.tensor([K - 1, 0, K, -3, 524287, 524288, 7, 7])])
+    for segments in (1, "auto"):
+        mod.segments = segments
+        got = mod(ids.cuda()).cpu()
+        assert torch.equal(got.view(torch.int16), _expected(table, ids).view(torch.int16)), segments
