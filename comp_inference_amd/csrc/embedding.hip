@@ -177,6 +177,183 @@ __global__ __launch_bounds__(1024) void embed_sort_kernel(EmbedArgs a) {
     }
 }
 
+// The same lists by counting instead of sorting, for tables of up to kGroupMaxSlots counting slots: the
+// gather needs its requests grouped by bucket, and in row order only inside a chunk, which the wavefront
+// that serves the chunk establishes itself (sort_chunk_rows).  A slot is a run of `fine_rows` rows (a
+// divisor of the bucket's rows, 1 for small tables): one pass counts the requests of every slot (LDS
+// atomics; the value returned is the request's rank in its slot), a scan gives every slot its first
+// position, the buckets' request counts follow from the slots' positions, a second scan gives every
+// bucket its first chunk, and a last pass scatters.  Requests thus lie in slot order -- the chunks of a
+// bucket many ids fall into cover ascending row ranges, as after a sort -- and in the order the atomics
+// came inside a slot, which changes from run to run; the gathered rows do not.
+constexpr uint32_t kGroupMaxSlots = 16384;  // two words of LDS per slot
+
+// Exclusive prefix of `mine` over the 1024 threads (via 16 wavefront totals in `wave_sum`); `total` = the sum.
+__device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t mine, uint32_t *wave_sum, uint32_t tid, uint32_t &total) {
+    const uint32_t lane = tid % 64, wv = tid / 64;
+    uint32_t incl = mine;
+#pragma unroll
+    for (uint32_t d = 1; d < 64; d <<= 1) {
+        const uint32_t up = (uint32_t)__shfl_up((int)incl, d, 64);
+        if (lane >= d) incl += up;
+    }
+    __syncthreads();  // (wave_sum may still be read from an earlier scan)
+    if (lane == 63) wave_sum[wv] = incl;
+    __syncthreads();
+    uint32_t before = incl - mine;
+    total = 0;
+    for (uint32_t w = 0; w < 16; ++w) {
+        const uint32_t t = wave_sum[w];
+        if (w < wv) before += t;
+        total += t;
+    }
+    return before;
+}
+
+__global__ __launch_bounds__(1024) void embed_group_kernel(EmbedArgs a, uint32_t fine_rows) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    const uint32_t nf = (a.K + fine_rows - 1) / fine_rows;  // slots of valid rows; slot nf collects the invalid ids
+    const uint32_t per_bucket = a.bucket_rows / fine_rows;  // slots of a bucket
+    uint32_t *cnt = reinterpret_cast<uint32_t *>(lds), *first = cnt + (nf + 1), *wave_sum = first + (nf + 2);
+    const uint32_t tid = threadIdx.x;
+    for (uint32_t f = tid; f <= nf; f += 1024) cnt[f] = 0;
+    __syncthreads();
+    uint32_t key[kEmbChunk / 1024], slot[kEmbChunk / 1024], rank[kEmbChunk / 1024];
+#pragma unroll
+    for (uint32_t r = 0; r < kEmbChunk / 1024; ++r) {
+        const uint32_t i = tid + 1024 * r;
+        key[r] = 0xFFFFFFFFu;
+        slot[r] = nf;
+        rank[r] = 0;
+        if (i < a.n_ids) {
+            const int64_t id = a.ids[i];
+            if (id >= 0 && id < (int64_t)a.K) {
+                key[r] = (uint32_t)id;
+                slot[r] = key[r] / fine_rows;
+            }
+            rank[r] = atomicAdd(&cnt[slot[r]], 1u);
+        }
+    }
+    __syncthreads();
+    // first position of every slot: every thread takes a run of neighbouring slots
+    {
+        const uint32_t per = (nf + 1 + 1023) / 1024, f0 = min(tid * per, nf + 1), f1 = min(f0 + per, nf + 1);
+        uint32_t mine = 0, total;
+        for (uint32_t f = f0; f < f1; ++f) mine += cnt[f];
+        uint32_t at = block_exclusive_scan(mine, wave_sum, tid, total);
+        for (uint32_t f = f0; f < f1; ++f) {
+            first[f] = at;
+            at += cnt[f];
+        }
+        if (tid == 0) first[nf + 1] = total;
+    }
+    __syncthreads();
+    // chunks: every thread takes a run of neighbouring buckets (bucket n_buckets = the invalid ids)
+    {
+        const uint32_t nb1 = a.n_buckets + 1, per = (nb1 + 1023) / 1024, b0 = min(tid * per, nb1), b1 = min(b0 + per, nb1);
+        auto span = [&](uint32_t b, uint32_t &lo, uint32_t &n) {  // the bucket's requests: positions lo .. lo + n
+            const uint32_t fa = b == a.n_buckets ? nf : min(b * per_bucket, nf);
+            const uint32_t fb = b == a.n_buckets ? nf + 1 : min((b + 1) * per_bucket, nf);
+            lo = first[fa];
+            n = first[fb] - lo;
+        };
+        uint32_t mine = 0, total;
+        for (uint32_t b = b0; b < b1; ++b) {
+            uint32_t lo, n;
+            span(b, lo, n);
+            mine += (n + kEmbRun - 1) / kEmbRun;
+        }
+        uint32_t at = block_exclusive_scan(mine, wave_sum, tid, total);
+        for (uint32_t b = b0; b < b1; ++b) {
+            uint32_t lo, n;
+            span(b, lo, n);
+            for (uint32_t q = 0; q * kEmbRun < n; ++q)
+                a.chunk_rec[at++] = make_uint2(lo + q * kEmbRun, b == a.n_buckets ? 0xFFFFFFFFu : b * a.bucket_rows);
+        }
+        if (tid == 0) {
+            a.chunk_rec[total] = make_uint2(a.n_ids, 0xFFFFFFFFu);  // end marker
+            *a.chunk_count = total;
+        }
+    }
+#pragma unroll
+    for (uint32_t r = 0; r < kEmbChunk / 1024; ++r) {
+        const uint32_t i = tid + 1024 * r;
+        if (i < a.n_ids) {
+            const uint32_t at = first[slot[r]] + rank[r];
+            a.keys[at] = key[r];
+            a.pos[at] = i;
+        }
+    }
+}
+
+// Value of lane (l ^ kXor) for every lane l of the wavefront, without a trip through memory: quad
+// permutes, row shifts and rotates inside a row of 16 lanes, and the two row / half swaps above that.
+template <int kXor>
+__device__ __forceinline__ uint32_t lane_xor(uint32_t x, uint32_t lane) {
+    if (kXor == 1) return (uint32_t)__builtin_amdgcn_update_dpp((int)x, (int)x, 0xB1, 0xF, 0xF, false);  // quad_perm [1,0,3,2]
+    if (kXor == 2) return (uint32_t)__builtin_amdgcn_update_dpp((int)x, (int)x, 0x4E, 0xF, 0xF, false);  // quad_perm [2,3,0,1]
+    if (kXor == 4) {
+        const uint32_t up = (uint32_t)__builtin_amdgcn_update_dpp((int)x, (int)x, 0x104, 0xF, 0xF, false);    // row_shl:4: from l + 4
+        const uint32_t down = (uint32_t)__builtin_amdgcn_update_dpp((int)x, (int)x, 0x114, 0xF, 0xF, false);  // row_shr:4: from l - 4
+        return (lane & 4u) ? down : up;
+    }
+    if (kXor == 8) return (uint32_t)__builtin_amdgcn_update_dpp((int)x, (int)x, 0x128, 0xF, 0xF, false);  // row_ror:8
+    if (kXor == 16) {
+        const auto r = __builtin_amdgcn_permlane16_swap(x, x, false, false);  // {rows 0 and 2 doubled, rows 1 and 3 doubled}
+        return (lane & 16u) ? r[0] : r[1];
+    }
+    const auto r = __builtin_amdgcn_permlane32_swap(x, x, false, false);  // {lower half doubled, upper half doubled}
+    return (lane & 32u) ? r[0] : r[1];
+}
+
+// One bitonic stage over the 64 lanes: ascending inside aligned blocks of 2 * kSize lanes ... with partner
+// l ^ kStride; x is the same kind of word in every lane (larger = later).
+template <int kSize, int kStride>
+__device__ __forceinline__ uint32_t sort_stage(uint32_t x, uint32_t lane) {
+    const uint32_t other = lane_xor<kStride>(x, lane);
+    const bool keep_min = ((lane & kStride) == 0) == ((lane & kSize) == 0);
+    return keep_min ? min(x, other) : max(x, other);
+}
+
+// The requests of a chunk (one per lane, `n` of them: row inside the bucket, < 2^26) in row order: returns
+// (row << 6 | lane that held it) ascending over the lanes 0 .. n - 1.  Every lane must be active.  Only the
+// stages that n needs are run; a chunk that arrives in order (the sorting kernel's) costs the same.
+__device__ __forceinline__ uint32_t sort_chunk_rows(uint32_t row, uint32_t n, uint32_t lane) {
+    uint32_t x = lane < n ? (row << 6) | lane : 0xFFFFFFFFu;
+    if (n > 1) x = sort_stage<2, 1>(x, lane);
+    if (n > 2) {
+        x = sort_stage<4, 2>(x, lane);
+        x = sort_stage<4, 1>(x, lane);
+    }
+    if (n > 4) {
+        x = sort_stage<8, 4>(x, lane);
+        x = sort_stage<8, 2>(x, lane);
+        x = sort_stage<8, 1>(x, lane);
+    }
+    if (n > 8) {
+        x = sort_stage<16, 8>(x, lane);
+        x = sort_stage<16, 4>(x, lane);
+        x = sort_stage<16, 2>(x, lane);
+        x = sort_stage<16, 1>(x, lane);
+    }
+    if (n > 16) {
+        x = sort_stage<32, 16>(x, lane);
+        x = sort_stage<32, 8>(x, lane);
+        x = sort_stage<32, 4>(x, lane);
+        x = sort_stage<32, 2>(x, lane);
+        x = sort_stage<32, 1>(x, lane);
+    }
+    if (n > 32) {
+        x = sort_stage<64, 32>(x, lane);
+        x = sort_stage<64, 16>(x, lane);
+        x = sort_stage<64, 8>(x, lane);
+        x = sort_stage<64, 4>(x, lane);
+        x = sort_stage<64, 2>(x, lane);
+        x = sort_stage<64, 1>(x, lane);
+    }
+    return x;
+}
+
 // One chunk of requests (all in one bucket = half tile of rows) for two neighbouring column tiles:
 // lanes 0..31 the first tile's 32 streams of that half, lanes 32..63 the second tile's.  Walks the
 // streams once, to the chunk's deepest row, and writes every requested row on the way as one
@@ -187,6 +364,7 @@ __device__ __forceinline__ void embed_one_item(const EmbedArgs &a, uint2 rec, ui
                                                const uint2 *tab, uint8_t *stage, int lane) {
     const uint32_t lo = rec.x;
     if (lo >= hi || hi > a.n_ids) return;
+    hi = min(hi, lo + kEmbRun);  // (chunks are cut at kEmbRun requests: one per lane)
     const uint32_t key0 = rec.y;
     const uint32_t b = key0 == 0xFFFFFFFFu ? a.n_buckets : min(key0 / a.bucket_rows, a.n_buckets - 1);
     const uint32_t c = lane % 32, side = lane / 32;
@@ -233,7 +411,13 @@ __device__ __forceinline__ void embed_one_item(const EmbedArgs &a, uint2 rec, ui
                    win_b = (uint32_t)max(min(w_hi + 1, (int32_t)depth_b) - w_lo, 0);
     const bool fast = __builtin_amdgcn_ballot_w64(!col_ok) == 0 && win_a >= 2 && win_b >= 2 && win_a < kStride &&
                       win_b < kStride && (uint32_t)(uintptr_t)tab == 0;
-    uint32_t j = lo;
+    // the chunk's requests in row order, one per lane: row inside the bucket and output position
+    const uint32_t nb = hi - lo;
+    const uint32_t raw_row = (uint32_t)lane < nb ? min(a.keys[lo + lane] - bucket_row0, rows_b - 1) : 0u;
+    const uint32_t raw_pos = (uint32_t)lane < nb ? a.pos[lo + lane] : 0u;
+    const uint32_t sorted = sort_chunk_rows(raw_row, nb, (uint32_t)lane);
+    const uint32_t my_row = (uint32_t)lane < nb ? sorted >> 6 : 0u;
+    const uint32_t my_pos = (uint32_t)__shfl((int)raw_pos, (int)(sorted & 63u), 64);
     if (fast) {
         StageRegs body;
         const uint32_t deepest = max(win_a, win_b), my_depth = (lane & 4) ? win_b : win_a;
@@ -246,14 +430,11 @@ __device__ __forceinline__ void embed_one_item(const EmbedArgs &a, uint2 rec, ui
             }
         FastLane st;
         st.init_at<kStride>(stage, row - w_lo + 1, lane, state);
-        // Requests are taken 64 at a time (one sorted key and output row per lane, read back with
-        // readlane) and their sign|mantissa bytes eight at a time, one group ahead of the decoding,
-        // so that no load sits on the chain of decode steps.
+        // The requests (read back from their lanes with readlane) are served in row order, their
+        // sign|mantissa bytes fetched eight at a time, one group ahead of the decoding, so that no load
+        // sits on the chain of decode steps.
         uint32_t done = 0, sym = 0;  // rows decoded so far, symbol of row done - 1
-        for (uint32_t jb = lo; jb < hi; jb += 64) {
-            const uint32_t nb = min(64u, hi - jb);
-            const uint32_t my_row = (uint32_t)lane < nb ? a.keys[jb + lane] - bucket_row0 : 0u;
-            const uint32_t my_pos = (uint32_t)lane < nb ? a.pos[jb + lane] : 0u;
+        {
             constexpr int kG = 8;
             uint32_t row_cur[kG] = {}, row_next[kG] = {};
             uint8_t man_cur[kG] = {}, man_next[kG] = {};
@@ -291,8 +472,8 @@ __device__ __forceinline__ void embed_one_item(const EmbedArgs &a, uint2 rec, ui
     GlobalBytes src;
     src.init(a.stream + base, (uint32_t)(row + 1), 64, q);
     uint32_t X = state << 3;
-    const uint32_t last_row = a.keys[hi - 1] - bucket_row0;  // deepest requested row of the bucket
-    uint32_t want = a.keys[j] - bucket_row0;
+    const uint32_t last_row = (uint32_t)__builtin_amdgcn_readlane((int)my_row, (int)(nb - 1));  // deepest requested row
+    uint32_t j = 0, want = (uint32_t)__builtin_amdgcn_readlane((int)my_row, 0);
     for (uint32_t i = 0; i <= last_row; ++i) {
         uint32_t sym = 0;
         if (col_ok) {
@@ -303,9 +484,10 @@ __device__ __forceinline__ void embed_one_item(const EmbedArgs &a, uint2 rec, ui
         if (i == want) {  // wave uniform
             const uint16_t v = col_ok ? (uint16_t)assemble_bf16(sym, man[(size_t)i * 32]) : 0;
             do {
-                if (col_ok) a.out[(size_t)a.pos[j] * a.out_stride + col] = v;
+                const uint32_t p = (uint32_t)__builtin_amdgcn_readlane((int)my_pos, (int)j);
+                if (col_ok) a.out[(size_t)p * a.out_stride + col] = v;
                 ++j;
-                want = j < hi ? a.keys[j] - bucket_row0 : 0xFFFFFFFFu;
+                want = j < nb ? (uint32_t)__builtin_amdgcn_readlane((int)my_row, (int)j) : 0xFFFFFFFFu;
             } while (want == i);
         }
     }
@@ -523,6 +705,7 @@ static int embedding_impl(const int64_t *d_ids, uint32_t n_ids, const uint8_t *d
     CI_ALLOW_FULL_LDS(embed_gather32_kernel);
     CI_ALLOW_FULL_LDS(embed_sort_kernel<true>);
     CI_ALLOW_FULL_LDS(embed_sort_kernel<false>);
+    CI_ALLOW_FULL_LDS(embed_group_kernel);
     uint32_t cus = 0;
     if (int rc = cu_count(&cus)) return rc;
     // as many work items as chunks x pairs of column tiles; the chunk count is known on the device only
@@ -532,11 +715,24 @@ static int embedding_impl(const int64_t *d_ids, uint32_t n_ids, const uint8_t *d
         a.n_ids = n_ids - first < kEmbChunk ? n_ids - first : kEmbChunk;
         a.out = d_out + (size_t)first * out_stride;
         a.n_pad = next_pow2(a.n_ids);
-        if (K < kEmbPackedInvalid)
-            hipLaunchKernelGGL(embed_sort_kernel<true>, dim3(1), dim3(1024), a.n_pad * 8 + 4096, s, a);
-        else
-            hipLaunchKernelGGL(embed_sort_kernel<false>, dim3(1), dim3(1024), a.n_pad * 8 + 4096, s, a);
-        CI_LAUNCH_CHECK("embed_sort_kernel");
+        // Counting slots: a bucket's rows, divided further (by powers of two) while there are no more slots
+        // than ids -- then the chunks of a bucket that many ids fall into still cover ascending row ranges;
+        // every slot costs time (0.7 ns: clearing, scanning), so few ids get few slots.
+        uint32_t fine_rows = a.bucket_rows;
+        while (fine_rows % 2 == 0 && ceil_div(K, fine_rows / 2) + 2 <= kGroupMaxSlots &&
+               ceil_div(K, fine_rows / 2) <= a.n_ids)
+            fine_rows /= 2;
+        const uint32_t slots = ceil_div(K, fine_rows) + 2;
+        if (slots <= kGroupMaxSlots) {
+            hipLaunchKernelGGL(embed_group_kernel, dim3(1), dim3(1024), slots * 8 + 256, s, a, fine_rows);
+            CI_LAUNCH_CHECK("embed_group_kernel");
+        } else {  // more buckets than the counters hold: a full sort
+            if (K < kEmbPackedInvalid)
+                hipLaunchKernelGGL(embed_sort_kernel<true>, dim3(1), dim3(1024), a.n_pad * 8 + 4096, s, a);
+            else
+                hipLaunchKernelGGL(embed_sort_kernel<false>, dim3(1), dim3(1024), a.n_pad * 8 + 4096, s, a);
+            CI_LAUNCH_CHECK("embed_sort_kernel");
+        }
         const uint64_t most = (uint64_t)emb_max_chunks(a.n_ids, a.n_buckets) * ceil_div(a.tiles_n, 2u);
         const uint32_t gather_grid = (uint32_t)(most < (uint64_t)cus ? most : (uint64_t)cus);
         hipLaunchKernelGGL(embed_gather32_kernel, dim3(gather_grid), dim3(kPersistWaves * kWave), kLdsLimit, s, a);

@@ -156,22 +156,27 @@ def test_embedding_with_checkpoints(oracle, K, N, th, segments):
     assert torch.equal(got, plain)
 
 
-def test_table_with_more_rows_than_a_one_word_sort_key_holds():
-    """The ids of a pass are sorted as (row << 13 | position) in one word while rows fit 19 bits, and as
-    (row, position) pairs beyond: a table of 530,000 rows takes the second form.  Both orders are the same
-    total order; duplicates, the last row, invalid ids and more ids than one sorting pass holds."""
+@pytest.mark.parametrize("K,th", [(530000, 1024), (530000, 64), (300000, 32)])
+def test_tables_with_many_rows_and_buckets(K, th):
+    """How the requests of a pass are put in order depends on the table: by counting per bucket while the
+    counters fit the LDS (530,000 rows under 1024-row tiles), else by a full sort whose elements are one
+    word (row << 13 | position) while rows fit 19 bits (300,000 rows, 16-row buckets) and (row, position)
+    pairs beyond (530,000 rows, 32-row buckets).  All give table[ids]: duplicates, the last row, invalid
+    ids, more ids than one pass holds."""
     import torch.nn as nn
 
     import comp_inference_amd as ci
 
-    K, N = 530000, 32
+    N = 32
     g = torch.Generator().manual_seed(8)
     table = (torch.randn(K, N, generator=g) * 0.02).to(torch.bfloat16)
     emb = nn.Embedding(K, N).to(torch.bfloat16)
     emb.weight.data = table.clone()
-    ci.rans_compress_module_weight(emb, transpose_weight=False)
+    ci.rans_compress_module_weight(emb, tile_height=th, tile_width=32, transpose_weight=False)
     mod = ci.RansEmbedding.from_compressed(emb).cuda()
-    ids = torch.cat([torch.randint(0, K, (9000,), generator=g), torch.tensor([K - 1, 0, K, -3, 524287, 524288, 7, 7])])
+    assert mod.tile_k == th
+    ids = torch.cat([torch.randint(0, K, (9000,), generator=g), torch.tensor([K - 1, 0, K, -3, 262143, 262144, 7, 7]),
+                     torch.randint(0, 40, (300,), generator=g)])
     for segments in (1, "auto"):
         mod.segments = segments
         got = mod(ids.cuda()).cpu()
