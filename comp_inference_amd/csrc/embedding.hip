@@ -6,11 +6,12 @@
 // (comp_inference/embedding_triton.py:170-330) and the dense-layout variant (:333-483).
 //
 // The reference starts one program per (token, column tile) and discards row % (th/2) decode
-// steps in each.  Here the ids are sorted once (one workgroup, bitonic sort in LDS); a "bucket"
-// is one half tile of rows, i.e. the row range of one stream.  A work item is one bucket of two
-// neighbouring column tiles (32 + 32 lanes, all on the same half): a wavefront walks the two half
-// tiles once up to the deepest requested row and writes every requested row on the way as one
-// 128-byte store.  Items of buckets nobody asked for are skipped before touching the stream.
+// steps in each.  Here the ids are first grouped by "bucket" (one workgroup: counting, or a bitonic
+// sort for tables with more buckets than the counters hold); a bucket is one half tile of rows, i.e.
+// the row range of one stream.  A work item is one bucket of two neighbouring column tiles (32 + 32
+// lanes, all on the same half): a wavefront walks the two half tiles once up to the deepest requested
+// row and writes every requested row on the way as one 128-byte store.  Items of buckets nobody
+// asked for are skipped before touching the stream.
 // With decoder checkpoints (ci_build_checkpoints_ilp2) a bucket is one *segment* of a half tile: the
 // walk starts at the segment's checkpoint instead of the top of the stream, so a requested row costs at
 // most th / (2 segments) decode steps instead of th / 2.
