@@ -80,7 +80,7 @@ __global__ __launch_bounds__(1024) void embed_sort_kernel(EmbedArgs a) {
         if (!kPacked) val[i] = i;
     }
     __syncthreads();
-    // Compare-exchange t works on elements inside the aligned block of 2 * stride elements around 2 t.  For
+    // Compare-exchange t works on elements inside the aligned block of 2 * stride elements that holds 2 t.  For
     // strides up to 64 the 64 exchanges of a wavefront stay inside that wavefront's own 128 elements (and
     // exchange t belongs to the same thread in every stage), so those stages need no workgroup barrier:
     // the LDS serves one wavefront's accesses in order.  Barriers remain around the stages with longer
