@@ -628,7 +628,9 @@ extern "C" size_t ci_fused_linear_workspace_bytes_segmented(uint32_t M, uint32_t
     const LinearPlan fast = plan_linear(M, K, tile_height, tile_width, tiles_n, dense != 0, true, segments);
     const LinearPlan slow = plan_linear(M, K, tile_height, tile_width, tiles_n, dense != 0, false, segments);
     const uint32_t P = fast.P > slow.P ? fast.P : slow.P;
-    const size_t partial = P > 1 ? (size_t)P * M * N * sizeof(float) : 0;
+    // (the one-thread-per-stream kernel always goes through the workspace, also with a single partial sum:
+    // the dense layout with one tile row)
+    const size_t partial = (P > 1 || !slow.fast) ? (size_t)P * M * N * sizeof(float) : 0;
     return ((partial + 15) & ~(size_t)15) + x_fragment_bytes(M, K, fast.fast);
 }
 
@@ -715,8 +717,11 @@ static int fused_linear_impl(const uint16_t *d_x, uint32_t M, uint32_t K, uint32
     a.nw = p.nw;
     a.P = p.P;
     a.partial = static_cast<float *>(d_workspace);
+    // The one-thread-per-stream kernel writes fp32 partial sums and leaves output, bias and rounding to the
+    // reduction, also when there is a single partial sum per output.
+    const bool via_workspace = p.P > 1 || (!p.fast && !p.resident);
     size_t partial_bytes = 0;
-    if (p.P > 1) {
+    if (via_workspace) {
         partial_bytes = (size_t)p.P * M * N * sizeof(float);
         if (!d_workspace || workspace_bytes < partial_bytes)
             return fail(CI_ERR_CAPACITY, "fused linear: workspace needs %zu bytes, got %zu", partial_bytes, workspace_bytes);
@@ -773,7 +778,7 @@ static int fused_linear_impl(const uint16_t *d_x, uint32_t M, uint32_t K, uint32
             hipLaunchKernelGGL(fused_linear_generic_kernel<false>, grid, block, 0, s, a);
         CI_LAUNCH_CHECK("fused_linear_generic_kernel");
     }
-    if (p.P > 1) {
+    if (via_workspace) {
         launch_splitk_reduce(a.partial, p.P, M, N, d_bias, d_out, out_stride, s);
         CI_LAUNCH_CHECK("splitk_reduce_kernel");
     }

@@ -93,10 +93,13 @@ def test_fused_linear_is_deterministic(oracle):
     assert torch.equal(a, b)
 
 
-def test_fused_linear_dense_layout(oracle):
+@pytest.mark.parametrize("K,N,th,tw,M", [(1024, 64, 512, 32, 3), (1024, 96, 1024, 32, 1), (700, 64, 1024, 32, 9),
+                                         (1024, 4096, 1024, 32, 64), (256, 128, 256, 64, 5)])
+def test_fused_linear_dense_layout(oracle, K, N, th, tw, M):
+    """One stream per column and tile; with K <= tile_height there is a single partial sum per output,
+    which still goes through the workspace and the reduction kernel."""
     from comp_inference_amd import fused_rans_linear_triton_uncoalesced
 
-    K, N, th, tw, M = 1024, 64, 512, 32, 3
     w = make_weight_kn(N, K, seed=31)
     e, m = oracle.split_bf16(bf16_bits(w))
     f, c = oracle.get_lut(e)

@@ -94,3 +94,48 @@ def test_module_integration_on_the_fused_kernels(data, always_fused, tile_height
     result_compressed = _fused(module, x[:128], tile_height, tile_width)
     assert torch.allclose(result_golden[:128], result_compressed, atol=1e-2, rtol=1e-2), \
         (result_golden[:128] - result_compressed).abs().max()
+
+
+@pytest.mark.parametrize("Kw,Nw", [(4096, 1024), (1024, 4096)])
+def test_split_k_sweep(Kw, Nw):
+    """The reference's SPLIT_K sweep (tests/test_split_k.py:94-230) with its own call pattern: both tiled
+    layouts, batch sizes 1-64, SPLIT_K 1-16, stream sizes of the one-stream-per-column layout taken as
+    successive differences of the offsets (:142-147).  The reference only times these calls; here the
+    result must not depend on SPLIT_K at all (partitioning is chosen from the shape) and must meet the
+    allclose(1e-2, 1e-2) bar against torch.matmul."""
+    from comp_inference_amd import (fused_rans_linear_triton, fused_rans_linear_triton_uncoalesced,
+                                    rans_compress_module_weight)
+
+    g = torch.Generator("cuda").manual_seed(Kw)
+    weights_kn = (torch.randn((Kw, Nw), device="cuda", generator=g) * 0.02).to(torch.bfloat16)
+    mods = {}
+    for uncoalesced in (False, True):
+        mod = torch.nn.Module()
+        mod.weight = torch.nn.Parameter(weights_kn.clone())
+        mod.bias = None
+        rans_compress_module_weight(mod, tile_height=1024, tile_width=32, transpose_weight=False,
+                                    uncoalesced_interleaving=uncoalesced)
+        mods[uncoalesced] = mod
+    c, u = mods[False], mods[True]
+    u_off = u.exponent_stream_offsets.cuda()
+    u_tot = torch.tensor([u.exponent_compressed_weight.numel()], dtype=torch.int64, device="cuda")
+    u_sizes = (torch.cat([u_off.to(torch.int64)[1:], u_tot]) - u_off.to(torch.int64)).to(torch.uint32)
+    for bs in (1, 8, 64):
+        x = torch.randn((bs, Kw), dtype=torch.bfloat16, device="cuda", generator=g)
+        want = torch.matmul(x, weights_kn).float()
+        first = {}
+        for sk in (1, 2, 4, 8, 16):
+            coal = fused_rans_linear_triton(
+                x=x, compressed_data=c.exponent_compressed_weight.cuda(), initial_states=c.exponent_states.cuda(),
+                tables=c.exponent_tables.cuda(), slot_map=c.exponent_slot_map.cuda(), weight_shape=(Kw, Nw),
+                tile_offsets=c.exponent_tile_offsets.cuda(), tile_max_lens=c.exponent_tile_max_lens.cuda(),
+                tile_k=1024, tile_n=32, mantissas=c.mantissa_raw.cuda(), accum_block_size=32, SPLIT_K=sk)
+            unco = fused_rans_linear_triton_uncoalesced(
+                x=x, compressed_data=u.exponent_compressed_weight.cuda(), initial_states=u.exponent_states.cuda(),
+                tables=u.exponent_tables.cuda(), slot_map=u.exponent_slot_map.cuda(), weight_shape=(Kw, Nw),
+                stream_offsets=u_off, stream_sizes=u_sizes, tile_k=1024, tile_n=32, mantissas=u.mantissa_raw.cuda(),
+                accum_block_size=32, SPLIT_K=sk)
+            for name, got in (("coalesced", coal), ("uncoalesced", unco)):
+                assert torch.allclose(got.float(), want, atol=1e-2, rtol=1e-2), (name, bs, sk)
+                ref = first.setdefault(name, got)
+                assert torch.equal(got.view(torch.int16), ref.view(torch.int16)), (name, bs, sk)

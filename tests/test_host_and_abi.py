@@ -113,3 +113,27 @@ def test_embedding_oracle_equals_table_lookup(oracle):
     ok = (ids >= 0) & (ids < K)
     want[ok] = bf16_bits(table)[ids[ok]]
     assert np.array_equal(got, want)
+
+
+def test_every_linear_plan_that_writes_partial_sums_has_a_workspace():
+    """The one-thread-per-stream kernel (one-stream-per-column layout, tile widths other than 32, unaligned
+    streams) writes fp32 partial sums for the reduction kernel even when there is a single one per output
+    -- the one-stream-per-column layout with K <= tile_height.  The size query must cover that case, and
+    the entry point must refuse a missing workspace before anything is launched (checked here with
+    made-up, never dereferenced device addresses: no GPU is touched)."""
+    from comp_inference_amd import _lib
+
+    lib = _lib.lib()
+    M, N = 3, 96
+    for K, th, dense, planes in ((1024, 1024, 1, 1), (700, 1024, 1, 1), (4096, 1024, 1, 4), (1024, 1024, 0, 2),
+                                 (4096, 1024, 0, 8)):
+        need = lib.ci_fused_linear_workspace_bytes(M, K, N, th, 32, dense)
+        assert need >= planes * M * N * 4, (K, th, dense, need)
+    fake = ctypes.c_void_p(0x1000)
+    for K in (1024, 700):
+        rc = lib.ci_fused_linear_dense(fake, M, K, N, K, fake, ctypes.c_uint64(64), fake, fake, fake, fake, fake, fake,
+                                       1024, 32, None, fake, N, None, ctypes.c_size_t(0), None)
+        assert rc == 3 and b"workspace" in lib.ci_last_error(), K      # CI_ERR_CAPACITY
+        rc = lib.ci_fused_linear_dense(fake, M, K, N, K, fake, ctypes.c_uint64(64), fake, fake, fake, fake, fake, fake,
+                                       1024, 32, None, fake, N, fake, ctypes.c_size_t(M * N * 4 - 1), None)
+        assert rc == 3, K
