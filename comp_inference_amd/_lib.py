@@ -81,3 +81,21 @@ def as_u8(t: torch.Tensor, device) -> torch.Tensor:
     if t.dtype != torch.uint8:
         t = t.to(torch.uint8)
     return t.to(device).contiguous()
+
+
+def check_tiled_operands(rows: int, cols: int, tile_k: int, tile_n: int, initial_states, tables, slot_map, meta0, meta1,
+                         dense: bool) -> None:
+    """The kernels index these arrays by tile and stream without a bound of their own: a short one would be
+    read past its end.  Same condition and exception as the reference's decoder
+    (comp_inference/rans_triton.py:141-144), applied to every operand and every op."""
+    tiles = (-(-rows // tile_k)) * (-(-cols // tile_n))
+    streams = tiles * tile_n * (1 if dense else 2)
+    if initial_states.numel() != streams:
+        raise ValueError(f"Initial states size mismatch. Expected {streams}")
+    per_meta = streams if dense else tiles
+    if meta0.numel() != per_meta or meta1.numel() != per_meta:
+        what = "stream offsets / sizes" if dense else "tile offsets / max lens"
+        raise ValueError(f"{what} size mismatch. Expected {per_meta}")
+    if tables.numel() != 256 or slot_map.numel() != 4096:
+        raise ValueError("tables must hold 256 entries and slot_map 4096")
+

@@ -18,6 +18,7 @@ def _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, met
          mantissas, out, dense: bool, checkpoints=None, segments: int = 1):
     K, N = int(weight_shape[0]), int(weight_shape[1])  # K = vocabulary, N = hidden
     _lib.require_device(x)
+    _lib.check_tiled_operands(K, N, int(tile_k), int(tile_n), initial_states, tables, slot_map, meta0, meta1, dense)
     dev = x.device
     ids = x.reshape(-1)
     if ids.dtype != torch.int64:

@@ -83,6 +83,7 @@ def _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, met
          tile_n, mantissas, bias, out, workspace, dense: bool, checkpoints=None, segments: int = 1):
     K, N = int(weight_shape[0]), int(weight_shape[1])
     _lib.require_device(x)
+    _lib.check_tiled_operands(K, N, int(tile_k), int(tile_n), initial_states, tables, slot_map, meta0, meta1, dense)
     dev = x.device
     x2 = _prep_x(x, K)
     M = x2.shape[0]
@@ -147,6 +148,8 @@ class PreparedLinear:
         self.dev = dev
         self.K, self.N = int(weight_shape[0]), int(weight_shape[1])
         self.tile_k, self.tile_n = int(tile_k), int(tile_n)
+        _lib.check_tiled_operands(self.K, self.N, self.tile_k, self.tile_n, initial_states, tables, slot_map,
+                                  tile_offsets, tile_max_lens, False)
         man = _lib.as_u8(mantissas, dev).view(-1)
         need_man = (-(-self.K // self.tile_k)) * (-(-self.N // self.tile_n)) * self.tile_k * self.tile_n
         if man.numel() < need_man:

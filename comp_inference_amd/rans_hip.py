@@ -40,11 +40,10 @@ def rans_decomp_tiled(compressed_streams, initial_states, tables, slot_map, outp
     segments of every stream are then decoded side by side -- same bytes out, a shorter chain of steps."""
     K, N = int(output_shape[0]), int(output_shape[1])
     num_tiles_n, num_tiles_k = _tiles(K, N, tile_k, tile_n)
-    expected_streams = num_tiles_n * num_tiles_k * tile_n * 2
-    if initial_states.numel() != expected_streams:
-        # comp_inference/rans_triton.py:141-144
-        raise ValueError(f"Initial states size mismatch. Expected {expected_streams}")
     _lib.require_device(compressed_streams)
+    # comp_inference/rans_triton.py:141-144, extended to the other per-tile operands
+    _lib.check_tiled_operands(K, N, int(tile_k), int(tile_n), initial_states, tables, slot_map, tile_offsets,
+                              tile_max_lens, False)
     dev = compressed_streams.device
     stream_t = _lib.as_u8(compressed_streams, dev)
     merge = mantissas is not None
@@ -128,9 +127,7 @@ def rans_decomp_tiled_batch(items, tile_k=1024, tile_n=32):
         cs, st, tb, sm, shape, to, tl = item[:7]
         K, N = int(shape[0]), int(shape[1])
         ck, segs = _checked_checkpoints(*(item[7:9] if len(item) >= 9 else (None, 1)), K, N, tile_k, tile_n, dev)
-        expected = (-(-N // tile_n)) * (-(-K // tile_k)) * tile_n * 2
-        if st.numel() != expected:
-            raise ValueError(f"Initial states size mismatch. Expected {expected}")
+        _lib.check_tiled_operands(K, N, int(tile_k), int(tile_n), st, tb, sm, to, tl, False)
         t = (_lib.as_u8(cs, dev), _lib.as_u32(st, dev), _lib.as_u32(tb, dev), _lib.as_u8(sm, dev),
              _lib.as_u32(to, dev), _lib.as_u32(tl, dev))
         out = torch.empty((K, N), device=dev, dtype=torch.uint8)
@@ -167,6 +164,8 @@ def rans_decomp_tiled_uncoalesced(compressed_streams, initial_states, tables, sl
     _lib.require_device(compressed_streams)
     dev = compressed_streams.device
     K, N = int(output_shape[0]), int(output_shape[1])
+    _lib.check_tiled_operands(K, N, int(tile_k), int(tile_n), initial_states, tables, slot_map, stream_offsets,
+                              stream_sizes, True)
     stream_t = _lib.as_u8(compressed_streams, dev)
     merge = mantissas is not None
     man = _lib.as_u8(mantissas, dev).view(-1) if merge else None

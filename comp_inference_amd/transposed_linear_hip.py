@@ -24,6 +24,7 @@ def _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, met
          mantissas, bias, out, dense: bool):
     V, H = int(weight_shape[0]), int(weight_shape[1])  # weight is [vocab, hidden]
     _lib.require_device(x)
+    _lib.check_tiled_operands(V, H, int(tile_k), int(tile_n), initial_states, tables, slot_map, meta0, meta1, dense)
     dev = x.device
     x2 = _prep_x(x, H)
     M = x2.shape[0]

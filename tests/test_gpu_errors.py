@@ -91,7 +91,11 @@ def test_python_layer_raises_runtime_error(oracle):
     K, N = 1024, 64
     e, _ = _dev_enc(oracle, K, N)
     x = make_x(1, K, seed=1).cuda()
-    with pytest.raises(RuntimeError):
+    odd = torch.zeros(4097, dtype=torch.uint8, device="cuda")[1:]      # 4096 entries at an odd address
+    odd.copy_(e["slot_map"])
+    with pytest.raises(RuntimeError, match="slot_map"):                 # the library's message, raised in Python
+        fused_rans_linear(x, e["stream"], e["states"], e["tables"], odd, (K, N), e["offs"], e["lens"], 1024, 32, e["man"])
+    with pytest.raises(ValueError, match="size mismatch"):              # operand lengths are checked before that
         fused_rans_linear(x, e["stream"], e["states"], e["tables"], e["slot_map"], (K, N), e["offs"], e["lens"], 1023, 32,
                           e["man"])
 

@@ -137,3 +137,22 @@ def test_every_linear_plan_that_writes_partial_sums_has_a_workspace():
         rc = lib.ci_fused_linear_dense(fake, M, K, N, K, fake, ctypes.c_uint64(64), fake, fake, fake, fake, fake, fake,
                                        1024, 32, None, fake, N, fake, ctypes.c_size_t(M * N * 4 - 1), None)
         assert rc == 3, K
+
+
+def test_operand_sizes_are_checked_before_a_kernel_sees_them():
+    """The kernels index states, offsets and tables by tile and stream without a bound of their own; the
+    Python operators refuse arrays of the wrong length (ValueError, like the reference's decoder,
+    comp_inference/rans_triton.py:141-144)."""
+    from comp_inference_amd._lib import check_tiled_operands as chk
+
+    z = lambda n: torch.zeros(n, dtype=torch.int32)  # noqa: E731
+    chk(1300, 80, 1024, 32, z(2 * 3 * 64), z(256), z(4096), z(6), z(6), False)           # 2 x 3 tiles
+    chk(1300, 80, 1024, 32, z(2 * 3 * 32), z(256), z(4096), z(192), z(192), True)         # one stream per column
+    for bad in (lambda: chk(1300, 80, 1024, 32, z(383), z(256), z(4096), z(6), z(6), False),
+                lambda: chk(1300, 80, 1024, 32, z(384), z(256), z(4096), z(5), z(6), False),
+                lambda: chk(1300, 80, 1024, 32, z(384), z(256), z(4096), z(6), z(7), False),
+                lambda: chk(1300, 80, 1024, 32, z(384), z(255), z(4096), z(6), z(6), False),
+                lambda: chk(1300, 80, 1024, 32, z(384), z(256), z(4095), z(6), z(6), False),
+                lambda: chk(1300, 80, 1024, 32, z(192), z(256), z(4096), z(6), z(6), True)):
+        with pytest.raises(ValueError):
+            bad()
