@@ -235,6 +235,9 @@ def decompress(stream, states, sizes, num_streams: int, tables, slot_map, output
         raise RuntimeError("Output buffer must be on GPU")
     _lib.require_device(output)
     dev = output.device
+    if states.numel() < int(num_streams) or sizes.numel() < int(num_streams) or tables.numel() != 256 \
+            or slot_map.numel() != 4096:
+        raise ValueError(f"states and sizes must hold {int(num_streams)} entries, tables 256, slot_map 4096")
     # device copies must stay referenced until the launch has been enqueued
     st, sz = _lib.as_u32(states, dev), _lib.as_u32(sizes, dev)
     tb, sm = _lib.as_u32(tables, dev), _lib.as_u8(slot_map, dev)

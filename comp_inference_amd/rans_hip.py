@@ -147,6 +147,8 @@ def rans_decomp_flat(compressed_streams, initial_states, tables, slot_map, strea
     dev = compressed_streams.device
     K, N = int(output_shape[0]), int(output_shape[1])
     num_streams = len(initial_states)
+    if stream_sizes.numel() != num_streams or tables.numel() != 256 or slot_map.numel() != 4096:
+        raise ValueError(f"stream_sizes must hold {num_streams} entries, tables 256, slot_map 4096")
     out = torch.empty((K, N), device=dev, dtype=torch.uint8)
     stream_t = _lib.as_u8(compressed_streams, dev)
     st, sz = _lib.as_u32(initial_states, dev), _lib.as_u32(stream_sizes, dev)
