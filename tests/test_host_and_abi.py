@@ -156,3 +156,74 @@ def test_operand_sizes_are_checked_before_a_kernel_sees_them():
                 lambda: chk(1300, 80, 1024, 32, z(192), z(256), z(4096), z(6), z(6), True)):
         with pytest.raises(ValueError):
             bad()
+
+
+def test_entry_points_refuse_bad_arguments_before_any_launch():
+    """Argument checks come before the first HIP call, so they can be exercised without a GPU: made-up,
+    never dereferenced device addresses; every call must come back with CI_ERR_ARG (1) or
+    CI_ERR_CAPACITY (3) and a message."""
+    from comp_inference_amd import _lib
+
+    lib = _lib.lib()
+    P = ctypes.c_void_p
+    fake, null = P(0x1000), P(0)
+    u64, sz = ctypes.c_uint64, ctypes.c_size_t
+    K, N, M = 14336, 96, 2
+
+    def lin(ws, ws_bytes, th=1024, x_stride=K, states=fake, segs=None, ck=null):
+        head = (fake, M, K, N, x_stride, fake, u64(64), states, fake, fake, fake, fake, fake, th, 32)
+        tail = (None, fake, N, ws, sz(ws_bytes), None)
+        if segs is None:
+            return lib.ci_fused_linear_ilp2(*head, *tail)
+        return lib.ci_fused_linear_ilp2_segmented(*head, ck, segs, *tail)
+
+    need = lib.ci_fused_linear_workspace_bytes(M, K, N, 1024, 32, 0)
+    assert need >= 2 * M * N * 4
+    assert lin(null, 0) == 3 and b"workspace" in lib.ci_last_error()          # 14 k-tiles: two partial sums
+    assert lin(fake, 2 * M * N * 4 - 1) == 3
+    assert lin(fake, need, th=1023) == 1                                       # odd tile height
+    assert lin(fake, need, x_stride=K - 8) == 1                                # row stride shorter than the row
+    assert lin(fake, need, states=null) == 1
+    assert lin(fake, need, segs=4, ck=null) == 1                               # segments without checkpoints
+    assert lin(fake, need, segs=3, ck=fake) == 1                               # 512 rows do not split in 3 x 16 n
+    assert lin(fake, need, segs=4, ck=P(0x1004)) == 1                          # checkpoints not 8-byte aligned
+
+    V, H = 5000, 256
+    tneed = lib.ci_fused_linear_transposed_workspace_bytes(M, H, V, 32)
+    assert tneed == (H // 32) * M * V * 4
+
+    def trans(ws, ws_bytes, x_stride=H):
+        return lib.ci_fused_linear_transposed_ilp2(fake, M, H, V, x_stride, fake, u64(64), fake, fake, fake, fake, fake, fake,
+                                                   1024, 32, None, fake, V, ws, sz(ws_bytes), None)
+
+    assert trans(null, 0) == 3 and trans(fake, tneed - 1) == 3 and trans(fake, tneed, x_stride=H - 1) == 1
+
+    def emb(ws, ws_bytes, out_stride=H, segs=None, ck=null, th=1024):
+        head = (fake, 7, fake, u64(64), fake, fake, fake, fake, fake, fake, V, H, th, 32)
+        tail = (fake, out_stride, ws, sz(ws_bytes), None)
+        if segs is None:
+            return lib.ci_fused_embedding_ilp2(*head, *tail)
+        return lib.ci_fused_embedding_ilp2_segmented(*head, ck, segs, *tail)
+
+    eneed = lib.ci_fused_embedding_workspace_bytes(7, V, 1024)
+    assert eneed > 7 * 8
+    assert emb(null, 0) == 3 and emb(fake, eneed - 1) == 3
+    assert emb(fake, eneed, out_stride=H - 1) == 1
+    assert emb(fake, eneed, segs=8, ck=null) == 1 and emb(fake, eneed, segs=3, ck=fake) == 1
+    assert emb(fake, eneed, th=1023) == 1
+
+    def dec(out, th=1024, segs=None, ck=null, states=fake):
+        head = (fake, u64(64), states, fake, fake, fake, fake, 2048, 64, th, 32)
+        if segs is None:
+            return lib.ci_decode_tiled_ilp2(*head, out, None, None, None)
+        return lib.ci_decode_tiled_ilp2_segmented(*head, ck, segs, out, None, None, None)
+
+    assert dec(null) == 1 and dec(fake, th=1023) == 1 and dec(fake, states=null) == 1
+    assert dec(fake, segs=4, ck=null) == 1 and dec(fake, segs=3, ck=fake) == 1
+    assert lib.ci_build_checkpoints_ilp2(fake, u64(64), fake, fake, fake, fake, fake, 2048, 64, 1024, 32, 4, fake,
+                                         sz(lib.ci_checkpoint_bytes(2048, 64, 1024, 32, 4) - 1), None) == 3
+    assert lib.ci_build_checkpoints_ilp2(fake, u64(64), fake, fake, fake, fake, fake, 2048, 64, 1024, 32, 3, fake,
+                                         sz(1 << 20), None) == 1                # 512 rows do not split in 3
+    assert lib.ci_splitk_reduce(null, 0, 4, M, N, None, fake, N, None) == 1
+    assert lib.ci_splitk_reduce(fake, 0, 4, M, N, None, fake, N - 1, None) == 1
+    assert lib.ci_last_error() != b""
