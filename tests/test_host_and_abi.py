@@ -227,3 +227,29 @@ def test_entry_points_refuse_bad_arguments_before_any_launch():
     assert lib.ci_splitk_reduce(null, 0, 4, M, N, None, fake, N, None) == 1
     assert lib.ci_splitk_reduce(fake, 0, 4, M, N, None, fake, N - 1, None) == 1
     assert lib.ci_last_error() != b""
+
+
+def test_public_header_is_plain_c(tmp_path):
+    """The boundary is a C ABI: the header compiles as C99 on its own and a C program links against the
+    library's host-only entry points."""
+    import shutil
+    import subprocess
+
+    from comp_inference_amd import _lib
+
+    if shutil.which("gcc") is None:
+        pytest.skip("no C compiler")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    src = tmp_path / "use.c"
+    src.write_text('#include "comp_inference_hip.h"\n'
+                   "int main(void) {\n"
+                   "    ci_tiling t;\n"
+                   "    if (ci_tiling_init(&t, 4096, 14336, 1024, 32, 1) != 0 || t.num_tiles != 1792) return 1;\n"
+                   "    if (ci_fused_linear_workspace_bytes(1, 14336, 4096, 1024, 32, 0) == 0) return 2;\n"
+                   "    return ci_abi_version() >= 1 ? 0 : 3;\n"
+                   "}\n")
+    exe = tmp_path / "use"
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", os.path.join(root, "include"),
+                    str(src), "-o", str(exe), _lib.LIB_PATH, "-Wl,-rpath," + os.path.dirname(_lib.LIB_PATH),
+                    "-Wl,-rpath,/opt/rocm/lib"], check=True)
+    assert subprocess.run([str(exe)]).returncode == 0
