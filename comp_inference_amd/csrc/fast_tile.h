@@ -6,16 +6,17 @@
 //         or shifts them away).  With this scaling the LDS address of the 8-byte slot-table
 //         entry is X & 0x7ff8: one instruction on the serial chain instead of two.
 //   tab = slot table with .x = 8*freq | symbol << 24, .y = 8*(slot - cdf), at LDS address 0.
-//   q   = LDS address of the byte after the next one of this lane's stream.  The tile body is
-//         staged transposed (each lane's bytes contiguous, ascending with the stored row), so
-//         consuming k bytes is q -= k, done with subtract-with-borrow on the compare results.
-//   n1, n2 = the next two stream bytes (at q+1 and q), read one step ahead.
+//   q   = LDS address of the next byte of this lane's stream.  The tile body is staged transposed
+//         (each lane's bytes contiguous, ascending with the stored row), so consuming a byte is q -= 1.
+//   n1  = that byte, read one step ahead.
 //
-// One decode step is branch free.  t = freq * (X >> 15) + bias needs 0, 1 or 2 more bytes
-// (t >= 2^16, t < 2^16, t < 2^8 in unscaled terms); both candidates are formed and selected:
-//   X = t < 2^8 ? (t << 16 | n1 << 8 | n2) : t < 2^16 ? (t << 8 | n1) : t
-// The serial chain per symbol is v_and -> ds_read_b64 -> v_mad_u32_u24 -> v_cmp -> 2 x v_cndmask;
-// everything else is placed in the latency shadow of the table read.
+// t = freq * (X >> 15) + bias needs 0, 1 or 2 more bytes (t >= 2^16, t < 2^16, t < 2^8 in unscaled
+// terms).  The lanes that need one take it under an execution mask (X = t << 8 | n1, q -= 1, next
+// byte requested); needing two takes a symbol of frequency < 16 and is rare, so that case leaves the
+// straight line: one compare says whether any lane is still below 2^16, and only then a branch is
+// taken to the code that waits for the byte just requested and repeats the step for those lanes.
+// Eight VALU instructions and two LDS reads per symbol; the serial chain is v_and -> ds_read_b64 ->
+// v_mad_u32_u24 -> v_cmp -> v_lshl_or; the rest sits in the latency shadow of the table read.
 //
 // Inline-asm rule kept throughout: no LDS or global load issued inside an asm statement is
 // still in flight when the statement ends (the compiler does not know about them and may
@@ -194,9 +195,9 @@ __device__ __forceinline__ void stage_body(uint8_t *stage, const uint8_t *__rest
 // ---- assembly building blocks ----------------------------------------------------------------
 // Fixed temporaries (declared as clobbers by every user):
 //   v[72:73], v[74:75]  slot-table entries of the even / odd step of a pair
-//   v76 address, v77 quotient, v78 n1 << 3, v79 n2 << 3, v80 t, v81 t<<8|n1, v82 ..<<8|n2
-//   s[20:21] second compare
-// Operands by name: X q n1 n2 (lane state), L8 B8 (scaled 2^16 and 2^8 in SGPRs).
+//   v76 address, v77 quotient, v78 n1 << 3
+//   s[20:21] execution mask saved around the masked part of a step
+// Operands by name: X q n1 (lane state), L8 (scaled 2^16 in an SGPR).  Every lane must be active on entry.
 
 // Issue the table read and prepare everything that does not depend on it.
 #define CI_STEP_ISSUE(E)                       \
@@ -204,27 +205,36 @@ __device__ __forceinline__ void stage_body(uint8_t *stage, const uint8_t *__rest
     "ds_read_b64 " E ", v76\n"                \
     "v_lshrrev_b32 v77, 15, %[X]\n"           \
     "s_waitcnt lgkmcnt(1)\n"                   \
-    "v_lshlrev_b32 v78, 3, %[n1]\n"           \
-    "v_lshlrev_b32 v79, 3, %[n2]\n"
+    "v_lshlrev_b32 v78, 3, %[n1]\n"
 
-// Consume the table entry (ELO/EHI = its two dwords): new state, pointer, next two bytes.
+// Consume the table entry (ELO/EHI = its two dwords): new state, pointer, next byte.  The lanes whose
+// state fell below 2^16 take a byte under an execution mask; the few that are still below it afterwards
+// (a symbol of frequency < 16 met a small quotient: about one step in a thousand on bf16 weight exponents)
+// take their second byte out of line.
 #define CI_STEP_FINISH(ELO, EHI)                        \
     "s_waitcnt lgkmcnt(0)\n"                            \
-    "v_mad_u32_u24 v80, " ELO ", v77, " EHI "\n"      \
-    "v_cmp_gt_u32 vcc, %[L8], v80\n"                   \
-    "v_cmp_gt_u32 s[20:21], %[B8], v80\n"              \
-    "v_lshl_or_b32 v81, v80, 8, v78\n"               \
-    "v_lshl_or_b32 v82, v81, 8, v79\n"               \
-    "v_cndmask_b32 %[X], v80, v81, vcc\n"             \
-    "v_subbrev_co_u32 %[q], vcc, 0, %[q], vcc\n"        \
-    "v_cndmask_b32 %[X], %[X], v82, s[20:21]\n"        \
-    "v_subbrev_co_u32 %[q], vcc, 0, %[q], s[20:21]\n"   \
-    "ds_read_u8 %[n1], %[q] offset:1\n"                 \
-    "ds_read_u8 %[n2], %[q]\n"
+    "v_mad_u32_u24 %[X], " ELO ", v77, " EHI "\n"     \
+    "v_cmp_gt_u32 vcc, %[L8], %[X]\n"                  \
+    "s_and_saveexec_b64 s[20:21], vcc\n"               \
+    "v_lshl_or_b32 %[X], %[X], 8, v78\n"              \
+    "v_add_u32 %[q], -1, %[q]\n"                       \
+    "ds_read_u8 %[n1], %[q]\n"                         \
+    "v_cmpx_gt_u32 vcc, %[L8], %[X]\n"                 \
+    "s_cbranch_execnz 8f\n"                            \
+    "9:\n"                                             \
+    "s_mov_b64 exec, s[20:21]\n"                       \
+    ".subsection 1\n"                                  \
+    "8:\n"                                             \
+    "s_waitcnt lgkmcnt(0)\n"                           \
+    "v_lshlrev_b32 v78, 3, %[n1]\n"                   \
+    "v_lshl_or_b32 %[X], %[X], 8, v78\n"              \
+    "v_add_u32 %[q], -1, %[q]\n"                       \
+    "ds_read_u8 %[n1], %[q]\n"                         \
+    "s_branch 9b\n"                                    \
+    ".subsection 0\n"
 
 #define CI_STEP_CLOBBERS                                                                                  \
-    "vcc", "s20", "s21", "v72", "v73", "v74", "v75", "v76", "v77", "v78", "v79", "v80", "v81", "v82", \
-        "memory"
+    "vcc", "s20", "s21", "v72", "v73", "v74", "v75", "v76", "v77", "v78", "memory"
 
 // Two decoded symbols (top bytes of ELO0, ELO1) and their sign|mantissa bytes (byte %[msel] of the
 // dwords M0, M1) -> one dword holding two bf16 (first row in the low half).  v83/v112 temporaries.
@@ -308,7 +318,7 @@ __device__ __forceinline__ void stage_body(uint8_t *stage, const uint8_t *__rest
 
 // Per-lane decoder state of the hand-scheduled loops.
 struct FastLane {
-    uint32_t X, q, n1, n2;
+    uint32_t X, q, n1;
     // `stage` = this wave's staging area, q_lane = this lane's stream inside the tile.
     // kStride = bytes of LDS per lane in the staging area (must exceed the tile's depth).
     template <uint32_t kStride = kFastStride>
@@ -322,9 +332,8 @@ struct FastLane {
     __device__ __forceinline__ void init_at(const uint8_t *stage, int32_t have, uint32_t q_lane, uint32_t state) {
         X = state << 3;
         const uint8_t *col = stage + q_lane * kStride;
-        q = (uint32_t)(uintptr_t)col + (uint32_t)have - 2;  // low 32 bits of an LDS pointer are its LDS address
+        q = (uint32_t)(uintptr_t)col + (uint32_t)have - 1;  // low 32 bits of an LDS pointer are its LDS address
         n1 = have >= 1 ? col[have - 1] : 0;
-        n2 = have >= 2 ? col[have - 2] : 0;
     }
 };
 
@@ -360,9 +369,9 @@ __device__ __forceinline__ void linear_tile_asm(FastLane &st, f32x16_t &acc, uin
         CI_TAIL("v98", "v99", "v[104:107]")
         "s_nop 15\n"
         "s_nop 15\n"
-        : [X] "+v"(st.X), [q] "+v"(st.q), [n1] "+v"(st.n1), [n2] "+v"(st.n2), [acc] "+v"(acc), [moff] "+v"(moff),
+        : [X] "+v"(st.X), [q] "+v"(st.q), [n1] "+v"(st.n1), [acc] "+v"(acc), [moff] "+v"(moff),
           [xoff] "+v"(xoff)
-        : [L8] "s"(kRansL << 3), [B8] "s"(256u << 3), [selE] "s"(0x070C030Cu), [mask] "s"(0x807F807Fu),
+        : [L8] "s"(kRansL << 3), [selE] "s"(0x070C030Cu), [mask] "s"(0x807F807Fu),
           [msel] "v"(man_sel), [mbase] "s"(mbase), [xbase] "s"(xbase), [nblk] "s"(nblocks), [wrapM] "s"(wrap_m),
           [wrapX] "s"(wrap_x), [xstep] "s"(xstep)
         : CI_STEP_CLOBBERS, "scc", "s22", "s23", "s24", "s25", "v83", "v84", "v85", "v86", "v87", "v88",
@@ -401,9 +410,9 @@ __device__ __forceinline__ void linear_tile_asm2(FastLane &st, f32x16_t &acc, f3
         CI_TAIL2("v98", "v99", "v[104:107]", "v[124:127]")
         "s_nop 15\n"
         "s_nop 15\n"
-        : [X] "+v"(st.X), [q] "+v"(st.q), [n1] "+v"(st.n1), [n2] "+v"(st.n2), [acc] "+v"(acc), [acc2] "+v"(acc2),
+        : [X] "+v"(st.X), [q] "+v"(st.q), [n1] "+v"(st.n1), [acc] "+v"(acc), [acc2] "+v"(acc2),
           [moff] "+v"(moff), [xoff] "+v"(xoff), [xoff2] "+v"(xoff2)
-        : [L8] "s"(kRansL << 3), [B8] "s"(256u << 3), [selE] "s"(0x070C030Cu), [mask] "s"(0x807F807Fu),
+        : [L8] "s"(kRansL << 3), [selE] "s"(0x070C030Cu), [mask] "s"(0x807F807Fu),
           [msel] "v"(man_sel), [mbase] "s"(mbase), [xbase] "s"(xbase), [nblk] "s"(nblocks), [wrapM] "s"(wrap_m),
           [wrapX] "s"(wrap_x), [xstep] "s"(xstep)
         : CI_STEP_CLOBBERS, "scc", "s22", "s23", "s24", "s25", "v83", "v84", "v85", "v86", "v87", "v88",
@@ -436,8 +445,8 @@ __device__ __forceinline__ void decode_tile_asm(FastLane &st, uint64_t obase, ui
         CI_STEP_ISSUE("v[74:75]") CI_STORE_SYM("v72") CI_STEP_FINISH("v74", "v75")
         CI_STORE_SYM("v74")
         "s_waitcnt vmcnt(0) lgkmcnt(0)\n"
-        : [X] "+v"(st.X), [q] "+v"(st.q), [n1] "+v"(st.n1), [n2] "+v"(st.n2), [off] "+v"(off)
-        : [L8] "s"(kRansL << 3), [B8] "s"(256u << 3), [obase] "s"(obase), [stride] "s"(stride), [npairs] "s"(npairs)
+        : [X] "+v"(st.X), [q] "+v"(st.q), [n1] "+v"(st.n1), [off] "+v"(off)
+        : [L8] "s"(kRansL << 3), [obase] "s"(obase), [stride] "s"(stride), [npairs] "s"(npairs)
         : CI_STEP_CLOBBERS, "scc", "s22", "v83");
 }
 
@@ -447,9 +456,9 @@ __device__ __forceinline__ void decode_tile_asm(FastLane &st, uint64_t obase, ui
 __device__ __forceinline__ void decode8_weights_asm(FastLane &st, const uint32_t (&m)[8], uint32_t man_sel,
                                                     uint32_t (&w)[4]) {
     asm volatile(CI_BLOCK8_OUT
-                 : [X] "+v"(st.X), [q] "+v"(st.q), [n1] "+v"(st.n1), [n2] "+v"(st.n2), [w0] "=&v"(w[0]),
+                 : [X] "+v"(st.X), [q] "+v"(st.q), [n1] "+v"(st.n1), [w0] "=&v"(w[0]),
                    [w1] "=&v"(w[1]), [w2] "=&v"(w[2]), [w3] "=&v"(w[3])
-                 : [L8] "s"(kRansL << 3), [B8] "s"(256u << 3), [selE] "s"(0x070C030Cu), [mask] "s"(0x807F807Fu),
+                 : [L8] "s"(kRansL << 3), [selE] "s"(0x070C030Cu), [mask] "s"(0x807F807Fu),
                    [msel] "v"(man_sel), [m0] "v"(m[0]), [m1] "v"(m[1]), [m2] "v"(m[2]), [m3] "v"(m[3]), [m4] "v"(m[4]),
                    [m5] "v"(m[5]), [m6] "v"(m[6]), [m7] "v"(m[7])
                  : CI_STEP_CLOBBERS, "v83", "v112", "v116", "v117", "v118", "v119");
@@ -469,8 +478,8 @@ __device__ __forceinline__ uint32_t advance_asm(FastLane &st, uint32_t n) {
         "s_cbranch_scc1 ci_adv_loop%=\n"
         "s_waitcnt lgkmcnt(0)\n"
         "v_mov_b32 %[e], v72\n"
-        : [X] "+v"(st.X), [q] "+v"(st.q), [n1] "+v"(st.n1), [n2] "+v"(st.n2), [e] "=&v"(e)
-        : [L8] "s"(kRansL << 3), [B8] "s"(256u << 3), [n] "s"(n)
+        : [X] "+v"(st.X), [q] "+v"(st.q), [n1] "+v"(st.n1), [e] "=&v"(e)
+        : [L8] "s"(kRansL << 3), [n] "s"(n)
         : CI_STEP_CLOBBERS, "scc", "s22");
     return e;
 }

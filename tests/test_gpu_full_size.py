@@ -1,6 +1,6 @@
-"""Parity at the sizes the benchmarks run at (one Llama-3-8B-shaped gate projection, the 128256-row
-embedding table): bit-exact round trips through the HIP encoder and decoders, the oracle's stream for
-the whole tensor, and size-independent properties of the fused operators (tolerance against
+"""Parity at the sizes the benchmarks run at (the seven tensors of one Llama-3-8B-shaped layer, the
+128256-row embedding table): bit-exact round trips through the HIP encoder and decoders, the oracle's
+stream for a whole tensor, and size-independent properties of the fused operators (tolerance against
 torch.matmul, linearity, gather == indexing)."""
 import numpy as np
 import pytest
@@ -11,13 +11,26 @@ pytestmark = pytest.mark.gpu
 ATOL = RTOL = 1e-2  # the reference's own bar (tests/test_mat_mul.py:220,238)
 
 
+LAYER = [("q", 4096, 4096), ("k", 1024, 4096), ("v", 1024, 4096), ("o", 4096, 4096),
+         ("gate", 14336, 4096), ("up", 14336, 4096), ("down", 4096, 14336)]  # (name, out, in)
+
+
 @pytest.fixture(scope="module")
-def gate():
-    """gate projection of the bench layer: [K=4096, N=14336] bf16 N(0, 0.02), compressed on the GPU."""
+def layer_weights():
+    """The seven weights of the bench layer, drawn in this order from ONE generator (seed 1), nn.Linear
+    orientation, returned transposed to [K=in, N=out]."""
+    g = torch.Generator("cpu").manual_seed(1)
+    return {name: (torch.randn(o, i, generator=g, dtype=torch.float32) * 0.02).to(torch.bfloat16).t().contiguous()
+            for name, o, i in LAYER}
+
+
+@pytest.fixture(scope="module")
+def gate(layer_weights):
+    """gate projection of the bench layer (its fifth draw): [K=4096, N=14336] bf16 N(0, 0.02), compressed on
+    the GPU."""
     import comp_inference_amd as ci
 
-    g = torch.Generator("cpu").manual_seed(1)
-    w = (torch.randn(14336, 4096, generator=g, dtype=torch.float32) * 0.02).to(torch.bfloat16).t().contiguous()
+    w = layer_weights["gate"]
     exp, man = ci.extract_exp_and_mantissa(w)
     f, c = ci.get_rans_lut(exp)
     r = ci.ccore.RansManager(exp.numel()).compress_tiled(exp, f, c, 1024, 32)
@@ -44,6 +57,35 @@ def test_full_size_encoder_equals_oracle_and_round_trips(oracle, gate):
     assert torch.equal(both[0], out) and torch.equal(both[1], out)
     w = ci.rans_decomp_tiled(*gate["args"], tile_k=1024, tile_n=32, mantissas=gate["man_t"])
     assert torch.equal(w.cpu().view(torch.int16), gate["w"].view(torch.int16))
+
+
+def test_whole_layer_decodes_bit_exact_in_one_launch(oracle, layer_weights):
+    """Every tensor of the layer: HIP-encoded, decoded by the oracle's decoder and by one batched HIP launch,
+    both equal to the exponent plane of the weight; the smallest tensor's stream also byte for byte against
+    the oracle's encoder (the largest is compared in the test above)."""
+    import comp_inference_amd as ci
+
+    dev = "cuda"
+    items, planes = [], []
+    for name, w in layer_weights.items():
+        exp, _ = ci.extract_exp_and_mantissa(w)
+        f, c = ci.get_rans_lut(exp)
+        r = ci.ccore.RansManager(exp.numel()).compress_tiled(exp, f, c, 1024, 32)
+        u32 = lambda t: t.view(torch.int32).numpy().view(np.uint32)  # noqa: E731
+        K, N = w.shape
+        back = oracle.decode_tiled_ilp2(r.stream.numpy(), u32(r.states), u32(r.tables), r.slot_map.numpy(),
+                                        u32(r.tile_offsets), u32(r.tile_max_lens), K, N, 1024, 32)
+        assert np.array_equal(back, exp.numpy()), name
+        if name == "k":
+            fo, co = oracle.get_lut(exp.numpy())
+            ref = oracle.encode_tiled_ilp2(exp.numpy(), fo, co, 1024, 32)
+            assert np.array_equal(r.stream.numpy(), ref.stream) and np.array_equal(u32(r.states), ref.states)
+        items.append((r.stream.to(dev), r.states.to(dev), r.tables.to(dev), r.slot_map.to(dev), (K, N),
+                      r.tile_offsets.to(dev), r.tile_max_lens.to(dev)))
+        planes.append(exp)
+    outs = ci.rans_decomp_tiled_batch(items, tile_k=1024, tile_n=32)
+    for (name, _), o, e in zip(layer_weights.items(), outs, planes):
+        assert torch.equal(o.cpu(), e), name
 
 
 @pytest.mark.parametrize("M", [1, 4, 16, 64])
@@ -84,12 +126,17 @@ def test_full_size_embedding_gather_is_indexing():
     ids = np.random.default_rng(4).choice(V, 2048, p=p / p.sum())
     ids = np.concatenate([ids, [0, V - 1, V - 256, V - 257, 1023, 1024, V, -1]])  # edges of the ragged last tile row
     ids_t = torch.from_numpy(ids.astype(np.int64))
-    got = ci.fused_rans_embedding(ids_t.to(dev), r.stream.to(dev), r.states.to(dev), r.tables.to(dev),
-                                  r.slot_map.to(dev), (V, H), r.tile_offsets.to(dev), r.tile_max_lens.to(dev), 1024, 32,
-                                  ci.interleave_mantissas(man, 1024, 32).to(dev)).cpu()
+    dargs = (r.stream.to(dev), r.states.to(dev), r.tables.to(dev), r.slot_map.to(dev), (V, H), r.tile_offsets.to(dev),
+             r.tile_max_lens.to(dev), 1024, 32)
+    man_t = ci.interleave_mantissas(man, 1024, 32).to(dev)
+    got = ci.fused_rans_embedding(ids_t.to(dev), *dargs, man_t).cpu()
     ok = (ids_t >= 0) & (ids_t < V)
     want = torch.zeros(ids_t.numel(), H, dtype=torch.bfloat16)
     want[ok] = table[ids_t[ok]]
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    # the path RansEmbedding takes by default: decoder checkpoints, 8 segments per stream
+    ck = ci.build_checkpoints(*dargs, 8)
+    got = ci.fused_rans_embedding(ids_t.to(dev), *dargs, man_t, checkpoints=ck, segments=8).cpu()
     assert torch.equal(got.view(torch.int16), want.view(torch.int16))
     # the same table as LM head: logits of one hidden state against torch on the bf16 table
     h = torch.randn(1, H, generator=g, dtype=torch.float32).to(torch.bfloat16)

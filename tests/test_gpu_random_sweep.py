@@ -1,7 +1,8 @@
 """A seeded sweep over shapes, tile heights, weight statistics and segment counts, through the module-level
 compressor and every fused operator: decode and gather bit-exact, the two linears bit-identical to the
-same contraction on the plain weight and within 1e-2 (relative to sum |x||w|, the reference's allclose
-bar scaled to the data) of the fp32 product.  Weight statistics include the cases that leave the
+same contraction on the plain weight and within the reference's allclose(1e-2, 1e-2) of the fp32 product
+(for the two weight kinds whose magnitudes span many binades, "wide" and "cols", where sums cancel far
+below their terms, the same bar scaled to sum |x||w|).  Weight statistics include the cases that leave the
 hand-scheduled paths: near-constant planes (streams of a few bytes), mostly-zero weights, columns of very
 different compressibility inside one tile (ragged stream lengths), wide exponent ranges (deep bodies)."""
 import random
@@ -64,11 +65,15 @@ def _same(a, b):
     return torch.equal(a.view(torch.int16), b.view(torch.int16))
 
 
-def _within(got, x, w_kn, bias):
+def _within(got, x, w_kn, bias, kind):
     want = x.float() @ w_kn.float()
+    if bias is not None:
+        want = want + bias.float()
+    if kind not in ("wide", "cols"):
+        return bool(torch.allclose(got.float(), want, atol=1e-2, rtol=1e-2))  # tests/test_mat_mul.py:220,238
     bound = 1e-2 * (x.float().abs() @ w_kn.float().abs()) + 1e-2
     if bias is not None:
-        want, bound = want + bias.float(), bound + 1e-2 * bias.float().abs()
+        bound = bound + 1e-2 * bias.float().abs()
     return bool(((got.float() - want).abs() <= bound).all())
 
 
@@ -98,7 +103,7 @@ def _one_case(ci, rng, big):
         got = ci.fused_rans_linear(x.cuda(), **a, bias=bias_d, checkpoints=_checkpoints(ci, a, segs), segments=segs)
         ref = ci.plain_linear_same_order(x.cuda(), w.cuda(), tile_k=th, tile_n=32, bias=bias_d, segments=segs)
         assert _same(got, ref), what
-        assert _within(got.cpu(), x, w, bias), what
+        assert _within(got.cpu(), x, w, bias, kind), what
     elif op == "embed":
         K = rng.choice([th, 2 * th + 5, rng.randrange(th, 5 * th), rng.randrange(th, 40 * th)])
         N = rng.choice([32, 64, 128, rng.randrange(32, 600)])
@@ -140,7 +145,7 @@ def _one_case(ci, rng, big):
         x = torch.randn(M, H, generator=g).to(torch.bfloat16)
         got = ci.fused_rans_linear_transposed(x.cuda(), **a)
         assert _same(got, ci.plain_linear_transposed_same_order(x.cuda(), w.cuda(), tile_k=th, tile_n=32)), what
-        assert _within(got.cpu(), x, w.t(), None), what
+        assert _within(got.cpu(), x, w.t(), None, kind), what
     else:
         K = max(th, rng.choice([th, rng.randrange(1, 4 * th), rng.randrange(th, 20 * th)]))
         N = max(32, rng.choice([1, 31, 32, 33, 64, rng.randrange(1, 900)]))
