@@ -118,13 +118,16 @@ class Compressed:
         import comp_inference_amd as ci
 
         if not hasattr(self, "segments"):
+            from comp_inference_amd.linear_hip import PreparedLinear
+
             self.segments = ci.suggest_segments((self.K, self.N), self.th, self.tw)
             self.checkpoints = ci.build_checkpoints(self.stream, self.states, self.tables, self.slot_map,
                                                     (self.K, self.N), self.tile_offsets, self.tile_max_lens,
                                                     self.th, self.tw, self.segments)
-        return ci.fused_rans_linear(x, self.stream, self.states, self.tables, self.slot_map, (self.K, self.N),
-                                    self.tile_offsets, self.tile_max_lens, self.th, self.tw, self.man,
-                                    checkpoints=self.checkpoints, segments=self.segments)
+            self.prepared = PreparedLinear(self.stream.device, self.stream, self.states, self.tables, self.slot_map,
+                                           (self.K, self.N), self.tile_offsets, self.tile_max_lens, self.th, self.tw,
+                                           self.man, checkpoints=self.checkpoints, segments=self.segments)
+        return self.prepared(x)
 
 
 def event_times_us(fn, warmup: int, iters: int):
@@ -310,14 +313,15 @@ def main() -> int:
         rows = []
         for M in (1, 4, 16, 64):
             x = x_all[:M].contiguous()
-            got = gate.linear(x).float()
+            got = gate.linear_segmented(x).float()
             want = torch.matmul(x, w_dense).float()
             ok = bool(torch.allclose(got, want, atol=1e-2, rtol=1e-2))
-            us = batched_time_us(lambda: gate.linear(x), 25, 100)
+            us = batched_time_us(lambda: gate.linear_segmented(x), 25, 100)
+            us_plain = batched_time_us(lambda: gate.linear(x), 25, 100)
             us_ref = batched_time_us(lambda: torch.matmul(x, w_dense), 25, 100)
             nbytes = gate.linear_bytes(M)
             sb = step_bound_us(gate.wave_steps(), gate.th // 2)
-            rows.append({"M": M, "us": round(us, 2), "allclose_1e-2": ok,
+            rows.append({"M": M, "us": round(us, 2), "us_without_checkpoints": round(us_plain, 2), "allclose_1e-2": ok,
                          "step_rate_bound_us": max(sb["throughput_us"], sb["latency_us"]),
                          "hbm_frac_compressed_bytes": round(nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
                          "effective_weight_GBs": round(2 * gate.K * gate.N / (us * 1e-6) / 1e9, 1),

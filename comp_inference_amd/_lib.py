@@ -22,6 +22,43 @@ class Tiling(C.Structure):
         "streams_per_tile", "num_streams", "capacity")]
 
 
+class TiledWeight(C.Structure):
+    """ci_tiled_weight: a compressed weight with the length of every array (include/comp_inference_hip.h)."""
+    _fields_ = [("K", C.c_uint32), ("N", C.c_uint32), ("tile_height", C.c_uint32), ("tile_width", C.c_uint32),
+                ("d_stream", C.c_void_p), ("stream_len", C.c_uint64),
+                ("d_states", C.c_void_p), ("n_states", C.c_uint64),
+                ("d_tables", C.c_void_p), ("d_slot_map", C.c_void_p),
+                ("d_tile_offsets", C.c_void_p), ("d_tile_max_lens", C.c_void_p), ("n_tiles", C.c_uint64),
+                ("d_man_tiled", C.c_void_p), ("man_len", C.c_uint64),
+                ("d_checkpoints", C.c_void_p), ("checkpoint_bytes", C.c_uint64), ("segments", C.c_uint32),
+                ("d_slot_table", C.c_void_p), ("slot_table_bytes", C.c_uint64)]
+
+
+SLOT_TABLE_BYTES = 32768
+
+
+def tiled_weight(K, N, tile_k, tile_n, stream, states, tables, slot_map, tile_offsets, tile_max_lens, man,
+                 checkpoints=None, segments=1, slot_table=None) -> TiledWeight:
+    """Descriptor over device tensors (which the caller keeps alive for as long as it is used)."""
+    w = TiledWeight()
+    w.K, w.N, w.tile_height, w.tile_width = int(K), int(N), int(tile_k), int(tile_n)
+    w.d_stream, w.stream_len = stream.data_ptr() if stream.numel() else None, stream.numel()
+    w.d_states, w.n_states = states.data_ptr(), states.numel()
+    w.d_tables, w.d_slot_map = tables.data_ptr(), slot_map.data_ptr()
+    w.d_tile_offsets, w.d_tile_max_lens = tile_offsets.data_ptr(), tile_max_lens.data_ptr()
+    w.n_tiles = min(tile_offsets.numel(), tile_max_lens.numel())
+    w.d_man_tiled, w.man_len = man.data_ptr(), man.numel()
+    if checkpoints is not None and segments > 1:
+        w.d_checkpoints, w.checkpoint_bytes, w.segments = checkpoints.data_ptr(), checkpoints.numel() * 8, int(segments)
+    else:
+        w.d_checkpoints, w.checkpoint_bytes, w.segments = None, 0, 1
+    if slot_table is not None:
+        w.d_slot_table, w.slot_table_bytes = slot_table.data_ptr(), slot_table.numel() * slot_table.element_size()
+    else:
+        w.d_slot_table, w.slot_table_bytes = None, 0
+    return w
+
+
 def lib() -> C.CDLL:
     """The shared library; raises RuntimeError when it has not been built."""
     global _lib

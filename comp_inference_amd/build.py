@@ -20,6 +20,7 @@ FLAGS = [
     # packed-fp32 code generation is switched off for every kernel in this library
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function",
+    *os.environ.get("CI_EXTRA_HIPCC_FLAGS", "").split(),
 ]
 
 

@@ -197,7 +197,9 @@ __device__ __forceinline__ void stage_body(uint8_t *stage, const uint8_t *__rest
 //   v[72:73], v[74:75]  slot-table entries of the even / odd step of a pair
 //   v76 address, v77 quotient, v78 n1 << 3
 //   s[20:21] execution mask saved around the masked part of a step
-// Operands by name: X q n1 (lane state), L8 (scaled 2^16 in an SGPR).  Every lane must be active on entry.
+// Operands by name: X q n1 (lane state), L8 (scaled 2^16 in an SGPR), qdec (LDS bytes from one byte of a
+// lane's stream down to the next: 1 in a transposed staging area, 64 where body rows are staged as they
+// lie in memory).
 
 // Issue the table read and prepare everything that does not depend on it.
 #define CI_STEP_ISSUE(E)                       \
@@ -217,7 +219,7 @@ __device__ __forceinline__ void stage_body(uint8_t *stage, const uint8_t *__rest
     "v_cmp_gt_u32 vcc, %[L8], %[X]\n"                  \
     "s_and_saveexec_b64 s[20:21], vcc\n"               \
     "v_lshl_or_b32 %[X], %[X], 8, v78\n"              \
-    "v_add_u32 %[q], -1, %[q]\n"                       \
+    "v_subrev_u32 %[q], %[qdec], %[q]\n"                \
     "ds_read_u8 %[n1], %[q]\n"                         \
     "v_cmpx_gt_u32 vcc, %[L8], %[X]\n"                 \
     "s_cbranch_execnz 8f\n"                            \
@@ -228,7 +230,7 @@ __device__ __forceinline__ void stage_body(uint8_t *stage, const uint8_t *__rest
     "s_waitcnt lgkmcnt(0)\n"                           \
     "v_lshlrev_b32 v78, 3, %[n1]\n"                   \
     "v_lshl_or_b32 %[X], %[X], 8, v78\n"              \
-    "v_add_u32 %[q], -1, %[q]\n"                       \
+    "v_subrev_u32 %[q], %[qdec], %[q]\n"                \
     "ds_read_u8 %[n1], %[q]\n"                         \
     "s_branch 9b\n"                                    \
     ".subsection 0\n"
@@ -346,7 +348,7 @@ typedef float f32x16_t __attribute__((ext_vector_type(16)));
 // fragment to the next (16 in a plain row of x).  acc accumulates W^T-tile x x^T.
 __device__ __forceinline__ void linear_tile_asm(FastLane &st, f32x16_t &acc, uint64_t mbase, uint32_t moff,
                                                 uint64_t xbase, uint32_t xoff, uint32_t xstep, uint32_t man_sel,
-                                                uint32_t nblocks) {
+                                                uint32_t nblocks, uint32_t qdec = 1) {
     const uint32_t wrap_m = 0u - (nblocks - 1) * 256u, wrap_x = 0u - (nblocks - 1) * xstep;
     asm volatile(
         "s_mov_b32 s23, 0\n"
@@ -373,7 +375,7 @@ __device__ __forceinline__ void linear_tile_asm(FastLane &st, f32x16_t &acc, uin
           [xoff] "+v"(xoff)
         : [L8] "s"(kRansL << 3), [selE] "s"(0x070C030Cu), [mask] "s"(0x807F807Fu),
           [msel] "v"(man_sel), [mbase] "s"(mbase), [xbase] "s"(xbase), [nblk] "s"(nblocks), [wrapM] "s"(wrap_m),
-          [wrapX] "s"(wrap_x), [xstep] "s"(xstep)
+          [wrapX] "s"(wrap_x), [xstep] "s"(xstep), [qdec] "s"(qdec)
         : CI_STEP_CLOBBERS, "scc", "s22", "s23", "s24", "s25", "v83", "v84", "v85", "v86", "v87", "v88",
           "v89", "v90", "v91", "v92", "v93", "v94", "v95", "v96", "v97", "v98", "v99", "v100", "v101",
           "v102", "v103", "v104", "v105", "v106", "v107", "v108", "v109", "v110", "v111", "v112", "v116", "v117",
@@ -384,7 +386,7 @@ __device__ __forceinline__ void linear_tile_asm(FastLane &st, f32x16_t &acc, uin
 // buffers v[120:123] / v[124:127]) and a second accumulator fed with the same decoded weights.
 __device__ __forceinline__ void linear_tile_asm2(FastLane &st, f32x16_t &acc, f32x16_t &acc2, uint64_t mbase,
                                                  uint32_t moff, uint64_t xbase, uint32_t xoff, uint32_t xoff2,
-                                                 uint32_t xstep, uint32_t man_sel, uint32_t nblocks) {
+                                                 uint32_t xstep, uint32_t man_sel, uint32_t nblocks, uint32_t qdec = 1) {
     const uint32_t wrap_m = 0u - (nblocks - 1) * 256u, wrap_x = 0u - (nblocks - 1) * xstep;
     asm volatile(
         "s_mov_b32 s23, 0\n"
@@ -414,7 +416,7 @@ __device__ __forceinline__ void linear_tile_asm2(FastLane &st, f32x16_t &acc, f3
           [moff] "+v"(moff), [xoff] "+v"(xoff), [xoff2] "+v"(xoff2)
         : [L8] "s"(kRansL << 3), [selE] "s"(0x070C030Cu), [mask] "s"(0x807F807Fu),
           [msel] "v"(man_sel), [mbase] "s"(mbase), [xbase] "s"(xbase), [nblk] "s"(nblocks), [wrapM] "s"(wrap_m),
-          [wrapX] "s"(wrap_x), [xstep] "s"(xstep)
+          [wrapX] "s"(wrap_x), [xstep] "s"(xstep), [qdec] "s"(qdec)
         : CI_STEP_CLOBBERS, "scc", "s22", "s23", "s24", "s25", "v83", "v84", "v85", "v86", "v87", "v88",
           "v89", "v90", "v91", "v92", "v93", "v94", "v95", "v96", "v97", "v98", "v99", "v100", "v101",
           "v102", "v103", "v104", "v105", "v106", "v107", "v108", "v109", "v110", "v111", "v112", "v116", "v117",
@@ -430,7 +432,7 @@ __device__ __forceinline__ void linear_tile_asm2(FastLane &st, f32x16_t &acc, f3
 // Stand-alone decode of one half tile per lane: `npairs` >= 1 pairs of steps, symbol i stored at
 // obase + off + i * stride (bytes).  The store of a symbol sits in the shadow of the next step.
 __device__ __forceinline__ void decode_tile_asm(FastLane &st, uint64_t obase, uint32_t off, uint32_t stride,
-                                                uint32_t npairs) {
+                                                uint32_t npairs, uint32_t qdec = 1) {
     asm volatile(
         "s_sub_u32 s22, %[npairs], 1\n"
         CI_STEP_ISSUE("v[72:73]") CI_STEP_FINISH("v72", "v73")
@@ -446,7 +448,7 @@ __device__ __forceinline__ void decode_tile_asm(FastLane &st, uint64_t obase, ui
         CI_STORE_SYM("v74")
         "s_waitcnt vmcnt(0) lgkmcnt(0)\n"
         : [X] "+v"(st.X), [q] "+v"(st.q), [n1] "+v"(st.n1), [off] "+v"(off)
-        : [L8] "s"(kRansL << 3), [obase] "s"(obase), [stride] "s"(stride), [npairs] "s"(npairs)
+        : [L8] "s"(kRansL << 3), [obase] "s"(obase), [stride] "s"(stride), [npairs] "s"(npairs), [qdec] "s"(qdec)
         : CI_STEP_CLOBBERS, "scc", "s22", "v83");
 }
 
@@ -454,19 +456,19 @@ __device__ __forceinline__ void decode_tile_asm(FastLane &st, uint64_t obase, ui
 // block.  m[r] = aligned dword holding this lane's sign|mantissa byte of row r, man_sel = the
 // per-lane byte selector 0x04040000 + (column & 3) * 0x01010101.
 __device__ __forceinline__ void decode8_weights_asm(FastLane &st, const uint32_t (&m)[8], uint32_t man_sel,
-                                                    uint32_t (&w)[4]) {
+                                                    uint32_t (&w)[4], uint32_t qdec = 1) {
     asm volatile(CI_BLOCK8_OUT
                  : [X] "+v"(st.X), [q] "+v"(st.q), [n1] "+v"(st.n1), [w0] "=&v"(w[0]),
                    [w1] "=&v"(w[1]), [w2] "=&v"(w[2]), [w3] "=&v"(w[3])
                  : [L8] "s"(kRansL << 3), [selE] "s"(0x070C030Cu), [mask] "s"(0x807F807Fu),
                    [msel] "v"(man_sel), [m0] "v"(m[0]), [m1] "v"(m[1]), [m2] "v"(m[2]), [m3] "v"(m[3]), [m4] "v"(m[4]),
-                   [m5] "v"(m[5]), [m6] "v"(m[6]), [m7] "v"(m[7])
+                   [m5] "v"(m[5]), [m6] "v"(m[6]), [m7] "v"(m[7]), [qdec] "s"(qdec)
                  : CI_STEP_CLOBBERS, "v83", "v112", "v116", "v117", "v118", "v119");
 }
 
 // Advance the lane's stream by n >= 1 symbols; returns the table word (symbol in the top byte) of
 // the last one.  n must be the same for every lane of the wave.
-__device__ __forceinline__ uint32_t advance_asm(FastLane &st, uint32_t n) {
+__device__ __forceinline__ uint32_t advance_asm(FastLane &st, uint32_t n, uint32_t qdec = 1) {
     uint32_t e;
     n = (uint32_t)__builtin_amdgcn_readfirstlane((int)n);  // the loop counter is scalar
     asm volatile(
@@ -479,7 +481,7 @@ __device__ __forceinline__ uint32_t advance_asm(FastLane &st, uint32_t n) {
         "s_waitcnt lgkmcnt(0)\n"
         "v_mov_b32 %[e], v72\n"
         : [X] "+v"(st.X), [q] "+v"(st.q), [n1] "+v"(st.n1), [e] "=&v"(e)
-        : [L8] "s"(kRansL << 3), [n] "s"(n)
+        : [L8] "s"(kRansL << 3), [n] "s"(n), [qdec] "s"(qdec)
         : CI_STEP_CLOBBERS, "scc", "s22");
     return e;
 }

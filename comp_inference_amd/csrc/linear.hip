@@ -58,6 +58,10 @@ struct LinearArgs {
     // null / 1: with them the resident kernel gives every (tile, segment) its own wavefront.
     const uint2 *ckpt;
     uint32_t segs;
+    // The 32 KB slot table of the scaled state (build_slot_table_x8) kept beside the weight, or null: then
+    // every workgroup builds it from tables and slot_map.
+    const uint2 *slot_table;
+    uint32_t rounds;  // fused_linear32_seg_kernel: items of a job per wavefront
 };
 
 // x [M, K] -> the fragment order described at LinearArgs::xf.  In a plain row-major x the 64 lanes of
@@ -287,9 +291,11 @@ __global__ __launch_bounds__(kLinMaxWaves *kWave) void fused_linear32_kernel(Lin
 // Item vk * tiles_n + tn, vk = tk * segs + seg: rows [seg, seg + 1) * th / (2 segs) of both halves of tile
 // (tk, tn).  A segment's bytes are the rows between its own checkpoint and the next one's, about
 // depth / segs of them per lane plus the spread between lanes; only that window of the body is staged.
-template <int MB, uint32_t kStride>
+// kKeep: the item's products are added to acc / acc2 and stay there (the caller owns the sum); otherwise the
+// item starts from zero and writes its own partial sums to the workspace.
+template <int MB, uint32_t kStride, bool kKeep = false>
 __device__ __forceinline__ void linear_one_item(const LinearArgs &a, uint32_t vk, uint32_t tn, const uint2 *tab,
-                                                uint8_t *stage, int lane) {
+                                                uint8_t *stage, int lane, f32x16 &acc, f32x16 &acc2) {
     const uint32_t tk = vk / a.segs, seg = vk % a.segs, tile = tk * a.tiles_n + tn;
     const uint32_t half = a.th / 2, seglen = half / a.segs, hsel = lane / 32, c = lane % 32;
     const uint32_t col0 = tn * 32, k0 = tk * a.th + hsel * half + seg * seglen;
@@ -317,17 +323,20 @@ __device__ __forceinline__ void linear_one_item(const LinearArgs &a, uint32_t vk
     // highest start row
     const int32_t lo = max(wave_min_i32(row_end) - 1, 0), hi = wave_max_i32(row);
     const uint32_t window = hi >= lo ? (uint32_t)(hi - lo + 1) : 0u;
-    const bool fast = full && a.fast_ok && window >= 2 && window < kStride && seglen % 16 == 0 &&
+    // (kStride == 0: a caller without a transposed staging area; every item takes the guarded path)
+    const bool fast = kStride != 0 && full && a.fast_ok && window >= 2 && window < kStride && seglen % 16 == 0 &&
                       (uint32_t)(uintptr_t)tab == 0 && !a.dense_w;
     const uint32_t m = c;  // row of x this lane feeds to the (first) MFMA
     const bool m_ok = m < a.M, m2_ok = MB == 2 && m + 32 < a.M;
-    f32x16 acc, acc2;
+    if (!kKeep) {
 #pragma unroll
-    for (int v = 0; v < 16; ++v) acc[v] = acc2[v] = 0.f;
+        for (int v = 0; v < 16; ++v) acc[v] = acc2[v] = 0.f;
+    }
     const uint32_t xrow_elems = (m_ok ? m : 0) * a.x_stride + k0;
     const uint32_t xrow2_elems = (m2_ok ? m + 32 : 0) * a.x_stride + k0;
     const size_t man_tile = (size_t)tile * a.th * 32;
     if (fast) {
+        if constexpr (kStride != 0) {
         stage_body<kStride>(stage, a.stream + base + (size_t)lo * 64, window, lane);
         FastLane st;
         st.init_at<kStride>(stage, row - lo + 1, lane, state);
@@ -351,6 +360,7 @@ __device__ __forceinline__ void linear_one_item(const LinearArgs &a, uint32_t vk
             linear_tile_asm2(st, acc, acc2, mb_u, moff, xb, xo, xo2, xstep, man_sel, seglen / 8);
         else
             linear_tile_asm(st, acc, mb_u, moff, xb, xo, xstep, man_sel, seglen / 8);
+        }
     } else {
         const uint8_t *man = a.man_tiled + man_tile + (size_t)(hsel * half + seg * seglen) * 32 + c;
         const uint16_t *wd = a.dense_w ? a.dense_w + (size_t)k0 * a.N + col0 + c : nullptr;
@@ -363,6 +373,7 @@ __device__ __forceinline__ void linear_one_item(const LinearArgs &a, uint32_t vk
                                 a.N);
         }
     }
+    if (kKeep) return;
     // MFMA 32x32 result layout: register v of lane l is row (v/4)*8 + (l/32)*4 + v%4 (= column of
     // the tile), column l%32 (= row m of x)
 #pragma unroll
@@ -388,8 +399,10 @@ __device__ __forceinline__ void linear_wave_tiles(const LinearArgs &a, const uin
     const uint32_t active = rounds ? (mine + rounds - 1) / rounds : 0u;
     if ((uint32_t)wave >= active) return;
     uint8_t *stage = persist_stage<kWaves, kStride>(lds, wave);
+    f32x16 acc, acc2;
     for (uint64_t item = (uint64_t)wave * gridDim.x + blockIdx.x; item < num_items; item += (uint64_t)active * gridDim.x)
-        linear_one_item<MB, kStride>(a, (uint32_t)(item / a.tiles_n), (uint32_t)(item % a.tiles_n), tab, stage, lane);
+        linear_one_item<MB, kStride>(a, (uint32_t)(item / a.tiles_n), (uint32_t)(item % a.tiles_n), tab, stage, lane, acc,
+                                     acc2);
 }
 
 template <int MB>
@@ -418,6 +431,330 @@ __global__ __launch_bounds__(kPersistWaves *kWave) void fused_linear32_resident_
     else
         linear_wave_tiles<MB, 12, kDepthTiny>(a, tab, lds, wave, lane);
 }
+
+// ---- sixteen wavefronts per CU on short items ---------------------------------------------------
+// The decode step is bound by how many wavefronts a CU keeps in flight (a step is a chain of dependent
+// instructions; four wavefronts per SIMD are what hides it), and sixteen wavefronts leave each 128
+// VGPRs and, next to the 32 KB slot table, 7 KB of LDS.  So this kernel takes items whose stream bytes
+// are few: a segment of the 64 streams of a tile (decoder checkpoints), or a whole tile when tiles are
+// low.  What such an item reads of the tile body is a window of at most kWinRows rows, staged as it lies
+// in memory (row r of the window at 64 r, one byte per lane: the stream pointer of a lane moves by 64),
+// which takes no lane exchanges and no VALU work.  A wavefront walks its list of items with what an item
+// needs from memory asked for ahead: the checkpoints of the item after the next are requested, and the
+// cache lines of the next item's window and first sign|mantissa rows are touched, before the current
+// item's loop starts, so that between two items a wavefront waits for cache hits, not for HBM.
+constexpr int kSegWaves = 16;
+constexpr uint32_t kWinRows = 112;
+constexpr int kWinPieces = (int)(kWinRows * 64 / 1024);  // 16 bytes per lane each
+constexpr uint32_t kWinBytes = kWinRows * 64;
+static_assert(kWinRows * 64 % 1024 == 0 && kSlotTableBytes + kSegWaves * kWinBytes <= kLdsLimit, "windows exceed the LDS");
+
+// What an item reads before its window is known (requested two items ahead, looked at one item ahead).
+struct SegRaw {
+    uint32_t state, row, row_end;  // per lane, as stored: decoder state, row of the next unread byte at the
+                                   // item's first row and at its end
+    uint32_t off, depth;           // the tile's body: byte offset in the stream, rows
+};
+// An item ready to be staged: lane state, window, and whether the hand-scheduled loop can take it.
+struct SegItem {
+    uint32_t vk, tn;
+    uint32_t state;
+    int32_t row;
+    uint32_t lo, rows;  // first body row of the window, rows in it
+    uint64_t base;      // byte offset of the tile body
+    bool fast;
+};
+
+__device__ __forceinline__ void seg_request(const LinearArgs &a, uint32_t vk, uint32_t tn, int lane, SegRaw &m) {
+    const uint32_t tk = vk / a.segs, seg = vk % a.segs, tile = tk * a.tiles_n + tn;
+    m.off = a.tile_offsets[tile];
+    m.depth = a.tile_max_lens[tile];
+    const uint2 *ck = a.ckpt + ((size_t)tile * (a.segs - 1)) * 64 + lane;  // (only read when segs > 1)
+    if (seg == 0) {
+        m.state = a.states[(size_t)tile * 64 + lane];
+        m.row = 0x7fffffffu;
+    } else {
+        const uint2 v = ck[(size_t)(seg - 1) * 64];
+        m.state = v.x;
+        m.row = v.y;
+    }
+    m.row_end = seg + 1 < a.segs ? ck[(size_t)seg * 64].y : 0xffffffffu;
+}
+
+__device__ __forceinline__ void seg_resolve(const LinearArgs &a, uint32_t vk, uint32_t tn, int lane, const SegRaw &m,
+                                            SegItem &it) {
+    const uint32_t tk = vk / a.segs, seg = vk % a.segs;
+    const uint32_t half = a.th / 2, seglen = half / a.segs, hsel = lane / 32, c = lane % 32;
+    const uint32_t k0 = tk * a.th + hsel * half + seg * seglen;
+    it.vk = vk;
+    it.tn = tn;
+    it.base = m.off;
+    uint32_t depth = m.depth;
+    if (it.base + (uint64_t)depth * 64 > a.stream_len) depth = 0;  // a body that would run past the stream is not read
+    it.state = m.state;
+    it.row = min((int32_t)m.row, (int32_t)depth - 1);
+    const int32_t row_end = min((int32_t)m.row_end, it.row);
+    uint32_t my_steps = 0;
+    if (tn * 32 + c < a.N && k0 < a.K) my_steps = min(seglen, a.K - k0);
+    const bool full = __builtin_amdgcn_ballot_w64(my_steps != seglen) == 0;
+    // rows of the body the item can touch: from the lowest row a lane has reached by the item's end (the byte
+    // there is fetched ahead, never used) to the highest row a lane starts at
+    const int32_t lo = max(wave_min_i32(row_end), 0), hi = wave_max_i32(it.row);
+    it.lo = (uint32_t)lo;
+    it.rows = hi >= lo ? (uint32_t)(hi - lo + 1) : 0u;
+    it.fast = full && a.fast_ok && it.rows <= kWinRows && seglen % 16 == 0;
+}
+
+// Touches the cache lines the item's start will read: its window of the body (lanes 0..55, a 128-byte line
+// each) and the first 128 rows of both halves of its sign|mantissa rows (all lanes).  The values are not
+// used; the loads bring the lines next to the CU while the previous item still decodes.
+__device__ __forceinline__ uint32_t seg_touch(const LinearArgs &a, const SegItem &it, int lane) {
+    uint32_t t = 0;
+    if (!it.fast) return t;
+    const uint32_t tk = it.vk / a.segs, seg = it.vk % a.segs, tile = tk * a.tiles_n + it.tn;
+    const uint32_t half = a.th / 2, seglen = half / a.segs;
+    if ((uint32_t)lane * 128 < it.rows * 64)
+        t = *reinterpret_cast<const volatile uint32_t *>(a.stream + it.base + (size_t)it.lo * 64 + lane * 128);
+    const uint32_t hsel = lane / 32, line = lane % 32;  // 4 sign|mantissa rows of a tile make a line
+    if (line * 4 < seglen)
+        t += *reinterpret_cast<const volatile uint32_t *>(a.man_tiled + (size_t)tile * a.th * 32 +
+                                                          (size_t)(hsel * half + seg * seglen + line * 4) * 32);
+    return t;
+}
+
+// The item's window, memory -> LDS as it lies (piece g = bytes [1024 g + 16 lane, + 16) of the window).
+// Every lane loads every piece, from the window's first bytes where its own lie outside: loads without
+// conditions can all be in flight together.
+__device__ __forceinline__ void seg_stage(const LinearArgs &a, const SegItem &it, uint8_t *stage, int lane) {
+    const uint32_t bytes = it.rows * 64;
+    if (bytes == 0) return;
+    const uint8_t *src = a.stream + it.base + (size_t)it.lo * 64;
+    u32x4 w[kWinPieces];
+#pragma unroll
+    for (int g = 0; g < kWinPieces; ++g) {
+        const uint32_t o = (uint32_t)g * 1024 + lane * 16;
+        w[g] = *reinterpret_cast<const u32x4 *>(src + (o < bytes ? o : 0u));
+    }
+#pragma unroll
+    for (int g = 0; g < kWinPieces; ++g) {
+        const uint32_t o = (uint32_t)g * 1024 + lane * 16;
+        if (o < bytes) *reinterpret_cast<u32x4 *>(stage + o) = w[g];
+    }
+}
+
+// One staged item through the hand-scheduled loop, accumulating into acc (and acc2 for x rows 32..63).
+template <int MB>
+__device__ __forceinline__ void seg_run(const LinearArgs &a, const SegItem &it, const uint8_t *stage, int lane,
+                                        f32x16 &acc, f32x16 &acc2) {
+    const uint32_t tk = it.vk / a.segs, seg = it.vk % a.segs, tile = tk * a.tiles_n + it.tn;
+    const uint32_t half = a.th / 2, seglen = half / a.segs, hsel = lane / 32, c = lane % 32;
+    const uint32_t k0 = tk * a.th + hsel * half + seg * seglen;
+    FastLane st;
+    st.X = it.state << 3;
+    const int32_t rel = it.row - (int32_t)it.lo;  // this lane's next byte, in rows of the window (< 0: none left)
+    st.q = (uint32_t)(uintptr_t)stage + (uint32_t)(rel * 64 + lane);
+    st.n1 = rel >= 0 ? stage[rel * 64 + lane] : 0;
+    const uint32_t m = c;  // row of x this lane feeds to the (first) MFMA
+    const bool m_ok = m < a.M, m2_ok = MB == 2 && m + 32 < a.M;
+    const uint64_t mbase = reinterpret_cast<uint64_t>(a.man_tiled + (size_t)tile * a.th * 32);
+    // readfirstlane returns a signed int: widen through uint32_t, not by sign extension
+    const uint32_t mb_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(mbase >> 32));
+    const uint32_t mb_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)mbase);
+    const uint64_t mb_u = ((uint64_t)mb_hi << 32) | (uint64_t)mb_lo;
+    const uint32_t moff = (hsel * half + seg * seglen) * 32 + (c & ~3u);
+    const uint32_t man_sel = 0x04040000u + (c & 3u) * 0x01010101u;
+    uint64_t xb = reinterpret_cast<uint64_t>(a.x);
+    uint32_t xo = ((m_ok ? m : 0) * a.x_stride + k0) * 2u, xo2 = ((m2_ok ? m + 32 : 0) * a.x_stride + k0) * 2u, xstep = 16;
+    if (a.xf) {
+        const uint32_t kbs = a.K / 8;
+        xb = reinterpret_cast<uint64_t>(a.xf);
+        xo = ((k0 / 8) * 32 + c) * 16;
+        xo2 = xo + kbs * 32 * 16;
+        xstep = 32 * 16;
+    }
+    if (MB == 2)
+        linear_tile_asm2(st, acc, acc2, mb_u, moff, xb, xo, xo2, xstep, man_sel, seglen / 8, 64);
+    else
+        linear_tile_asm(st, acc, mb_u, moff, xb, xo, xstep, man_sel, seglen / 8, 64);
+}
+
+// An item that the loop above cannot take (ragged edges, a window larger than kWinRows, a plain-weight run).
+template <int MB>
+__device__ __forceinline__ void seg_cold_item(const LinearArgs &a, uint32_t vk, uint32_t tn, const uint2 *tab,
+                                                        uint8_t *stage, int lane, f32x16 &acc, f32x16 &acc2) {
+    linear_one_item<MB, 0, true>(a, vk, tn, tab, stage, lane, acc, acc2);
+}
+
+// Jobs.  With VK = tiles_k * segs items per column tile:
+//   VK >= 16: a job is one column tile and one chunk of its items, vk in [chunk * 16 R, (chunk + 1) * 16 R);
+//     wavefront w takes item chunk * 16 R + 16 r + w in its round r and keeps one accumulator over its R items;
+//   VK < 16: a job is 16 / VK neighbouring column tiles with all their items, wavefront w item w % VK of
+//     column tile w / VK (R = 1, one chunk).
+// At the end of a job the accumulators that belong to one column tile are added through LDS in wavefront
+// order and the sum goes to the output (one chunk per column tile) or to plane `chunk` of the fp32
+// workspace.  Which wavefront adds what is fixed by the shape and the CU count alone, so the same job on
+// a plain bf16 weight (LinearArgs::dense_w) gives the same bits.
+struct SegJobs {
+    uint32_t VK, R, chunk_items, chunks, cols, per_col, jobs;
+    __device__ __forceinline__ void init(const LinearArgs &a) {
+        VK = a.tiles_k * a.segs;
+        if (VK >= (uint32_t)kSegWaves) {
+            R = a.rounds;
+            chunk_items = kSegWaves * R;
+            chunks = (VK + chunk_items - 1) / chunk_items;  // == a.P
+            cols = 1;
+            per_col = kSegWaves;
+            jobs = a.tiles_n * chunks;
+        } else {
+            R = 1;
+            chunk_items = VK;
+            chunks = 1;
+            cols = kSegWaves / VK;
+            per_col = VK;
+            jobs = (a.tiles_n + cols - 1) / cols;
+        }
+    }
+    // item of wavefront `wave` in round r of job `job`: false if there is none
+    __device__ __forceinline__ bool item(const LinearArgs &a, uint32_t job, uint32_t r, uint32_t wave, uint32_t &vk,
+                                         uint32_t &tn) const {
+        if (cols == 1) {
+            tn = job % a.tiles_n;
+            vk = (job / a.tiles_n) * chunk_items + r * kSegWaves + wave;
+            return vk < VK;
+        }
+        tn = job * cols + wave / per_col;
+        vk = wave % per_col;
+        return wave < cols * per_col && tn < a.tiles_n;
+    }
+};
+
+// grid: any number of workgroups (one per CU); workgroup j takes jobs j, j + gridDim.x, ...
+#ifdef CI_PROBE
+__device__ uint64_t g_probe[64 * 64];
+#define PROBE(k) do { if (blockIdx.x == 0 && lane == 0 && pcount < 60) g_probe[wave * 64 + pcount++] = ((uint64_t)(k) << 56) | (wall_clock64() & 0xffffffffffffffull); } while (0)
+#else
+#define PROBE(k) do { } while (0)
+#endif
+template <int MB>
+__global__ __launch_bounds__(kSegWaves *kWave) void fused_linear32_seg_kernel(LinearArgs a) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    const uint2 *tab = reinterpret_cast<const uint2 *>(lds);
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+#ifdef CI_PROBE
+    int pcount = 0;
+#endif
+    PROBE(1);
+    uint8_t *stage = lds + kSlotTableBytes + (size_t)wave * kWinBytes;
+    SegJobs jb;
+    jb.init(a);
+    const uint32_t my_jobs = blockIdx.x < jb.jobs ? (jb.jobs - blockIdx.x + gridDim.x - 1) / gridDim.x : 0u;
+    const uint32_t slots = my_jobs * jb.R;  // this wavefront's sequence of (job, round) slots, some without an item
+    auto slot_item = [&](uint32_t sl, uint32_t &vk, uint32_t &tn) {
+        return jb.item(a, blockIdx.x + (sl / jb.R) * gridDim.x, sl % jb.R, (uint32_t)wave, vk, tn);
+    };
+    auto next_slot = [&](uint32_t sl, uint32_t &vk, uint32_t &tn) {  // first slot >= sl that has an item, or `slots`
+        while (sl < slots && !slot_item(sl, vk, tn)) ++sl;
+        return sl;
+    };
+    const bool coded = a.dense_w == nullptr;
+
+    // the first item's inputs are on their way while the table is copied
+    SegRaw raw;
+    SegItem nxt;
+    nxt.fast = false;
+    uint32_t vk_n = 0, tn_n = 0, vk_nn = 0, tn_nn = 0;
+    uint32_t s_nxt = next_slot(0, vk_n, tn_n), s_nn = slots;  // the next slot with an item, and the one after
+    if (coded && s_nxt < slots) seg_request(a, vk_n, tn_n, lane, raw);
+    if (coded && a.slot_table) {
+        const u32x4 *src = reinterpret_cast<const u32x4 *>(a.slot_table);
+        u32x4 *dst = reinterpret_cast<u32x4 *>(lds);
+        const u32x4 e0 = src[threadIdx.x * 2], e1 = src[threadIdx.x * 2 + 1];
+        dst[threadIdx.x * 2] = e0;
+        dst[threadIdx.x * 2 + 1] = e1;
+    } else if (coded) {
+        build_slot_table_x8(reinterpret_cast<uint2 *>(lds), a.tables, a.slot_map, threadIdx.x, kSegWaves * kWave);
+    }
+    if (coded && s_nxt < slots) {
+        seg_resolve(a, vk_n, tn_n, lane, raw, nxt);
+        s_nn = next_slot(s_nxt + 1, vk_nn, tn_nn);
+        if (s_nn < slots) seg_request(a, vk_nn, tn_nn, lane, raw);
+    }
+    __syncthreads();
+    PROBE(2);
+
+    const uint32_t hsel = lane / 32, c = lane % 32;
+    f32x16 acc, acc2;
+    for (uint32_t sl = 0; sl < slots; ++sl) {
+        if (sl % jb.R == 0) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[v] = acc2[v] = 0.f;
+        }
+        const uint32_t job = blockIdx.x + (sl / jb.R) * gridDim.x;
+        uint32_t vk, tn;
+        if (slot_item(sl, vk, tn)) {
+            if (!coded) {
+                seg_cold_item<MB>(a, vk, tn, tab, stage, lane, acc, acc2);
+            } else {
+                // (sl == s_nxt: the slots with an item are visited in order)
+                const SegItem cur = nxt;
+                PROBE(3);
+                if (cur.fast) seg_stage(a, cur, stage, lane);
+                PROBE(4);
+                uint32_t touched = 0;
+                s_nxt = s_nn;
+                vk_n = vk_nn;
+                tn_n = tn_nn;
+                if (s_nxt < slots) {
+                    seg_resolve(a, vk_n, tn_n, lane, raw, nxt);
+                    touched = seg_touch(a, nxt, lane);
+                    s_nn = next_slot(s_nxt + 1, vk_nn, tn_nn);
+                    if (s_nn < slots) seg_request(a, vk_nn, tn_nn, lane, raw);
+                }
+                PROBE(cur.fast ? 5 : 9);
+                if (cur.fast)
+                    seg_run<MB>(a, cur, stage, lane, acc, acc2);  // (a wavefront's LDS operations complete in order)
+                else
+                    seg_cold_item<MB>(a, vk, tn, tab, stage, lane, acc, acc2);
+                asm volatile("" ::"v"(touched));  // the touching loads end here
+                PROBE(6);
+            }
+        }
+        if (sl % jb.R != jb.R - 1) continue;
+        // End of a job: add the accumulators of each column tile in wavefront order.  Every wavefront stores
+        // its fragment as [v][lane] floats in its own window area; wavefront w then adds row v = w of the
+        // fragments of each column tile of the job, which is column (w/4)*8 + (lane/32)*4 + w%4 of that tile
+        // for x row lane%32 (MFMA 32x32 result layout: register v of lane l is row (v/4)*8 + (l/32)*4 + v%4,
+        // column l%32).
+        const uint32_t chunk = jb.cols == 1 ? job / a.tiles_n : 0u;
+        float *red = reinterpret_cast<float *>(lds + kSlotTableBytes);
+#pragma unroll
+        for (int g = 0; g < MB; ++g) {
+            const f32x16 &part = g ? acc2 : acc;
+            __syncthreads();  // the window areas are free: every wavefront has left its loop
+#pragma unroll
+            for (int v = 0; v < 16; ++v) red[(size_t)wave * (kWinBytes / 4) + v * kWave + lane] = part[v];
+            __syncthreads();
+            for (uint32_t t = 0; t < jb.cols; ++t) {
+                const uint32_t col_tile = jb.cols == 1 ? job % a.tiles_n : job * jb.cols + t;
+                float sum = 0.f;
+                for (uint32_t i = 0; i < jb.per_col; ++i)
+                    sum += red[(size_t)(t * jb.per_col + i) * (kWinBytes / 4) + wave * kWave + lane];
+                const uint32_t n = col_tile * 32 + (wave / 4) * 8 + hsel * 4 + (wave % 4), mg = c + 32 * g;
+                if (col_tile < a.tiles_n && mg < a.M && n < a.N) {
+                    if (a.P == 1)
+                        a.out[(size_t)mg * a.out_stride + n] = finish_bf16(sum, a.bias, n);
+                    else
+                        a.partial[((size_t)chunk * a.M + mg) * a.N + n] = sum;
+                }
+            }
+        }
+        __syncthreads();  // before the next window is written over the fragments
+        PROBE(7);
+    }
+}
+#ifdef CI_PROBE
+extern "C" int ci_debug_probe(uint64_t *h_out) { return hipMemcpyFromSymbol(h_out, HIP_SYMBOL(g_probe), sizeof(uint64_t) * 64 * 64) == hipSuccess ? 0 : 2; }
+#endif
 
 // Any tile width, either tiled layout: one thread per stream, eight rows of x per pass.
 // Partial sums (one per stream, i.e. per (k-tile[, half])) go to the fp32 workspace.
@@ -581,26 +918,59 @@ static size_t x_fragment_bytes(uint32_t M, uint32_t K, bool fast_plan) {
 }
 
 struct LinearPlan {
-    bool fast, resident;
+    bool fast, resident, seg16;
     uint32_t kw, nw, P, segs;
+    uint32_t rounds;  // seg16: items of a job per wavefront
 };
+
+// Rows (decode steps) of the longest item the sixteen-wavefront kernel is given: bf16 weight exponents take
+// about 0.35 bytes per symbol, and the lanes of a tile drift apart by some twenty rows, so 256 rows stay
+// below kWinRows.  (An item whose window turns out larger takes the guarded path.)
+constexpr uint32_t kSegMaxRows = 256;
+
+// fused_linear32_seg_kernel: items per wavefront and job (R) for a weight of VK = tiles_k * segs items per
+// column tile on `cus` CUs, by the time the jobs take (rounds of jobs on the chip x R item lengths, and
+// about half an item for the reduction launch when a column tile is cut into several chunks); the largest
+// R among equals, which leaves the fewest chunks.
+static uint32_t seg_rounds(uint32_t VK, uint32_t tiles_n, uint32_t cus) {
+    const uint32_t r_max = ceil_div(VK, (uint32_t)kSegWaves);
+    uint32_t best = 1;
+    uint64_t best_cost = ~0ull;
+    for (uint32_t R = 1; R <= r_max; ++R) {
+        const uint32_t chunks = ceil_div(VK, kSegWaves * R);
+        const uint64_t jobs = (uint64_t)tiles_n * chunks;
+        const uint64_t cost = 2 * ((jobs + cus - 1) / cus) * R + (chunks > 1 ? 1 : 0);
+        if (cost <= best_cost) {
+            best_cost = cost;
+            best = R;
+        }
+    }
+    return best;
+}
 
 // Tiles from which every tile gets its own wavefront of a resident workgroup: more than a chip of
 // 8-wavefront workgroups holds at once (256 CUs x 8).
 constexpr uint32_t kResidentMinTiles = 2049;
-constexpr uint32_t kPlanCus = 256;  // CUs assumed when segments are suggested
 
 // segments: 1, or the number of segments the caller's checkpoints cut every stream into.
+// cus: CUs of the device, or 0 for the plan that needs the largest workspace.
 static LinearPlan plan_linear(uint32_t M, uint32_t K, uint32_t th, uint32_t tw, uint32_t tiles_n, bool dense,
-                              bool stream_aligned, uint32_t segments = 1) {
+                              bool stream_aligned, uint32_t segments = 1, uint32_t cus = 0) {
     LinearPlan p;
     const uint32_t tiles_k = ceil_div(K, th);
     p.fast = !dense && tw == 32 && th % 16 == 0 && stream_aligned;
     p.segs = 1;
+    p.rounds = 1;
     if (p.fast && M <= 64 && segments > 1 && (th / 2) % (16 * segments) == 0) p.segs = segments;
-    p.resident = p.fast && M <= 64 &&
+    // items short enough for their windows of the body to fit 7 KB of LDS go to the sixteen-wavefront kernel
+    p.seg16 = p.fast && M <= 64 && (th / 2) % (16 * p.segs) == 0 && th / 2 / p.segs <= kSegMaxRows;
+    p.resident = !p.seg16 && p.fast && M <= 64 &&
                  (p.segs > 1 || (tiles_k >= 2 && (uint64_t)tiles_k * tiles_n >= kResidentMinTiles));
-    if (p.resident) {
+    if (p.seg16) {
+        p.kw = p.nw = 1;
+        p.rounds = cus ? seg_rounds(tiles_k * p.segs, tiles_n, cus) : 1;
+        p.P = ceil_div(tiles_k * p.segs, kSegWaves * p.rounds);
+    } else if (p.resident) {
         p.kw = p.nw = 1;
         p.P = tiles_k * p.segs;
     } else if (p.fast) {
@@ -639,20 +1009,22 @@ extern "C" size_t ci_fused_linear_workspace_bytes(uint32_t M, uint32_t K, uint32
     return ci_fused_linear_workspace_bytes_segmented(M, K, N, tile_height, tile_width, dense, 1);
 }
 
-// Segments per stream for a weight of this shape, from measurements on 256 CUs x 12 wavefronts: as many
-// (2, 4 or 8) as still give every (tile, segment) a wavefront of its own in one round -- the time is
-// then one chain of th / (2 segments) steps instead of th / 2 -- and 2 for weights that take several
-// rounds anyway (shorter items fill the last round better); 1 in between, where the chip is busy with
-// whole tiles.
+// Segments per stream for a weight of this shape: the fewest (items as long as possible: every item pays
+// for its own start) that make an item kSegMaxRows rows or less and the items at least 70 % of the
+// wavefronts a chip of 256 CUs x 16 holds; the most that keep an item 64 rows or more if none gets
+// there; 1 if the tile shape allows none.
 extern "C" uint32_t ci_suggest_segments(uint32_t K, uint32_t N, uint32_t tile_height, uint32_t tile_width) {
     if (tile_height == 0 || tile_width != 32 || tile_height % 16) return 1;
     const uint64_t tiles = (uint64_t)ceil_div(K, tile_height) * ceil_div(N, tile_width);
-    const uint64_t one_round = (uint64_t)kPlanCus * kPersistWaves;
-    auto fits = [&](uint32_t segs) { return (tile_height / 2) % (16 * segs) == 0; };
-    for (uint32_t segs = 8; segs >= 2; segs /= 2)
-        if (tiles * segs <= one_round && fits(segs)) return segs;
-    if (tiles >= kResidentMinTiles && fits(2)) return 2;
-    return 1;
+    const uint32_t half = tile_height / 2;
+    uint32_t best = 1;
+    for (uint32_t segs = 1; segs <= 64; segs *= 2) {
+        if (half % (16 * segs) || half / segs < 64) break;
+        if (half / segs > kSegMaxRows) continue;
+        best = segs;
+        if (tiles * segs * 10 >= 7ull * 256 * kSegWaves) break;
+    }
+    return best;
 }
 
 static int fused_linear_impl(const uint16_t *d_x, uint32_t M, uint32_t K, uint32_t N, uint32_t x_stride,
@@ -661,7 +1033,8 @@ static int fused_linear_impl(const uint16_t *d_x, uint32_t M, uint32_t K, uint32
                              const uint32_t *d_meta1, const uint8_t *d_man_tiled, uint32_t th, uint32_t tw,
                              const uint16_t *d_bias, uint16_t *d_out, uint32_t out_stride, void *d_workspace,
                              size_t workspace_bytes, bool dense, hipStream_t s, const uint16_t *d_plain_w = nullptr,
-                             const void *d_checkpoints = nullptr, uint32_t segments = 1) {
+                             const void *d_checkpoints = nullptr, uint32_t segments = 1,
+                             const void *d_slot_table = nullptr) {
     if (M == 0 || N == 0) return CI_OK;
     if (K == 0) return fail(CI_ERR_ARG, "fused linear: K is 0");
     if (!d_x || !d_out) return fail(CI_ERR_ARG, "fused linear: null pointer");
@@ -708,10 +1081,13 @@ static int fused_linear_impl(const uint16_t *d_x, uint32_t M, uint32_t K, uint32
         if (!d_plain_w && (!d_checkpoints || !aligned(d_checkpoints, 8)))
             return fail(CI_ERR_ARG, "fused linear: segments without (8-byte aligned) checkpoints");
     }
-    const LinearPlan p = plan_linear(M, K, th, tw, a.tiles_n, dense, d_plain_w || aligned(d_stream, 16), segments);
+    // (planned for no device in particular first: the checks below run before the first HIP call)
+    LinearPlan p = plan_linear(M, K, th, tw, a.tiles_n, dense, d_plain_w || aligned(d_stream, 16), segments);
     if (d_plain_w && !p.fast)
         return fail(CI_ERR_ARG, "plain-weight linear: only the 32-column tiling (tile height a multiple of 16)");
     a.ckpt = static_cast<const uint2 *>(d_checkpoints);
+    a.slot_table = static_cast<const uint2 *>(d_slot_table);
+    a.rounds = p.rounds;
     a.segs = p.segs;
     a.kw = p.kw;
     a.nw = p.nw;
@@ -719,13 +1095,22 @@ static int fused_linear_impl(const uint16_t *d_x, uint32_t M, uint32_t K, uint32
     a.partial = static_cast<float *>(d_workspace);
     // The one-thread-per-stream kernel writes fp32 partial sums and leaves output, bias and rounding to the
     // reduction, also when there is a single partial sum per output.
-    const bool via_workspace = p.P > 1 || (!p.fast && !p.resident);
+    bool via_workspace = p.P > 1 || (!p.fast && !p.resident);
     size_t partial_bytes = 0;
     if (via_workspace) {
         partial_bytes = (size_t)p.P * M * N * sizeof(float);
         if (!d_workspace || workspace_bytes < partial_bytes)
             return fail(CI_ERR_CAPACITY, "fused linear: workspace needs %zu bytes, got %zu", partial_bytes, workspace_bytes);
         if (!aligned(d_workspace, 4)) return fail(CI_ERR_ARG, "fused linear: workspace must be 4-byte aligned");
+    }
+    uint32_t cus = 0;
+    if (int rc = cu_count(&cus)) return rc;
+    if (p.seg16) {  // how a column tile's items are cut into jobs depends on the CUs there are to fill
+        p = plan_linear(M, K, th, tw, a.tiles_n, dense, d_plain_w || aligned(d_stream, 16), segments, cus);
+        a.P = p.P;
+        a.rounds = p.rounds;
+        via_workspace = p.P > 1;
+        partial_bytes = via_workspace ? (size_t)p.P * M * N * sizeof(float) : 0;
     }
     // the fragment copy of x goes behind the partials when the caller's workspace has room for it
     a.xf = nullptr;
@@ -742,9 +1127,19 @@ static int fused_linear_impl(const uint16_t *d_x, uint32_t M, uint32_t K, uint32
         }
     }
 
-    if (p.resident) {
-        uint32_t cus = 0;
-        if (int rc = cu_count(&cus)) return rc;
+    if (p.seg16) {
+        CI_ALLOW_FULL_LDS(fused_linear32_seg_kernel<1>);
+        CI_ALLOW_FULL_LDS(fused_linear32_seg_kernel<2>);
+        const uint32_t VK = a.tiles_k * p.segs;
+        const uint32_t jobs = VK >= (uint32_t)kSegWaves ? a.tiles_n * p.P : ceil_div(a.tiles_n, kSegWaves / VK);
+        const dim3 grid(jobs < cus ? jobs : cus), block(kSegWaves * kWave);
+        const uint32_t lds_bytes = kSlotTableBytes + kSegWaves * kWinBytes;
+        if (M > 32)
+            hipLaunchKernelGGL(fused_linear32_seg_kernel<2>, grid, block, lds_bytes, s, a);
+        else
+            hipLaunchKernelGGL(fused_linear32_seg_kernel<1>, grid, block, lds_bytes, s, a);
+        CI_LAUNCH_CHECK("fused_linear32_seg_kernel");
+    } else if (p.resident) {
         CI_ALLOW_FULL_LDS(fused_linear32_resident_kernel<1>);
         CI_ALLOW_FULL_LDS(fused_linear32_resident_kernel<2>);
         const dim3 grid(cus), block(kPersistWaves * kWave);
@@ -821,6 +1216,69 @@ extern "C" int ci_fused_linear_ilp2_segmented(const uint16_t *d_x, uint32_t M, u
                              d_tile_offsets, d_tile_max_lens, d_man_tiled, tile_height, tile_width, d_bias, d_out,
                              out_stride, d_workspace, workspace_bytes, false, static_cast<hipStream_t>(stream), nullptr,
                              d_checkpoints, segments);
+}
+
+namespace ci {
+__global__ __launch_bounds__(256) void slot_table_kernel(const uint32_t *tables, const uint8_t *slot_map, uint2 *out) {
+    build_slot_table_x8(out, tables, slot_map, blockIdx.x * 256 + threadIdx.x, gridDim.x * 256);
+}
+}  // namespace ci
+
+extern "C" int ci_build_slot_table(const uint32_t *d_tables, const uint8_t *d_slot_map, void *d_slot_table,
+                                   size_t slot_table_bytes, ci_stream_t stream) {
+    if (!d_tables || !d_slot_map || !d_slot_table) return fail(CI_ERR_ARG, "ci_build_slot_table: null pointer");
+    if (slot_table_bytes < CI_SLOT_TABLE_BYTES)
+        return fail(CI_ERR_CAPACITY, "ci_build_slot_table: the table takes %d bytes, got %zu", CI_SLOT_TABLE_BYTES,
+                    slot_table_bytes);
+    if (!aligned(d_slot_map, 4) || !aligned(d_slot_table, 16))
+        return fail(CI_ERR_ARG, "ci_build_slot_table: slot_map must be 4-byte, the table 16-byte aligned");
+    hipLaunchKernelGGL(slot_table_kernel, dim3(4), dim3(256), 0, static_cast<hipStream_t>(stream), d_tables, d_slot_map,
+                       static_cast<uint2 *>(d_slot_table));
+    CI_LAUNCH_CHECK("slot_table_kernel");
+    return CI_OK;
+}
+
+extern "C" int ci_tiled_weight_check(const ci_tiled_weight *w) {
+    if (!w) return fail(CI_ERR_ARG, "weight descriptor: null");
+    if (w->K == 0 || w->N == 0 || w->tile_height == 0 || w->tile_width == 0 || (w->tile_height & 1))
+        return fail(CI_ERR_ARG, "weight descriptor: bad shape %u x %u, tile %u x %u", w->K, w->N, w->tile_height,
+                    w->tile_width);
+    const uint64_t tiles = (uint64_t)ceil_div(w->K, w->tile_height) * ceil_div(w->N, w->tile_width);
+    if (!w->d_states || !w->d_tables || !w->d_slot_map || !w->d_tile_offsets || !w->d_tile_max_lens || !w->d_man_tiled)
+        return fail(CI_ERR_ARG, "weight descriptor: null pointer");
+    if (w->stream_len && !w->d_stream) return fail(CI_ERR_ARG, "weight descriptor: null stream");
+    if (!aligned(w->d_slot_map, 4)) return fail(CI_ERR_ARG, "weight descriptor: slot_map must be 4-byte aligned");
+    if (w->n_states < tiles * 2 * w->tile_width)
+        return fail(CI_ERR_ARG, "weight descriptor: %llu states, the shape has %llu streams",
+                    (unsigned long long)w->n_states, (unsigned long long)(tiles * 2 * w->tile_width));
+    if (w->n_tiles < tiles)
+        return fail(CI_ERR_ARG, "weight descriptor: tile metadata for %llu tiles, the shape has %llu",
+                    (unsigned long long)w->n_tiles, (unsigned long long)tiles);
+    if (w->man_len < tiles * w->tile_height * w->tile_width)
+        return fail(CI_ERR_ARG, "weight descriptor: sign|mantissa plane of %llu bytes, the tiles take %llu",
+                    (unsigned long long)w->man_len, (unsigned long long)(tiles * w->tile_height * w->tile_width));
+    if (w->segments > 1) {
+        if (!w->d_checkpoints || !aligned(w->d_checkpoints, 8))
+            return fail(CI_ERR_ARG, "weight descriptor: segments without (8-byte aligned) checkpoints");
+        const size_t need = ci_checkpoint_bytes(w->K, w->N, w->tile_height, w->tile_width, w->segments);
+        if (need == 0 || w->checkpoint_bytes != need)
+            return fail(CI_ERR_ARG, "weight descriptor: checkpoints of %llu bytes, %u segments of this shape take %zu",
+                        (unsigned long long)w->checkpoint_bytes, w->segments, need);
+    }
+    if (w->d_slot_table && (w->slot_table_bytes != CI_SLOT_TABLE_BYTES || !aligned(w->d_slot_table, 16)))
+        return fail(CI_ERR_ARG, "weight descriptor: the slot table is %d bytes, 16-byte aligned", CI_SLOT_TABLE_BYTES);
+    return CI_OK;
+}
+
+extern "C" int ci_fused_linear_tiled(const ci_tiled_weight *w, const uint16_t *d_x, uint32_t M, uint32_t x_stride,
+                                     const uint16_t *d_bias, uint16_t *d_out, uint32_t out_stride, void *d_workspace,
+                                     size_t workspace_bytes, ci_stream_t stream) {
+    if (int rc = ci_tiled_weight_check(w)) return rc;
+    return fused_linear_impl(d_x, M, w->K, w->N, x_stride, w->d_stream, w->stream_len, w->d_states, w->d_tables,
+                             w->d_slot_map, w->d_tile_offsets, w->d_tile_max_lens, w->d_man_tiled, w->tile_height,
+                             w->tile_width, d_bias, d_out, out_stride, d_workspace, workspace_bytes, false,
+                             static_cast<hipStream_t>(stream), nullptr, w->segments > 1 ? w->d_checkpoints : nullptr,
+                             w->segments > 1 ? w->segments : 1, w->d_slot_table);
 }
 
 extern "C" int ci_plain_linear_same_order(const uint16_t *d_x, uint32_t M, uint32_t K, uint32_t N, uint32_t x_stride,

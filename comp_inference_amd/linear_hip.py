@@ -119,19 +119,21 @@ def _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, met
     # device copies must stay referenced until the launch has been enqueued
     st, tb, sm = _lib.as_u32(initial_states, dev), _lib.as_u32(tables, dev), _lib.as_u8(slot_map, dev)
     m0, m1 = _lib.as_u32(meta0, dev), _lib.as_u32(meta1, dev)
-    if segments > 1:
-        ck = checkpoints.to(dev).contiguous()
-        if ck.dtype != torch.int64 or ck.numel() * 8 != lib().ci_checkpoint_bytes(K, N, int(tile_k), int(tile_n), segments):
-            raise RuntimeError("checkpoints do not belong to this weight shape, tiling and segment count")
-        check(lib().ci_fused_linear_ilp2_segmented(
-            ptr(x2), M, K, N, x2.stride(0), ptr(stream_t), C.c_uint64(stream_t.numel()), ptr(st), ptr(tb), ptr(sm),
-            ptr(m0), ptr(m1), ptr(man), int(tile_k), int(tile_n), ptr(ck), segments, ptr(b), ptr(result),
-            result.stride(0), ptr(ws), C.c_size_t(ws_bytes), _lib.stream_handle(dev)))
+    if not dense:
+        ck = None
+        if segments > 1:
+            ck = checkpoints.to(dev).contiguous()
+            if ck.dtype != torch.int64:
+                raise RuntimeError("checkpoints do not belong to this weight shape, tiling and segment count")
+        # the lengths of every operand travel with it and are checked by the library before the launch
+        w = _lib.tiled_weight(K, N, tile_k, tile_n, stream_t, st, tb, sm, m0, m1, man, ck, segments)
+        check(lib().ci_fused_linear_tiled(C.byref(w), ptr(x2), M, x2.stride(0), ptr(b), ptr(result), result.stride(0),
+                                          ptr(ws), C.c_size_t(ws_bytes), _lib.stream_handle(dev)))
     else:
-        fn = lib().ci_fused_linear_dense if dense else lib().ci_fused_linear_ilp2
-        check(fn(ptr(x2), M, K, N, x2.stride(0), ptr(stream_t), C.c_uint64(stream_t.numel()),
-                 ptr(st), ptr(tb), ptr(sm), ptr(m0), ptr(m1), ptr(man), int(tile_k), int(tile_n), ptr(b), ptr(result),
-                 result.stride(0), ptr(ws), C.c_size_t(ws_bytes), _lib.stream_handle(dev)))
+        check(lib().ci_fused_linear_dense(
+            ptr(x2), M, K, N, x2.stride(0), ptr(stream_t), C.c_uint64(stream_t.numel()), ptr(st), ptr(tb), ptr(sm),
+            ptr(m0), ptr(m1), ptr(man), int(tile_k), int(tile_n), ptr(b), ptr(result), result.stride(0), ptr(ws),
+            C.c_size_t(ws_bytes), _lib.stream_handle(dev)))
     if out is not None:
         return out
     return result.view(*x.shape[:-1], N)
@@ -165,18 +167,25 @@ class PreparedLinear:
         self.keep = (_lib.as_u8(compressed_data, dev), _lib.as_u32(initial_states, dev), _lib.as_u32(tables, dev),
                      _lib.as_u8(slot_map, dev), _lib.as_u32(tile_offsets, dev), _lib.as_u32(tile_max_lens, dev), man,
                      None if bias is None else bias.to(device=dev, dtype=torch.bfloat16).contiguous(), ck)
+        # the decoder's lookup table in the form the kernels keep in LDS: built once, copied by every launch
+        self.slot_table = torch.empty(_lib.SLOT_TABLE_BYTES, dtype=torch.uint8, device=dev)
+        with torch.cuda.device(dev):
+            check(lib().ci_build_slot_table(ptr(self.keep[2]), ptr(self.keep[3]), ptr(self.slot_table),
+                                            C.c_size_t(_lib.SLOT_TABLE_BYTES), _lib.stream_handle(dev)))
         self.need = {}
         self._bind()
 
     def _bind(self) -> None:
-        self.p = [ptr(t) for t in self.keep]
-        self.stream_len = C.c_uint64(self.keep[0].numel())
+        o = self.keep
+        self.p = [ptr(t) for t in o]
+        self.w = _lib.tiled_weight(self.K, self.N, self.tile_k, self.tile_n, o[0], o[1], o[2], o[3], o[4], o[5], o[6],
+                                   o[8], self.segments, self.slot_table)
 
     # A copy (copy.deepcopy of the owning module, pickling) gets its own tensors: the pointers are taken
     # again from them instead of travelling as numbers.
     def __getstate__(self):
         state = dict(self.__dict__)
-        del state["p"], state["stream_len"]
+        del state["p"], state["w"]
         return state
 
     def __setstate__(self, state):
@@ -198,17 +207,8 @@ class PreparedLinear:
             need = self.need[M] = lib().ci_fused_linear_workspace_bytes_segmented(M, self.K, self.N, self.tile_k,
                                                                                    self.tile_n, 0, self.segments)
         ws, ws_bytes = _pick_workspace(None, need, self.dev)
-        p = self.p
-        if self.segments > 1:
-            check(lib().ci_fused_linear_ilp2_segmented(
-                ptr(x2), M, self.K, self.N, x2.stride(0), p[0], self.stream_len, p[1], p[2], p[3], p[4], p[5], p[6],
-                self.tile_k, self.tile_n, p[8], self.segments, p[7], ptr(result), self.N, ptr(ws),
-                C.c_size_t(ws_bytes), _lib.stream_handle(self.dev)))
-        else:
-            check(lib().ci_fused_linear_ilp2(
-                ptr(x2), M, self.K, self.N, x2.stride(0), p[0], self.stream_len, p[1], p[2], p[3], p[4], p[5], p[6],
-                self.tile_k, self.tile_n, p[7], ptr(result), self.N, ptr(ws), C.c_size_t(ws_bytes),
-                _lib.stream_handle(self.dev)))
+        check(lib().ci_fused_linear_tiled(C.byref(self.w), ptr(x2), M, x2.stride(0), self.p[7], ptr(result), self.N,
+                                          ptr(ws), C.c_size_t(ws_bytes), _lib.stream_handle(self.dev)))
         return result.view(*x.shape[:-1], self.N)
 
 

@@ -357,6 +357,59 @@ int ci_decode_tiled_ilp2_segmented(const uint8_t *d_stream, uint64_t stream_len,
                                    const uint8_t *d_man_tiled, uint16_t *d_out_bf16, ci_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------
+ * A compressed weight as one descriptor with the length of every array in it.  The entry points
+ * that take it check those lengths against the shape on the host before anything is launched
+ * (CI_ERR_ARG), where the bare-pointer entry points above trust the caller: a kernel indexes
+ * states by stream, tile metadata by tile, the sign|mantissa plane by tile and row, checkpoints by
+ * (tile, segment, stream), and a short array would be read out of bounds on the GPU.  The operands are
+ * those of the reference's fused_rans_linear_triton (comp_inference/linear_triton.py:229-246), which
+ * passes torch tensors and checks nothing.  Default format only (two streams per column).
+ *
+ * d_checkpoints / segments: NULL / 0 or 1, or the index made by ci_build_checkpoints_ilp2.
+ * d_slot_table: NULL, or the 32 KB made by ci_build_slot_table; a kernel then copies the table
+ * instead of building it from d_tables and d_slot_map in every workgroup.
+ * ------------------------------------------------------------------------------------- */
+typedef struct ci_tiled_weight {
+    uint32_t K, N, tile_height, tile_width;
+    const uint8_t *d_stream;
+    uint64_t stream_len;              /* bytes */
+    const uint32_t *d_states;
+    uint64_t n_states;                /* >= tiles * 2 * tile_width */
+    const uint32_t *d_tables;         /* 256 entries */
+    const uint8_t *d_slot_map;        /* 4096 entries, 4-byte aligned */
+    const uint32_t *d_tile_offsets;
+    const uint32_t *d_tile_max_lens;
+    uint64_t n_tiles;                 /* entries in each of the two, >= tiles */
+    const uint8_t *d_man_tiled;
+    uint64_t man_len;                 /* bytes, >= tiles * tile_height * tile_width */
+    const void *d_checkpoints;
+    uint64_t checkpoint_bytes;        /* == ci_checkpoint_bytes(K, N, tile_height, tile_width, segments) */
+    uint32_t segments;
+    const void *d_slot_table;
+    uint64_t slot_table_bytes;        /* == CI_SLOT_TABLE_BYTES when d_slot_table is given */
+} ci_tiled_weight;
+
+#define CI_SLOT_TABLE_BYTES 32768
+
+/* CI_OK if every array of the descriptor is present, aligned and long enough for its shape.  Runs on
+ * the host alone (no device needed). */
+int ci_tiled_weight_check(const ci_tiled_weight *w);
+
+/* The decoder's lookup table as the kernels keep it in LDS (one 8-byte entry per 12-bit slot: the
+ * reference's slot_map and tables folded into one read, src/cuda/rans_kernels.cuh:677-690), written to
+ * d_slot_table (CI_SLOT_TABLE_BYTES, 16-byte aligned).  Derived data kept beside the weight, like the
+ * checkpoints. */
+int ci_build_slot_table(const uint32_t *d_tables, const uint8_t *d_slot_map, void *d_slot_table,
+                        size_t slot_table_bytes, ci_stream_t stream);
+
+/* Fused decompress-GEMV/GEMM on a descriptor: what ci_fused_linear_ilp2 / _segmented compute, with the
+ * lengths checked.  Workspace: ci_fused_linear_workspace_bytes_segmented(M, K, N, tile_height,
+ * tile_width, 0, segments) bytes. */
+int ci_fused_linear_tiled(const ci_tiled_weight *w, const uint16_t *d_x, uint32_t M, uint32_t x_stride,
+                          const uint16_t *d_bias, uint16_t *d_out, uint32_t out_stride, void *d_workspace,
+                          size_t workspace_bytes, ci_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------
  * Verification aids: the contraction of the fused kernels applied to a plain (uncompressed) bf16
  * weight.  No counterpart in the reference, whose tests compare the fused kernels with
  * torch.matmul within allclose(1e-2, 1e-2) (tests/test_mat_mul.py:220, :238) -- a bar that a wrong

@@ -403,7 +403,7 @@ def test_segmented_fused_linear(oracle, K, N, th, M, segments):
 def test_segment_arguments_are_checked(oracle):
     from comp_inference_amd import build_checkpoints, suggest_segments
 
-    assert suggest_segments((4096, 4096)) == 4 and suggest_segments((4096, 14336)) == 1
+    assert suggest_segments((4096, 4096)) == 8 and suggest_segments((4096, 14336)) == 2
     assert suggest_segments((4096, 28672)) == 2 and suggest_segments((4096, 4096), 1024, 64) == 1
     K, N, th = 1024, 64, 1024
     w = make_weight_kn(N, K, seed=71)
