@@ -39,9 +39,10 @@ def test_greedy_ids_equal_the_run_on_decompressed_weights(small_decoder):
 def test_logits_match_torch_matmul_on_decompressed_weights(small_decoder):
     """Teacher-forced logits of every step: bit-identical to the same-order run on the decompressed weights
     (what losslessness means for the model), and close to the decoder that runs torch.matmul on them.  The
-    two bf16 pipelines add in different orders, and a one-ulp difference in a hidden state is carried through
-    the layers behind it, so the operator-level bar (1e-2 / 1e-2) is asked of 99.9 % of the logits and every
-    logit must stay within four bf16 steps at the largest logit's magnitude."""
+    two bf16 pipelines add in different orders, and a one-step difference in a bf16 hidden state is carried
+    through the layers behind it, so element-wise operator tolerances do not apply to logits; the bar is
+    1e-2 relative on the whole logit matrix (Frobenius norm) and four bf16 steps at the largest logit's
+    magnitude on every single logit."""
     bm, dev, comp, ref, same, prompt = small_decoder
     n_new, max_len = 16, 8 + 16 + 1
     with torch.no_grad():
@@ -51,7 +52,7 @@ def test_logits_match_torch_matmul_on_decompressed_weights(small_decoder):
         ls = bm.teacher_forced(bm.Decoder(same, 2, max_len, dev), prompt, ids)
     assert lc.shape == (n_new, bm.Shape.vocab)
     assert torch.equal(lc, ls)
-    diff, bound = (lc.float() - lr.float()).abs(), ATOL + RTOL * lr.float().abs()
-    assert float((diff <= bound).float().mean()) >= 0.999
+    diff = (lc.float() - lr.float()).abs()
+    assert float(diff.norm() / lr.float().norm()) <= RTOL
     ulp = 2.0 ** (torch.floor(torch.log2(lr.float().abs().max())) - 7)
     assert float(diff.max()) <= 4 * float(ulp), (float(diff.max()), float(ulp))
