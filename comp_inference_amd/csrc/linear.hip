@@ -1281,6 +1281,56 @@ extern "C" int ci_fused_linear_tiled(const ci_tiled_weight *w, const uint16_t *d
                              w->segments > 1 ? w->segments : 1, w->d_slot_table);
 }
 
+// ---- an entry point that allocates nothing ----------------------------------------------------------
+// For callers that cannot allocate device memory (code under graph capture, tight serving loops): the
+// fused linear with its workspace -- fp32 partial sums and the fragment copy of x -- in a fixed array of
+// device memory that belongs to the library.  Every GPU the library runs on holds its own copy of the
+// array at its own address until the process ends; the address is asked for once per device.  Calls on one
+// GPU share that GPU's array, so two of them must not overlap in time (different streams, or threads).
+static __device__ __align__(256) uint8_t scratch[CI_NOALLOC_SCRATCH_BYTES];
+
+namespace ci {
+constexpr int kMaxScratchDevices = 64;
+static std::atomic<void *> g_scratch_ptr[kMaxScratchDevices];
+
+// Device address of `scratch` on the current device.
+static int scratch_address(void **out) {
+    int dev = 0;
+    CI_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxScratchDevices) return fail(CI_ERR_ARG, "no-allocation linear: device index %d", dev);
+    void *ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!ptr) {
+        CI_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));  // (two threads asking at once get the same answer)
+        if (!ptr) return fail(CI_ERR_HIP, "no-allocation linear: the scratch array has no device address");
+        g_scratch_ptr[dev].store(ptr, std::memory_order_release);
+    }
+    *out = ptr;
+    return CI_OK;
+}
+}  // namespace ci
+
+extern "C" int ci_fused_linear_tiled_noalloc(const ci_tiled_weight *w, const uint16_t *d_x, uint32_t M,
+                                             uint32_t x_stride, const uint16_t *d_bias, uint16_t *d_out,
+                                             uint32_t out_stride, ci_stream_t stream) {
+    if (int rc = ci_tiled_weight_check(w)) return rc;
+    const uint32_t segments = w->segments > 1 ? w->segments : 1;
+    const size_t need = ci_fused_linear_workspace_bytes_segmented(M, w->K, w->N, w->tile_height, w->tile_width, 0, segments);
+    if (need > (size_t)CI_NOALLOC_SCRATCH_BYTES)
+        return fail(CI_ERR_CAPACITY,
+                    "no-allocation linear: %u rows of x on a %u x %u weight take %zu bytes of workspace, the library's "
+                    "fixed scratch array has %zu; use ci_fused_linear_tiled with a workspace of the caller's",
+                    M, w->K, w->N, need, (size_t)CI_NOALLOC_SCRATCH_BYTES);
+    void *ws = nullptr;
+    if (int rc = scratch_address(&ws)) return rc;
+    // (every kernel of the plan writes the partial sums it later reads, or clears them first with a kernel of
+    // its own: what an earlier call left in the array is never read)
+    return fused_linear_impl(d_x, M, w->K, w->N, x_stride, w->d_stream, w->stream_len, w->d_states, w->d_tables,
+                             w->d_slot_map, w->d_tile_offsets, w->d_tile_max_lens, w->d_man_tiled, w->tile_height,
+                             w->tile_width, d_bias, d_out, out_stride, ws, (size_t)CI_NOALLOC_SCRATCH_BYTES, false,
+                             static_cast<hipStream_t>(stream), nullptr, segments > 1 ? w->d_checkpoints : nullptr,
+                             segments, w->d_slot_table);
+}
+
 extern "C" int ci_plain_linear_same_order(const uint16_t *d_x, uint32_t M, uint32_t K, uint32_t N, uint32_t x_stride,
                                           const uint16_t *d_w, uint32_t tile_height, uint32_t tile_width,
                                           uint32_t segments, const uint16_t *d_bias, uint16_t *d_out,

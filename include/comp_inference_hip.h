@@ -409,6 +409,21 @@ int ci_fused_linear_tiled(const ci_tiled_weight *w, const uint16_t *d_x, uint32_
                           const uint16_t *d_bias, uint16_t *d_out, uint32_t out_stride, void *d_workspace,
                           size_t workspace_bytes, ci_stream_t stream);
 
+/* The same fused linear for callers that cannot allocate device memory -- code under HIP graph
+ * capture, tight serving loops, harnesses that forbid allocation.  It has no counterpart in the
+ * reference (whose fused_rans_linear_triton allocates its split-K workspace through torch on every
+ * call, comp_inference/linear_triton.py:258-263).  It calls no hipMalloc / hipFree or other allocating
+ * routine and takes no workspace: partial sums and the fragment copy of x go to a fixed array of
+ * CI_NOALLOC_SCRATCH_BYTES of device memory inside the library, one copy per GPU, held until the
+ * process ends.  Shapes whose workspace (ci_fused_linear_workspace_bytes_segmented) is larger are
+ * refused with CI_ERR_CAPACITY.  All calls on one GPU share that GPU's array: calls that overlap in
+ * time on one GPU (two streams, two threads) race; calls queued on one stream do not.  Results are
+ * bit-identical to ci_fused_linear_tiled. */
+#define CI_NOALLOC_SCRATCH_BYTES (16u << 20)
+int ci_fused_linear_tiled_noalloc(const ci_tiled_weight *w, const uint16_t *d_x, uint32_t M, uint32_t x_stride,
+                                  const uint16_t *d_bias, uint16_t *d_out, uint32_t out_stride,
+                                  ci_stream_t stream);
+
 /* ---------------------------------------------------------------------------------------
  * Verification aids: the contraction of the fused kernels applied to a plain (uncompressed) bf16
  * weight.  No counterpart in the reference, whose tests compare the fused kernels with
