@@ -14,6 +14,12 @@ The JSON line also carries
   fused_gemv    fused decompress-GEMV/GEMM on the gate projection for M = 1, 4, 16, 64:
                 time, share of the HBM roofline on compressed bytes, and torch.matmul (hipBLASLt)
                 on the uncompressed bf16 weight for comparison
+  fused_gemv_layer_M1, fused_embedding, lm_head   the other operators at their full sizes
+  fused_model   batch-1 greedy decode of a 32-layer Llama-3-8B-shaped decoder on compressed weights
+                (bench_model.run), tok/s next to the same decoder on bf16 weights
+  cpu_roundtrip one 4096x4096 tensor (seed 0) through the CPU oracle's encoder and decoder
+Every fraction of the HBM peak in the line is repeated in roofline.kernels with the bytes and the time
+it was computed from.
 """
 from __future__ import annotations
 
@@ -36,17 +42,18 @@ HBM_PEAK_GBS = 8000.0
 # CU), and a lone wavefront needs about 65 ns per step.  Reported next to every HBM fraction.
 STEP_NS_PER_CU = 9.4
 STEP_NS_LATENCY = 65.0
-NUM_CUS = 256
+NUM_CUS = 256  # replaced by the device's own count in main()
 
 
 def step_bound_us(wave_steps: int, chain: int) -> dict:
     """Lower bounds from the step rate: throughput (all CUs busy) and latency (one chain)."""
     return {"throughput_us": round(wave_steps * STEP_NS_PER_CU / NUM_CUS * 1e-3, 1),
             "latency_us": round(chain * STEP_NS_LATENCY * 1e-3, 1)}
-# HBM bytes of one batched decode launch on this workload, from rocprofv3 FETCH_SIZE and WRITE_SIZE
-# passes scaled by what the same counters read for a plain copy of known size (profiles/ holds the
-# runs): 38115.2 KiB x 1.9991 fetched + 212992.0 KiB x 1.0 written.
+# HBM bytes of one batched decode launch on this workload.  Not measured by this program: taken from
+# offline rocprofv3 FETCH_SIZE and WRITE_SIZE passes over this same command, scaled by what the same
+# counters read for a plain copy of known size: 38115.2 KiB x 1.9991 fetched + 212992.0 KiB x 1.0 written.
 MEASURED_TRAFFIC_BYTES = 296_130_080
+TRAFFIC_SOURCE = "profiles/decode_tiled32_persist_kernel_llama8b_layer.md (offline counter passes, not this run)"
 LAYER = [("q", 4096, 4096), ("k", 1024, 4096), ("v", 1024, 4096), ("o", 4096, 4096),
          ("gate", 14336, 4096), ("up", 14336, 4096), ("down", 4096, 14336)]  # (name, out, in)
 
@@ -207,6 +214,37 @@ def cpu_baseline(layer: list[Compressed], budget_s: float = 15.0):
                                 "torch_matmul_bf16": round(t_mm * 1e3, 2)}}
 
 
+def cpu_roundtrip(seed: int = 0, n: int = 4096):
+    """One n x n bf16 tensor, N(0, 0.02) from `seed`, through the CPU oracle alone: planes split, exponent
+    plane rANS-coded in the default tiling, decoded and joined again; bit-exact check, whole-tensor
+    compression ratio and decode rate on the host cores."""
+    from oracle import rans_oracle as ro
+
+    g = torch.Generator("cpu").manual_seed(seed)
+    w = (torch.randn(n, n, generator=g, dtype=torch.float32) * 0.02).to(torch.bfloat16)
+    bits = w.view(torch.int16).numpy().view(np.uint16)
+    t0 = time.time()
+    enc, man = ro.compress_bf16(bits, 1024, 32)
+    t_enc = time.time() - t0
+    dec_args = (enc.stream, enc.states, enc.tables, enc.slot_map, enc.tile_offsets, enc.tile_max_lens, n, n, 1024, 32)
+    times = []
+    for _ in range(5):
+        t0 = time.time()
+        e = ro.decode_tiled_ilp2(*dec_args)
+        times.append(time.time() - t0)
+    t_dec = float(np.median(times))
+    back = ro.merge_bf16(e, ro.uninterleave_plane(man, n, n, 1024, 32))
+    stored = enc.stream.size + man.size + 4 * enc.states.size + 4 * enc.tile_offsets.size + 4 * enc.tile_max_lens.size + 5120
+    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else os.cpu_count()
+    cores = min(cores or 1, int(os.environ.get("OMP_NUM_THREADS", cores or 1)))
+    return {"tensor": f"{n}x{n} bf16 N(0,0.02) seed {seed}, tile 1024x32", "bit_exact": bool(np.array_equal(back, bits)),
+            "compression_ratio": round(2.0 * n * n / stored, 4),
+            "exponent_plane_ratio": round(n * n / enc.stream.size, 4),
+            "cpu_decode_GBs_exponent_bytes": round(n * n / t_dec / 1e9, 3),
+            "cpu_decode_GBs_bf16_bytes": round(2.0 * n * n / t_dec / 1e9, 3),
+            "cpu_encode_s": round(t_enc, 3), "cores": int(cores), "kind": "port"}
+
+
 def ci_uninterleave(c: "Compressed") -> np.ndarray:
     """Row-major sign|mantissa plane of a compressed tensor (host)."""
     import comp_inference_amd as ci
@@ -222,6 +260,7 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-gemv", action="store_true")
     ap.add_argument("--no-embedding", action="store_true")
+    ap.add_argument("--no-model", action="store_true", help="skip the 32-layer decoder (about a minute)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three 64 MiB device-to-device copies, so that a counter run has a "
                          "kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
@@ -237,6 +276,15 @@ def main() -> int:
 
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
+    global NUM_CUS
+    NUM_CUS = torch.cuda.get_device_properties(dev).multi_processor_count
+    kernels = []  # every HBM fraction of the line with the bytes and the time behind it
+
+    def record(kernel: str, config: str, nbytes: int, us: float) -> float:
+        frac = nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS
+        kernels.append({"kernel": kernel, "config": config, "bytes": int(nbytes), "us": round(us, 2), "frac": round(frac, 4)})
+        return frac
+
     if a.copy_calibration:
         src = torch.full((64 << 20,), 7, device=dev, dtype=torch.uint8)
         dst = torch.empty_like(src)
@@ -286,9 +334,11 @@ def main() -> int:
     achieved = algo_bytes / (launch_us * 1e-6) / 1e9
     roofline = {"bound": "hbm", "kernel": "decode_tiled32_persist_kernel", "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                "traffic": MEASURED_TRAFFIC_BYTES, "bytes_per_launch": int(algo_bytes),
+                "traffic": MEASURED_TRAFFIC_BYTES, "traffic_source": TRAFFIC_SOURCE,
+                "bytes_per_launch": int(algo_bytes), "cus": int(NUM_CUS),
                 "launch_us": round(launch_us, 2), "single_tensor_launch_us": per_kernel,
                 "compressed_read_GBs": round(total_stream / (launch_us * 1e-6) / 1e9, 1)}
+    record("decode_tiled32_persist_kernel", "one layer, seven tensors, one launch", algo_bytes, launch_us)
     wave_steps = sum(c.wave_steps() for c in layer)
     sb = step_bound_us(wave_steps, th // 2)
     roofline["step_rate_bound"] = dict(sb, wavefront_steps=wave_steps, ns_per_wavefront_step_per_cu=STEP_NS_PER_CU,
@@ -320,6 +370,7 @@ def main() -> int:
             us_plain = batched_time_us(lambda: gate.linear(x), 25, 100)
             us_ref = batched_time_us(lambda: torch.matmul(x, w_dense), 25, 100)
             nbytes = gate.linear_bytes(M)
+            record("fused linear (checkpoints)", f"gate K=4096 N=14336 M={M}", nbytes, us)
             sb = step_bound_us(gate.wave_steps(), gate.th // 2)
             rows.append({"M": M, "us": round(us, 2), "us_without_checkpoints": round(us_plain, 2), "allclose_1e-2": ok,
                          "step_rate_bound_us": max(sb["throughput_us"], sb["latency_us"]),
@@ -348,6 +399,7 @@ def main() -> int:
             us_plain = batched_time_us(lambda: c.linear(x), 25, 100)
             us_ref = batched_time_us(lambda: torch.matmul(x, w_dense), 25, 100)
             total, total_ref = total + us, total_ref + us_ref
+            record("fused linear (checkpoints)", f"{name} K={c.K} N={c.N} M=1", c.linear_bytes(1), us)
             rows.append({"layer": f"{name} K={c.K} N={c.N}", "segments": int(c.segments), "us": round(us, 2),
                          "us_without_checkpoints": round(us_plain, 2), "allclose_1e-2": ok,
                          "checkpoint_bytes": 0 if c.checkpoints is None else int(c.checkpoints.numel() * 8),
@@ -392,11 +444,49 @@ def main() -> int:
                                   "gathered_GBs": round(T * H * 2 / (us * 1e-6) / 1e9, 2),
                                   "compressed_table_bytes": int(emb.stream.numel() + emb.man.numel()),
                                   "torch_index_bf16_us": round(us_ref, 1)}
+        # useful bytes of the gather: the rows written and, per distinct (half tile of rows, pair of column
+        # tiles) touched, nothing less than the rows themselves in compressed form -- counted as output only
+        record("embed_gather32_kernel (+ grouping)", f"{V}x{H} table, {T} Zipf ids, 8 segments", T * H * 2 + T * 8, us)
+
+        # --- the same table as a tied LM head: logits = x W^T, M = 1
+        xh = torch.randn(1, H, generator=torch.Generator("cpu").manual_seed(2), dtype=torch.float32).to(torch.bfloat16).to(dev)
+
+        def head():
+            return ci.fused_rans_linear_transposed(xh, emb.stream, emb.states, emb.tables, emb.slot_map, (V, H),
+                                                   emb.tile_offsets, emb.tile_max_lens, emb.th, emb.tw, emb.man)
+
+        want_logits = torch.matmul(xh, table_dev.t()).float()
+        ok = bool(torch.allclose(head().float(), want_logits, atol=1e-2, rtol=1e-2))
+        us_h = batched_time_us(head, 5, 20)
+        us_h_ref = batched_time_us(lambda: torch.matmul(xh, table_dev.t()), 5, 20)
+        head_bytes = emb.stream.numel() + emb.man.numel() + 4 * emb.n_streams + 8 * emb.n_tiles + 5120 + 2 * H + 2 * V
+        out["lm_head"] = {"weight": f"{V}x{H} (the embedding table, tied)", "M": 1, "us": round(us_h, 1), "allclose_1e-2": ok,
+                          "hbm_frac_compressed_bytes": round(record("trans32_kernel (+ reduction)", f"{V}x{H} head M=1", head_bytes, us_h), 4),
+                          "effective_weight_GBs": round(2 * V * H / (us_h * 1e-6) / 1e9, 1),
+                          "torch_matmul_bf16_us": round(us_h_ref, 1)}
         del emb, table_dev, table, ck
 
+    roofline["kernels"] = kernels
     if not a.no_cpu_baseline:
         log("timing the CPU oracle ...")
         out["cpu_baseline"] = cpu_baseline(layer)
+        out["cpu_roundtrip"] = cpu_roundtrip()
+    del layer, items
+    torch.cuda.empty_cache()
+
+    # --- the whole decoder: 32 layers, 128-token prompt, 256 greedy tokens, weights from the CPU generator
+    if not a.no_model:
+        import bench_model
+
+        m = bench_model.run(32, 128, 256, 1024, 32, "cpu")
+        out["fused_model"] = {k: m[k] for k in (
+            "model", "prompt_tokens", "new_tokens", "weight_bytes_compressed", "weight_bytes_bf16",
+            "checkpoint_index_bytes", "tok_per_s_compressed_graph", "tok_per_s_compressed_eager",
+            "tok_per_s_reference_bf16_graph", "tok_per_s_reference_bf16_eager",
+            "ids_equal_to_decompressed_same_order_run", "graph_ids_equal_to_decompressed_same_order_run",
+            "teacher_forced_logits_bit_identical_to_same_order_run", "ids_equal_to_reference",
+            "teacher_forced_top1_agreement", "teacher_forced_max_abs_logit_diff",
+            "reference_smallest_top1_top2_logit_gap")}
 
     print(json.dumps(out))
     return 0
