@@ -31,14 +31,14 @@ class TiledWeight(C.Structure):
                 ("d_tile_offsets", C.c_void_p), ("d_tile_max_lens", C.c_void_p), ("n_tiles", C.c_uint64),
                 ("d_man_tiled", C.c_void_p), ("man_len", C.c_uint64),
                 ("d_checkpoints", C.c_void_p), ("checkpoint_bytes", C.c_uint64), ("segments", C.c_uint32),
-                ("d_slot_table", C.c_void_p), ("slot_table_bytes", C.c_uint64)]
+                ("d_slot_table", C.c_void_p), ("slot_table_bytes", C.c_uint64), ("max_window_rows", C.c_uint32)]
 
 
 SLOT_TABLE_BYTES = 32768
 
 
 def tiled_weight(K, N, tile_k, tile_n, stream, states, tables, slot_map, tile_offsets, tile_max_lens, man,
-                 checkpoints=None, segments=1, slot_table=None) -> TiledWeight:
+                 checkpoints=None, segments=1, slot_table=None, max_window_rows=0) -> TiledWeight:
     """Descriptor over device tensors (which the caller keeps alive for as long as it is used)."""
     w = TiledWeight()
     w.K, w.N, w.tile_height, w.tile_width = int(K), int(N), int(tile_k), int(tile_n)
@@ -56,6 +56,7 @@ def tiled_weight(K, N, tile_k, tile_n, stream, states, tables, slot_map, tile_of
         w.d_slot_table, w.slot_table_bytes = slot_table.data_ptr(), slot_table.numel() * slot_table.element_size()
     else:
         w.d_slot_table, w.slot_table_bytes = None, 0
+    w.max_window_rows = int(max_window_rows)
     return w
 
 

@@ -9,7 +9,7 @@ thread_local char g_err[512] = "";
 
 extern "C" const char *ci_last_error(void) { return ci::g_err; }
 
-extern "C" int ci_abi_version(void) { return 2; }
+extern "C" int ci_abi_version(void) { return 3; }
 
 extern "C" int ci_check_device(void) {
     int dev = 0;

@@ -62,6 +62,7 @@ struct LinearArgs {
     // every workgroup builds it from tables and slot_map.
     const uint2 *slot_table;
     uint32_t rounds;  // fused_linear32_seg_kernel: items of a job per wavefront
+    bool all_fast;    // every item of the weight takes the hand-scheduled loop (known from the descriptor)
 };
 
 // x [M, K] -> the fragment order described at LinearArgs::xf.  In a plain row-major x the 64 lanes of
@@ -507,19 +508,20 @@ __device__ __forceinline__ void seg_resolve(const LinearArgs &a, uint32_t vk, ui
 
 // Touches the cache lines the item's start will read: its window of the body (lanes 0..55, a 128-byte line
 // each) and the first 128 rows of both halves of its sign|mantissa rows (all lanes).  The values are not
-// used; the loads bring the lines next to the CU while the previous item still decodes.
-__device__ __forceinline__ uint32_t seg_touch(const LinearArgs &a, const SegItem &it, int lane) {
-    uint32_t t = 0;
-    if (!it.fast) return t;
+// used; the loads bring the lines next to the CU while the previous item still decodes.  Plain global loads
+// (a volatile access would become a flat, system-scope load, which the LDS counter of every decode step
+// would wait for): the caller keeps the two values alive until the item's loop has run.
+__device__ __forceinline__ void seg_touch(const LinearArgs &a, const SegItem &it, int lane, uint32_t &t, uint32_t &t2) {
+    t = t2 = 0;
+    if (!it.fast) return;
     const uint32_t tk = it.vk / a.segs, seg = it.vk % a.segs, tile = tk * a.tiles_n + it.tn;
     const uint32_t half = a.th / 2, seglen = half / a.segs;
     if ((uint32_t)lane * 128 < it.rows * 64)
-        t = *reinterpret_cast<const volatile uint32_t *>(a.stream + it.base + (size_t)it.lo * 64 + lane * 128);
+        t = *reinterpret_cast<const uint32_t *>(a.stream + it.base + (size_t)it.lo * 64 + lane * 128);
     const uint32_t hsel = lane / 32, line = lane % 32;  // 4 sign|mantissa rows of a tile make a line
     if (line * 4 < seglen)
-        t += *reinterpret_cast<const volatile uint32_t *>(a.man_tiled + (size_t)tile * a.th * 32 +
-                                                          (size_t)(hsel * half + seg * seglen + line * 4) * 32);
-    return t;
+        t2 = *reinterpret_cast<const uint32_t *>(a.man_tiled + (size_t)tile * a.th * 32 +
+                                                 (size_t)(hsel * half + seg * seglen + line * 4) * 32);
 }
 
 // The item's window, memory -> LDS as it lies (piece g = bytes [1024 g + 16 lane, + 16) of the window).
@@ -543,6 +545,11 @@ __device__ __forceinline__ void seg_stage(const LinearArgs &a, const SegItem &it
 }
 
 // One staged item through the hand-scheduled loop, accumulating into acc (and acc2 for x rows 32..63).
+#ifdef CI_EXP_MANHOT
+#define CI_EXP_TILE(t) ((t) & 7)
+#else
+#define CI_EXP_TILE(t) (t)
+#endif
 template <int MB>
 __device__ __forceinline__ void seg_run(const LinearArgs &a, const SegItem &it, const uint8_t *stage, int lane,
                                         f32x16 &acc, f32x16 &acc2) {
@@ -556,7 +563,7 @@ __device__ __forceinline__ void seg_run(const LinearArgs &a, const SegItem &it, 
     st.n1 = rel >= 0 ? stage[rel * 64 + lane] : 0;
     const uint32_t m = c;  // row of x this lane feeds to the (first) MFMA
     const bool m_ok = m < a.M, m2_ok = MB == 2 && m + 32 < a.M;
-    const uint64_t mbase = reinterpret_cast<uint64_t>(a.man_tiled + (size_t)tile * a.th * 32);
+    const uint64_t mbase = reinterpret_cast<uint64_t>(a.man_tiled + (size_t)CI_EXP_TILE(tile) * a.th * 32);
     // readfirstlane returns a signed int: widen through uint32_t, not by sign extension
     const uint32_t mb_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(mbase >> 32));
     const uint32_t mb_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)mbase);
@@ -631,15 +638,23 @@ struct SegJobs {
 // grid: any number of workgroups (one per CU); workgroup j takes jobs j, j + gridDim.x, ...
 #ifdef CI_PROBE
 __device__ uint64_t g_probe[64 * 64];
+#define PROBEW(k) do { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory"); PROBE(k); } while (0)
 #define PROBE(k) do { if (blockIdx.x == 0 && lane == 0 && pcount < 60) g_probe[wave * 64 + pcount++] = ((uint64_t)(k) << 56) | (wall_clock64() & 0xffffffffffffffull); } while (0)
 #else
 #define PROBE(k) do { } while (0)
+#define PROBEW(k) do { } while (0)
 #endif
-template <int MB>
+// kCold = false: the instance for weights whose every item is known to take the hand-scheduled loop (full
+// tiles, windows of at most kWinRows rows: LinearArgs::all_fast).  It holds no code for the guarded path,
+// whose registers would otherwise be spilled around every item; an item that does not qualify after all
+// (a descriptor that promised too much) is left out rather than staged beyond its window area.
+template <int MB, bool kCold>
 __global__ __launch_bounds__(kSegWaves *kWave) void fused_linear32_seg_kernel(LinearArgs a) {
     extern __shared__ __align__(16) uint8_t lds[];
     const uint2 *tab = reinterpret_cast<const uint2 *>(lds);
-    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    // (the wavefront's index through readfirstlane: everything derived from it -- jobs, items, tiles -- is then
+    // uniform for the compiler too and lives in scalar registers)
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWave)), lane = threadIdx.x % kWave;
 #ifdef CI_PROBE
     int pcount = 0;
 #endif
@@ -656,7 +671,7 @@ __global__ __launch_bounds__(kSegWaves *kWave) void fused_linear32_seg_kernel(Li
         while (sl < slots && !slot_item(sl, vk, tn)) ++sl;
         return sl;
     };
-    const bool coded = a.dense_w == nullptr;
+    const bool coded = !kCold || a.dense_w == nullptr;
 
     // the first item's inputs are on their way while the table is copied
     SegRaw raw;
@@ -665,6 +680,7 @@ __global__ __launch_bounds__(kSegWaves *kWave) void fused_linear32_seg_kernel(Li
     uint32_t vk_n = 0, tn_n = 0, vk_nn = 0, tn_nn = 0;
     uint32_t s_nxt = next_slot(0, vk_n, tn_n), s_nn = slots;  // the next slot with an item, and the one after
     if (coded && s_nxt < slots) seg_request(a, vk_n, tn_n, lane, raw);
+    PROBE(20);
     if (coded && a.slot_table) {
         const u32x4 *src = reinterpret_cast<const u32x4 *>(a.slot_table);
         u32x4 *dst = reinterpret_cast<u32x4 *>(lds);
@@ -674,11 +690,14 @@ __global__ __launch_bounds__(kSegWaves *kWave) void fused_linear32_seg_kernel(Li
     } else if (coded) {
         build_slot_table_x8(reinterpret_cast<uint2 *>(lds), a.tables, a.slot_map, threadIdx.x, kSegWaves * kWave);
     }
+    PROBE(21);
     if (coded && s_nxt < slots) {
         seg_resolve(a, vk_n, tn_n, lane, raw, nxt);
+        PROBE(22);
         s_nn = next_slot(s_nxt + 1, vk_nn, tn_nn);
         if (s_nn < slots) seg_request(a, vk_nn, tn_nn, lane, raw);
     }
+    PROBE(23);
     __syncthreads();
     PROBE(2);
 
@@ -689,33 +708,36 @@ __global__ __launch_bounds__(kSegWaves *kWave) void fused_linear32_seg_kernel(Li
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[v] = acc2[v] = 0.f;
         }
+        PROBE(10);
         const uint32_t job = blockIdx.x + (sl / jb.R) * gridDim.x;
         uint32_t vk, tn;
         if (slot_item(sl, vk, tn)) {
-            if (!coded) {
+            PROBE(11);
+            if (kCold && !coded) {
                 seg_cold_item<MB>(a, vk, tn, tab, stage, lane, acc, acc2);
             } else {
                 // (sl == s_nxt: the slots with an item are visited in order)
                 const SegItem cur = nxt;
                 PROBE(3);
                 if (cur.fast) seg_stage(a, cur, stage, lane);
-                PROBE(4);
-                uint32_t touched = 0;
+                PROBEW(4);
+                uint32_t touched = 0, touched2 = 0;  // (kept apart: adding them would wait for both loads)
                 s_nxt = s_nn;
                 vk_n = vk_nn;
                 tn_n = tn_nn;
                 if (s_nxt < slots) {
                     seg_resolve(a, vk_n, tn_n, lane, raw, nxt);
-                    touched = seg_touch(a, nxt, lane);
+                    seg_touch(a, nxt, lane, touched, touched2);
                     s_nn = next_slot(s_nxt + 1, vk_nn, tn_nn);
                     if (s_nn < slots) seg_request(a, vk_nn, tn_nn, lane, raw);
                 }
                 PROBE(cur.fast ? 5 : 9);
+                PROBEW(12);
                 if (cur.fast)
                     seg_run<MB>(a, cur, stage, lane, acc, acc2);  // (a wavefront's LDS operations complete in order)
-                else
+                else if (kCold)
                     seg_cold_item<MB>(a, vk, tn, tab, stage, lane, acc, acc2);
-                asm volatile("" ::"v"(touched));  // the touching loads end here
+                asm volatile("" ::"v"(touched), "v"(touched2));  // the touching loads end here
                 PROBE(6);
             }
         }
@@ -1034,7 +1056,7 @@ static int fused_linear_impl(const uint16_t *d_x, uint32_t M, uint32_t K, uint32
                              const uint16_t *d_bias, uint16_t *d_out, uint32_t out_stride, void *d_workspace,
                              size_t workspace_bytes, bool dense, hipStream_t s, const uint16_t *d_plain_w = nullptr,
                              const void *d_checkpoints = nullptr, uint32_t segments = 1,
-                             const void *d_slot_table = nullptr) {
+                             const void *d_slot_table = nullptr, uint32_t max_window_rows = 0) {
     if (M == 0 || N == 0) return CI_OK;
     if (K == 0) return fail(CI_ERR_ARG, "fused linear: K is 0");
     if (!d_x || !d_out) return fail(CI_ERR_ARG, "fused linear: null pointer");
@@ -1087,6 +1109,9 @@ static int fused_linear_impl(const uint16_t *d_x, uint32_t M, uint32_t K, uint32
         return fail(CI_ERR_ARG, "plain-weight linear: only the 32-column tiling (tile height a multiple of 16)");
     a.ckpt = static_cast<const uint2 *>(d_checkpoints);
     a.slot_table = static_cast<const uint2 *>(d_slot_table);
+    // no item is ragged (whole tiles in both directions) and none has a window larger than its staging area
+    a.all_fast = !d_plain_w && a.fast_ok && K % th == 0 && N % tw == 0 && max_window_rows != 0 &&
+                 max_window_rows <= kWinRows;
     a.rounds = p.rounds;
     a.segs = p.segs;
     a.kw = p.kw;
@@ -1128,16 +1153,21 @@ static int fused_linear_impl(const uint16_t *d_x, uint32_t M, uint32_t K, uint32
     }
 
     if (p.seg16) {
-        CI_ALLOW_FULL_LDS(fused_linear32_seg_kernel<1>);
-        CI_ALLOW_FULL_LDS(fused_linear32_seg_kernel<2>);
         const uint32_t VK = a.tiles_k * p.segs;
         const uint32_t jobs = VK >= (uint32_t)kSegWaves ? a.tiles_n * p.P : ceil_div(a.tiles_n, kSegWaves / VK);
         const dim3 grid(jobs < cus ? jobs : cus), block(kSegWaves * kWave);
         const uint32_t lds_bytes = kSlotTableBytes + kSegWaves * kWinBytes;
-        if (M > 32)
-            hipLaunchKernelGGL(fused_linear32_seg_kernel<2>, grid, block, lds_bytes, s, a);
-        else
-            hipLaunchKernelGGL(fused_linear32_seg_kernel<1>, grid, block, lds_bytes, s, a);
+#define CI_LAUNCH_SEG(MB_, COLD_)                                                                   \
+    do {                                                                                            \
+        CI_ALLOW_FULL_LDS((fused_linear32_seg_kernel<MB_, COLD_>));                                 \
+        hipLaunchKernelGGL((fused_linear32_seg_kernel<MB_, COLD_>), grid, block, lds_bytes, s, a);  \
+    } while (0)
+        if (M > 32) {
+            if (a.all_fast) CI_LAUNCH_SEG(2, false); else CI_LAUNCH_SEG(2, true);
+        } else {
+            if (a.all_fast) CI_LAUNCH_SEG(1, false); else CI_LAUNCH_SEG(1, true);
+        }
+#undef CI_LAUNCH_SEG
         CI_LAUNCH_CHECK("fused_linear32_seg_kernel");
     } else if (p.resident) {
         CI_ALLOW_FULL_LDS(fused_linear32_resident_kernel<1>);
@@ -1238,6 +1268,53 @@ extern "C" int ci_build_slot_table(const uint32_t *d_tables, const uint8_t *d_sl
     return CI_OK;
 }
 
+namespace ci {
+// One wavefront per item (segment of the 64 streams of a tile): the rows of the tile body the item can touch,
+// as the sixteen-wavefront kernel works them out before staging; the maximum over all items, at least 1.
+__global__ __launch_bounds__(256) void window_rows_kernel(LinearArgs a, uint32_t num_items, uint32_t *out) {
+    const uint32_t item = blockIdx.x * 4 + threadIdx.x / kWave;
+    const int lane = threadIdx.x % kWave;
+    if (item >= num_items) return;  // (whole wavefronts)
+    const uint32_t vk = item / a.tiles_n, tn = item % a.tiles_n;
+    SegRaw raw;
+    seg_request(a, vk, tn, lane, raw);
+    SegItem it;
+    seg_resolve(a, vk, tn, lane, raw, it);
+    if (lane == 0) atomicMax(out, it.rows > 1u ? it.rows : 1u);
+}
+}  // namespace ci
+
+extern "C" int ci_max_window_rows(const ci_tiled_weight *w, uint32_t *d_rows, ci_stream_t stream) {
+    if (int rc = ci_tiled_weight_check(w)) return rc;
+    if (!d_rows || !aligned(d_rows, 4)) return fail(CI_ERR_ARG, "ci_max_window_rows: null or unaligned result pointer");
+    if (w->tile_width != 32) return fail(CI_ERR_ARG, "ci_max_window_rows: 32-column tiles only");
+    const uint32_t segs = w->segments > 1 ? w->segments : 1;
+    if ((w->tile_height / 2) % segs) return fail(CI_ERR_ARG, "ci_max_window_rows: half a tile does not split into %u segments", segs);
+    LinearArgs a{};
+    a.K = w->K;
+    a.N = w->N;
+    a.th = w->tile_height;
+    a.tw = w->tile_width;
+    a.tiles_n = ceil_div(w->N, w->tile_width);
+    a.tiles_k = ceil_div(w->K, w->tile_height);
+    a.segs = segs;
+    a.stream = w->d_stream;
+    a.stream_len = w->stream_len;
+    a.states = w->d_states;
+    a.tile_offsets = w->d_tile_offsets;
+    a.tile_max_lens = w->d_tile_max_lens;
+    a.ckpt = static_cast<const uint2 *>(segs > 1 ? w->d_checkpoints : nullptr);
+    a.fast_ok = true;
+    const uint64_t items = (uint64_t)a.tiles_k * segs * a.tiles_n;
+    if (items > 0xffffffffull / 4) return fail(CI_ERR_ARG, "ci_max_window_rows: too many items");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipLaunchKernelGGL(zero_f32_kernel, dim3(1), dim3(256), 0, s, reinterpret_cast<float *>(d_rows), (uint64_t)1);
+    CI_LAUNCH_CHECK("zero_f32_kernel");
+    hipLaunchKernelGGL(window_rows_kernel, dim3((uint32_t)((items + 3) / 4)), dim3(256), 0, s, a, (uint32_t)items, d_rows);
+    CI_LAUNCH_CHECK("window_rows_kernel");
+    return CI_OK;
+}
+
 extern "C" int ci_tiled_weight_check(const ci_tiled_weight *w) {
     if (!w) return fail(CI_ERR_ARG, "weight descriptor: null");
     if (w->K == 0 || w->N == 0 || w->tile_height == 0 || w->tile_width == 0 || (w->tile_height & 1))
@@ -1278,7 +1355,7 @@ extern "C" int ci_fused_linear_tiled(const ci_tiled_weight *w, const uint16_t *d
                              w->d_slot_map, w->d_tile_offsets, w->d_tile_max_lens, w->d_man_tiled, w->tile_height,
                              w->tile_width, d_bias, d_out, out_stride, d_workspace, workspace_bytes, false,
                              static_cast<hipStream_t>(stream), nullptr, w->segments > 1 ? w->d_checkpoints : nullptr,
-                             w->segments > 1 ? w->segments : 1, w->d_slot_table);
+                             w->segments > 1 ? w->segments : 1, w->d_slot_table, w->max_window_rows);
 }
 
 // ---- an entry point that allocates nothing ----------------------------------------------------------
@@ -1328,7 +1405,7 @@ extern "C" int ci_fused_linear_tiled_noalloc(const ci_tiled_weight *w, const uin
                              w->d_slot_map, w->d_tile_offsets, w->d_tile_max_lens, w->d_man_tiled, w->tile_height,
                              w->tile_width, d_bias, d_out, out_stride, ws, (size_t)CI_NOALLOC_SCRATCH_BYTES, false,
                              static_cast<hipStream_t>(stream), nullptr, segments > 1 ? w->d_checkpoints : nullptr,
-                             segments, w->d_slot_table);
+                             segments, w->d_slot_table, w->max_window_rows);
 }
 
 extern "C" int ci_plain_linear_same_order(const uint16_t *d_x, uint32_t M, uint32_t K, uint32_t N, uint32_t x_stride,

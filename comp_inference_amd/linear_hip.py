@@ -173,13 +173,22 @@ class PreparedLinear:
             check(lib().ci_build_slot_table(ptr(self.keep[2]), ptr(self.keep[3]), ptr(self.slot_table),
                                             C.c_size_t(_lib.SLOT_TABLE_BYTES), _lib.stream_handle(dev)))
         self.need = {}
+        self.max_window_rows = 0
         self._bind()
+        # the most rows of a tile body one item reads, worked out once (one small launch and a read-back): with
+        # it in the descriptor the library knows that every item fits its staging area before it launches
+        if self.tile_n == 32 and self.tile_k % 2 == 0 and (self.tile_k // 2) % self.segments == 0:
+            rows = torch.zeros(1, dtype=torch.int32, device=dev)
+            with torch.cuda.device(dev):
+                check(lib().ci_max_window_rows(C.byref(self.w), ptr(rows), _lib.stream_handle(dev)))
+            self.max_window_rows = int(rows.item())
+            self._bind()
 
     def _bind(self) -> None:
         o = self.keep
         self.p = [ptr(t) for t in o]
         self.w = _lib.tiled_weight(self.K, self.N, self.tile_k, self.tile_n, o[0], o[1], o[2], o[3], o[4], o[5], o[6],
-                                   o[8], self.segments, self.slot_table)
+                                   o[8], self.segments, self.slot_table, self.max_window_rows)
 
     # A copy (copy.deepcopy of the owning module, pickling) gets its own tensors: the pointers are taken
     # again from them instead of travelling as numbers.

@@ -387,6 +387,7 @@ typedef struct ci_tiled_weight {
     uint32_t segments;
     const void *d_slot_table;
     uint64_t slot_table_bytes;        /* == CI_SLOT_TABLE_BYTES when d_slot_table is given */
+    uint32_t max_window_rows;         /* 0 (not known), or what ci_max_window_rows wrote for these arrays */
 } ci_tiled_weight;
 
 #define CI_SLOT_TABLE_BYTES 32768
@@ -401,6 +402,15 @@ int ci_tiled_weight_check(const ci_tiled_weight *w);
  * checkpoints. */
 int ci_build_slot_table(const uint32_t *d_tables, const uint8_t *d_slot_map, void *d_slot_table,
                         size_t slot_table_bytes, ci_stream_t stream);
+
+/* The largest number of rows of a tile body that one item -- a segment of the 64 streams of a tile, or
+ * the whole streams without checkpoints -- reads, written to *d_rows (device memory, 4 bytes) on `stream`.
+ * Derived data like the checkpoints: computed once per weight, copied back by the caller and kept in
+ * ci_tiled_weight::max_window_rows.  With it the fused linear knows before the launch that every item
+ * fits its staging area and runs a kernel without the guarded path; with 0 there it runs the kernel that
+ * checks every item.  A value smaller than the true one makes the kernel leave out the items that do not
+ * fit (wrong sums, no out-of-bounds access). */
+int ci_max_window_rows(const ci_tiled_weight *w, uint32_t *d_rows, ci_stream_t stream);
 
 /* Fused decompress-GEMV/GEMM on a descriptor: what ci_fused_linear_ilp2 / _segmented compute, with the
  * lengths checked.  Workspace: ci_fused_linear_workspace_bytes_segmented(M, K, N, tile_height,

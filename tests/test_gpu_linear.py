@@ -418,3 +418,95 @@ def test_segment_arguments_are_checked(oracle):
     x = make_x(2, K, seed=1)
     with pytest.raises(RuntimeError):
         _call(enc, man, x, K, N, th, 32, checkpoints=ck, segments=2)   # index made for 4 segments
+
+
+def _window_rows_numpy(ck, depths, segments):
+    """Rows of a tile body that item (tile, segment) can touch, from the checkpoint index alone: from the lowest
+    row any lane has reached at the segment's end to the highest row a lane starts at; maximum over all items."""
+    best = 1
+    tiles = depths.shape[0]
+    rows = None if ck is None else (ck >> 32).astype(np.int64)  # (int64 words: the shift keeps the row's sign)
+    for t in range(tiles):
+        d = int(depths[t])
+        for seg in range(segments):
+            start = np.full(64, d - 1, np.int64) if seg == 0 else np.minimum(rows[t, seg - 1], d - 1)
+            end = np.minimum(rows[t, seg], start) if seg + 1 < segments else np.full(64, -1, np.int64)
+            lo, hi = max(int(end.min()), 0), int(start.max())
+            best = max(best, hi - lo + 1 if hi >= lo else 0)
+    return best
+
+
+@pytest.mark.parametrize("K,N,th,M,segments", [
+    (4096, 256, 1024, 1, 2), (4096, 256, 1024, 5, 4), (4096, 256, 1024, 40, 8), (8192, 64, 1024, 1, 2),
+    (18432, 64, 1024, 3, 2),  # 36 items per column tile: two chunks, partial sums through the workspace
+    (2048, 96, 512, 1, 1),    # no checkpoints: whole streams of a 256-row half tile
+])
+def test_prepared_weight_runs_the_kernel_without_guarded_path(oracle, K, N, th, M, segments):
+    """A prepared weight knows its largest window (ci_max_window_rows, checked here against the checkpoint
+    index) and, on whole tiles, runs the kernel instance that has no guarded path: its output is the same bits
+    as the checking instance's, which the operator without a prepared weight runs."""
+    from comp_inference_amd import build_checkpoints
+    from comp_inference_amd.linear_hip import PreparedLinear
+
+    w = make_weight_kn(N, K, seed=K + N + segments)
+    enc, man, wdec = _compress(oracle, w, th, 32)
+    x = make_x(M, K, seed=M).cuda()
+    dev = torch.device("cuda", 0)
+    args = (torch.from_numpy(enc.stream).to(dev), _t32(enc.states).to(dev), _t32(enc.tables).to(dev),
+            torch.from_numpy(enc.slot_map).to(dev), (K, N), _t32(enc.tile_offsets).to(dev), _t32(enc.tile_max_lens).to(dev))
+    ck = build_checkpoints(*args, th, 32, segments)
+    p = PreparedLinear(dev, *args, th, 32, torch.from_numpy(man).to(dev), checkpoints=ck, segments=segments)
+    want_rows = _window_rows_numpy(None if ck is None else ck.cpu().numpy(), enc.tile_max_lens.astype(np.int64), segments)
+    assert p.max_window_rows == want_rows
+    assert 0 < p.max_window_rows <= 112
+    got = p(x)
+    same = _call(enc, man, x, K, N, th, 32, checkpoints=ck, segments=segments)
+    assert torch.equal(got.view(torch.int16), same.view(torch.int16))
+    want = torch.matmul(x.float().cpu(), wdec.float())
+    assert torch.allclose(got.float().cpu(), want, atol=ATOL, rtol=RTOL)
+
+
+def test_a_window_promise_that_is_too_small_loses_items_but_stays_in_bounds(oracle):
+    """Exponents spread evenly over sixteen values cost half a byte per symbol, so a 256-row half tile reads
+    more rows of its body than an item's staging area holds.  With no promise in the descriptor the checking
+    kernel sends such items down the guarded path and the result is right; with a promise that is too small the
+    kernel without guarded path leaves them out: wrong sums, but nothing out of bounds, and the next call is
+    unharmed."""
+    import ctypes as C
+
+    from comp_inference_amd import _lib
+
+    K, N, th = 1024, 64, 512
+    rng = np.random.default_rng(17)
+    bits = (rng.integers(0, 2, (K, N)) << 15 | rng.integers(118, 134, (K, N)) << 7 | rng.integers(0, 128, (K, N))).astype(np.uint16)
+    w = bits_to_bf16(bits)
+    enc, man, wdec = _compress(oracle, w, th, 32)
+    dev = torch.device("cuda", 0)
+    t = [torch.from_numpy(enc.stream).to(dev), _t32(enc.states).to(dev), _t32(enc.tables).to(dev),
+         torch.from_numpy(enc.slot_map).to(dev), _t32(enc.tile_offsets).to(dev), _t32(enc.tile_max_lens).to(dev),
+         torch.from_numpy(man).to(dev)]
+    x = make_x(2, K, seed=3).to(dev)
+    lib, ptr = _lib.lib(), _lib.ptr
+    need = lib.ci_fused_linear_workspace_bytes_segmented(2, K, N, th, 32, 0, 1)
+    ws = torch.empty(max(need, 16), dtype=torch.uint8, device=dev)
+
+    def run(promise):
+        desc = _lib.tiled_weight(K, N, th, 32, t[0], t[1], t[2], t[3], t[4], t[5], t[6], None, 1, None, promise)
+        out = torch.zeros(2, N, dtype=torch.bfloat16, device=dev)
+        _lib.check(lib.ci_fused_linear_tiled(C.byref(desc), ptr(x), 2, K, None, ptr(out), N, ptr(ws), C.c_size_t(ws.numel()),
+                                             _lib.stream_handle(dev)))
+        torch.cuda.synchronize()
+        return out.float().cpu()
+
+    rows = torch.zeros(1, dtype=torch.int32, device=dev)
+    desc = _lib.tiled_weight(K, N, th, 32, t[0], t[1], t[2], t[3], t[4], t[5], t[6])
+    _lib.check(lib.ci_max_window_rows(C.byref(desc), ptr(rows), _lib.stream_handle(dev)))
+    true_rows = int(rows.item())
+    assert true_rows == int(enc.tile_max_lens.max()) and true_rows > 112
+    want = torch.matmul(x.float().cpu(), wdec.float())
+    right = run(0)
+    assert torch.allclose(right, want, atol=ATOL, rtol=RTOL)
+    assert torch.equal(run(true_rows), right)   # the true figure is beyond the staging area: the checking kernel again
+    lost = run(100)
+    assert bool(torch.isfinite(lost).all()) and not torch.equal(lost, right)
+    assert torch.equal(run(0), right)
