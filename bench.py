@@ -301,8 +301,14 @@ def main() -> int:
     for c in layer:
         assert np.array_equal(c.decode().cpu().numpy(), c.exp_host), f"decode mismatch on {c.name}"
 
-    items = [(c.stream, c.states, c.tables, c.slot_map, (c.K, c.N), c.tile_offsets, c.tile_max_lens) for c in layer]
+    plain_items = [(c.stream, c.states, c.tables, c.slot_map, (c.K, c.N), c.tile_offsets, c.tile_max_lens) for c in layer]
     th, tw = layer[0].th, layer[0].tw
+    # decoder checkpoints: the decoder's state and position in the middle of every stream (an index of 8 bytes per
+    # stream and checkpoint beside the compressed tensor, derived from it once; the stream itself is unchanged).
+    # With them an item is half a stream and its window of the tile body fits sixteen wavefronts on a CU.
+    DECODE_SEGMENTS = 2
+    items = [it + (ci.build_checkpoints(*it, th, tw, DECODE_SEGMENTS), DECODE_SEGMENTS) for it in plain_items]
+    checkpoint_bytes = sum(int(it[7].numel()) * 8 for it in items)
 
     # one step = the whole layer decoded by one batched launch (every tensor, every tile)
     def step():
@@ -330,15 +336,21 @@ def main() -> int:
     per_kernel = {}
     for c in layer:
         per_kernel[c.name] = round(float(np.median(event_times_us(c.decode, 5, 30))), 2)
-    algo_bytes = sum(c.decode_bytes() for c in layer)
+    algo_bytes = sum(c.decode_bytes() for c in layer) + checkpoint_bytes
     achieved = algo_bytes / (launch_us * 1e-6) / 1e9
-    roofline = {"bound": "hbm", "kernel": "decode_tiled32_persist_kernel", "achieved": round(achieved, 1),
+    for o, c in zip(ci.rans_decomp_tiled_batch(plain_items, tile_k=th, tile_n=tw), layer):
+        assert np.array_equal(o.cpu().numpy(), c.exp_host), f"decode without checkpoints: mismatch on {c.name}"
+    us_whole_streams = batched_time_us(lambda: ci.rans_decomp_tiled_batch(plain_items, tile_k=th, tile_n=tw), 5, 20)
+    roofline = {"bound": "hbm", "kernel": "decode_tiled32_seg_kernel", "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                 "traffic": MEASURED_TRAFFIC_BYTES, "traffic_source": TRAFFIC_SOURCE,
                 "bytes_per_launch": int(algo_bytes), "cus": int(NUM_CUS),
                 "launch_us": round(launch_us, 2), "single_tensor_launch_us": per_kernel,
+                "decoder_checkpoint_segments": DECODE_SEGMENTS, "checkpoint_bytes": checkpoint_bytes,
+                "launch_us_whole_streams_no_checkpoints": round(us_whole_streams, 2),
                 "compressed_read_GBs": round(total_stream / (launch_us * 1e-6) / 1e9, 1)}
-    record("decode_tiled32_persist_kernel", "one layer, seven tensors, one launch", algo_bytes, launch_us)
+    record("decode_tiled32_seg_kernel", "one layer, seven tensors, one launch, 2 segments per stream", algo_bytes, launch_us)
+    record("decode_tiled32_persist_kernel", "the same without checkpoints (whole streams)", algo_bytes - checkpoint_bytes, us_whole_streams)
     wave_steps = sum(c.wave_steps() for c in layer)
     sb = step_bound_us(wave_steps, th // 2)
     roofline["step_rate_bound"] = dict(sb, wavefront_steps=wave_steps, ns_per_wavefront_step_per_cu=STEP_NS_PER_CU,
@@ -348,7 +360,8 @@ def main() -> int:
            "warmup": a.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
            "vs_baseline": None, "dtype": "u8", "data": "synthetic",
            "config": {"workload": "standalone rANS decode of one Llama-3-8B-shaped layer (q,k,v,o,gate,up,down), "
-                                  "bf16 N(0,0.02) seed 1, tile 1024x32, two streams per column, 12-bit tables",
+                                  "bf16 N(0,0.02) seed 1, tile 1024x32, two streams per column, 12-bit tables, "
+                                  "decoder checkpoints at the middle of every stream",
                       "symbols_per_step": total_syms, "compressed_stream_bytes": total_stream,
                       "exponent_plane_ratio": round(total_syms / total_stream, 3)},
            "roofline": roofline}
@@ -471,7 +484,7 @@ def main() -> int:
         log("timing the CPU oracle ...")
         out["cpu_baseline"] = cpu_baseline(layer)
         out["cpu_roundtrip"] = cpu_roundtrip()
-    del layer, items
+    del layer, items, plain_items
     torch.cuda.empty_cache()
 
     # --- the whole decoder: 32 layers, 128-token prompt, 256 greedy tokens, weights from the CPU generator

@@ -45,6 +45,41 @@ struct DecodeArgs {
 // bytes and writes bf16.  Items that do not qualify for the hand-scheduled loop (ragged, odd block
 // counts, a window deeper than a lane stride) take the same arithmetic with guarded byte reads from
 // global memory.
+// ---- sixteen wavefronts per CU ------------------------------------------------------------------------
+// The decode step is a chain of dependent instructions, and what hides it is the number of wavefronts a
+// CU keeps in flight: sixteen leave each 128 VGPRs and, next to the slot table, 7 KB of LDS.  That holds
+// the window of a short item -- a segment of the streams (decoder checkpoints) or the whole streams of a low
+// tile -- staged as the rows lie in memory: LDS row r of the window = the item's 32 bytes of row r of body A,
+// then those of body B, so lane l finds its bytes at 64 r + l and its pointer moves by 64 per byte.  No
+// transposition, no lane exchanges.  kStride == 0 selects this staging in decode_one_item.
+constexpr int kDecSegWaves = 16;
+constexpr uint32_t kDecWinRows = 112;
+constexpr uint32_t kDecWinBytes = kDecWinRows * 64;
+constexpr int kDecWinPieces = (int)(kDecWinRows / 16);  // one 16-byte load per lane covers 16 rows
+static_assert(kDecWinRows % 16 == 0 && kSlotTableBytes + kDecSegWaves * kDecWinBytes <= kLdsLimit, "windows exceed the LDS");
+
+// Rows [0, rows) of the window: lane l loads 16 bytes of row 16 g + l / 4 -- body A for l % 4 < 2, body B
+// otherwise, columns hsel * 32 + 16 * (l % 2) on -- and writes them where they belong.  A body shorter than
+// the window (win_x < rows) repeats its last row: those bytes belong to no lane.
+__device__ __forceinline__ void stage_window_pair(uint8_t *stage, const uint8_t *__restrict__ src_a, uint32_t win_a,
+                                                  const uint8_t *__restrict__ src_b, uint32_t win_b, uint32_t hsel,
+                                                  uint32_t rows, int lane) {
+    const uint32_t r0 = lane / 4, side = (lane % 4) / 2, part = lane % 2;
+    const uint8_t *src = (side ? src_b : src_a) + hsel * 32 + part * 16;
+    const uint32_t win = side ? win_b : win_a;  // >= 1
+    u32x4 w[kDecWinPieces];
+#pragma unroll
+    for (int g = 0; g < kDecWinPieces; ++g) {
+        const uint32_t r = min((uint32_t)g * 16 + r0, win - 1);
+        w[g] = *reinterpret_cast<const u32x4 *>(src + (size_t)r * 64);
+    }
+#pragma unroll
+    for (int g = 0; g < kDecWinPieces; ++g) {
+        const uint32_t r = (uint32_t)g * 16 + r0;
+        if (r < rows) *reinterpret_cast<u32x4 *>(stage + r * 64 + side * 32 + part * 16) = w[g];
+    }
+}
+
 template <uint32_t kStride, bool kMerge>
 __device__ __forceinline__ void decode_one_item(const DecodeArgs &a, uint32_t item, const uint2 *tab,
                                                 uint8_t *stage, int lane) {
@@ -85,25 +120,36 @@ __device__ __forceinline__ void decode_one_item(const DecodeArgs &a, uint32_t it
     const int32_t w_lo = max(wave_min_i32(row_end) - 1, 0), w_hi = wave_max_i32(row);
     const uint32_t win_a = (uint32_t)max(min(w_hi + 1, (int32_t)depth_a) - w_lo, 0),
                    win_b = (uint32_t)max(min(w_hi + 1, (int32_t)depth_b) - w_lo, 0);
+    constexpr uint32_t kWinLimit = kStride ? kStride : kDecWinRows + 1;  // (rows of a window must stay below it)
     const bool fast = __builtin_amdgcn_ballot_w64(!col_ok) == 0 && steps == seglen && win_a >= 2 && win_b >= 2 &&
-                      win_a < kStride && win_b < kStride && seglen % (kMerge ? 8 : 2) == 0 && seglen >= 2 &&
+                      win_a < kWinLimit && win_b < kWinLimit && seglen % (kMerge ? 8 : 2) == 0 && seglen >= 2 &&
                       (uint64_t)a.K * a.N < (1ull << (kMerge ? 31 : 32)) && (uint32_t)(uintptr_t)tab == 0 &&
                       (!kMerge || a.man_aligned);
     const uint8_t *man_seg =
         kMerge ? a.man_tiled + (size_t)tile * a.th * 32 + (size_t)(hsel * half + seg * seglen) * 32 : nullptr;
     if (fast) {
-        StageRegs body;
-        const uint32_t deepest = max(win_a, win_b), my_depth = (lane & 4) ? win_b : win_a;
+        const uint32_t deepest = max(win_a, win_b);
         const uint8_t *src_a = a.stream + base_a + (size_t)w_lo * 64, *src_b = a.stream + base_b + (size_t)w_lo * 64;
-#pragma unroll
-        for (int grp = 0; grp < stage_groups(kStride); ++grp)
-            if ((uint32_t)grp * 128 < deepest) {
-                stage_fetch_pair(body, src_a, win_a, src_b, win_b, hsel, grp * 128, lane);
-                stage_commit<kStride>(body, stage, grp * 128, my_depth, lane);
-            }
-        // LDS operations of one wavefront complete in order: the reads below see the writes above
         FastLane st;
-        st.init_at<kStride>(stage, row - w_lo + 1, lane, state);
+        constexpr uint32_t qdec = kStride ? 1u : 64u;
+        if constexpr (kStride != 0) {
+            StageRegs body;
+            const uint32_t my_depth = (lane & 4) ? win_b : win_a;
+#pragma unroll
+            for (int grp = 0; grp < stage_groups(kStride); ++grp)
+                if ((uint32_t)grp * 128 < deepest) {
+                    stage_fetch_pair(body, src_a, win_a, src_b, win_b, hsel, grp * 128, lane);
+                    stage_commit<kStride>(body, stage, grp * 128, my_depth, lane);
+                }
+            // LDS operations of one wavefront complete in order: the reads below see the writes above
+            st.init_at<kStride>(stage, row - w_lo + 1, lane, state);
+        } else {
+            stage_window_pair(stage, src_a, win_a, src_b, win_b, hsel, deepest, lane);
+            const int32_t rel = row - w_lo;  // this lane's next byte, in rows of the window (< 0: none left)
+            st.X = state << 3;
+            st.q = (uint32_t)(uintptr_t)stage + (uint32_t)(rel * 64 + lane);
+            st.n1 = rel >= 0 ? stage[rel * 64 + lane] : 0;
+        }
         if (kMerge) {
             // blocks of eight rows: sign|mantissa dwords of the next block are loaded while this one decodes
             const uint32_t man_sel = 0x04040000u + (c & 3u) * 0x01010101u;
@@ -118,7 +164,7 @@ __device__ __forceinline__ void decode_one_item(const DecodeArgs &a, uint32_t it
 #pragma unroll
                 for (int r = 0; r < 8; ++r) mnext[r] = nrow[r * 8];
                 uint32_t w[4];
-                decode8_weights_asm(st, mcur, man_sel, w);
+                decode8_weights_asm(st, mcur, man_sel, w, qdec);
 #pragma unroll
                 for (int d = 0; d < 4; ++d) {
                     o[(size_t)(blk * 8 + 2 * d) * a.N] = (uint16_t)w[d];
@@ -132,7 +178,7 @@ __device__ __forceinline__ void decode_one_item(const DecodeArgs &a, uint32_t it
             // readfirstlane returns a signed int: widen through uint32_t
             const uint32_t ob_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(ob >> 32));
             const uint32_t ob_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)ob);
-            decode_tile_asm(st, ((uint64_t)ob_hi << 32) | (uint64_t)ob_lo, lane, a.N, seglen / 2);
+            decode_tile_asm(st, ((uint64_t)ob_hi << 32) | (uint64_t)ob_lo, lane, a.N, seglen / 2, qdec);
         }
     } else if (col_ok) {
         GlobalBytes src;
@@ -216,6 +262,183 @@ __global__ __launch_bounds__(kPersistWaves *kWave) void decode_tiled32_persist_k
         decode_wave_tiles<8, kDepthDeep, kMerge>(a, j, n_wg, tab, lds, wave, lane);
     else
         decode_wave_tiles<10, kDepthMedium, kMerge>(a, j, n_wg, tab, lds, wave, lane);
+}
+
+// ---- items of the sixteen-wavefront kernel, with what they read from memory asked for ahead ------------
+// What an item reads before its window is known (requested two items ahead, looked at one item ahead) ...
+struct DecRaw {
+    uint32_t state, row, row_end;               // per lane, as stored (row: 0x7fffffff = from the body's last row)
+    uint32_t off_a, depth_a, off_b, depth_b;    // the two tile bodies
+};
+// ... and the item ready to be staged.
+struct DecItem {
+    uint32_t item;
+    uint32_t state;
+    int32_t row;
+    uint32_t w_lo, rows, win_a, win_b;  // first body row of the window, rows in it (both bodies / each)
+    uint64_t base_a, base_b;
+    bool fast;
+};
+
+__device__ __forceinline__ void dec_indices(const DecodeArgs &a, uint32_t item, uint32_t &hsel, uint32_t &seg, uint32_t &p,
+                                            uint32_t &tk) {
+    const uint32_t pairs = (a.tiles_n + 1) / 2;
+    hsel = item & 1u;
+    seg = (item >> 1) % a.segs;
+    const uint32_t pr = (item >> 1) / a.segs;
+    p = pr % pairs;
+    tk = pr / pairs;
+}
+
+__device__ __forceinline__ void dec_request(const DecodeArgs &a, uint32_t item, int lane, DecRaw &m) {
+    uint32_t hsel, seg, p, tk;
+    dec_indices(a, item, hsel, seg, p, tk);
+    const uint32_t side = lane / 32, c = lane % 32;
+    const bool have_b = 2 * p + 1 < a.tiles_n;
+    const uint32_t tile_a = tk * a.tiles_n + 2 * p, tile_b = have_b ? tile_a + 1 : tile_a;
+    m.off_a = a.tile_offsets[tile_a];
+    m.depth_a = a.tile_max_lens[tile_a];
+    m.off_b = a.tile_offsets[tile_b];
+    m.depth_b = a.tile_max_lens[tile_b];
+    const uint32_t tile = side ? tile_b : tile_a, q = hsel * 32 + c;
+    const uint2 *ck = a.ckpt + ((size_t)tile * (a.segs - 1)) * 64 + q;  // (only read when segs > 1)
+    if (seg == 0) {
+        m.state = a.states[(size_t)tile * 64 + q];
+        m.row = 0x7fffffffu;
+    } else {
+        const uint2 v = ck[(size_t)(seg - 1) * 64];
+        m.state = v.x;
+        m.row = v.y;
+    }
+    m.row_end = seg + 1 < a.segs ? ck[(size_t)seg * 64].y : 0xffffffffu;
+}
+
+// Same conditions as decode_one_item's.
+template <bool kMerge>
+__device__ __forceinline__ void dec_resolve(const DecodeArgs &a, uint32_t item, int lane, const DecRaw &m, DecItem &it) {
+    uint32_t hsel, seg, p, tk;
+    dec_indices(a, item, hsel, seg, p, tk);
+    const uint32_t half = a.th / 2, seglen = half / a.segs, side = lane / 32, c = lane % 32;
+    const uint32_t tn = 2 * p + side, col = tn * 32 + c, row_first = tk * a.th + hsel * half + seg * seglen;
+    it.item = item;
+    it.base_a = m.off_a;
+    it.base_b = m.off_b;
+    uint32_t depth_a = m.depth_a, depth_b = m.depth_b;
+    if (it.base_a + (uint64_t)depth_a * 64 > a.stream_len) depth_a = 0;
+    if (it.base_b + (uint64_t)depth_b * 64 > a.stream_len) depth_b = 0;
+    const uint32_t depth = side ? depth_b : depth_a;
+    it.state = m.state;
+    it.row = min((int32_t)m.row, (int32_t)depth - 1);
+    const int32_t row_end = min((int32_t)m.row_end, it.row);
+    const bool col_ok = tn < a.tiles_n && col < a.N;
+    const bool whole = row_first < a.K && a.K - row_first >= seglen;
+    const int32_t w_lo = max(wave_min_i32(row_end) - 1, 0), w_hi = wave_max_i32(it.row);
+    it.w_lo = (uint32_t)w_lo;
+    it.win_a = (uint32_t)max(min(w_hi + 1, (int32_t)depth_a) - w_lo, 0);
+    it.win_b = (uint32_t)max(min(w_hi + 1, (int32_t)depth_b) - w_lo, 0);
+    it.rows = max(it.win_a, it.win_b);
+    it.fast = __builtin_amdgcn_ballot_w64(!col_ok) == 0 && whole && it.win_a >= 2 && it.win_b >= 2 &&
+              it.rows <= kDecWinRows && seglen % (kMerge ? 8 : 2) == 0 && seglen >= 2 &&
+              (uint64_t)a.K * a.N < (1ull << (kMerge ? 31 : 32)) && (!kMerge || a.man_aligned);
+}
+
+// Touches the cache lines of the item's two windows (a 128-byte line per lane and body); the values are not
+// used, the caller keeps them alive until the current item has been decoded.
+__device__ __forceinline__ void dec_touch(const DecodeArgs &a, const DecItem &it, int lane, uint32_t &t, uint32_t &t2) {
+    t = t2 = 0;
+    if (!it.fast) return;
+    if ((uint32_t)lane * 128 < it.win_a * 64)
+        t = *reinterpret_cast<const uint32_t *>(a.stream + it.base_a + (size_t)it.w_lo * 64 + lane * 128);
+    if ((uint32_t)lane * 128 < it.win_b * 64)
+        t2 = *reinterpret_cast<const uint32_t *>(a.stream + it.base_b + (size_t)it.w_lo * 64 + lane * 128);
+}
+
+// A resolved, fast item: its window into the wavefront's area (before anything of the next item is asked
+// for: loads complete in the order they were issued) ...
+__device__ __forceinline__ void dec_stage(const DecodeArgs &a, const DecItem &it, uint8_t *stage, int lane) {
+    stage_window_pair(stage, a.stream + it.base_a + (size_t)it.w_lo * 64, it.win_a,
+                      a.stream + it.base_b + (size_t)it.w_lo * 64, it.win_b, it.item & 1u, it.rows, lane);
+}
+
+// ... then decode, store the exponent bytes.
+__device__ __forceinline__ void dec_run(const DecodeArgs &a, const DecItem &it, uint8_t *stage, int lane) {
+    uint32_t hsel, seg, p, tk;
+    dec_indices(a, it.item, hsel, seg, p, tk);
+    const uint32_t half = a.th / 2, seglen = half / a.segs, row_first = tk * a.th + hsel * half + seg * seglen;
+    FastLane st;
+    const int32_t rel = it.row - (int32_t)it.w_lo;  // this lane's next byte, in rows of the window (< 0: none left)
+    st.X = it.state << 3;
+    st.q = (uint32_t)(uintptr_t)stage + (uint32_t)(rel * 64 + lane);
+    st.n1 = rel >= 0 ? stage[rel * 64 + lane] : 0;  // (a wavefront's LDS operations complete in order)
+    const uint64_t ob = reinterpret_cast<uint64_t>(a.out_exp + (size_t)row_first * a.N + 2 * p * 32);
+    // readfirstlane returns a signed int: widen through uint32_t
+    const uint32_t ob_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(ob >> 32));
+    const uint32_t ob_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)ob);
+    decode_tile_asm(st, ((uint64_t)ob_hi << 32) | (uint64_t)ob_lo, lane, a.N, seglen / 2, 64);
+}
+
+// The same batch on sixteen wavefronts per workgroup, for tensors whose items are short (see kDecSegWaves).
+// A wavefront walks its items with the next one's checkpoints requested and its windows touched before the
+// current one is decoded; an item whose window turns out larger than its area, a ragged one, and every item
+// of a merging decode take decode_one_item.
+template <bool kMerge>
+__global__ __launch_bounds__(kDecSegWaves *kWave) void decode_tiled32_seg_kernel(DecodeBatchArgs b) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    const uint2 *tab = reinterpret_cast<const uint2 *>(lds);
+    const int tid = threadIdx.x, lane = tid % kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    uint32_t i = 0;
+    while (i + 1 < b.n && blockIdx.x >= b.first_block[i + 1]) ++i;
+    const DecodeArgs &a = b.item[i];
+    const uint32_t j = blockIdx.x - b.first_block[i], n_wg = b.first_block[i + 1] - b.first_block[i];
+    const uint64_t n_units = decode_num_pairs(a) * a.segs;  // unit = one segment of a pair, both halves
+    uint8_t *stage = lds + kSlotTableBytes + (size_t)wave * kDecWinBytes;
+    // this wavefront's items: slot = wave, wave + 16, ...; slot / 2 picks the workgroup's unit, slot % 2 the half
+    auto item_of = [&](uint32_t slot, uint32_t &item) {
+        const uint64_t unit = (uint64_t)(slot >> 1) * n_wg + j;
+        item = (uint32_t)unit * 2 + (slot & 1u);
+        return unit < n_units;
+    };
+    if (kMerge) {
+        build_slot_table_x8(reinterpret_cast<uint2 *>(lds), a.tables, a.slot_map, tid, kDecSegWaves * kWave);
+        __syncthreads();
+        uint32_t item;
+        for (uint32_t slot = wave; item_of(slot, item); slot += kDecSegWaves)
+            decode_one_item<0, true>(a, item, tab, stage, lane);
+        return;
+    }
+    DecRaw raw;
+    DecItem nxt;
+    nxt.fast = false;
+    uint32_t slot = wave, item_n = 0, item_nn = 0;
+    bool have_n = item_of(slot, item_n), have_nn = false;
+    if (have_n) dec_request(a, item_n, lane, raw);  // on its way while the table is built
+    build_slot_table_x8(reinterpret_cast<uint2 *>(lds), a.tables, a.slot_map, tid, kDecSegWaves * kWave);
+    if (have_n) {
+        dec_resolve<false>(a, item_n, lane, raw, nxt);
+        have_nn = item_of(slot + kDecSegWaves, item_nn);
+        if (have_nn) dec_request(a, item_nn, lane, raw);
+    }
+    __syncthreads();
+    while (have_n) {
+        const DecItem cur = nxt;
+        if (cur.fast) dec_stage(a, cur, stage, lane);
+        uint32_t touched = 0, touched2 = 0;
+        have_n = have_nn;
+        item_n = item_nn;
+        slot += kDecSegWaves;
+        if (have_n) {
+            dec_resolve<false>(a, item_n, lane, raw, nxt);
+            dec_touch(a, nxt, lane, touched, touched2);
+            have_nn = item_of(slot + kDecSegWaves, item_nn);
+            if (have_nn) dec_request(a, item_nn, lane, raw);
+        }
+        if (cur.fast)
+            dec_run(a, cur, stage, lane);
+        else
+            decode_one_item<0, false>(a, cur.item, tab, stage, lane);
+        asm volatile("" ::"v"(touched), "v"(touched2));  // the touching loads end here
+    }
 }
 
 // Any tile width: one thread per stream, bytes read where they lie.  Used for widths other
@@ -352,6 +575,11 @@ static int check_segments(const char *who, uint32_t tile_height, uint32_t segmen
 
 // Launch the persistent kernel over the (already checked) tensors of `b`: the device's CUs are
 // divided among the tensors in proportion to their tile counts.
+// Rows of the longest item the sixteen-wavefront kernel is given (bf16 weight exponents take about a third
+// of a byte per symbol and the lanes of a tile drift apart by some twenty rows: 256 rows stay below the
+// window area; an item whose window is larger takes the guarded path).
+constexpr uint32_t kDecSegRows = 256;
+
 static int launch_persist(DecodeBatchArgs &b, bool merge, hipStream_t s) {
     uint32_t cus = 0;
     if (int rc = cu_count(&cus)) return rc;
@@ -386,9 +614,26 @@ static int launch_persist(DecodeBatchArgs &b, bool merge, hipStream_t s) {
         blocks += share[i];
     }
     b.first_block[b.n] = blocks;
+    // Items of at most kDecSegRows rows (segments of streams, or low tiles) have windows that fit 7 KB: such a
+    // batch runs on sixteen wavefronts per CU.
+    bool short_items = true;
+    for (uint32_t i = 0; i < b.n; ++i) short_items = short_items && b.item[i].th / 2 / b.item[i].segs <= kDecSegRows;
+    const dim3 grid(blocks);
+    if (short_items) {
+        CI_ALLOW_FULL_LDS(decode_tiled32_seg_kernel<false>);
+        CI_ALLOW_FULL_LDS(decode_tiled32_seg_kernel<true>);
+        const dim3 block(kDecSegWaves * kWave);
+        const uint32_t lds_bytes = kSlotTableBytes + kDecSegWaves * kDecWinBytes;
+        if (merge)
+            hipLaunchKernelGGL(decode_tiled32_seg_kernel<true>, grid, block, lds_bytes, s, b);
+        else
+            hipLaunchKernelGGL(decode_tiled32_seg_kernel<false>, grid, block, lds_bytes, s, b);
+        CI_LAUNCH_CHECK("decode_tiled32_seg_kernel");
+        return CI_OK;
+    }
     CI_ALLOW_FULL_LDS(decode_tiled32_persist_kernel<false>);
     CI_ALLOW_FULL_LDS(decode_tiled32_persist_kernel<true>);
-    const dim3 grid(blocks), block(kPersistWaves * kWave);
+    const dim3 block(kPersistWaves * kWave);
     if (merge)
         hipLaunchKernelGGL(decode_tiled32_persist_kernel<true>, grid, block, kLdsLimit, s, b);
     else

@@ -424,10 +424,16 @@ __device__ __forceinline__ void linear_tile_asm2(FastLane &st, f32x16_t &acc, f3
 }
 
 // Symbol of the step that used table entry ELO -> one byte at obase + off; off advances a row.
+#ifdef CI_EXP_NOSTORE
+#define CI_STORE_SYM(ELO)                                  \
+    "v_lshrrev_b32 v83, 24, " ELO "\n"                    \
+    "v_add_u32 %[off], %[stride], %[off]\n"
+#else
 #define CI_STORE_SYM(ELO)                                  \
     "v_lshrrev_b32 v83, 24, " ELO "\n"                    \
     "global_store_byte %[off], v83, %[obase]\n"           \
     "v_add_u32 %[off], %[stride], %[off]\n"
+#endif
 
 // Stand-alone decode of one half tile per lane: `npairs` >= 1 pairs of steps, symbol i stored at
 // obase + off + i * stride (bytes).  The store of a symbol sits in the shadow of the next step.

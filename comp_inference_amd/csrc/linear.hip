@@ -448,7 +448,13 @@ constexpr int kSegWaves = 16;
 constexpr uint32_t kWinRows = 112;
 constexpr int kWinPieces = (int)(kWinRows * 64 / 1024);  // 16 bytes per lane each
 constexpr uint32_t kWinBytes = kWinRows * 64;
-static_assert(kWinRows * 64 % 1024 == 0 && kSlotTableBytes + kSegWaves * kWinBytes <= kLdsLimit, "windows exceed the LDS");
+// Behind the windows: for up to kSmallM rows of x, the sums a wavefront hands over at the end of a job (32
+// tile columns per row of x), and two words of bookkeeping (wavefronts arrived, jobs added up).
+constexpr uint32_t kSmallM = 4;
+constexpr uint32_t kSmallBufOff = kSlotTableBytes + kSegWaves * kWinBytes;
+constexpr uint32_t kSmallFlagsOff = kSmallBufOff + kSegWaves * kSmallM * 32 * 4;
+constexpr uint32_t kSegLdsBytes = kSmallFlagsOff + 16;
+static_assert(kWinRows * 64 % 1024 == 0 && kSegLdsBytes <= kLdsLimit, "windows exceed the LDS");
 
 // What an item reads before its window is known (requested two items ahead, looked at one item ahead).
 struct SegRaw {
@@ -659,6 +665,14 @@ __global__ __launch_bounds__(kSegWaves *kWave) void fused_linear32_seg_kernel(Li
     int pcount = 0;
 #endif
     PROBE(1);
+    // the slot table is asked for before anything else: the job arithmetic below runs while it travels
+    const bool copy_table = (!kCold || a.dense_w == nullptr) && a.slot_table;
+    u32x4 tab0 = {0, 0, 0, 0}, tab1 = {0, 0, 0, 0};
+    if (copy_table) {
+        const u32x4 *src = reinterpret_cast<const u32x4 *>(a.slot_table);
+        tab0 = src[threadIdx.x * 2];
+        tab1 = src[threadIdx.x * 2 + 1];
+    }
     uint8_t *stage = lds + kSlotTableBytes + (size_t)wave * kWinBytes;
     SegJobs jb;
     jb.init(a);
@@ -681,12 +695,10 @@ __global__ __launch_bounds__(kSegWaves *kWave) void fused_linear32_seg_kernel(Li
     uint32_t s_nxt = next_slot(0, vk_n, tn_n), s_nn = slots;  // the next slot with an item, and the one after
     if (coded && s_nxt < slots) seg_request(a, vk_n, tn_n, lane, raw);
     PROBE(20);
-    if (coded && a.slot_table) {
-        const u32x4 *src = reinterpret_cast<const u32x4 *>(a.slot_table);
+    if (copy_table) {
         u32x4 *dst = reinterpret_cast<u32x4 *>(lds);
-        const u32x4 e0 = src[threadIdx.x * 2], e1 = src[threadIdx.x * 2 + 1];
-        dst[threadIdx.x * 2] = e0;
-        dst[threadIdx.x * 2 + 1] = e1;
+        dst[threadIdx.x * 2] = tab0;
+        dst[threadIdx.x * 2 + 1] = tab1;
     } else if (coded) {
         build_slot_table_x8(reinterpret_cast<uint2 *>(lds), a.tables, a.slot_map, threadIdx.x, kSegWaves * kWave);
     }
@@ -696,6 +708,10 @@ __global__ __launch_bounds__(kSegWaves *kWave) void fused_linear32_seg_kernel(Li
         PROBE(22);
         s_nn = next_slot(s_nxt + 1, vk_nn, tn_nn);
         if (s_nn < slots) seg_request(a, vk_nn, tn_nn, lane, raw);
+    }
+    if (threadIdx.x == 0) {
+        uint32_t *flags = reinterpret_cast<uint32_t *>(lds + kSmallFlagsOff);
+        flags[0] = flags[1] = 0;
     }
     PROBE(23);
     __syncthreads();
@@ -748,6 +764,47 @@ __global__ __launch_bounds__(kSegWaves *kWave) void fused_linear32_seg_kernel(Li
         // for x row lane%32 (MFMA 32x32 result layout: register v of lane l is row (v/4)*8 + (l/32)*4 + v%4,
         // column l%32).
         const uint32_t chunk = jb.cols == 1 ? job / a.tiles_n : 0u;
+        if (MB == 1 && a.M <= kSmallM) {
+            // Few rows of x: only the lanes of those rows hold sums, 32 per row and wavefront.  They go to a small
+            // area of their own and the last wavefront to arrive adds them up -- in wavefront order, like the
+            // general case below -- while the others are already on their next job: no barrier.  The area is
+            // handed from job to job by the count of jobs added up.
+            float *buf = reinterpret_cast<float *>(lds + kSmallBufOff);
+            uint32_t *flags = reinterpret_cast<uint32_t *>(lds + kSmallFlagsOff);
+            const uint32_t jn = sl / jb.R;  // which of this workgroup's jobs
+            while (__hip_atomic_load(&flags[1], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) != jn)
+                __builtin_amdgcn_s_sleep(2);  // (the wavefront adding up the job before this one is not waiting for us)
+            if (c < a.M) {
+#pragma unroll
+                for (int v = 0; v < 16; ++v)
+                    buf[((uint32_t)wave * kSmallM + c) * 32 + (v / 4) * 8 + hsel * 4 + (v % 4)] = acc[v];
+            }
+            uint32_t arrived = 0;
+            if (lane == 0) arrived = __hip_atomic_fetch_add(&flags[0], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_WORKGROUP);
+            arrived = (uint32_t)__builtin_amdgcn_readfirstlane((int)arrived);
+            if (arrived == (uint32_t)kSegWaves - 1) {
+                const uint32_t per_tile = 32 * a.M;
+                for (uint32_t o = lane; o < jb.cols * per_tile; o += kWave) {
+                    const uint32_t t = o / per_tile, mg = (o % per_tile) / 32, n32 = o % 32;
+                    const uint32_t col_tile = jb.cols == 1 ? job % a.tiles_n : job * jb.cols + t;
+                    float sum = 0.f;
+                    for (uint32_t i = 0; i < jb.per_col; ++i) sum += buf[((t * jb.per_col + i) * kSmallM + mg) * 32 + n32];
+                    const uint32_t n = col_tile * 32 + n32;
+                    if (col_tile < a.tiles_n && n < a.N) {
+                        if (a.P == 1)
+                            a.out[(size_t)mg * a.out_stride + n] = finish_bf16(sum, a.bias, n);
+                        else
+                            a.partial[((size_t)chunk * a.M + mg) * a.N + n] = sum;
+                    }
+                }
+                if (lane == 0) {
+                    __hip_atomic_store(&flags[0], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    __hip_atomic_store(&flags[1], jn + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+                }
+            }
+            PROBE(7);
+            continue;
+        }
         float *red = reinterpret_cast<float *>(lds + kSlotTableBytes);
 #pragma unroll
         for (int g = 0; g < MB; ++g) {
@@ -1156,7 +1213,7 @@ static int fused_linear_impl(const uint16_t *d_x, uint32_t M, uint32_t K, uint32
         const uint32_t VK = a.tiles_k * p.segs;
         const uint32_t jobs = VK >= (uint32_t)kSegWaves ? a.tiles_n * p.P : ceil_div(a.tiles_n, kSegWaves / VK);
         const dim3 grid(jobs < cus ? jobs : cus), block(kSegWaves * kWave);
-        const uint32_t lds_bytes = kSlotTableBytes + kSegWaves * kWinBytes;
+        const uint32_t lds_bytes = kSegLdsBytes;
 #define CI_LAUNCH_SEG(MB_, COLD_)                                                                   \
     do {                                                                                            \
         CI_ALLOW_FULL_LDS((fused_linear32_seg_kernel<MB_, COLD_>));                                 \

@@ -86,6 +86,12 @@ def test_whole_layer_decodes_bit_exact_in_one_launch(oracle, layer_weights):
     outs = ci.rans_decomp_tiled_batch(items, tile_k=1024, tile_n=32)
     for (name, _), o, e in zip(layer_weights.items(), outs, planes):
         assert torch.equal(o.cpu(), e), name
+    # the same launch with decoder checkpoints (two segments per stream: sixteen wavefronts per CU on windows of
+    # the bodies, what the benchmark times)
+    with_ck = [it + (ci.build_checkpoints(*it, 1024, 32, 2), 2) for it in items]
+    outs = ci.rans_decomp_tiled_batch(with_ck, tile_k=1024, tile_n=32)
+    for (name, _), o, e in zip(layer_weights.items(), outs, planes):
+        assert torch.equal(o.cpu(), e), name
 
 
 @pytest.mark.parametrize("M", [1, 4, 16, 64])
