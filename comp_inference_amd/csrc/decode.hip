@@ -28,6 +28,7 @@ struct DecodeArgs {
     // that are decoded as work items of their own.
     const uint2 *ckpt;
     uint32_t segs;
+    uint32_t seglen;  // th / (2 segs): rows of an item (kept here: the kernels would divide for it per item)
 };
 
 // Work item of the 32-column kernels: one half (top or bottom rows) of two neighbouring column
@@ -86,7 +87,7 @@ __device__ __forceinline__ void decode_one_item(const DecodeArgs &a, uint32_t it
     const uint32_t pairs = (a.tiles_n + 1) / 2;
     const uint32_t hsel = item & 1u, seg = (item >> 1) % a.segs, pr = (item >> 1) / a.segs;
     const uint32_t p = pr % pairs, tk = pr / pairs;
-    const uint32_t half = a.th / 2, seglen = half / a.segs, side = lane / 32, c = lane % 32;
+    const uint32_t half = a.th / 2, seglen = a.seglen, side = lane / 32, c = lane % 32;
     const uint32_t tn = 2 * p + side, col = tn * 32 + c, row_first = tk * a.th + hsel * half + seg * seglen;
     if (row_first >= a.K) return;  // past the end of a short last tile row
     const bool have_b = 2 * p + 1 < a.tiles_n;
@@ -264,6 +265,10 @@ __global__ __launch_bounds__(kPersistWaves *kWave) void decode_tiled32_persist_k
         decode_wave_tiles<10, kDepthMedium, kMerge>(a, j, n_wg, tab, lds, wave, lane);
 }
 
+// Where an item lies: worked out once per item (the divisions are long instruction sequences) and handed on.
+struct DecCoord {
+    uint32_t item, hsel, seg, p, tk;
+};
 // ---- items of the sixteen-wavefront kernel, with what they read from memory asked for ahead ------------
 // What an item reads before its window is known (requested two items ahead, looked at one item ahead) ...
 struct DecRaw {
@@ -272,7 +277,7 @@ struct DecRaw {
 };
 // ... and the item ready to be staged.
 struct DecItem {
-    uint32_t item;
+    DecCoord co;
     uint32_t state;
     int32_t row;
     uint32_t w_lo, rows, win_a, win_b;  // first body row of the window, rows in it (both bodies / each)
@@ -280,19 +285,20 @@ struct DecItem {
     bool fast;
 };
 
-__device__ __forceinline__ void dec_indices(const DecodeArgs &a, uint32_t item, uint32_t &hsel, uint32_t &seg, uint32_t &p,
-                                            uint32_t &tk) {
+__device__ __forceinline__ DecCoord dec_coord(const DecodeArgs &a, uint32_t item) {
     const uint32_t pairs = (a.tiles_n + 1) / 2;
-    hsel = item & 1u;
-    seg = (item >> 1) % a.segs;
-    const uint32_t pr = (item >> 1) / a.segs;
-    p = pr % pairs;
-    tk = pr / pairs;
+    DecCoord c;
+    c.item = item;
+    c.hsel = item & 1u;
+    const uint32_t us = item >> 1, pr = us / a.segs;
+    c.seg = us - pr * a.segs;
+    c.tk = pr / pairs;
+    c.p = pr - c.tk * pairs;
+    return c;
 }
 
-__device__ __forceinline__ void dec_request(const DecodeArgs &a, uint32_t item, int lane, DecRaw &m) {
-    uint32_t hsel, seg, p, tk;
-    dec_indices(a, item, hsel, seg, p, tk);
+__device__ __forceinline__ void dec_request(const DecodeArgs &a, const DecCoord &co, int lane, DecRaw &m) {
+    const uint32_t hsel = co.hsel, seg = co.seg, p = co.p, tk = co.tk;
     const uint32_t side = lane / 32, c = lane % 32;
     const bool have_b = 2 * p + 1 < a.tiles_n;
     const uint32_t tile_a = tk * a.tiles_n + 2 * p, tile_b = have_b ? tile_a + 1 : tile_a;
@@ -315,12 +321,11 @@ __device__ __forceinline__ void dec_request(const DecodeArgs &a, uint32_t item, 
 
 // Same conditions as decode_one_item's.
 template <bool kMerge>
-__device__ __forceinline__ void dec_resolve(const DecodeArgs &a, uint32_t item, int lane, const DecRaw &m, DecItem &it) {
-    uint32_t hsel, seg, p, tk;
-    dec_indices(a, item, hsel, seg, p, tk);
-    const uint32_t half = a.th / 2, seglen = half / a.segs, side = lane / 32, c = lane % 32;
+__device__ __forceinline__ void dec_resolve(const DecodeArgs &a, const DecCoord &co, int lane, const DecRaw &m, DecItem &it) {
+    const uint32_t hsel = co.hsel, seg = co.seg, p = co.p, tk = co.tk;
+    const uint32_t half = a.th / 2, seglen = a.seglen, side = lane / 32, c = lane % 32;
     const uint32_t tn = 2 * p + side, col = tn * 32 + c, row_first = tk * a.th + hsel * half + seg * seglen;
-    it.item = item;
+    it.co = co;
     it.base_a = m.off_a;
     it.base_b = m.off_b;
     uint32_t depth_a = m.depth_a, depth_b = m.depth_b;
@@ -357,14 +362,13 @@ __device__ __forceinline__ void dec_touch(const DecodeArgs &a, const DecItem &it
 // for: loads complete in the order they were issued) ...
 __device__ __forceinline__ void dec_stage(const DecodeArgs &a, const DecItem &it, uint8_t *stage, int lane) {
     stage_window_pair(stage, a.stream + it.base_a + (size_t)it.w_lo * 64, it.win_a,
-                      a.stream + it.base_b + (size_t)it.w_lo * 64, it.win_b, it.item & 1u, it.rows, lane);
+                      a.stream + it.base_b + (size_t)it.w_lo * 64, it.win_b, it.co.hsel, it.rows, lane);
 }
 
 // ... then decode, store the exponent bytes.
 __device__ __forceinline__ void dec_run(const DecodeArgs &a, const DecItem &it, uint8_t *stage, int lane) {
-    uint32_t hsel, seg, p, tk;
-    dec_indices(a, it.item, hsel, seg, p, tk);
-    const uint32_t half = a.th / 2, seglen = half / a.segs, row_first = tk * a.th + hsel * half + seg * seglen;
+    const uint32_t hsel = it.co.hsel, seg = it.co.seg, p = it.co.p, tk = it.co.tk;
+    const uint32_t half = a.th / 2, seglen = a.seglen, row_first = tk * a.th + hsel * half + seg * seglen;
     FastLane st;
     const int32_t rel = it.row - (int32_t)it.w_lo;  // this lane's next byte, in rows of the window (< 0: none left)
     st.X = it.state << 3;
@@ -389,7 +393,9 @@ __global__ __launch_bounds__(kDecSegWaves *kWave) void decode_tiled32_seg_kernel
     const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
     uint32_t i = 0;
     while (i + 1 < b.n && blockIdx.x >= b.first_block[i + 1]) ++i;
-    const DecodeArgs &a = b.item[i];
+    // (a copy: the tensor's description then sits in scalar registers, where a reference into the kernel
+    // arguments at a variable index would be read from memory again wherever a field is used)
+    const DecodeArgs a = b.item[i];
     const uint32_t j = blockIdx.x - b.first_block[i], n_wg = b.first_block[i + 1] - b.first_block[i];
     const uint64_t n_units = decode_num_pairs(a) * a.segs;  // unit = one segment of a pair, both halves
     uint8_t *stage = lds + kSlotTableBytes + (size_t)wave * kDecWinBytes;
@@ -412,12 +418,16 @@ __global__ __launch_bounds__(kDecSegWaves *kWave) void decode_tiled32_seg_kernel
     nxt.fast = false;
     uint32_t slot = wave, item_n = 0, item_nn = 0;
     bool have_n = item_of(slot, item_n), have_nn = false;
-    if (have_n) dec_request(a, item_n, lane, raw);  // on its way while the table is built
+    DecCoord co_n = dec_coord(a, item_n), co_nn = co_n;
+    if (have_n) dec_request(a, co_n, lane, raw);  // on its way while the table is built
     build_slot_table_x8(reinterpret_cast<uint2 *>(lds), a.tables, a.slot_map, tid, kDecSegWaves * kWave);
     if (have_n) {
-        dec_resolve<false>(a, item_n, lane, raw, nxt);
+        dec_resolve<false>(a, co_n, lane, raw, nxt);
         have_nn = item_of(slot + kDecSegWaves, item_nn);
-        if (have_nn) dec_request(a, item_nn, lane, raw);
+        if (have_nn) {
+            co_nn = dec_coord(a, item_nn);
+            dec_request(a, co_nn, lane, raw);
+        }
     }
     __syncthreads();
     while (have_n) {
@@ -425,21 +435,25 @@ __global__ __launch_bounds__(kDecSegWaves *kWave) void decode_tiled32_seg_kernel
         if (cur.fast) dec_stage(a, cur, stage, lane);
         uint32_t touched = 0, touched2 = 0;
         have_n = have_nn;
-        item_n = item_nn;
+        co_n = co_nn;
         slot += kDecSegWaves;
         if (have_n) {
-            dec_resolve<false>(a, item_n, lane, raw, nxt);
+            dec_resolve<false>(a, co_n, lane, raw, nxt);
             dec_touch(a, nxt, lane, touched, touched2);
             have_nn = item_of(slot + kDecSegWaves, item_nn);
-            if (have_nn) dec_request(a, item_nn, lane, raw);
+            if (have_nn) {
+                co_nn = dec_coord(a, item_nn);
+                dec_request(a, co_nn, lane, raw);
+            }
         }
         if (cur.fast)
             dec_run(a, cur, stage, lane);
         else
-            decode_one_item<0, false>(a, cur.item, tab, stage, lane);
+            decode_one_item<0, false>(a, cur.co.item, tab, stage, lane);
         asm volatile("" ::"v"(touched), "v"(touched2));  // the touching loads end here
     }
 }
+
 
 // Any tile width: one thread per stream, bytes read where they lie.  Used for widths other
 // than 32 (the reference's tests sweep 16..128, tests/test_mat_mul.py:263-264).
@@ -686,11 +700,13 @@ extern "C" int ci_decode_tiled_ilp2_batch(const ci_decode_item *h_items, uint32_
             a.man_aligned = 0;
             a.ckpt = nullptr;
             a.segs = 1;
+            a.seglen = it.tile_height / 2;
             if (it.segments > 1) {
                 if (int rc = check_segments("ci_decode_tiled_ilp2_batch", it.tile_height, it.segments, it.d_checkpoints))
                     return rc;
                 a.ckpt = static_cast<const uint2 *>(it.d_checkpoints);
                 a.segs = it.segments;
+                a.seglen = it.tile_height / 2 / it.segments;
             }
             ++b.n;
         }
@@ -753,10 +769,12 @@ extern "C" int ci_decode_tiled_ilp2_segmented(const uint8_t *d_stream, uint64_t 
     a.man_aligned = merge && aligned(d_man_tiled, 4) ? 1u : 0u;
     a.ckpt = nullptr;
     a.segs = 1;
+    a.seglen = tile_height / 2;
     if (segments > 1 && tile_width == 32) {  // (other widths decode one thread per stream: nothing to split)
         if (int rc = check_segments("ci_decode_tiled_ilp2_segmented", tile_height, segments, d_checkpoints)) return rc;
         a.ckpt = static_cast<const uint2 *>(d_checkpoints);
         a.segs = segments;
+        a.seglen = tile_height / 2 / segments;
     }
     if (tile_width == 32 && aligned(d_stream, 16)) {
         DecodeBatchArgs b;

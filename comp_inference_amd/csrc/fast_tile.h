@@ -424,16 +424,10 @@ __device__ __forceinline__ void linear_tile_asm2(FastLane &st, f32x16_t &acc, f3
 }
 
 // Symbol of the step that used table entry ELO -> one byte at obase + off; off advances a row.
-#ifdef CI_EXP_NOSTORE
-#define CI_STORE_SYM(ELO)                                  \
-    "v_lshrrev_b32 v83, 24, " ELO "\n"                    \
-    "v_add_u32 %[off], %[stride], %[off]\n"
-#else
 #define CI_STORE_SYM(ELO)                                  \
     "v_lshrrev_b32 v83, 24, " ELO "\n"                    \
     "global_store_byte %[off], v83, %[obase]\n"           \
     "v_add_u32 %[off], %[stride], %[off]\n"
-#endif
 
 // Stand-alone decode of one half tile per lane: `npairs` >= 1 pairs of steps, symbol i stored at
 // obase + off + i * stride (bytes).  The store of a symbol sits in the shadow of the next step.
@@ -452,7 +446,9 @@ __device__ __forceinline__ void decode_tile_asm(FastLane &st, uint64_t obase, ui
         "ci_dec_done%=:\n"
         CI_STEP_ISSUE("v[74:75]") CI_STORE_SYM("v72") CI_STEP_FINISH("v74", "v75")
         CI_STORE_SYM("v74")
-        "s_waitcnt vmcnt(0) lgkmcnt(0)\n"
+        // (the stores may still be on their way: they hold no register the compiler could reuse too early, and
+        // the next reader of these bytes is another kernel)
+        "s_waitcnt lgkmcnt(0)\n"
         : [X] "+v"(st.X), [q] "+v"(st.q), [n1] "+v"(st.n1), [off] "+v"(off)
         : [L8] "s"(kRansL << 3), [obase] "s"(obase), [stride] "s"(stride), [npairs] "s"(npairs), [qdec] "s"(qdec)
         : CI_STEP_CLOBBERS, "scc", "s22", "v83");

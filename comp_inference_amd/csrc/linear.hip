@@ -551,11 +551,6 @@ __device__ __forceinline__ void seg_stage(const LinearArgs &a, const SegItem &it
 }
 
 // One staged item through the hand-scheduled loop, accumulating into acc (and acc2 for x rows 32..63).
-#ifdef CI_EXP_MANHOT
-#define CI_EXP_TILE(t) ((t) & 7)
-#else
-#define CI_EXP_TILE(t) (t)
-#endif
 template <int MB>
 __device__ __forceinline__ void seg_run(const LinearArgs &a, const SegItem &it, const uint8_t *stage, int lane,
                                         f32x16 &acc, f32x16 &acc2) {
@@ -569,7 +564,7 @@ __device__ __forceinline__ void seg_run(const LinearArgs &a, const SegItem &it, 
     st.n1 = rel >= 0 ? stage[rel * 64 + lane] : 0;
     const uint32_t m = c;  // row of x this lane feeds to the (first) MFMA
     const bool m_ok = m < a.M, m2_ok = MB == 2 && m + 32 < a.M;
-    const uint64_t mbase = reinterpret_cast<uint64_t>(a.man_tiled + (size_t)CI_EXP_TILE(tile) * a.th * 32);
+    const uint64_t mbase = reinterpret_cast<uint64_t>(a.man_tiled + (size_t)tile * a.th * 32);
     // readfirstlane returns a signed int: widen through uint32_t, not by sign extension
     const uint32_t mb_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(mbase >> 32));
     const uint32_t mb_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)mbase);
