@@ -37,11 +37,11 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 # The binding limit of byte-wise rANS on this chip is not HBM but the rate of dependent decode steps:
-# one step of one wavefront (64 streams) occupies a CU's LDS pipe for about 9.4 ns (one random 8-byte
-# table read and two byte reads; measured with a micro-benchmark, the same from 8 to 16 wavefronts per
-# CU), and a lone wavefront needs about 65 ns per step.  Reported next to every HBM fraction.
-STEP_NS_PER_CU = 9.4
-STEP_NS_LATENCY = 65.0
+# one step of one wavefront (64 streams) takes about 6.0 ns of a CU that sixteen wavefronts share (one
+# random 8-byte table read and one byte read from LDS, eight VALU instructions), and a lone wavefront needs
+# about 87 ns per step (profiles/step_rate_microbench.md).  Reported next to every HBM fraction.
+STEP_NS_PER_CU = 6.0
+STEP_NS_LATENCY = 87.0
 NUM_CUS = 256  # replaced by the device's own count in main()
 
 
@@ -51,9 +51,9 @@ def step_bound_us(wave_steps: int, chain: int) -> dict:
             "latency_us": round(chain * STEP_NS_LATENCY * 1e-3, 1)}
 # HBM bytes of one batched decode launch on this workload.  Not measured by this program: taken from
 # offline rocprofv3 FETCH_SIZE and WRITE_SIZE passes over this same command, scaled by what the same
-# counters read for a plain copy of known size: 38115.2 KiB x 1.9991 fetched + 212992.0 KiB x 1.0 written.
-MEASURED_TRAFFIC_BYTES = 296_130_080
-TRAFFIC_SOURCE = "profiles/decode_tiled32_persist_kernel_llama8b_layer.md (offline counter passes, not this run)"
+# counters read for a plain copy of known size: 72735.3 KiB x 1.9988 fetched + 212992.0 KiB x 1.0 written.
+MEASURED_TRAFFIC_BYTES = 366_978_000
+TRAFFIC_SOURCE = "profiles/decode_tiled32_seg_kernel_llama8b_layer.md (offline counter passes, not this run)"
 LAYER = [("q", 4096, 4096), ("k", 1024, 4096), ("v", 1024, 4096), ("o", 4096, 4096),
          ("gate", 14336, 4096), ("up", 14336, 4096), ("down", 4096, 14336)]  # (name, out, in)
 
@@ -352,7 +352,7 @@ def main() -> int:
     record("decode_tiled32_seg_kernel", "one layer, seven tensors, one launch, 2 segments per stream", algo_bytes, launch_us)
     record("decode_tiled32_persist_kernel", "the same without checkpoints (whole streams)", algo_bytes - checkpoint_bytes, us_whole_streams)
     wave_steps = sum(c.wave_steps() for c in layer)
-    sb = step_bound_us(wave_steps, th // 2)
+    sb = step_bound_us(wave_steps, th // 2 // DECODE_SEGMENTS)
     roofline["step_rate_bound"] = dict(sb, wavefront_steps=wave_steps, ns_per_wavefront_step_per_cu=STEP_NS_PER_CU,
                                        frac=round(sb["throughput_us"] / launch_us, 3))
 
@@ -384,7 +384,7 @@ def main() -> int:
             us_ref = batched_time_us(lambda: torch.matmul(x, w_dense), 25, 100)
             nbytes = gate.linear_bytes(M)
             record("fused linear (checkpoints)", f"gate K=4096 N=14336 M={M}", nbytes, us)
-            sb = step_bound_us(gate.wave_steps(), gate.th // 2)
+            sb = step_bound_us(gate.wave_steps(), gate.th // 2 // int(gate.segments))
             rows.append({"M": M, "us": round(us, 2), "us_without_checkpoints": round(us_plain, 2), "allclose_1e-2": ok,
                          "step_rate_bound_us": max(sb["throughput_us"], sb["latency_us"]),
                          "hbm_frac_compressed_bytes": round(nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
