@@ -47,7 +47,7 @@ def tiled_weight(K, N, tile_k, tile_n, stream, states, tables, slot_map, tile_of
     w.d_tables, w.d_slot_map = tables.data_ptr(), slot_map.data_ptr()
     w.d_tile_offsets, w.d_tile_max_lens = tile_offsets.data_ptr(), tile_max_lens.data_ptr()
     w.n_tiles = min(tile_offsets.numel(), tile_max_lens.numel())
-    w.d_man_tiled, w.man_len = man.data_ptr(), man.numel()
+    w.d_man_tiled, w.man_len = (man.data_ptr(), man.numel()) if man is not None else (None, 0)
     if checkpoints is not None and segments > 1:
         w.d_checkpoints, w.checkpoint_bytes, w.segments = checkpoints.data_ptr(), checkpoints.numel() * 8, int(segments)
     else:

@@ -792,3 +792,14 @@ extern "C" int ci_decode_tiled_ilp2_segmented(const uint8_t *d_stream, uint64_t 
     }
     return CI_OK;
 }
+
+extern "C" int ci_decode_tiled(const ci_tiled_weight *w, uint8_t *d_out_exp, uint16_t *d_out_bf16, ci_stream_t stream) {
+    if (int rc = ci_tiled_weight_check(w)) return rc;
+    if (d_out_bf16 && !w->d_man_tiled) return fail(CI_ERR_ARG, "ci_decode_tiled: bf16 asked of a weight without sign|mantissa plane");
+    const uint32_t segments = w->segments > 1 ? w->segments : 1;
+    return ci_decode_tiled_ilp2_segmented(w->d_stream, w->stream_len, w->d_states, w->d_tables, w->d_slot_map,
+                                          w->d_tile_offsets, w->d_tile_max_lens, w->K, w->N, w->tile_height,
+                                          w->tile_width, segments > 1 ? w->d_checkpoints : nullptr, segments,
+                                          d_out_bf16 ? nullptr : d_out_exp, d_out_bf16 ? w->d_man_tiled : nullptr,
+                                          d_out_bf16, stream);
+}

@@ -769,6 +769,18 @@ extern "C" int ci_fused_embedding_ilp2_segmented(const int64_t *d_ids, uint32_t 
                           segments);
 }
 
+extern "C" int ci_fused_embedding_tiled(const ci_tiled_weight *w, const int64_t *d_ids, uint32_t n_ids, uint16_t *d_out,
+                                        uint32_t out_stride, void *d_workspace, size_t workspace_bytes,
+                                        ci_stream_t stream) {
+    if (int rc = ci_tiled_weight_check(w)) return rc;
+    if (!w->d_man_tiled) return fail(CI_ERR_ARG, "fused embedding: the weight has no sign|mantissa plane");
+    const uint32_t segments = w->segments > 1 ? w->segments : 1;
+    return embedding_impl(d_ids, n_ids, w->d_stream, w->stream_len, w->d_states, w->d_tables, w->d_slot_map,
+                          w->d_tile_offsets, w->d_tile_max_lens, w->d_man_tiled, w->K, w->N, w->tile_height,
+                          w->tile_width, d_out, out_stride, d_workspace, workspace_bytes, false,
+                          static_cast<hipStream_t>(stream), segments > 1 ? w->d_checkpoints : nullptr, segments);
+}
+
 extern "C" int ci_fused_embedding_dense(const int64_t *d_ids, uint32_t n_ids, const uint8_t *d_stream,
                                         uint64_t stream_len, const uint32_t *d_states, const uint32_t *d_tables,
                                         const uint8_t *d_slot_map, const uint32_t *d_stream_offsets,

@@ -1373,8 +1373,11 @@ extern "C" int ci_tiled_weight_check(const ci_tiled_weight *w) {
         return fail(CI_ERR_ARG, "weight descriptor: bad shape %u x %u, tile %u x %u", w->K, w->N, w->tile_height,
                     w->tile_width);
     const uint64_t tiles = (uint64_t)ceil_div(w->K, w->tile_height) * ceil_div(w->N, w->tile_width);
-    if (!w->d_states || !w->d_tables || !w->d_slot_map || !w->d_tile_offsets || !w->d_tile_max_lens || !w->d_man_tiled)
+    if (!w->d_states || !w->d_tables || !w->d_slot_map || !w->d_tile_offsets || !w->d_tile_max_lens)
         return fail(CI_ERR_ARG, "weight descriptor: null pointer");
+    // (a weight without sign|mantissa plane can only be decoded to its exponent plane)
+    if (!w->d_man_tiled && w->man_len) return fail(CI_ERR_ARG, "weight descriptor: null sign|mantissa plane of %llu bytes",
+                                                  (unsigned long long)w->man_len);
     if (w->stream_len && !w->d_stream) return fail(CI_ERR_ARG, "weight descriptor: null stream");
     if (!aligned(w->d_slot_map, 4)) return fail(CI_ERR_ARG, "weight descriptor: slot_map must be 4-byte aligned");
     if (w->n_states < tiles * 2 * w->tile_width)
@@ -1383,7 +1386,7 @@ extern "C" int ci_tiled_weight_check(const ci_tiled_weight *w) {
     if (w->n_tiles < tiles)
         return fail(CI_ERR_ARG, "weight descriptor: tile metadata for %llu tiles, the shape has %llu",
                     (unsigned long long)w->n_tiles, (unsigned long long)tiles);
-    if (w->man_len < tiles * w->tile_height * w->tile_width)
+    if (w->d_man_tiled && w->man_len < tiles * w->tile_height * w->tile_width)
         return fail(CI_ERR_ARG, "weight descriptor: sign|mantissa plane of %llu bytes, the tiles take %llu",
                     (unsigned long long)w->man_len, (unsigned long long)(tiles * w->tile_height * w->tile_width));
     if (w->segments > 1) {
@@ -1403,6 +1406,7 @@ extern "C" int ci_fused_linear_tiled(const ci_tiled_weight *w, const uint16_t *d
                                      const uint16_t *d_bias, uint16_t *d_out, uint32_t out_stride, void *d_workspace,
                                      size_t workspace_bytes, ci_stream_t stream) {
     if (int rc = ci_tiled_weight_check(w)) return rc;
+    if (!w->d_man_tiled) return fail(CI_ERR_ARG, "fused linear: the weight has no sign|mantissa plane");
     return fused_linear_impl(d_x, M, w->K, w->N, x_stride, w->d_stream, w->stream_len, w->d_states, w->d_tables,
                              w->d_slot_map, w->d_tile_offsets, w->d_tile_max_lens, w->d_man_tiled, w->tile_height,
                              w->tile_width, d_bias, d_out, out_stride, d_workspace, workspace_bytes, false,
@@ -1442,6 +1446,7 @@ extern "C" int ci_fused_linear_tiled_noalloc(const ci_tiled_weight *w, const uin
                                              uint32_t x_stride, const uint16_t *d_bias, uint16_t *d_out,
                                              uint32_t out_stride, ci_stream_t stream) {
     if (int rc = ci_tiled_weight_check(w)) return rc;
+    if (!w->d_man_tiled) return fail(CI_ERR_ARG, "fused linear: the weight has no sign|mantissa plane");
     const uint32_t segments = w->segments > 1 ? w->segments : 1;
     const size_t need = ci_fused_linear_workspace_bytes_segmented(M, w->K, w->N, w->tile_height, w->tile_width, 0, segments);
     if (need > (size_t)CI_NOALLOC_SCRATCH_BYTES)

@@ -395,6 +395,18 @@ extern "C" int ci_fused_linear_transposed_ilp2(const uint16_t *d_x, uint32_t M, 
                            out_stride, d_workspace, workspace_bytes, false, stream);
 }
 
+extern "C" int ci_fused_linear_transposed_tiled(const ci_tiled_weight *w, const uint16_t *d_x, uint32_t M,
+                                                uint32_t x_stride, const uint16_t *d_bias, uint16_t *d_out,
+                                                uint32_t out_stride, void *d_workspace, size_t workspace_bytes,
+                                                ci_stream_t stream) {
+    if (int rc = ci_tiled_weight_check(w)) return rc;
+    if (!w->d_man_tiled) return fail(CI_ERR_ARG, "transposed linear: the weight has no sign|mantissa plane");
+    // (the weight is stored [V, H]: its rows are the outputs)
+    return transposed_impl(d_x, M, w->N, w->K, x_stride, w->d_stream, w->stream_len, w->d_states, w->d_tables,
+                           w->d_slot_map, w->d_tile_offsets, w->d_tile_max_lens, w->d_man_tiled, w->tile_height,
+                           w->tile_width, d_bias, d_out, out_stride, d_workspace, workspace_bytes, false, stream);
+}
+
 extern "C" int ci_fused_linear_transposed_dense(const uint16_t *d_x, uint32_t M, uint32_t H, uint32_t V,
                                                 uint32_t x_stride, const uint8_t *d_stream, uint64_t stream_len,
                                                 const uint32_t *d_states, const uint32_t *d_tables,

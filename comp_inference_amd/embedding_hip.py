@@ -43,24 +43,18 @@ def _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, met
         check(lib().ci_fused_embedding_dense(
             ptr(ids), n, ptr(stream_t), C.c_uint64(stream_t.numel()), ptr(st), ptr(tb), ptr(sm), ptr(m0), ptr(m1),
             ptr(man), K, N, int(tile_k), int(tile_n), ptr(result), result.stride(0), _lib.stream_handle(dev)))
-    elif checkpoints is not None and int(segments) > 1:
-        segments = int(segments)
-        ck = checkpoints.to(dev).contiguous()
-        if ck.dtype != torch.int64 or ck.numel() * 8 != lib().ci_checkpoint_bytes(K, N, int(tile_k), int(tile_n), segments):
-            raise RuntimeError("checkpoints do not belong to this table shape, tiling and segment count")
+    else:
+        ck, segments = None, 1 if checkpoints is None else int(segments)
+        if segments > 1:
+            ck = checkpoints.to(dev).contiguous()
+            if ck.dtype != torch.int64:
+                raise RuntimeError("checkpoints do not belong to this table shape, tiling and segment count")
         need = lib().ci_fused_embedding_workspace_bytes_segmented(n, K, int(tile_k), segments)
         ws = _Scratch.get(need, ("emb", dev))
-        check(lib().ci_fused_embedding_ilp2_segmented(
-            ptr(ids), n, ptr(stream_t), C.c_uint64(stream_t.numel()), ptr(st), ptr(tb), ptr(sm), ptr(m0), ptr(m1),
-            ptr(man), K, N, int(tile_k), int(tile_n), ptr(ck), segments, ptr(result), result.stride(0), ptr(ws),
-            C.c_size_t(ws.numel() if ws is not None else 0), _lib.stream_handle(dev)))
-    else:
-        need = lib().ci_fused_embedding_workspace_bytes(n, K, int(tile_k))
-        ws = _Scratch.get(need, ("emb", dev))
-        check(lib().ci_fused_embedding_ilp2(
-            ptr(ids), n, ptr(stream_t), C.c_uint64(stream_t.numel()), ptr(st), ptr(tb), ptr(sm), ptr(m0), ptr(m1),
-            ptr(man), K, N, int(tile_k), int(tile_n), ptr(result), result.stride(0), ptr(ws),
-            C.c_size_t(ws.numel() if ws is not None else 0), _lib.stream_handle(dev)))
+        # the lengths of every operand travel with it and are checked by the library before the launch
+        w = _lib.tiled_weight(K, N, tile_k, tile_n, stream_t, st, tb, sm, m0, m1, man, ck, segments)
+        check(lib().ci_fused_embedding_tiled(C.byref(w), ptr(ids), n, ptr(result), result.stride(0), ptr(ws),
+                                             C.c_size_t(ws.numel() if ws is not None else 0), _lib.stream_handle(dev)))
     if out is not None:
         return out.view(*x.shape, N)
     return result.view(*x.shape, N)

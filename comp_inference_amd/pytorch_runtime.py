@@ -145,6 +145,7 @@ class RansLMHead(nn.Module):
                      "rans_exp_tile_offsets", "rans_exp_tile_max_lens", "rans_man_raw", "rans_info"):
             setattr(self, name, getattr(emb, name))
         self.tile_k, self.tile_n = emb.tile_k, emb.tile_n
+        self.tied_to_embedding = True
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         device = x.device
@@ -239,6 +240,20 @@ def swap_in_rans_modules(model: nn.Module, state_dict: dict, quant_config: dict 
     if hasattr(model, "lm_head") and "lm_head.rans_exp_stream" in state_dict:
         th, tw = tile_of("lm_head")
         model.lm_head = RansLMHead(model.lm_head.in_features, model.lm_head.out_features, tile_k=th, tile_n=tw)
+    elif hasattr(model, "lm_head") and not any(k in state_dict for k in ("lm_head.weight", "model.lm_head.weight")):
+        # A package written with a tied head holds neither lm_head.weight nor a compressed head: the head is the
+        # embedding table.  The reference gets there through from_pretrained's own tying; a model built from its
+        # config alone (or handed in) would keep a randomly initialised head once the embedding has been
+        # replaced, so the head is tied to the compressed table here -- or the load fails.
+        emb = model.get_input_embeddings() if hasattr(model, "get_input_embeddings") else None
+        if isinstance(emb, RansEmbedding):
+            head = RansLMHead(model.lm_head.in_features, model.lm_head.out_features, tile_k=emb.tile_k, tile_n=emb.tile_n)
+            head.tie_to(emb)
+            model.lm_head = head
+        elif isinstance(emb, nn.Embedding) and isinstance(model.lm_head, nn.Linear):
+            model.lm_head.weight = emb.weight
+        else:
+            raise RuntimeError("the file holds no lm_head weights and the model has no embedding to tie the head to")
 
     targets = dict(model.named_buffers())
     targets.update(dict(model.named_parameters()))
@@ -273,4 +288,10 @@ def load_compressed_model_with_auto_model(model_id: str, safetensors_path: str, 
             quant_config = json.load(open(cfg_path)).get("quantization_config", {})
     state_dict = load_file(safetensors_path, device="cpu")
     model = swap_in_rans_modules(model, state_dict, quant_config, split_k)
-    return model.cuda()
+    model = model.cuda()
+    # (moving a module gives each of its buffers a tensor of its own: a head tied to the table is tied again,
+    # so that the table is on the GPU once)
+    head, emb = getattr(model, "lm_head", None), model.get_input_embeddings() if hasattr(model, "get_input_embeddings") else None
+    if isinstance(head, RansLMHead) and getattr(head, "tied_to_embedding", False) and isinstance(emb, RansEmbedding):
+        head.tie_to(emb)
+    return model

@@ -63,10 +63,10 @@ def rans_decomp_tiled(compressed_streams, initial_states, tables, slot_map, outp
     st, tb, sm = _lib.as_u32(initial_states, dev), _lib.as_u32(tables, dev), _lib.as_u8(slot_map, dev)
     to, tl = _lib.as_u32(tile_offsets, dev), _lib.as_u32(tile_max_lens, dev)
     ck, segments = _checked_checkpoints(checkpoints, segments, K, N, tile_k, tile_n, dev)
-    check(lib().ci_decode_tiled_ilp2_segmented(
-        ptr(stream_t), C.c_uint64(stream_t.numel()), ptr(st), ptr(tb), ptr(sm), ptr(to), ptr(tl),
-        K, N, int(tile_k), int(tile_n), ptr(ck), segments, None if merge else ptr(out), ptr(man) if merge else None,
-        ptr(out) if merge else None, _lib.stream_handle(dev)))
+    # the lengths of every operand travel with it and are checked by the library before the launch
+    w = _lib.tiled_weight(K, N, tile_k, tile_n, stream_t, st, tb, sm, to, tl, man, ck, segments)
+    check(lib().ci_decode_tiled(C.byref(w), None if merge else ptr(out), ptr(out) if merge else None,
+                                _lib.stream_handle(dev)))
     return out
 
 
@@ -170,7 +170,13 @@ def rans_decomp_tiled_uncoalesced(compressed_streams, initial_states, tables, sl
                               stream_sizes, True)
     stream_t = _lib.as_u8(compressed_streams, dev)
     merge = mantissas is not None
-    man = _lib.as_u8(mantissas, dev).view(-1) if merge else None
+    man = None
+    if merge:
+        man = _lib.as_u8(mantissas, dev).view(-1)
+        num_tiles_n, num_tiles_k = _tiles(K, N, tile_k, tile_n)
+        need = num_tiles_k * num_tiles_n * tile_k * tile_n
+        if man.numel() < need:  # a truncated tail reads as zero padding, as in rans_decomp_tiled
+            man = torch.nn.functional.pad(man, (0, need - man.numel()))
     out = torch.empty((K, N), device=dev, dtype=torch.bfloat16 if merge else torch.uint8)
     st, tb, sm = _lib.as_u32(initial_states, dev), _lib.as_u32(tables, dev), _lib.as_u8(slot_map, dev)
     so, sz = _lib.as_u32(stream_offsets, dev), _lib.as_u32(stream_sizes, dev)

@@ -60,8 +60,8 @@ def collect_tensors(model, tied_lm_head: bool = False) -> dict:
         handled.update({"lm_head.weight", "model.lm_head.weight"})
     for name, module in model.named_modules():
         if getattr(module, "compressed", None) == "rans_bfloat16":
-            if tied_lm_head and "lm_head" in name:
-                continue
+            # (a compressed lm_head keeps its tensors also when the head is tied, as in
+            # comp_inference/rans_saving.py:193-227: only the plain lm_head.weight is dropped)
             tensors.update(rans_tensors_for_module(name + ".", module))
             handled.update({f"{name}.weight", f"{name}.bias"})
     for pname, param in model.named_parameters():

@@ -55,10 +55,17 @@ def _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, met
     # device copies must stay referenced until the launch has been enqueued
     st, tb, sm = _lib.as_u32(initial_states, dev), _lib.as_u32(tables, dev), _lib.as_u8(slot_map, dev)
     m0, m1 = _lib.as_u32(meta0, dev), _lib.as_u32(meta1, dev)
-    fn = lib().ci_fused_linear_transposed_dense if dense else lib().ci_fused_linear_transposed_ilp2
-    check(fn(ptr(x2), M, H, V, x2.stride(0), ptr(stream_t), C.c_uint64(stream_t.numel()), ptr(st), ptr(tb),
-             ptr(sm), ptr(m0), ptr(m1), ptr(man), int(tile_k), int(tile_n), ptr(b), ptr(result),
-             result.stride(0), ptr(ws), C.c_size_t(ws.numel()), _lib.stream_handle(dev)))
+    if dense:
+        check(lib().ci_fused_linear_transposed_dense(
+            ptr(x2), M, H, V, x2.stride(0), ptr(stream_t), C.c_uint64(stream_t.numel()), ptr(st), ptr(tb), ptr(sm),
+            ptr(m0), ptr(m1), ptr(man), int(tile_k), int(tile_n), ptr(b), ptr(result), result.stride(0), ptr(ws),
+            C.c_size_t(ws.numel()), _lib.stream_handle(dev)))
+    else:
+        # the lengths of every operand travel with it and are checked by the library before the launch
+        w = _lib.tiled_weight(V, H, tile_k, tile_n, stream_t, st, tb, sm, m0, m1, man)
+        check(lib().ci_fused_linear_transposed_tiled(C.byref(w), ptr(x2), M, x2.stride(0), ptr(b), ptr(result),
+                                                     result.stride(0), ptr(ws), C.c_size_t(ws.numel()),
+                                                     _lib.stream_handle(dev)))
     if out is not None:
         return out
     return result.view(*x.shape[:-1], V)

@@ -380,7 +380,7 @@ typedef struct ci_tiled_weight {
     const uint32_t *d_tile_offsets;
     const uint32_t *d_tile_max_lens;
     uint64_t n_tiles;                 /* entries in each of the two, >= tiles */
-    const uint8_t *d_man_tiled;
+    const uint8_t *d_man_tiled;       /* NULL (with man_len 0): exponent plane only */
     uint64_t man_len;                 /* bytes, >= tiles * tile_height * tile_width */
     const void *d_checkpoints;
     uint64_t checkpoint_bytes;        /* == ci_checkpoint_bytes(K, N, tile_height, tile_width, segments) */
@@ -418,6 +418,22 @@ int ci_max_window_rows(const ci_tiled_weight *w, uint32_t *d_rows, ci_stream_t s
 int ci_fused_linear_tiled(const ci_tiled_weight *w, const uint16_t *d_x, uint32_t M, uint32_t x_stride,
                           const uint16_t *d_bias, uint16_t *d_out, uint32_t out_stride, void *d_workspace,
                           size_t workspace_bytes, ci_stream_t stream);
+
+/* The other operators on a descriptor, lengths checked before the launch like ci_fused_linear_tiled:
+ * ci_decode_tiled = ci_decode_tiled_ilp2[_segmented] (exponent plane to d_out_exp, or, with d_out_bf16
+ * given, the bf16 tensor from the weight's own sign|mantissa plane; a descriptor with d_man_tiled NULL and
+ * man_len 0 is accepted for the exponent plane alone), ci_fused_embedding_tiled =
+ * ci_fused_embedding_ilp2[_segmented] (workspace: ci_fused_embedding_workspace_bytes_segmented),
+ * ci_fused_linear_transposed_tiled = ci_fused_linear_transposed_ilp2 with the weight stored [V, H]
+ * (K = V rows, N = H columns in the descriptor). */
+int ci_decode_tiled(const ci_tiled_weight *w, uint8_t *d_out_exp, uint16_t *d_out_bf16, ci_stream_t stream);
+
+int ci_fused_embedding_tiled(const ci_tiled_weight *w, const int64_t *d_ids, uint32_t n_ids, uint16_t *d_out,
+                             uint32_t out_stride, void *d_workspace, size_t workspace_bytes, ci_stream_t stream);
+
+int ci_fused_linear_transposed_tiled(const ci_tiled_weight *w, const uint16_t *d_x, uint32_t M, uint32_t x_stride,
+                                     const uint16_t *d_bias, uint16_t *d_out, uint32_t out_stride,
+                                     void *d_workspace, size_t workspace_bytes, ci_stream_t stream);
 
 /* The same fused linear for callers that cannot allocate device memory -- code under HIP graph
  * capture, tight serving loops, harnesses that forbid allocation.  It has no counterpart in the

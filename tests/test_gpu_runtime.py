@@ -364,3 +364,52 @@ def test_gguf_export_holds_the_weights(tmp_path):
         got = ci.reconstruct_from_exp_and_mantissa(exp.cpu(), man)
         assert torch.equal(got.view(torch.int16), w.view(torch.int16)), base
     assert torch.equal(u("blk.0.ffn_up.bias", torch.float32), up.bias.detach().float())
+
+
+def test_tied_head_package_ties_the_head_to_the_compressed_table(tmp_path):
+    """A model whose head shares the embedding table, saved with tied_lm_head=True: the file holds the compressed
+    table once and no lm_head.weight (comp_inference/rans_saving.py:186-191); loaded into a freshly built model
+    (nothing pretrained behind it) the head must be tied to the compressed table, not left at its random
+    initialisation.  With the head compressed as well its tensors stay in the file, as in the reference."""
+    import comp_inference_amd as ci
+    from safetensors import safe_open
+
+    class TinyTied(Tiny):
+        def get_input_embeddings(self):
+            return self.embed_tokens
+
+    def make(seed):
+        torch.manual_seed(seed)
+        m = TinyTied().to(torch.bfloat16)
+        with torch.no_grad():
+            for p in m.parameters():
+                if p.ndim == 2:
+                    p.mul_(0.3)
+        m.lm_head.weight = m.embed_tokens.weight
+        return m
+
+    ref = make(0)
+    ids = torch.tensor([[3, 17, 1299, 640]])
+    want = _forward_fp32_linears(ref.cuda(), ids.cuda()).float().cpu()
+    comp = make(0)
+    ci.rans_compress_module_weight(comp.embed_tokens, tile_height=256, tile_width=32, transpose_weight=False)
+    for name in ("up_proj", "down_proj"):
+        ci.rans_compress_module_weight(getattr(comp, name), tile_height=64, tile_width=32)
+    out_dir = ci.save_rans_model_package(comp, None, str(tmp_path / "tied"), tied_lm_head=True)
+    path = os.path.join(out_dir, "model.safetensors")
+    with safe_open(path, "pt") as f:
+        keys = set(f.keys())
+    assert "embed_tokens.rans_exp_stream" in keys and "lm_head.weight" not in keys and "lm_head.rans_exp_stream" not in keys
+    model = ci.load_compressed_model_with_auto_model("unused", path, model=make(77))
+    assert isinstance(model.lm_head, ci.RansLMHead) and isinstance(model.embed_tokens, ci.RansEmbedding)
+    assert model.lm_head.rans_exp_stream.data_ptr() == model.embed_tokens.rans_exp_stream.data_ptr()  # on the GPU once
+    got = model(ids.cuda()).float().cpu()
+    assert torch.allclose(got, want, atol=1e-2, rtol=1e-2), (got - want).abs().max()
+
+    # head compressed too: its tensors are written although the head is tied
+    both = make(0)
+    both.lm_head.weight = nn.Parameter(both.embed_tokens.weight.detach().clone())
+    ci.rans_compress_module_weight(both.embed_tokens, tile_height=256, tile_width=32, transpose_weight=False)
+    ci.rans_compress_module_weight(both.lm_head, tile_height=256, tile_width=32, transpose_weight=False)
+    tensors = ci.rans_saving.collect_tensors(both, tied_lm_head=True)
+    assert "lm_head.rans_exp_stream" in tensors and "lm_head.weight" not in tensors

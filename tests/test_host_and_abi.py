@@ -253,3 +253,66 @@ def test_public_header_is_plain_c(tmp_path):
                     str(src), "-o", str(exe), _lib.LIB_PATH, "-Wl,-rpath," + os.path.dirname(_lib.LIB_PATH),
                     "-Wl,-rpath,/opt/rocm/lib"], check=True)
     assert subprocess.run([str(exe)]).returncode == 0
+
+
+def test_a_descriptor_with_a_short_array_is_refused_on_the_host():
+    """ci_tiled_weight carries the length of every array; the check runs on the host alone, so every kind of short
+    or missing array is tried here with made-up addresses, and the entry points that take a descriptor refuse it
+    with CI_ERR_ARG (1) before any device call."""
+    from comp_inference_amd import _lib
+
+    lib = _lib.lib()
+    K, N, th, tw = 4096, 96, 1024, 32
+    tiles = (K // th) * (N // tw)
+
+    def desc(**over):
+        w = _lib.TiledWeight()
+        w.K, w.N, w.tile_height, w.tile_width = K, N, th, tw
+        w.d_stream, w.stream_len = 0x10000, 1 << 20
+        w.d_states, w.n_states = 0x20000, tiles * 64
+        w.d_tables, w.d_slot_map = 0x30000, 0x40000
+        w.d_tile_offsets, w.d_tile_max_lens, w.n_tiles = 0x50000, 0x60000, tiles
+        w.d_man_tiled, w.man_len = 0x70000, tiles * th * tw
+        w.d_checkpoints, w.checkpoint_bytes, w.segments = None, 0, 1
+        w.d_slot_table, w.slot_table_bytes, w.max_window_rows = None, 0, 0
+        for k, v in over.items():
+            setattr(w, k, v)
+        return w
+
+    def rc(**over):
+        return lib.ci_tiled_weight_check(ctypes.byref(desc(**over)))
+
+    assert rc() == 0
+    assert rc(n_states=tiles * 64 - 1) == 1 and b"states" in lib.ci_last_error()
+    assert rc(n_tiles=tiles - 1) == 1 and b"tile metadata" in lib.ci_last_error()
+    assert rc(man_len=tiles * th * tw - 1) == 1 and b"mantissa" in lib.ci_last_error()
+    assert rc(d_man_tiled=None, man_len=0) == 0            # exponent plane only
+    assert rc(d_man_tiled=None) == 1
+    assert rc(d_states=None) == 1 and rc(d_tile_offsets=None) == 1 and rc(d_stream=None) == 1
+    assert rc(d_slot_map=0x40002) == 1                     # not 4-byte aligned
+    assert rc(tile_height=1023) == 1 and rc(K=0) == 1
+    ck = lib.ci_checkpoint_bytes(K, N, th, tw, 4)
+    assert ck == tiles * 3 * 64 * 8
+    assert rc(segments=4, d_checkpoints=0x80000, checkpoint_bytes=ck) == 0
+    assert rc(segments=4, d_checkpoints=0x80000, checkpoint_bytes=ck - 8) == 1 and b"checkpoints" in lib.ci_last_error()
+    assert rc(segments=4, d_checkpoints=None, checkpoint_bytes=ck) == 1
+    assert rc(segments=4, d_checkpoints=0x80004, checkpoint_bytes=ck) == 1
+    assert rc(d_slot_table=0x90000, slot_table_bytes=32768) == 0 and rc(d_slot_table=0x90000, slot_table_bytes=4096) == 1
+    assert lib.ci_tiled_weight_check(None) == 1
+
+    # every entry point that takes a descriptor checks it first
+    fake = ctypes.c_void_p(0x1000)
+    short = ctypes.byref(desc(n_states=5))
+    sz = ctypes.c_size_t
+    assert lib.ci_fused_linear_tiled(short, fake, 1, K, None, fake, N, fake, sz(1 << 20), None) == 1
+    assert lib.ci_fused_linear_tiled_noalloc(short, fake, 1, K, None, fake, N, None) == 1
+    assert lib.ci_fused_embedding_tiled(short, fake, 3, fake, N, fake, sz(1 << 20), None) == 1
+    assert lib.ci_fused_linear_transposed_tiled(short, fake, 1, N, None, fake, K, fake, sz(1 << 20), None) == 1
+    assert lib.ci_decode_tiled(short, fake, None, None) == 1
+    assert lib.ci_max_window_rows(short, fake, None) == 1
+    # operators that need the sign|mantissa plane refuse a weight without one
+    bare = ctypes.byref(desc(d_man_tiled=None, man_len=0))
+    assert lib.ci_fused_linear_tiled(bare, fake, 1, K, None, fake, N, fake, sz(1 << 20), None) == 1
+    assert lib.ci_fused_embedding_tiled(bare, fake, 3, fake, N, fake, sz(1 << 20), None) == 1
+    assert lib.ci_fused_linear_transposed_tiled(bare, fake, 1, N, None, fake, K, fake, sz(1 << 20), None) == 1
+    assert lib.ci_decode_tiled(bare, None, fake, None) == 1
