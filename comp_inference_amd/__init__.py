@@ -29,6 +29,7 @@ from .linear_hip import (
     fused_rans_linear_triton_uncoalesced,
     fused_rans_linear_uncoalesced,
     plain_linear_same_order,
+    release_scratch,
     splitk_reduce,
     triton_matmul,
 )

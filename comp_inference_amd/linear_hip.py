@@ -15,10 +15,12 @@ from ._lib import check, lib, ptr
 
 
 class _Scratch:
-    """Grow-only scratch areas (split-K partials, decoded weights, sort keys), one per device and purpose
-    (the reference keeps a class-level buffer too, comp_inference/pytorch_runtime.py:386-394).  Calls that
-    follow each other on one stream share them safely; calls that run at the same time on different
-    streams of one device would overwrite each other's scratch -- pass `workspace=` of your own there."""
+    """Scratch areas (split-K partials, decoded weights, sort keys), one per purpose, device and stream (the
+    reference keeps a class-level buffer too, comp_inference/pytorch_runtime.py:386-394).  Calls that follow
+    each other on one stream share an area safely; calls on different streams get areas of their own.  An
+    area grows to the largest request it has seen and stays: the decode-once path of a many-row linear keeps
+    one bf16 weight (117 MB for a 4096 x 14336 projection, 1 GB for a 128256 x 4096 head) until
+    `release_scratch()` is called or `DECODE_ONCE_ABOVE_ROWS` is set to None."""
     _buf: dict = {}
 
     @classmethod
@@ -27,11 +29,25 @@ class _Scratch:
         if nbytes == 0:
             return None
         device = key[1] if isinstance(key, tuple) else key
+        key = (key, torch.cuda.current_stream(device).cuda_stream)
         b = cls._buf.get(key)
         if b is None or b.numel() < nbytes:
             b = torch.empty(nbytes, dtype=torch.uint8, device=device)
             cls._buf[key] = b
         return b
+
+    @classmethod
+    def release(cls) -> int:
+        """Drops every scratch area; returns the bytes given back to torch's allocator."""
+        n = sum(b.numel() for b in cls._buf.values())
+        cls._buf.clear()
+        return n
+
+
+def release_scratch() -> int:
+    """Frees the scratch areas the operators keep between calls (they are allocated again on demand).  Not
+    while a captured graph that uses them may still be replayed."""
+    return _Scratch.release()
 
 
 # Rows of x above which the fused linear decodes the weight ONCE into a bf16 scratch and multiplies with

@@ -60,8 +60,9 @@ def _cached_checkpoints(mod: nn.Module, device, shape, segments: int):
     """(checkpoints, segments) of `mod`'s compressed weight as it lies on `device`: built on first use from
     the stream (one pass of the decoder) and kept beside it; derived data, not part of the saved state."""
     cached = getattr(mod, "_ckpt_cache", None)
-    if cached is not None and cached[0][0] is mod.rans_exp_stream and cached[0][1] == device \
-            and cached[0][2] == segments:
+    st = mod.rans_exp_stream
+    key = ((st.data_ptr(), st.numel(), st._version), device, segments)  # (a reload swaps the storage, not the tensor)
+    if cached is not None and cached[0] == key:
         return cached[1], cached[2]
     ck = None
     if segments > 1:
@@ -69,7 +70,7 @@ def _cached_checkpoints(mod: nn.Module, device, shape, segments: int):
                                mod.rans_exp_tables.to(device), mod.rans_exp_slot_map.to(device), shape,
                                mod.rans_exp_tile_offsets.to(device), mod.rans_exp_tile_max_lens.to(device),
                                mod.tile_k, mod.tile_n, segments)
-    mod._ckpt_cache = ((mod.rans_exp_stream, device, segments), ck, segments if ck is not None else 1)
+    mod._ckpt_cache = (key, ck, segments if ck is not None else 1)
     return mod._ckpt_cache[1], mod._ckpt_cache[2]
 
 
@@ -106,11 +107,18 @@ class RansLinear(nn.Module):
         segs = suggest_segments(shape, self.tile_k, self.tile_n) if self.segments == "auto" else int(self.segments)
         return _cached_checkpoints(self, device, shape, segs)
 
+    def _buffers_key(self):
+        """What the prepared call was made from: storage, length and version of every buffer, so that a reload
+        that swaps `tensor.data` under an unchanged tensor object (the loader's own idiom) or an in-place update
+        is noticed."""
+        ts = (self.rans_exp_stream, self.rans_exp_states, self.rans_man_raw, self.bias)  # (a reload replaces them all)
+        return tuple((t.data_ptr(), t.numel(), t._version) if t is not None else None for t in ts)
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         device = x.device
         prepared = getattr(self, "_prepared", None)
-        if prepared is None or prepared[0] is not self.rans_exp_stream or prepared[1] != device \
-                or prepared[2] is not self.bias or prepared[3] != self.segments:
+        key = (self._buffers_key(), device, self.segments)
+        if prepared is None or prepared[0] != key:
             from . import _lib
 
             _lib.require_device(x)
@@ -119,8 +127,8 @@ class RansLinear(nn.Module):
                                   self.rans_exp_slot_map, (self.in_features, self.out_features),
                                   self.rans_exp_tile_offsets, self.rans_exp_tile_max_lens, self.tile_k, self.tile_n,
                                   self.rans_man_raw, self.bias, checkpoints, segments)
-            prepared = self._prepared = (self.rans_exp_stream, device, self.bias, self.segments, call)
-        return prepared[4](x)
+            prepared = self._prepared = (key, call)
+        return prepared[1](x)
 
 
 class RansLMHead(nn.Module):

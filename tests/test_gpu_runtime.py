@@ -262,12 +262,12 @@ def test_rans_linear_prepares_once_and_follows_its_buffers():
     xs = {M: torch.randn(M, K).to(torch.bfloat16).cuda() for M in (1, 5, 64, 70)}
     for M in (1, 5, 1, 64, 70, 5):                       # buffers on the host: device copies are kept
         assert same(rl(xs[M]), entry(xs[M], bias, segs)), M
-    first = rl._prepared[4]
-    assert rl(xs[1][None]).shape == (1, 1, N) and rl._prepared[4] is first
+    first = rl._prepared[1]
+    assert rl(xs[1][None]).shape == (1, 1, N) and rl._prepared[1] is first
 
     rl = rl.cuda()                                       # the buffers are new tensors now
-    assert same(rl(xs[5]), entry(xs[5], bias, segs)) and rl._prepared[4] is not first
-    assert rl._prepared[4].keep[0].data_ptr() == rl.rans_exp_stream.data_ptr()      # no second copy
+    assert same(rl(xs[5]), entry(xs[5], bias, segs)) and rl._prepared[1] is not first
+    assert rl._prepared[1].keep[0].data_ptr() == rl.rans_exp_stream.data_ptr()      # no second copy
 
     rl.bias = (bias.float() + 1).to(torch.bfloat16).cuda()
     assert same(rl(xs[5]), entry(xs[5], rl.bias, segs))
@@ -276,13 +276,13 @@ def test_rans_linear_prepares_once_and_follows_its_buffers():
     with pytest.raises(RuntimeError):
         rl(xs[5].cpu())
     with pytest.raises(RuntimeError):
-        rl._prepared[4](xs[5].cpu())
+        rl._prepared[1](xs[5].cpu())
 
     import copy                                          # a copy of the module points at its own tensors
     want = rl(xs[5])
     twin = copy.deepcopy(rl)
-    call = twin._prepared[4]
-    assert call is not rl._prepared[4] and call.keep[0] is twin.rans_exp_stream
+    call = twin._prepared[1]
+    assert call is not rl._prepared[1] and call.keep[0] is twin.rans_exp_stream
     assert call.keep[0].data_ptr() != rl.rans_exp_stream.data_ptr()
     assert call.p[0].value == call.keep[0].data_ptr() and call.p[6].value == call.keep[6].data_ptr()
     del rl
@@ -413,3 +413,28 @@ def test_tied_head_package_ties_the_head_to_the_compressed_table(tmp_path):
     ci.rans_compress_module_weight(both.lm_head, tile_height=256, tile_width=32, transpose_weight=False)
     tensors = ci.rans_saving.collect_tensors(both, tied_lm_head=True)
     assert "lm_head.rans_exp_stream" in tensors and "lm_head.weight" not in tensors
+
+
+def test_reloading_buffers_in_place_is_noticed():
+    """The loader's idiom replaces `tensor.data` under the same tensor objects: a module that has already run
+    must drop what it prepared from the old storage (pointers, checkpoints, slot table) and use the new weight."""
+    import comp_inference_amd as ci
+
+    def compressed(seed):
+        torch.manual_seed(seed)
+        lin = nn.Linear(2048, 64, bias=False).to(torch.bfloat16)
+        w = lin.weight.detach().clone()
+        ci.rans_compress_module_weight(lin, tile_height=1024, tile_width=32)
+        return ci.RansLinear.from_compressed(lin).cuda(), w
+
+    a, wa = compressed(1)
+    b, wb = compressed(2)
+    x = torch.randn(2, 2048).to(torch.bfloat16).cuda()
+    ya = a(x).float().cpu()
+    assert torch.allclose(ya, x.float().cpu() @ wa.float().t(), atol=1e-2, rtol=1e-2)
+    for name, buf in a.named_buffers():
+        buf.data = dict(b.named_buffers())[name].data.clone()
+    yb = a(x).float().cpu()
+    assert torch.allclose(yb, x.float().cpu() @ wb.float().t(), atol=1e-2, rtol=1e-2)
+    assert torch.equal(yb, b(x).float().cpu())
+    assert ci.release_scratch() >= 0
