@@ -235,8 +235,10 @@ __device__ __forceinline__ void stage_body(uint8_t *stage, const uint8_t *__rest
     "s_branch 9b\n"                                    \
     ".subsection 0\n"
 
+// (scc: s_and_saveexec_b64 writes it -- a loop compare the compiler placed before a statement must not be
+// trusted after it)
 #define CI_STEP_CLOBBERS                                                                                  \
-    "vcc", "s20", "s21", "v72", "v73", "v74", "v75", "v76", "v77", "v78", "memory"
+    "vcc", "scc", "s20", "s21", "v72", "v73", "v74", "v75", "v76", "v77", "v78", "memory"
 
 // Two decoded symbols (top bytes of ELO0, ELO1) and their sign|mantissa bytes (byte %[msel] of the
 // dwords M0, M1) -> one dword holding two bf16 (first row in the low half).  v83/v112 temporaries.
@@ -376,7 +378,7 @@ __device__ __forceinline__ void linear_tile_asm(FastLane &st, f32x16_t &acc, uin
         : [L8] "s"(kRansL << 3), [selE] "s"(0x070C030Cu), [mask] "s"(0x807F807Fu),
           [msel] "v"(man_sel), [mbase] "s"(mbase), [xbase] "s"(xbase), [nblk] "s"(nblocks), [wrapM] "s"(wrap_m),
           [wrapX] "s"(wrap_x), [xstep] "s"(xstep), [qdec] "s"(qdec)
-        : CI_STEP_CLOBBERS, "scc", "s22", "s23", "s24", "s25", "v83", "v84", "v85", "v86", "v87", "v88",
+        : CI_STEP_CLOBBERS, "s22", "s23", "s24", "s25", "v83", "v84", "v85", "v86", "v87", "v88",
           "v89", "v90", "v91", "v92", "v93", "v94", "v95", "v96", "v97", "v98", "v99", "v100", "v101",
           "v102", "v103", "v104", "v105", "v106", "v107", "v108", "v109", "v110", "v111", "v112", "v116", "v117",
           "v118", "v119");
@@ -417,7 +419,7 @@ __device__ __forceinline__ void linear_tile_asm2(FastLane &st, f32x16_t &acc, f3
         : [L8] "s"(kRansL << 3), [selE] "s"(0x070C030Cu), [mask] "s"(0x807F807Fu),
           [msel] "v"(man_sel), [mbase] "s"(mbase), [xbase] "s"(xbase), [nblk] "s"(nblocks), [wrapM] "s"(wrap_m),
           [wrapX] "s"(wrap_x), [xstep] "s"(xstep), [qdec] "s"(qdec)
-        : CI_STEP_CLOBBERS, "scc", "s22", "s23", "s24", "s25", "v83", "v84", "v85", "v86", "v87", "v88",
+        : CI_STEP_CLOBBERS, "s22", "s23", "s24", "s25", "v83", "v84", "v85", "v86", "v87", "v88",
           "v89", "v90", "v91", "v92", "v93", "v94", "v95", "v96", "v97", "v98", "v99", "v100", "v101",
           "v102", "v103", "v104", "v105", "v106", "v107", "v108", "v109", "v110", "v111", "v112", "v116", "v117",
           "v118", "v119", "v120", "v121", "v122", "v123", "v124", "v125", "v126", "v127");
@@ -451,7 +453,7 @@ __device__ __forceinline__ void decode_tile_asm(FastLane &st, uint64_t obase, ui
         "s_waitcnt lgkmcnt(0)\n"
         : [X] "+v"(st.X), [q] "+v"(st.q), [n1] "+v"(st.n1), [off] "+v"(off)
         : [L8] "s"(kRansL << 3), [obase] "s"(obase), [stride] "s"(stride), [npairs] "s"(npairs), [qdec] "s"(qdec)
-        : CI_STEP_CLOBBERS, "scc", "s22", "v83");
+        : CI_STEP_CLOBBERS, "s22", "v83");
 }
 
 // Eight symbols of this lane's stream as bf16 weights: w[d] = rows 2d (low half) and 2d + 1 of the
@@ -484,7 +486,7 @@ __device__ __forceinline__ uint32_t advance_asm(FastLane &st, uint32_t n, uint32
         "v_mov_b32 %[e], v72\n"
         : [X] "+v"(st.X), [q] "+v"(st.q), [n1] "+v"(st.n1), [e] "=&v"(e)
         : [L8] "s"(kRansL << 3), [n] "s"(n), [qdec] "s"(qdec)
-        : CI_STEP_CLOBBERS, "scc", "s22");
+        : CI_STEP_CLOBBERS, "s22");
     return e;
 }
 

@@ -38,6 +38,12 @@ struct TransArgs {
     // Verification aid: when set, the weights are read from this plain bf16 [V, H] matrix instead of
     // being decoded (same products, same reduction); none of the compressed operands is touched.
     const uint16_t *dense_w;
+    // Decoder checkpoints (the index of ci_build_checkpoints_ilp2) for the sixteen-wavefront kernel: every
+    // stream cut into segs segments of seglen rows; slot_table: the 32 KB table kept beside the weight, or null.
+    const uint2 *ckpt;
+    uint32_t segs, seglen;
+    const uint2 *slot_table;
+    uint32_t first_tile;  // trans32_kernel: tiles below this one are not its work
 };
 
 template <int kCtrl>
@@ -212,7 +218,8 @@ template <int MB, int kWaves, uint32_t kStride>
 __device__ __forceinline__ void trans_wave_tiles(const TransArgs &a, const uint2 *tab, uint8_t *lds, int wave, int lane) {
     if (wave >= kWaves) return;
     uint8_t *stage = persist_stage<kWaves, kStride>(lds, wave);
-    for (uint64_t tile = (uint64_t)wave * gridDim.x + blockIdx.x; tile < a.num_tiles; tile += (uint64_t)kWaves * gridDim.x)
+    for (uint64_t tile = (uint64_t)wave * gridDim.x + blockIdx.x + a.first_tile; tile < a.num_tiles;
+         tile += (uint64_t)kWaves * gridDim.x)
         trans_one_tile<MB, kStride>(a, (uint32_t)tile, tab, stage, lane);
 }
 
@@ -225,14 +232,123 @@ __global__ __launch_bounds__(kPersistWaves *kWave) void trans32_kernel(TransArgs
     const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
     // (a plain-weight run has no table to build; which wavefront takes which tile does not change a tile's sums)
     const uint32_t cls = a.dense_w ? 0u
-                                   : persist_prologue(lds, a.tables, a.slot_map, a.tile_max_lens, a.num_tiles,
-                                                      blockIdx.x, gridDim.x);
+                                   : persist_prologue(lds, a.tables, a.slot_map, a.tile_max_lens + a.first_tile,
+                                                      a.num_tiles - a.first_tile, blockIdx.x, gridDim.x);
     if (cls == 2u)
         trans_wave_tiles<MB, 8, kDepthDeep>(a, tab, lds, wave, lane);
     else if (cls == 1u)
         trans_wave_tiles<MB, 10, kDepthMedium>(a, tab, lds, wave, lane);
     else
         trans_wave_tiles<MB, 11, kDepthShallow>(a, tab, lds, wave, lane);
+}
+
+// ---- sixteen wavefronts per CU, one row of x --------------------------------------------------------------
+// The decode step is a chain of dependent instructions and what hides it is the number of wavefronts in flight:
+// sixteen leave each 128 VGPRs and, next to the slot table, 7 KB of LDS, which holds the window of the tile body
+// that one segment of the 64 streams reads (decoder checkpoints), staged as the rows lie in memory (pointer step
+// 64, no transposition).  An item = (tile, segment): seglen rows of both halves.  The caller guarantees, from the
+// weight's descriptor, that every item it sends here is whole and has a window of at most kTrWinRows rows; an
+// item that does not qualify after all is left out rather than staged beyond its area.  Tiles of a short last
+// tile row go to trans32_kernel (first_tile).
+constexpr int kTrSegWaves = 16;
+constexpr uint32_t kTrWinRows = 112;
+constexpr uint32_t kTrWinBytes = kTrWinRows * 64;
+constexpr int kTrWinPieces = (int)(kTrWinBytes / 1024);  // 16 bytes per lane each
+static_assert(kTrWinBytes % 1024 == 0 && kSlotTableBytes + kTrSegWaves * kTrWinBytes <= kLdsLimit, "windows exceed the LDS");
+
+__device__ __forceinline__ void trans_one_segment(const TransArgs &a, uint32_t tile, uint32_t seg, uint8_t *stage, int lane) {
+    const uint32_t tk = tile / a.tiles_n, tn = tile - tk * a.tiles_n;
+    const uint32_t half = a.th / 2, seglen = a.seglen, hsel = lane / 32, c = lane % 32;
+    const uint32_t v0 = tk * a.th + hsel * half + seg * seglen, h = tn * 32 + c;
+    const uint64_t base = a.tile_offsets[tile];
+    uint32_t depth = a.tile_max_lens[tile];
+    if (base + (uint64_t)depth * 64 > a.stream_len) depth = 0;  // a body that would run past the stream is not read
+    // decoder state and row of the next unread byte at the segment's first row, and the row reached at its end
+    uint32_t state;
+    int32_t row = (int32_t)depth - 1, row_end = -1;
+    {
+        const uint2 *ck = a.ckpt + ((size_t)tile * (a.segs - 1)) * 64 + lane;  // (only read when segs > 1)
+        if (seg == 0) {
+            state = a.states[(size_t)tile * 64 + lane];
+        } else {
+            const uint2 v = ck[(size_t)(seg - 1) * 64];
+            state = v.x;
+            row = min((int32_t)v.y, (int32_t)depth - 1);
+        }
+        if (seg + 1 < a.segs) row_end = min((int32_t)ck[(size_t)seg * 64].y, row);
+    }
+    const bool whole = __builtin_amdgcn_ballot_w64(v0 >= a.V || a.V - v0 < seglen || h >= a.H) == 0;
+    const int32_t lo = max(wave_min_i32(row_end), 0), hi = wave_max_i32(row);
+    const uint32_t rows = hi >= lo ? (uint32_t)(hi - lo + 1) : 0u;
+    if (!whole || rows == 0 || rows > kTrWinRows || seglen % 32 != 0) return;  // (promised not to happen)
+
+    // the window, memory -> LDS as it lies; every lane loads every piece (from the window's first bytes where its
+    // own lie outside), so that the loads are all in flight together
+    const uint8_t *src = a.stream + base + (size_t)lo * 64;
+    {
+        u32x4 w[kTrWinPieces];
+#pragma unroll
+        for (int g = 0; g < kTrWinPieces; ++g) {
+            const uint32_t o = (uint32_t)g * 1024 + lane * 16;
+            w[g] = *reinterpret_cast<const u32x4 *>(src + (o < rows * 64 ? o : 0u));
+        }
+#pragma unroll
+        for (int g = 0; g < kTrWinPieces; ++g) {
+            const uint32_t o = (uint32_t)g * 1024 + lane * 16;
+            if (o < rows * 64) *reinterpret_cast<u32x4 *>(stage + o) = w[g];
+        }
+    }
+    FastLane st;
+    const int32_t rel = row - lo;  // this lane's next byte, in rows of the window (< 0: none left)
+    st.X = state << 3;
+    st.q = (uint32_t)(uintptr_t)stage + (uint32_t)(rel * 64 + lane);
+    st.n1 = rel >= 0 ? stage[rel * 64 + lane] : 0;  // (a wavefront's LDS operations complete in order)
+
+    uint32_t xb[1] = {a.x[h]};  // bf16 bits of x[0, h]
+    const uint8_t *man_seg = a.man_tiled + (size_t)tile * a.th * 32 + (size_t)(hsel * half + seg * seglen) * 32;
+    float *dst = a.partial + (size_t)tn * a.V + v0;  // (M = 1)
+    const uint32_t man_sel = 0x04040000u + (c & 3u) * 0x01010101u;
+    const uint32_t *mrow = reinterpret_cast<const uint32_t *>(man_seg + (c & ~3u));  // + 8 dwords per row
+    const uint32_t nblk = seglen / 8;
+    uint32_t mcur[8], mnext[8];
+    float keep[1] = {0.f};
+#pragma unroll
+    for (int r = 0; r < 8; ++r) mcur[r] = mrow[r * 8];
+    for (uint32_t blk = 0; blk < nblk; ++blk) {
+        // rows of the next block (the last block re-reads its own: stays inside the segment)
+        const uint32_t *nrow = mrow + (size_t)(blk + 1 < nblk ? blk + 1 : blk) * 64;
+#pragma unroll
+        for (int r = 0; r < 8; ++r) mnext[r] = nrow[r * 8];
+        uint32_t w[4];
+        decode8_weights_asm(st, mcur, man_sel, w, 64);
+        trans_emit8_lines<1>(w, xb, 1, a.V, dst, blk, keep, lane);
+#pragma unroll
+        for (int r = 0; r < 8; ++r) mcur[r] = mnext[r];
+    }
+}
+
+// grid: at most one workgroup per CU; workgroup j's wavefront w takes the items w * gridDim + j, + 16 gridDim, ...
+// of the tiles below a.first_tile (item = tile * segs + segment).
+__global__ __launch_bounds__(kTrSegWaves *kWave) void trans32_seg_kernel(TransArgs a) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    const int lane = threadIdx.x % kWave;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWave));
+    if (a.slot_table) {
+        const u32x4 *src = reinterpret_cast<const u32x4 *>(a.slot_table);
+        u32x4 *dst = reinterpret_cast<u32x4 *>(lds);
+        const u32x4 e0 = src[threadIdx.x * 2], e1 = src[threadIdx.x * 2 + 1];
+        dst[threadIdx.x * 2] = e0;
+        dst[threadIdx.x * 2 + 1] = e1;
+    } else {
+        build_slot_table_x8(reinterpret_cast<uint2 *>(lds), a.tables, a.slot_map, threadIdx.x, kTrSegWaves * kWave);
+    }
+    __syncthreads();
+    uint8_t *stage = lds + kSlotTableBytes + (size_t)wave * kTrWinBytes;
+    const uint64_t n_items = (uint64_t)a.first_tile * a.segs;
+    for (uint64_t item = (uint64_t)wave * gridDim.x + blockIdx.x; item < n_items; item += (uint64_t)kTrSegWaves * gridDim.x) {
+        const uint32_t tile = (uint32_t)(item / a.segs), seg = (uint32_t)(item - (uint64_t)tile * a.segs);
+        trans_one_segment(a, tile, seg, stage, lane);
+    }
 }
 
 // Any tile width and the dense layout: one thread per (tile, half): it decodes the tile's columns
@@ -308,7 +424,8 @@ static int transposed_impl(const uint16_t *d_x, uint32_t M, uint32_t H, uint32_t
                            const uint32_t *d_meta1, const uint8_t *d_man_tiled, uint32_t th, uint32_t tw,
                            const uint16_t *d_bias, uint16_t *d_out, uint32_t out_stride, void *d_workspace,
                            size_t workspace_bytes, bool dense, ci_stream_t stream,
-                           const uint16_t *d_plain_w = nullptr) {
+                           const uint16_t *d_plain_w = nullptr, const void *d_checkpoints = nullptr,
+                           uint32_t segments = 1, uint32_t max_window_rows = 0, const void *d_slot_table = nullptr) {
     if (M == 0 || V == 0) return CI_OK;
     if (H == 0) return fail(CI_ERR_ARG, "transposed linear: hidden size is 0");
     if (!d_x || !d_out) return fail(CI_ERR_ARG, "transposed linear: null pointer");
@@ -346,6 +463,11 @@ static int transposed_impl(const uint16_t *d_x, uint32_t M, uint32_t H, uint32_t
     a.tiles_n = ceil_div(H, tw);  // column tiles run along the hidden dimension
     a.tiles_k = ceil_div(V, th);
     a.num_tiles = a.tiles_n * a.tiles_k;
+    a.ckpt = nullptr;
+    a.segs = 1;
+    a.seglen = th / 2;
+    a.slot_table = static_cast<const uint2 *>(d_slot_table);
+    a.first_tile = 0;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bool fast = !dense && tw == 32 && (d_plain_w || (aligned(d_stream, 16) && aligned(d_man_tiled, 4)));
     if (d_plain_w && !fast) return fail(CI_ERR_ARG, "plain-weight transposed linear: only the 32-column tiling");
@@ -355,12 +477,38 @@ static int transposed_impl(const uint16_t *d_x, uint32_t M, uint32_t H, uint32_t
         CI_ALLOW_FULL_LDS(trans32_kernel<1>);
         CI_ALLOW_FULL_LDS(trans32_kernel<kTrRows>);
     }
+    // One row of x on a weight with decoder checkpoints whose largest window is known to fit: the tile rows that
+    // are whole go to the sixteen-wavefront kernel, a short last tile row to the kernel below.
+    if (fast && M == 1 && !d_plain_w && segments > 1 && d_checkpoints && aligned(d_checkpoints, 8) && th % 2 == 0 &&
+        (th / 2) % (32 * segments) == 0 && th / 2 / segments <= 256 && max_window_rows != 0 &&
+        max_window_rows <= kTrWinRows && H % 32 == 0 && aligned(d_x, 2)) {
+        const uint32_t whole_rows = V / th;  // tile rows without a ragged edge
+        if (whole_rows > 0) {
+            a.x = d_x;
+            a.M = 1;
+            a.ckpt = static_cast<const uint2 *>(d_checkpoints);
+            a.segs = segments;
+            a.seglen = th / 2 / segments;
+            a.first_tile = whole_rows * a.tiles_n;
+            const uint64_t items = (uint64_t)a.first_tile * segments;
+            CI_ALLOW_FULL_LDS(trans32_seg_kernel);
+            const dim3 grid((uint32_t)(items < cus ? items : cus)), block(kTrSegWaves * kWave);
+            hipLaunchKernelGGL(trans32_seg_kernel, grid, block, kSlotTableBytes + kTrSegWaves * kTrWinBytes, s, a);
+            CI_LAUNCH_CHECK("trans32_seg_kernel");
+            a.ckpt = nullptr;
+            a.segs = 1;
+            a.seglen = th / 2;
+        }
+    }
     // passes of kTrRows rows of x reuse the workspace one after another on the stream
     for (uint32_t m0 = 0; m0 < M; m0 += kTrRows) {
         a.x = d_x + (size_t)m0 * x_stride;
         a.M = M - m0 < (uint32_t)kTrRows ? M - m0 : (uint32_t)kTrRows;
-        if (fast) {
-            const dim3 grid(a.num_tiles < cus ? a.num_tiles : cus), block(kPersistWaves * kWave);
+        if (fast && a.first_tile >= a.num_tiles) {
+            // (every tile went to the sixteen-wavefront kernel)
+        } else if (fast) {
+            const uint32_t left = a.num_tiles - a.first_tile;
+            const dim3 grid(left < cus ? left : cus), block(kPersistWaves * kWave);
             if (a.M == 1)
                 hipLaunchKernelGGL(trans32_kernel<1>, grid, block, kLdsLimit, s, a);
             else
@@ -404,7 +552,9 @@ extern "C" int ci_fused_linear_transposed_tiled(const ci_tiled_weight *w, const 
     // (the weight is stored [V, H]: its rows are the outputs)
     return transposed_impl(d_x, M, w->N, w->K, x_stride, w->d_stream, w->stream_len, w->d_states, w->d_tables,
                            w->d_slot_map, w->d_tile_offsets, w->d_tile_max_lens, w->d_man_tiled, w->tile_height,
-                           w->tile_width, d_bias, d_out, out_stride, d_workspace, workspace_bytes, false, stream);
+                           w->tile_width, d_bias, d_out, out_stride, d_workspace, workspace_bytes, false, stream, nullptr,
+                           w->segments > 1 ? w->d_checkpoints : nullptr, w->segments > 1 ? w->segments : 1,
+                           w->max_window_rows, w->d_slot_table);
 }
 
 extern "C" int ci_fused_linear_transposed_dense(const uint16_t *d_x, uint32_t M, uint32_t H, uint32_t V,

@@ -155,10 +155,45 @@ class RansLMHead(nn.Module):
         self.tile_k, self.tile_n = emb.tile_k, emb.tile_n
         self.tied_to_embedding = True
 
+    # Derived data kept beside the weight, built on first use: decoder checkpoints (so that one row of x runs on
+    # sixteen wavefronts per CU), the largest window an item reads, the slot table in its LDS form.  `auto`: as many
+    # segments as the library suggests for the shape; an int fixes them; 1 (the default) switches the index off.
+    segments = 1
+
+    def _derived(self, device):
+        import ctypes as C
+
+        from . import _lib
+
+        shape = (self.out_features, self.in_features)
+        segs = suggest_segments(shape, self.tile_k, self.tile_n) if self.segments == "auto" else int(self.segments)
+        ck, segs = _cached_checkpoints(self, device, shape, segs)
+        cached = getattr(self, "_derived_cache", None)
+        key = (self._ckpt_cache[0], segs)
+        if cached is not None and cached[0] == key:
+            return ck, segs, cached[1], cached[2]
+        max_rows, table = 0, None
+        if segs > 1 and self.tile_n == 32:
+            t = [b.to(device) for b in (self.rans_exp_stream, self.rans_exp_states, self.rans_exp_tables, self.rans_exp_slot_map,
+                                        self.rans_exp_tile_offsets, self.rans_exp_tile_max_lens)]
+            t = [_lib.as_u8(t[0], device), _lib.as_u32(t[1], device), _lib.as_u32(t[2], device), _lib.as_u8(t[3], device),
+                 _lib.as_u32(t[4], device), _lib.as_u32(t[5], device)]
+            table = torch.empty(_lib.SLOT_TABLE_BYTES, dtype=torch.uint8, device=device)
+            rows = torch.zeros(1, dtype=torch.int32, device=device)
+            w = _lib.tiled_weight(shape[0], shape[1], self.tile_k, self.tile_n, t[0], t[1], t[2], t[3], t[4], t[5], None, ck, segs)
+            with torch.cuda.device(device):
+                _lib.check(_lib.lib().ci_build_slot_table(_lib.ptr(t[2]), _lib.ptr(t[3]), _lib.ptr(table),
+                                                          C.c_size_t(_lib.SLOT_TABLE_BYTES), _lib.stream_handle(device)))
+                _lib.check(_lib.lib().ci_max_window_rows(C.byref(w), _lib.ptr(rows), _lib.stream_handle(device)))
+            max_rows = int(rows.item())
+        self._derived_cache = (key, max_rows, table)
+        return ck, segs, max_rows, table
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         device = x.device
+        ck, segs, max_rows, table = self._derived(device)
         return fused_rans_linear_transposed(
-            x=x,
+            x=x, checkpoints=ck, segments=segs, max_window_rows=max_rows, slot_table=table,
             compressed_data=self.rans_exp_stream.to(device, non_blocking=True),
             initial_states=self.rans_exp_states.to(device, non_blocking=True),
             tables=self.rans_exp_tables.to(device, non_blocking=True),

@@ -21,7 +21,8 @@ DECODE_ONCE_ABOVE_ROWS = 4
 
 
 def _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, meta0, meta1, tile_k, tile_n,
-         mantissas, bias, out, dense: bool):
+         mantissas, bias, out, dense: bool, checkpoints=None, segments: int = 1, max_window_rows: int = 0,
+         slot_table=None):
     V, H = int(weight_shape[0]), int(weight_shape[1])  # weight is [vocab, hidden]
     _lib.require_device(x)
     _lib.check_tiled_operands(V, H, int(tile_k), int(tile_n), initial_states, tables, slot_map, meta0, meta1, dense)
@@ -62,7 +63,13 @@ def _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, met
             C.c_size_t(ws.numel()), _lib.stream_handle(dev)))
     else:
         # the lengths of every operand travel with it and are checked by the library before the launch
-        w = _lib.tiled_weight(V, H, tile_k, tile_n, stream_t, st, tb, sm, m0, m1, man)
+        ck = None
+        if checkpoints is not None and int(segments) > 1:
+            ck = checkpoints.to(dev).contiguous()
+            if ck.dtype != torch.int64:
+                raise RuntimeError("checkpoints do not belong to this weight shape, tiling and segment count")
+        w = _lib.tiled_weight(V, H, tile_k, tile_n, stream_t, st, tb, sm, m0, m1, man, ck, int(segments) if ck is not None else 1,
+                              slot_table, int(max_window_rows))
         check(lib().ci_fused_linear_transposed_tiled(C.byref(w), ptr(x2), M, x2.stride(0), ptr(b), ptr(result),
                                                      result.stride(0), ptr(ws), C.c_size_t(ws.numel()),
                                                      _lib.stream_handle(dev)))
@@ -73,13 +80,15 @@ def _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, met
 
 def fused_rans_linear_transposed(x, compressed_data, initial_states, tables, slot_map, weight_shape,
                                  tile_offsets, tile_max_lens, tile_k, tile_n, mantissas, workspace=None,
-                                 bias=None, out=None, SPLIT_K=8):
+                                 bias=None, out=None, SPLIT_K=8, checkpoints=None, segments=1, max_window_rows=0,
+                                 slot_table=None):
     """x[..., H] @ W[V, H]^T (+ bias), W in the tiled two-streams-per-column format
     (comp_inference/transposed_linear_triton.py:361-435).  `workspace` and `SPLIT_K` are accepted
     for signature compatibility; the library keeps its own fp32 scratch (one partial per column
     tile, summed in tile order)."""
     return _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, tile_offsets, tile_max_lens,
-                tile_k, tile_n, mantissas, bias, out, dense=False)
+                tile_k, tile_n, mantissas, bias, out, dense=False, checkpoints=checkpoints, segments=segments,
+                max_window_rows=max_window_rows, slot_table=slot_table)
 
 
 def fused_rans_linear_transposed_uncoalesced(x, compressed_data, initial_states, tables, slot_map, weight_shape,

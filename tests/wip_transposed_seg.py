@@ -1,0 +1,50 @@
+"""The sixteen-wavefront LM-head kernel (one row of x, decoder checkpoints, largest window known) against the
+kernel that walks whole tiles: the same products and the same eight-row reduction, so the logits are compared bit
+for bit; and against torch.matmul on the oracle-decoded weight within the operator's tolerance."""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import bf16_bits, bits_to_bf16, make_weight_kn, make_x
+
+pytestmark = pytest.mark.gpu
+ATOL = RTOL = 1e-2
+
+
+def _t32(a):
+    return torch.from_numpy(np.ascontiguousarray(a).view(np.int32))
+
+
+@pytest.mark.parametrize("V,H,segments", [(2304, 128, 2), (4096, 64, 4), (1024, 96, 2), (3000, 64, 2)])
+def test_one_row_of_x_on_sixteen_wavefronts(oracle, V, H, segments):
+    import comp_inference_amd as ci
+    from comp_inference_amd import _lib
+
+    th = 1024
+    w = make_weight_kn(H, V, seed=V + H)           # [V, H]: rows are the outputs
+    enc, man = oracle.compress_bf16(bf16_bits(w), th, 32)
+    wdec = bits_to_bf16(oracle.decompress_bf16(enc, man, V, H))
+    dev = torch.device("cuda", 0)
+    t = [torch.from_numpy(enc.stream).to(dev), _t32(enc.states).to(dev), _t32(enc.tables).to(dev),
+         torch.from_numpy(enc.slot_map).to(dev), _t32(enc.tile_offsets).to(dev), _t32(enc.tile_max_lens).to(dev),
+         torch.from_numpy(man).to(dev)]
+    args = (t[0], t[1], t[2], t[3], (V, H), t[4], t[5], th, 32, t[6])
+    x = make_x(1, H, seed=7).to(dev)
+    whole = ci.fused_rans_linear_transposed(x, *args)
+    ck = ci.build_checkpoints(t[0], t[1], t[2], t[3], (V, H), t[4], t[5], th, 32, segments)
+    rows = torch.zeros(1, dtype=torch.int32, device=dev)
+    desc = _lib.tiled_weight(V, H, th, 32, t[0], t[1], t[2], t[3], t[4], t[5], None, ck, segments)
+    _lib.check(_lib.lib().ci_max_window_rows(C.byref(desc), _lib.ptr(rows), _lib.stream_handle(dev)))
+    max_rows = int(rows.item())
+    assert 0 < max_rows <= 112
+    got = ci.fused_rans_linear_transposed(x, *args, checkpoints=ck, segments=segments, max_window_rows=max_rows)
+    assert torch.equal(got.view(torch.int16), whole.view(torch.int16))
+    want = torch.matmul(x.float().cpu(), wdec.float().t())
+    assert torch.allclose(got.float().cpu(), want, atol=ATOL, rtol=RTOL), (got.float().cpu() - want).abs().max()
+    # more rows of x, or no promise about the windows, take the other kernel: same answer as without checkpoints
+    x3 = make_x(3, H, seed=8).to(dev)
+    assert torch.equal(ci.fused_rans_linear_transposed(x3, *args, checkpoints=ck, segments=segments, max_window_rows=max_rows),
+                       ci.fused_rans_linear_transposed(x3, *args))
+    assert torch.equal(ci.fused_rans_linear_transposed(x, *args, checkpoints=ck, segments=segments), whole)
