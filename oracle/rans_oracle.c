@@ -171,15 +171,18 @@ static uint32_t stream_capacity(uint64_t n_symbols, uint32_t n_streams) {
  * ---------------------------------------------------------------------------------- */
 void ro_free(void *p) { free(p); }
 
-int ro_encode_tiled_ilp2(const uint8_t *sym, uint32_t K, uint32_t N, const uint16_t *freq,
-                         const uint16_t *cdf, uint32_t th, uint32_t tw, uint32_t *states,
-                         uint32_t *sizes, uint32_t *tile_offsets, uint32_t *tile_max_lens,
-                         uint8_t **stream_out, uint64_t *stream_len_out) {
-    if (th == 0 || tw == 0 || th % 16 != 0 || K == 0 || N == 0) return RO_ERR_ARG;
+/* `halves` streams per column and tile: 2 = the default format above, 1 = one stream over the whole tile
+ * height (the reference's first tiled format: kernel src/cuda/rans_kernels.cuh:316-391, packing
+ * src/cuda/rans_ops.cu:522-566, the same interleave with rows of tw bytes). */
+static int encode_tiled(const uint8_t *sym, uint32_t K, uint32_t N, const uint16_t *freq,
+                        const uint16_t *cdf, uint32_t th, uint32_t tw, uint32_t halves, uint32_t *states,
+                        uint32_t *sizes, uint32_t *tile_offsets, uint32_t *tile_max_lens,
+                        uint8_t **stream_out, uint64_t *stream_len_out) {
+    if (th == 0 || tw == 0 || (halves == 2 && th % 16 != 0) || K == 0 || N == 0) return RO_ERR_ARG;
     const uint32_t tiles_k = (K + th - 1) / th, tiles_n = (N + tw - 1) / tw;
-    const uint32_t T = tiles_k * tiles_n, spt = 2 * tw, S = T * spt;
+    const uint32_t T = tiles_k * tiles_n, spt = halves * tw, S = T * spt;
     const uint32_t cap = stream_capacity((uint64_t)K * N, S);
-    const uint32_t half = th / 2;
+    const uint32_t half = th / halves;
     uint8_t **bodies = (uint8_t **)calloc(T, sizeof(uint8_t *));
     if (!bodies) return RO_ERR_NOMEM;
     int status = RO_OK;
@@ -202,7 +205,7 @@ int ro_encode_tiled_ilp2(const uint8_t *sym, uint32_t K, uint32_t N, const uint1
                 ro_bytes out = {tmp + (size_t)q * cap, 0, cap};
                 uint32_t x = RO_RANS_L;
                 if (col < N) {
-                    const int lo = is_b ? (int)half : 0, hi = is_b ? (int)th : (int)half;
+                    const int lo = (int)(is_b * half), hi = lo + (int)half;
                     for (int i = hi - 1; i >= lo; --i) { /* bottom-up */
                         uint32_t row = row0 + (uint32_t)i;
                         if (row >= K) continue;
@@ -259,19 +262,37 @@ int ro_encode_tiled_ilp2(const uint8_t *sym, uint32_t K, uint32_t N, const uint1
     return status;
 }
 
+int ro_encode_tiled_ilp2(const uint8_t *sym, uint32_t K, uint32_t N, const uint16_t *freq,
+                         const uint16_t *cdf, uint32_t th, uint32_t tw, uint32_t *states,
+                         uint32_t *sizes, uint32_t *tile_offsets, uint32_t *tile_max_lens,
+                         uint8_t **stream_out, uint64_t *stream_len_out) {
+    return encode_tiled(sym, K, N, freq, cdf, th, tw, 2, states, sizes, tile_offsets, tile_max_lens, stream_out,
+                        stream_len_out);
+}
+
+/* One stream per column and tile, packed into tile bodies (src/cuda/rans_kernels.cuh:316-391,
+ * src/cuda/rans_ops.cu:412-600): T * tw streams. */
+int ro_encode_tiled_one(const uint8_t *sym, uint32_t K, uint32_t N, const uint16_t *freq,
+                        const uint16_t *cdf, uint32_t th, uint32_t tw, uint32_t *states,
+                        uint32_t *sizes, uint32_t *tile_offsets, uint32_t *tile_max_lens,
+                        uint8_t **stream_out, uint64_t *stream_len_out) {
+    return encode_tiled(sym, K, N, freq, cdf, th, tw, 1, states, sizes, tile_offsets, tile_max_lens, stream_out,
+                        stream_len_out);
+}
+
 /* ------------------------------------------------------------------------------------
  * Decoder for the ILP2 format.  comp_inference/rans_triton.py:34-119.
  * Lanes of columns >= N and rows >= K take no step.  end_states (optional, S entries)
  * and bytes_left (optional) expose the final coder state for the invariant tests.
  * ---------------------------------------------------------------------------------- */
-int ro_decode_tiled_ilp2(const uint8_t *stream, uint64_t stream_len, const uint32_t *states,
-                         const uint32_t *tables, const uint8_t *slot_map,
-                         const uint32_t *tile_offsets, const uint32_t *tile_max_lens, uint32_t K,
-                         uint32_t N, uint32_t th, uint32_t tw, uint8_t *out, uint32_t *end_states,
-                         int32_t *rows_left) {
-    if (th == 0 || tw == 0 || (th & 1u)) return RO_ERR_ARG;
+static int decode_tiled(const uint8_t *stream, uint64_t stream_len, const uint32_t *states,
+                        const uint32_t *tables, const uint8_t *slot_map,
+                        const uint32_t *tile_offsets, const uint32_t *tile_max_lens, uint32_t K,
+                        uint32_t N, uint32_t th, uint32_t tw, uint32_t halves, uint8_t *out, uint32_t *end_states,
+                        int32_t *rows_left) {
+    if (th == 0 || tw == 0 || (halves == 2 && (th & 1u))) return RO_ERR_ARG;
     const uint32_t tiles_k = (K + th - 1) / th, tiles_n = (N + tw - 1) / tw;
-    const uint32_t T = tiles_k * tiles_n, spt = 2 * tw, half = th / 2;
+    const uint32_t T = tiles_k * tiles_n, spt = halves * tw, half = th / halves;
     int status = RO_OK;
 #pragma omp parallel for schedule(dynamic, 4)
     for (uint32_t t = 0; t < T; ++t) {
@@ -297,7 +318,7 @@ int ro_decode_tiled_ilp2(const uint8_t *stream, uint64_t stream_len, const uint3
         for (uint32_t i = 0; i < half; ++i) {
             for (uint32_t q = 0; q < spt; ++q) {
                 const uint32_t lane = q % tw, is_b = q / tw;
-                const uint32_t col = tn * tw + lane, row = row0 + i + (is_b ? half : 0);
+                const uint32_t col = tn * tw + lane, row = row0 + i + is_b * half;
                 if (col >= N || row >= K) continue;
                 uint32_t xs = x[q];
                 const uint32_t slot = xs & RO_PROB_MASK;
@@ -320,6 +341,26 @@ int ro_decode_tiled_ilp2(const uint8_t *stream, uint64_t stream_len, const uint3
         }
     }
     return status;
+}
+
+int ro_decode_tiled_ilp2(const uint8_t *stream, uint64_t stream_len, const uint32_t *states,
+                         const uint32_t *tables, const uint8_t *slot_map,
+                         const uint32_t *tile_offsets, const uint32_t *tile_max_lens, uint32_t K,
+                         uint32_t N, uint32_t th, uint32_t tw, uint8_t *out, uint32_t *end_states,
+                         int32_t *rows_left) {
+    return decode_tiled(stream, stream_len, states, tables, slot_map, tile_offsets, tile_max_lens, K, N, th, tw, 2, out,
+                        end_states, rows_left);
+}
+
+/* Decoder for the one-stream-per-column tiled format: comp_inference/rans_triton.py:399-464 (rows of tw bytes,
+ * one state per lane, the whole tile height in one chain). */
+int ro_decode_tiled_one(const uint8_t *stream, uint64_t stream_len, const uint32_t *states,
+                        const uint32_t *tables, const uint8_t *slot_map,
+                        const uint32_t *tile_offsets, const uint32_t *tile_max_lens, uint32_t K,
+                        uint32_t N, uint32_t th, uint32_t tw, uint8_t *out, uint32_t *end_states,
+                        int32_t *rows_left) {
+    return decode_tiled(stream, stream_len, states, tables, slot_map, tile_offsets, tile_max_lens, K, N, th, tw, 1, out,
+                        end_states, rows_left);
 }
 
 /* ------------------------------------------------------------------------------------

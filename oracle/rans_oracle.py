@@ -188,6 +188,44 @@ def decode_tiled_ilp2(stream, states, tables, slot_map, tile_offsets, tile_max_l
     return (out, end, left) if want_end else out
 
 
+def encode_tiled_one(sym: np.ndarray, freq, cdf, th: int = 1024, tw: int = 32) -> TiledResult:
+    """One stream per column and tile, packed into tile bodies of tw-byte rows (src/cuda/rans_kernels.cuh:316-391,
+    src/cuda/rans_ops.cu:412-600)."""
+    sym = _u8(sym)
+    K, N = sym.shape
+    tk, tn = -(-K // th), -(-N // tw)
+    T, S = tk * tn, tk * tn * tw
+    states = np.empty(S, np.uint32)
+    sizes = np.empty(S, np.uint32)
+    offs = np.empty(T, np.uint32)
+    lens = np.empty(T, np.uint32)
+    sp = C.c_void_p()
+    sl = C.c_uint64()
+    _check(lib().ro_encode_tiled_one(_p(sym), K, N, _p(_u16(freq)), _p(_u16(cdf)), th, tw,
+                                     _p(states), _p(sizes), _p(offs), _p(lens),
+                                     C.byref(sp), C.byref(sl)), "encode_tiled_one")
+    tables, slot_map = build_tables(freq, cdf)
+    return TiledResult(_take_stream(sp, sl.value), states, sizes, tables, slot_map, offs, lens,
+                       S, tk, tn, th, tw)
+
+
+def decode_tiled_one(stream, states, tables, slot_map, tile_offsets, tile_max_lens, K, N,
+                     th=1024, tw=32, want_end=False):
+    """comp_inference/rans_triton.py:399-464."""
+    stream = _u8(stream)
+    out = np.zeros((K, N), np.uint8)
+    S = -(-K // th) * -(-N // tw) * tw
+    states = _u32(states)
+    assert states.size == S
+    end = np.empty(S, np.uint32) if want_end else None
+    left = np.empty(S, np.int32) if want_end else None
+    _check(lib().ro_decode_tiled_one(_p(stream), C.c_uint64(stream.size), _p(states),
+                                     _p(_u32(tables)), _p(_u8(slot_map)), _p(_u32(tile_offsets)),
+                                     _p(_u32(tile_max_lens)), K, N, th, tw, _p(out), _p(end),
+                                     _p(left)), "decode_tiled_one")
+    return (out, end, left) if want_end else out
+
+
 def encode_tiled_dense(sym: np.ndarray, freq, cdf, th: int = 1024, tw: int = 32) -> DenseResult:
     sym = _u8(sym)
     K, N = sym.shape

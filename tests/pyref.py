@@ -22,9 +22,11 @@ def encode_stream(symbols, freq, cdf):
     return x, out
 
 
-def decode_tiled(stream, states, tables, slot_map, tile_offsets, tile_max_lens, K, N, th, tw):
+def decode_tiled(stream, states, tables, slot_map, tile_offsets, tile_max_lens, K, N, th, tw, halves=2):
+    """halves = 2: two streams per column and tile (rows [0, th/2) and [th/2, th)); halves = 1: one stream over
+    the whole tile height (comp_inference/rans_triton.py:399-464)."""
     tiles_k, tiles_n = -(-K // th), -(-N // tw)
-    half, spt = th // 2, 2 * tw
+    half, spt = th // halves, halves * tw
     out = np.zeros((K, N), np.uint8)
     freq = (tables & 0xFFFF).astype(np.int64)
     cdf = (tables >> 16).astype(np.int64)

@@ -192,3 +192,60 @@ def test_tile_height_must_be_multiple_of_16(oracle):
     f, c = _table(oracle, sym)
     with pytest.raises(RuntimeError):
         oracle.encode_tiled_ilp2(sym, f, c, 24, 32)
+
+
+# ---- one stream per column and tile (the reference's first tiled format) ------------------------------------
+@pytest.mark.parametrize("K,N,th,tw", [(80, 24, 32, 8), (700, 70, 256, 32), (1024, 64, 1024, 32), (50, 5, 64, 16)])
+def test_one_stream_layout_round_trips_and_agrees_with_the_second_implementation(oracle, K, N, th, tw):
+    """src/cuda/rans_kernels.cuh:316-391 + src/cuda/rans_ops.cu:522-566 + comp_inference/rans_triton.py:399-464:
+    decode(encode(x)) == x; every stream ends on 2^16 with exactly its own bytes consumed; the numpy decoder
+    written in the shape of the Triton kernel decodes the same bytes; the plain-integer encoder produces the same
+    stream, state and zero-prefixed body column for every stream; offsets are the scan of depth * tw."""
+    sym = zipf_bytes(K * N, 1.1, K + N).reshape(K, N)
+    f, c = _table(oracle, sym)
+    enc = oracle.encode_tiled_one(sym, f, c, th, tw)
+    tiles_k, tiles_n = -(-K // th), -(-N // tw)
+    assert enc.num_streams == tiles_k * tiles_n * tw and enc.states.size == enc.num_streams
+    out, end, left = oracle.decode_tiled_one(enc.stream, enc.states, enc.tables, enc.slot_map, enc.tile_offsets,
+                                             enc.tile_max_lens, K, N, th, tw, want_end=True)
+    assert np.array_equal(out, sym)
+    got = pyref.decode_tiled(enc.stream, enc.states, enc.tables, enc.slot_map, enc.tile_offsets, enc.tile_max_lens,
+                             K, N, th, tw, halves=1)
+    assert np.array_equal(got, sym)
+    lane_col = (np.arange(enc.num_streams) // tw % tiles_n) * tw + np.arange(enc.num_streams) % tw
+    live = lane_col < N
+    assert (end[live] == L).all()
+    pad_rows = np.repeat(enc.tile_max_lens, tw).astype(np.int64) - enc.sizes
+    assert np.array_equal(left.astype(np.int64)[live], pad_rows[live] - 1)     # exactly its own bytes
+    assert (enc.sizes[~live] == 0).all() and (enc.states[~live] == L).all()
+    assert np.array_equal(enc.tile_offsets.astype(np.int64),
+                          np.concatenate(([0], np.cumsum(enc.tile_max_lens.astype(np.int64) * tw)[:-1])))
+    assert enc.stream.size == int((enc.tile_max_lens.astype(np.int64) * tw).sum())
+    for sid in range(0, enc.num_streams, 3):
+        t, q = divmod(sid, tw)
+        tk, tn = divmod(t, tiles_n)
+        col = tn * tw + q
+        if col >= N:
+            continue
+        rows = [r for r in range(tk * th, tk * th + th) if r < K]
+        x, emitted = pyref.encode_stream(sym[rows, col], f, c)
+        assert enc.states[sid] == x and enc.sizes[sid] == len(emitted)
+        depth = int(enc.tile_max_lens[t])
+        body = enc.stream[enc.tile_offsets[t]:][: depth * tw].reshape(-1, tw)
+        pad = depth - len(emitted)
+        assert body[pad:, q].tolist() == emitted and not body[:pad, q].any()
+
+
+def test_one_stream_layout_is_the_two_stream_layout_of_twice_the_columns(oracle):
+    """A plane whose top and bottom half tiles are laid side by side: the one-stream coding of the [th/2, 2N]
+    arrangement has, stream for stream, the states and bytes of the two-stream coding of the [th, N] plane --
+    the two formats differ in how streams are grouped into bodies, not in the coder."""
+    th, tw, N = 64, 8, 16
+    sym = zipf_bytes(th * N, 1.2, 3).reshape(th, N)
+    f, c = _table(oracle, sym)
+    two = oracle.encode_tiled_ilp2(sym, f, c, th, tw)
+    side = np.concatenate([np.concatenate([sym[: th // 2, tn * tw:(tn + 1) * tw], sym[th // 2:, tn * tw:(tn + 1) * tw]], 1)
+                           for tn in range(N // tw)], 1)      # per column tile: [top | bottom]
+    one = oracle.encode_tiled_one(np.ascontiguousarray(side), f, c, th // 2, 2 * tw)
+    assert np.array_equal(one.states, two.states) and np.array_equal(one.sizes, two.sizes)
+    assert np.array_equal(one.stream, two.stream) and np.array_equal(one.tile_max_lens, two.tile_max_lens)
