@@ -637,14 +637,6 @@ struct SegJobs {
 };
 
 // grid: any number of workgroups (one per CU); workgroup j takes jobs j, j + gridDim.x, ...
-#ifdef CI_PROBE
-__device__ uint64_t g_probe[64 * 64];
-#define PROBEW(k) do { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory"); PROBE(k); } while (0)
-#define PROBE(k) do { if (blockIdx.x == 0 && lane == 0 && pcount < 60) g_probe[wave * 64 + pcount++] = ((uint64_t)(k) << 56) | (wall_clock64() & 0xffffffffffffffull); } while (0)
-#else
-#define PROBE(k) do { } while (0)
-#define PROBEW(k) do { } while (0)
-#endif
 // kCold = false: the instance for weights whose every item is known to take the hand-scheduled loop (full
 // tiles, windows of at most kWinRows rows: LinearArgs::all_fast).  It holds no code for the guarded path,
 // whose registers would otherwise be spilled around every item; an item that does not qualify after all
@@ -656,10 +648,6 @@ __global__ __launch_bounds__(kSegWaves *kWave) void fused_linear32_seg_kernel(Li
     // (the wavefront's index through readfirstlane: everything derived from it -- jobs, items, tiles -- is then
     // uniform for the compiler too and lives in scalar registers)
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWave)), lane = threadIdx.x % kWave;
-#ifdef CI_PROBE
-    int pcount = 0;
-#endif
-    PROBE(1);
     // the slot table is asked for before anything else: the job arithmetic below runs while it travels
     const bool copy_table = (!kCold || a.dense_w == nullptr) && a.slot_table;
     u32x4 tab0 = {0, 0, 0, 0}, tab1 = {0, 0, 0, 0};
@@ -689,7 +677,6 @@ __global__ __launch_bounds__(kSegWaves *kWave) void fused_linear32_seg_kernel(Li
     uint32_t vk_n = 0, tn_n = 0, vk_nn = 0, tn_nn = 0;
     uint32_t s_nxt = next_slot(0, vk_n, tn_n), s_nn = slots;  // the next slot with an item, and the one after
     if (coded && s_nxt < slots) seg_request(a, vk_n, tn_n, lane, raw);
-    PROBE(20);
     if (copy_table) {
         u32x4 *dst = reinterpret_cast<u32x4 *>(lds);
         dst[threadIdx.x * 2] = tab0;
@@ -697,10 +684,8 @@ __global__ __launch_bounds__(kSegWaves *kWave) void fused_linear32_seg_kernel(Li
     } else if (coded) {
         build_slot_table_x8(reinterpret_cast<uint2 *>(lds), a.tables, a.slot_map, threadIdx.x, kSegWaves * kWave);
     }
-    PROBE(21);
     if (coded && s_nxt < slots) {
         seg_resolve(a, vk_n, tn_n, lane, raw, nxt);
-        PROBE(22);
         s_nn = next_slot(s_nxt + 1, vk_nn, tn_nn);
         if (s_nn < slots) seg_request(a, vk_nn, tn_nn, lane, raw);
     }
@@ -708,9 +693,7 @@ __global__ __launch_bounds__(kSegWaves *kWave) void fused_linear32_seg_kernel(Li
         uint32_t *flags = reinterpret_cast<uint32_t *>(lds + kSmallFlagsOff);
         flags[0] = flags[1] = 0;
     }
-    PROBE(23);
     __syncthreads();
-    PROBE(2);
 
     const uint32_t hsel = lane / 32, c = lane % 32;
     f32x16 acc, acc2;
@@ -719,19 +702,15 @@ __global__ __launch_bounds__(kSegWaves *kWave) void fused_linear32_seg_kernel(Li
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[v] = acc2[v] = 0.f;
         }
-        PROBE(10);
         const uint32_t job = blockIdx.x + (sl / jb.R) * gridDim.x;
         uint32_t vk, tn;
         if (slot_item(sl, vk, tn)) {
-            PROBE(11);
             if (kCold && !coded) {
                 seg_cold_item<MB>(a, vk, tn, tab, stage, lane, acc, acc2);
             } else {
                 // (sl == s_nxt: the slots with an item are visited in order)
                 const SegItem cur = nxt;
-                PROBE(3);
                 if (cur.fast) seg_stage(a, cur, stage, lane);
-                PROBEW(4);
                 uint32_t touched = 0, touched2 = 0;  // (kept apart: adding them would wait for both loads)
                 s_nxt = s_nn;
                 vk_n = vk_nn;
@@ -742,14 +721,11 @@ __global__ __launch_bounds__(kSegWaves *kWave) void fused_linear32_seg_kernel(Li
                     s_nn = next_slot(s_nxt + 1, vk_nn, tn_nn);
                     if (s_nn < slots) seg_request(a, vk_nn, tn_nn, lane, raw);
                 }
-                PROBE(cur.fast ? 5 : 9);
-                PROBEW(12);
                 if (cur.fast)
                     seg_run<MB>(a, cur, stage, lane, acc, acc2);  // (a wavefront's LDS operations complete in order)
                 else if (kCold)
                     seg_cold_item<MB>(a, vk, tn, tab, stage, lane, acc, acc2);
                 asm volatile("" ::"v"(touched), "v"(touched2));  // the touching loads end here
-                PROBE(6);
             }
         }
         if (sl % jb.R != jb.R - 1) continue;
@@ -797,7 +773,6 @@ __global__ __launch_bounds__(kSegWaves *kWave) void fused_linear32_seg_kernel(Li
                     __hip_atomic_store(&flags[1], jn + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
                 }
             }
-            PROBE(7);
             continue;
         }
         float *red = reinterpret_cast<float *>(lds + kSlotTableBytes);
@@ -823,12 +798,8 @@ __global__ __launch_bounds__(kSegWaves *kWave) void fused_linear32_seg_kernel(Li
             }
         }
         __syncthreads();  // before the next window is written over the fragments
-        PROBE(7);
     }
 }
-#ifdef CI_PROBE
-extern "C" int ci_debug_probe(uint64_t *h_out) { return hipMemcpyFromSymbol(h_out, HIP_SYMBOL(g_probe), sizeof(uint64_t) * 64 * 64) == hipSuccess ? 0 : 2; }
-#endif
 
 // Any tile width, either tiled layout: one thread per stream, eight rows of x per pass.
 // Partial sums (one per stream, i.e. per (k-tile[, half])) go to the fp32 workspace.
