@@ -18,6 +18,7 @@ from .comp_inference import (
 )
 from .embedding_hip import (
     fused_rans_embedding,
+    fused_rans_embedding_one_stream,
     fused_rans_embedding_triton,
     fused_rans_embedding_triton_uncoalesced,
     fused_rans_embedding_uncoalesced,
@@ -25,6 +26,7 @@ from .embedding_hip import (
 from .linear_hip import (
     dense_matmul,
     fused_rans_linear,
+    fused_rans_linear_one_stream,
     fused_rans_linear_triton,
     fused_rans_linear_triton_uncoalesced,
     fused_rans_linear_uncoalesced,
@@ -38,6 +40,7 @@ from .rans_hip import (
     rans_decomp_flat,
     rans_decomp_tiled,
     rans_decomp_tiled_batch,
+    rans_decomp_tiled_one_stream,
     rans_decomp_tiled_uncoalesced,
     rans_decomp_triton,
     rans_decomp_triton_tiled,
@@ -45,6 +48,7 @@ from .rans_hip import (
 )
 from .transposed_linear_hip import (
     fused_rans_linear_transposed,
+    fused_rans_linear_transposed_one_stream,
     fused_rans_linear_transposed_triton,
     fused_rans_linear_transposed_triton_uncoalesced,
     fused_rans_linear_transposed_uncoalesced,

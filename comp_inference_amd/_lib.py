@@ -122,12 +122,14 @@ def as_u8(t: torch.Tensor, device) -> torch.Tensor:
 
 
 def check_tiled_operands(rows: int, cols: int, tile_k: int, tile_n: int, initial_states, tables, slot_map, meta0, meta1,
-                         dense: bool) -> None:
+                         dense: bool, one: bool = False) -> None:
     """The kernels index these arrays by tile and stream without a bound of their own: a short one would be
     read past its end.  Same condition and exception as the reference's decoder
-    (comp_inference/rans_triton.py:141-144), applied to every operand and every op."""
+    (comp_inference/rans_triton.py:141-144, :482-487), applied to every operand and every op.
+    `dense`: one stream per column with per-stream offsets and sizes; `one`: one stream per column in
+    tile bodies (per-tile offsets and depths); neither: two streams per column in tile bodies."""
     tiles = (-(-rows // tile_k)) * (-(-cols // tile_n))
-    streams = tiles * tile_n * (1 if dense else 2)
+    streams = tiles * tile_n * (1 if dense or one else 2)
     if initial_states.numel() != streams:
         raise ValueError(f"Initial states size mismatch. Expected {streams}")
     per_meta = streams if dense else tiles

@@ -86,6 +86,18 @@ class RansManager:
     # -- tiled, two streams per column: the default format --------------------------------
     def compress_tiled(self, data, freqs, cdf, tile_height: int, tile_width: int):
         """src/python_bindings.cpp:302-347 -> RansManager::compress_tiled_ilp2."""
+        return self._compress_bodies(data, freqs, cdf, tile_height, tile_width, two=True)
+
+    # -- tiled, one stream per column, tile bodies of tile_width bytes a row -----------------
+    def compress_tiled_one_stream(self, data, freqs, cdf, tile_height: int, tile_width: int):
+        """RansManager::compress_tiled of the C++ class (src/cuda/rans_ops.cu:412-600, kernel
+        src/cuda/rans_kernels.cuh:316-391), which the reference's Python module does not bind
+        (its `compress_tiled` is the two-stream encoder above).  Same result class; `states` and
+        `output_sizes` hold tile_width entries per tile.  Read by `rans_decomp_triton_tiled2` /
+        `_tiled_splitk`, `fused_rans_linear_triton_splitk` and `fused_rans_embedding_triton_2`."""
+        return self._compress_bodies(data, freqs, cdf, tile_height, tile_width, two=False)
+
+    def _compress_bodies(self, data, freqs, cdf, tile_height: int, tile_width: int, two: bool):
         dev = _dev()
         K, N = _shape2d(data)
         if data.numel() != K * N:
@@ -93,7 +105,7 @@ class RansManager:
         sym = _lib.as_u8(data, dev).reshape(K, N)
         f, c = _np_u16(freqs), _np_u16(cdf)
         t = Tiling()
-        check(lib().ci_tiling_init(C.byref(t), K, N, int(tile_height), int(tile_width), 1))
+        check(lib().ci_tiling_init(C.byref(t), K, N, int(tile_height), int(tile_width), 1 if two else 0))
         s = _lib.stream_handle(dev)
         nb = lib().ci_encode_scratch_bytes(t.num_streams, t.capacity)
         scratch = torch.empty(nb, dtype=torch.uint8, device=dev)
@@ -102,13 +114,14 @@ class RansManager:
         offs = torch.empty(t.num_tiles, dtype=torch.int32, device=dev)
         lens = torch.empty(t.num_tiles, dtype=torch.int32, device=dev)
         total = C.c_uint64(0)
-        check(lib().ci_encode_tiled_ilp2(ptr(sym), C.byref(t), f.ctypes.data_as(C.c_void_p),
-                                         c.ctypes.data_as(C.c_void_p), ptr(scratch), C.c_size_t(nb),
-                                         ptr(states), ptr(sizes), ptr(offs), ptr(lens),
-                                         C.byref(total), s))
+        encode = lib().ci_encode_tiled_ilp2 if two else lib().ci_encode_tiled_one
+        pack = lib().ci_pack_tiled_ilp2 if two else lib().ci_pack_tiled_one
+        check(encode(ptr(sym), C.byref(t), f.ctypes.data_as(C.c_void_p), c.ctypes.data_as(C.c_void_p),
+                     ptr(scratch), C.c_size_t(nb), ptr(states), ptr(sizes), ptr(offs), ptr(lens),
+                     C.byref(total), s))
         stream = torch.empty(total.value, dtype=torch.uint8, device=dev)
-        check(lib().ci_pack_tiled_ilp2(ptr(scratch), C.byref(t), ptr(sizes), ptr(offs), ptr(lens),
-                                       ptr(stream), C.c_uint64(total.value), s))
+        check(pack(ptr(scratch), C.byref(t), ptr(sizes), ptr(offs), ptr(lens), ptr(stream),
+                   C.c_uint64(total.value), s))
         tables, slot_map = _host_tables(f, c)
         return TiledTensorCompressResult(
             success=True, stream=stream.cpu(), states=states.cpu().view(torch.uint32),

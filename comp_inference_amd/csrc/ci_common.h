@@ -38,6 +38,12 @@ inline int hip_fail(hipError_t e, const char *what) {
         if (e_ != hipSuccess) return ci::hip_fail(e_, name);   \
     } while (0)
 
+// How the streams of a tile lie in the byte stream, for the kernels that take every layout.
+//   kBodyTwo   two streams per column (rows [0, th/2) and [th/2, th)), tile body of 2 tw bytes a row (default)
+//   kExactBytes one stream per column over the tile's height, each stream's bytes on their own at stream_offsets
+//   kBodyOne   one stream per column over the tile's height, tile body of tw bytes a row
+enum TileLayout { kBodyTwo = 0, kExactBytes = 1, kBodyOne = 2 };
+
 inline uint32_t ceil_div(uint32_t a, uint32_t b) { return (a + b - 1) / b; }
 
 inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }

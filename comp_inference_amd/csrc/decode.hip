@@ -456,18 +456,19 @@ __global__ __launch_bounds__(kDecSegWaves *kWave) void decode_tiled32_seg_kernel
 
 
 // Any tile width: one thread per stream, bytes read where they lie.  Used for widths other
-// than 32 (the reference's tests sweep 16..128, tests/test_mat_mul.py:263-264).
-template <bool kMerge>
+// than 32 (the reference's tests sweep 16..128, tests/test_mat_mul.py:263-264) and, with kHalves = 1, for
+// the layout of one stream per column and tile (comp_inference/rans_triton.py:399-464).
+template <bool kMerge, uint32_t kHalves>
 __global__ __launch_bounds__(256) void decode_tiled_generic_kernel(DecodeArgs a) {
     __shared__ uint2 tab[kProbScale];
     build_slot_table(tab, a.tables, a.slot_map, threadIdx.x, 256);
     __syncthreads();
-    const uint32_t spt = 2 * a.tw;
+    const uint32_t spt = kHalves * a.tw;
     const uint64_t sid = (uint64_t)blockIdx.x * 256 + threadIdx.x;
     if (sid >= (uint64_t)a.num_tiles * spt) return;
     const uint32_t tile = (uint32_t)(sid / spt), q = (uint32_t)(sid % spt);
     const uint32_t tk = tile / a.tiles_n, tn = tile % a.tiles_n;
-    const uint32_t half = a.th / 2, hsel = q / a.tw, c = q % a.tw;
+    const uint32_t half = a.th / kHalves, hsel = q / a.tw, c = q % a.tw;
     const uint32_t col = tn * a.tw + c, my_row0 = tk * a.th + hsel * half;
     if (col >= a.N || my_row0 >= a.K) return;
     const uint32_t my_steps = min(half, a.K - my_row0);
@@ -785,11 +786,56 @@ extern "C" int ci_decode_tiled_ilp2_segmented(const uint8_t *d_stream, uint64_t 
         const uint64_t streams = (uint64_t)a.num_tiles * 2 * tile_width;
         const dim3 grid((uint32_t)((streams + 255) / 256)), block(256);
         if (merge)
-            hipLaunchKernelGGL(decode_tiled_generic_kernel<true>, grid, block, 0, s, a);
+            hipLaunchKernelGGL((decode_tiled_generic_kernel<true, 2>), grid, block, 0, s, a);
         else
-            hipLaunchKernelGGL(decode_tiled_generic_kernel<false>, grid, block, 0, s, a);
+            hipLaunchKernelGGL((decode_tiled_generic_kernel<false, 2>), grid, block, 0, s, a);
         CI_LAUNCH_CHECK("decode_tiled_generic_kernel");
     }
+    return CI_OK;
+}
+
+extern "C" int ci_decode_tiled_one(const uint8_t *d_stream, uint64_t stream_len, const uint32_t *d_states,
+                                   const uint32_t *d_tables, const uint8_t *d_slot_map,
+                                   const uint32_t *d_tile_offsets, const uint32_t *d_tile_max_lens, uint32_t K,
+                                   uint32_t N, uint32_t tile_height, uint32_t tile_width, uint8_t *d_out_exp,
+                                   const uint8_t *d_man_tiled, uint16_t *d_out_bf16, ci_stream_t stream) {
+    if (K == 0 || N == 0) return CI_OK;
+    if (!d_states || !d_tables || !d_slot_map || !d_tile_offsets || !d_tile_max_lens)
+        return fail(CI_ERR_ARG, "ci_decode_tiled_one: null table or metadata pointer");
+    if (stream_len && !d_stream) return fail(CI_ERR_ARG, "ci_decode_tiled_one: null stream");
+    if (tile_height == 0 || tile_width == 0) return fail(CI_ERR_ARG, "ci_decode_tiled_one: empty tile");
+    const bool merge = d_man_tiled != nullptr;
+    if (merge ? !d_out_bf16 : !d_out_exp) return fail(CI_ERR_ARG, "ci_decode_tiled_one: null output");
+    if (!aligned(d_slot_map, 4)) return fail(CI_ERR_ARG, "ci_decode_tiled_one: slot_map must be 4-byte aligned");
+    DecodeArgs a;
+    a.stream = d_stream;
+    a.stream_len = stream_len;
+    a.states = d_states;
+    a.tables = d_tables;
+    a.slot_map = d_slot_map;
+    a.tile_offsets = d_tile_offsets;
+    a.tile_max_lens = d_tile_max_lens;
+    a.K = K;
+    a.N = N;
+    a.th = tile_height;
+    a.tw = tile_width;
+    a.tiles_n = ceil_div(N, tile_width);
+    a.num_tiles = ceil_div(K, tile_height) * a.tiles_n;
+    a.out_exp = d_out_exp;
+    a.man_tiled = d_man_tiled;
+    a.out_bf16 = d_out_bf16;
+    a.man_aligned = 0;
+    a.ckpt = nullptr;
+    a.segs = 1;
+    a.seglen = tile_height;
+    const uint64_t streams = (uint64_t)a.num_tiles * tile_width;
+    const dim3 grid((uint32_t)((streams + 255) / 256)), block(256);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (merge)
+        hipLaunchKernelGGL((decode_tiled_generic_kernel<true, 1>), grid, block, 0, s, a);
+    else
+        hipLaunchKernelGGL((decode_tiled_generic_kernel<false, 1>), grid, block, 0, s, a);
+    CI_LAUNCH_CHECK("decode_tiled_generic_kernel");
     return CI_OK;
 }
 

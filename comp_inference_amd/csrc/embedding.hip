@@ -558,9 +558,9 @@ __global__ __launch_bounds__(kPersistWaves *kWave) void embed_gather32_kernel(Em
         embed_wave_items<10, kDepthMedium>(a, tab, lds, wave, lane);
 }
 
-// Any tile width and the dense layout: one thread per (token, column), discarding the rows above
-// the requested one exactly as the reference does (comp_inference/embedding_triton.py:239-257).
-template <bool kDense>
+// Any tile width, any tiled layout (TileLayout): one thread per (token, column), discarding the rows above
+// the requested one exactly as the reference does (comp_inference/embedding_triton.py:239-257; one stream per column: :124-144).
+template <int kLayout>
 __global__ __launch_bounds__(256) void embed_generic_kernel(EmbedArgs a) {
     __shared__ uint2 tab[kProbScale];
     build_slot_table(tab, a.tables, a.slot_map, threadIdx.x, 256);
@@ -575,7 +575,8 @@ __global__ __launch_bounds__(256) void embed_generic_kernel(EmbedArgs a) {
     }
     const uint32_t tok = (uint32_t)id, tk = tok / a.th, rel = tok % a.th;
     const uint32_t tn = col / a.tw, c = col % a.tw, tile = tk * a.tiles_n + tn;
-    const uint32_t span = kDense ? a.th : a.th / 2, hsel = kDense ? 0 : rel / span, target = rel % span;
+    constexpr bool kOne = kLayout != kBodyTwo;  // one stream per column over the whole tile height
+    const uint32_t span = kOne ? a.th : a.th / 2, hsel = kOne ? 0 : rel / span, target = rel % span;
     uint32_t x, sym = 0;
     auto run = [&](auto &src) {
         for (uint32_t i = 0; i <= target; ++i) {
@@ -584,7 +585,7 @@ __global__ __launch_bounds__(256) void embed_generic_kernel(EmbedArgs a) {
             src.renorm(x);
         }
     };
-    if (kDense) {
+    if (kLayout == kExactBytes) {
         const uint32_t sid = tile * a.tw + c;
         x = a.states[sid];
         const uint64_t off = a.stream_offsets[sid];
@@ -594,7 +595,7 @@ __global__ __launch_bounds__(256) void embed_generic_kernel(EmbedArgs a) {
         src.init(a.stream + off, size);
         run(src);
     } else {
-        const uint32_t spt = 2 * a.tw, q = hsel * a.tw + c;
+        const uint32_t spt = (kOne ? 1 : 2) * a.tw, q = hsel * a.tw + c;
         x = a.states[(size_t)tile * spt + q];
         uint64_t base = a.tile_offsets[tile];
         uint32_t depth = a.tile_max_lens[tile];
@@ -635,8 +636,10 @@ static int embedding_impl(const int64_t *d_ids, uint32_t n_ids, const uint8_t *d
                           const uint32_t *d_states, const uint32_t *d_tables, const uint8_t *d_slot_map,
                           const uint32_t *d_meta0, const uint32_t *d_meta1, const uint8_t *d_man_tiled, uint32_t K,
                           uint32_t N, uint32_t th, uint32_t tw, uint16_t *d_out, uint32_t out_stride,
-                          void *d_workspace, size_t workspace_bytes, bool dense, hipStream_t s,
+                          void *d_workspace, size_t workspace_bytes, int layout, hipStream_t s,
                           const void *d_checkpoints = nullptr, uint32_t segments = 1) {
+    const bool dense = layout != kBodyTwo;     // one stream per column: the one-thread-per-column kernel
+    const bool exact = layout == kExactBytes;  // d_meta0 / d_meta1 are stream_offsets / stream_sizes
     if (n_ids == 0 || N == 0) return CI_OK;
     if (segments == 0) segments = 1;
     if (segments > 1) {
@@ -658,10 +661,10 @@ static int embedding_impl(const int64_t *d_ids, uint32_t n_ids, const uint8_t *d
     a.states = d_states;
     a.tables = d_tables;
     a.slot_map = d_slot_map;
-    a.tile_offsets = dense ? nullptr : d_meta0;
-    a.tile_max_lens = dense ? nullptr : d_meta1;
-    a.stream_offsets = dense ? d_meta0 : nullptr;
-    a.stream_sizes = dense ? d_meta1 : nullptr;
+    a.tile_offsets = exact ? nullptr : d_meta0;
+    a.tile_max_lens = exact ? nullptr : d_meta1;
+    a.stream_offsets = exact ? d_meta0 : nullptr;
+    a.stream_sizes = exact ? d_meta1 : nullptr;
     a.man_tiled = d_man_tiled;
     a.K = K;
     a.N = N;
@@ -680,10 +683,12 @@ static int embedding_impl(const int64_t *d_ids, uint32_t n_ids, const uint8_t *d
         a.out = d_out;
         a.n_buckets = 0;
         const dim3 grid(n_ids, ceil_div(N, 256)), block(256);
-        if (dense)
-            hipLaunchKernelGGL(embed_generic_kernel<true>, grid, block, 0, s, a);
+        if (layout == kExactBytes)
+            hipLaunchKernelGGL(embed_generic_kernel<kExactBytes>, grid, block, 0, s, a);
+        else if (layout == kBodyOne)
+            hipLaunchKernelGGL(embed_generic_kernel<kBodyOne>, grid, block, 0, s, a);
         else
-            hipLaunchKernelGGL(embed_generic_kernel<false>, grid, block, 0, s, a);
+            hipLaunchKernelGGL(embed_generic_kernel<kBodyTwo>, grid, block, 0, s, a);
         CI_LAUNCH_CHECK("embed_generic_kernel");
         return CI_OK;
     }
@@ -779,6 +784,17 @@ extern "C" int ci_fused_embedding_tiled(const ci_tiled_weight *w, const int64_t 
                           w->d_tile_offsets, w->d_tile_max_lens, w->d_man_tiled, w->K, w->N, w->tile_height,
                           w->tile_width, d_out, out_stride, d_workspace, workspace_bytes, false,
                           static_cast<hipStream_t>(stream), segments > 1 ? w->d_checkpoints : nullptr, segments);
+}
+
+extern "C" int ci_fused_embedding_one(const int64_t *d_ids, uint32_t n_ids, const uint8_t *d_stream,
+                                      uint64_t stream_len, const uint32_t *d_states, const uint32_t *d_tables,
+                                      const uint8_t *d_slot_map, const uint32_t *d_tile_offsets,
+                                      const uint32_t *d_tile_max_lens, const uint8_t *d_man_tiled, uint32_t K,
+                                      uint32_t N, uint32_t tile_height, uint32_t tile_width, uint16_t *d_out,
+                                      uint32_t out_stride, ci_stream_t stream) {
+    return embedding_impl(d_ids, n_ids, d_stream, stream_len, d_states, d_tables, d_slot_map, d_tile_offsets,
+                          d_tile_max_lens, d_man_tiled, K, N, tile_height, tile_width, d_out, out_stride, nullptr,
+                          0, kBodyOne, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int ci_fused_embedding_dense(const int64_t *d_ids, uint32_t n_ids, const uint8_t *d_stream,

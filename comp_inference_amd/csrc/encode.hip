@@ -3,9 +3,10 @@
 // to a per-stream slice of a scratch buffer; the packing that the reference does in a
 // single-threaded host loop runs here as small follow-up kernels on the same HIP stream.
 //
-// Three stream layouts share the one encode kernel:
+// Three stream shapes share the one encode kernel:
 //   kIlp2  two streams per (tile, column): rows [0,th/2) and [th/2,th)   (default format)
-//   kDense one stream per (tile, column) over the full tile height       ("uncoalesced")
+//   kDense one stream per (tile, column) over the full tile height       ("uncoalesced", and the first
+//          tiled format, which packs these streams into tile bodies like the default one)
 //   kFlat  stream gid = (512-row segment gid / N, column gid % N)         (legacy)
 #include "ci_common.h"
 #include "rans_device.h"
@@ -275,18 +276,18 @@ extern "C" size_t ci_encode_scratch_bytes(uint32_t num_streams, uint32_t capacit
     return scratch_needed(num_streams, capacity);
 }
 
-extern "C" int ci_encode_tiled_ilp2(const uint8_t *d_symbols, const ci_tiling *t,
-                                    const uint16_t *h_freqs, const uint16_t *h_cdf, uint8_t *d_scratch,
-                                    size_t scratch_bytes, uint32_t *d_states, uint32_t *d_sizes,
-                                    uint32_t *d_tile_offsets, uint32_t *d_tile_max_lens,
-                                    uint64_t *h_stream_len, ci_stream_t stream) {
-    if (!t || !d_tile_offsets || !d_tile_max_lens || !h_stream_len)
-        return fail(CI_ERR_ARG, "ci_encode_tiled_ilp2: null pointer");
-    if (t->streams_per_tile != 2 * t->tile_width)
-        return fail(CI_ERR_ARG, "ci_encode_tiled_ilp2: tiling was not initialised for two streams per column");
-    hipStream_t s = static_cast<hipStream_t>(stream);
+// Encode, then the tile metadata of the two body layouts: depth of every tile and the scan of depth * spt.
+static int encode_tiled_bodies(const char *who, int layout, const uint8_t *d_symbols, const ci_tiling *t,
+                               const uint16_t *h_freqs, const uint16_t *h_cdf, uint8_t *d_scratch,
+                               size_t scratch_bytes, uint32_t *d_states, uint32_t *d_sizes,
+                               uint32_t *d_tile_offsets, uint32_t *d_tile_max_lens, uint64_t *h_stream_len,
+                               hipStream_t s) {
+    if (!t || !d_tile_offsets || !d_tile_max_lens || !h_stream_len) return fail(CI_ERR_ARG, "%s: null pointer", who);
+    if (t->streams_per_tile != (layout == kIlp2 ? 2u : 1u) * t->tile_width)
+        return fail(CI_ERR_ARG, "%s: tiling was not initialised for %s per column", who,
+                    layout == kIlp2 ? "two streams" : "one stream");
     int rc = run_encode(d_symbols, t->K, t->N, t->tile_height, t->tile_width, t->num_tiles_n,
-                        t->num_streams, t->capacity, kIlp2, h_freqs, h_cdf, d_scratch, scratch_bytes,
+                        t->num_streams, t->capacity, layout, h_freqs, h_cdf, d_scratch, scratch_bytes,
                         d_states, d_sizes, nullptr, s);
     if (rc) return rc;
     uint32_t *header = reinterpret_cast<uint32_t *>(d_scratch);
@@ -303,19 +304,56 @@ extern "C" int ci_encode_tiled_ilp2(const uint8_t *d_symbols, const ci_tiling *t
     return CI_OK;
 }
 
-extern "C" int ci_pack_tiled_ilp2(const uint8_t *d_scratch, const ci_tiling *t, const uint32_t *d_sizes,
-                                  const uint32_t *d_tile_offsets, const uint32_t *d_tile_max_lens,
-                                  uint8_t *d_stream, uint64_t stream_len, ci_stream_t stream) {
-    if (!d_scratch || !t || !d_sizes || !d_tile_offsets || !d_tile_max_lens)
-        return fail(CI_ERR_ARG, "ci_pack_tiled_ilp2: null pointer");
+static int pack_tiled_bodies(const char *who, const uint8_t *d_scratch, const ci_tiling *t, const uint32_t *d_sizes,
+                             const uint32_t *d_tile_offsets, const uint32_t *d_tile_max_lens, uint8_t *d_stream,
+                             uint64_t stream_len, hipStream_t s) {
+    if (!d_scratch || !t || !d_sizes || !d_tile_offsets || !d_tile_max_lens) return fail(CI_ERR_ARG, "%s: null pointer", who);
     if (stream_len == 0) return CI_OK;
-    if (!d_stream) return fail(CI_ERR_ARG, "ci_pack_tiled_ilp2: null stream buffer");
-    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (!d_stream) return fail(CI_ERR_ARG, "%s: null stream buffer", who);
     hipLaunchKernelGGL(pack_tiled_kernel, dim3(t->num_tiles), dim3(256), 0, s,
                        d_scratch + kHeaderBytes + 1024, d_sizes, d_tile_offsets, d_tile_max_lens,
                        t->streams_per_tile, t->capacity, d_stream, stream_len);
     CI_LAUNCH_CHECK("pack_tiled_kernel");
     return CI_OK;
+}
+
+extern "C" int ci_encode_tiled_ilp2(const uint8_t *d_symbols, const ci_tiling *t,
+                                    const uint16_t *h_freqs, const uint16_t *h_cdf, uint8_t *d_scratch,
+                                    size_t scratch_bytes, uint32_t *d_states, uint32_t *d_sizes,
+                                    uint32_t *d_tile_offsets, uint32_t *d_tile_max_lens,
+                                    uint64_t *h_stream_len, ci_stream_t stream) {
+    return encode_tiled_bodies("ci_encode_tiled_ilp2", kIlp2, d_symbols, t, h_freqs, h_cdf, d_scratch, scratch_bytes,
+                               d_states, d_sizes, d_tile_offsets, d_tile_max_lens, h_stream_len,
+                               static_cast<hipStream_t>(stream));
+}
+
+extern "C" int ci_pack_tiled_ilp2(const uint8_t *d_scratch, const ci_tiling *t, const uint32_t *d_sizes,
+                                  const uint32_t *d_tile_offsets, const uint32_t *d_tile_max_lens,
+                                  uint8_t *d_stream, uint64_t stream_len, ci_stream_t stream) {
+    if (t && t->streams_per_tile != 2 * t->tile_width)
+        return fail(CI_ERR_ARG, "ci_pack_tiled_ilp2: tiling was not initialised for two streams per column");
+    return pack_tiled_bodies("ci_pack_tiled_ilp2", d_scratch, t, d_sizes, d_tile_offsets, d_tile_max_lens, d_stream,
+                             stream_len, static_cast<hipStream_t>(stream));
+}
+
+// src/cuda/rans_kernels.cuh:316-391 + src/cuda/rans_ops.cu:412-600
+extern "C" int ci_encode_tiled_one(const uint8_t *d_symbols, const ci_tiling *t,
+                                   const uint16_t *h_freqs, const uint16_t *h_cdf, uint8_t *d_scratch,
+                                   size_t scratch_bytes, uint32_t *d_states, uint32_t *d_sizes,
+                                   uint32_t *d_tile_offsets, uint32_t *d_tile_max_lens,
+                                   uint64_t *h_stream_len, ci_stream_t stream) {
+    return encode_tiled_bodies("ci_encode_tiled_one", kDense, d_symbols, t, h_freqs, h_cdf, d_scratch, scratch_bytes,
+                               d_states, d_sizes, d_tile_offsets, d_tile_max_lens, h_stream_len,
+                               static_cast<hipStream_t>(stream));
+}
+
+extern "C" int ci_pack_tiled_one(const uint8_t *d_scratch, const ci_tiling *t, const uint32_t *d_sizes,
+                                 const uint32_t *d_tile_offsets, const uint32_t *d_tile_max_lens,
+                                 uint8_t *d_stream, uint64_t stream_len, ci_stream_t stream) {
+    if (t && t->streams_per_tile != t->tile_width)
+        return fail(CI_ERR_ARG, "ci_pack_tiled_one: tiling was not initialised for one stream per column");
+    return pack_tiled_bodies("ci_pack_tiled_one", d_scratch, t, d_sizes, d_tile_offsets, d_tile_max_lens, d_stream,
+                             stream_len, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int ci_encode_tiled_dense(const uint8_t *d_symbols, const ci_tiling *t,

@@ -801,20 +801,21 @@ __global__ __launch_bounds__(kSegWaves *kWave) void fused_linear32_seg_kernel(Li
     }
 }
 
-// Any tile width, either tiled layout: one thread per stream, eight rows of x per pass.
+// Any tile width, any tiled layout (TileLayout): one thread per stream, eight rows of x per pass.
 // Partial sums (one per stream, i.e. per (k-tile[, half])) go to the fp32 workspace.
 // grid: (ceil(streams / 256), ceil(M / 8))
-template <bool kDense>
+template <int kLayout>
 __global__ __launch_bounds__(256) void fused_linear_generic_kernel(LinearArgs a) {
     __shared__ uint2 tab[kProbScale];
     build_slot_table(tab, a.tables, a.slot_map, threadIdx.x, 256);
     __syncthreads();
-    const uint32_t spt = (kDense ? 1 : 2) * a.tw;
+    constexpr bool kOne = kLayout != kBodyTwo;  // one stream per column over the whole tile height
+    const uint32_t spt = (kOne ? 1 : 2) * a.tw;
     const uint64_t sid = (uint64_t)blockIdx.x * 256 + threadIdx.x;
     if (sid >= (uint64_t)a.tiles_k * a.tiles_n * spt) return;
     const uint32_t tile = (uint32_t)(sid / spt), q = (uint32_t)(sid % spt);
     const uint32_t tk = tile / a.tiles_n, tn = tile % a.tiles_n;
-    const uint32_t span = kDense ? a.th : a.th / 2, hsel = kDense ? 0 : q / a.tw, c = q % a.tw;
+    const uint32_t span = kOne ? a.th : a.th / 2, hsel = kOne ? 0 : q / a.tw, c = q % a.tw;
     const uint32_t col = tn * a.tw + c, k0 = tk * a.th + hsel * span;
     if (col >= a.N) return;
     const uint32_t my_steps = k0 < a.K ? min(span, a.K - k0) : 0;
@@ -834,7 +835,7 @@ __global__ __launch_bounds__(256) void fused_linear_generic_kernel(LinearArgs a)
                 if (m0 + j < a.M) acc[j] += bf16_to_f32(a.x[(size_t)(m0 + j) * a.x_stride + k0 + i]) * w;
         }
     };
-    if (kDense) {
+    if (kLayout == kExactBytes) {
         const uint64_t off = a.stream_offsets[sid];
         uint32_t size = a.stream_sizes[sid];
         if (off + size > a.stream_len) size = 0;
@@ -849,7 +850,7 @@ __global__ __launch_bounds__(256) void fused_linear_generic_kernel(LinearArgs a)
         src.init(a.stream + base, depth, spt, q);
         run(src);
     }
-    const uint32_t p = kDense ? tk : tk * 2 + hsel;
+    const uint32_t p = kOne ? tk : tk * 2 + hsel;
 #pragma unroll
     for (int j = 0; j < 8; ++j)
         if (m0 + j < a.M) a.partial[((size_t)p * a.M + m0 + j) * a.N + col] = acc[j];
@@ -1077,9 +1078,11 @@ static int fused_linear_impl(const uint16_t *d_x, uint32_t M, uint32_t K, uint32
                              const uint32_t *d_tables, const uint8_t *d_slot_map, const uint32_t *d_meta0,
                              const uint32_t *d_meta1, const uint8_t *d_man_tiled, uint32_t th, uint32_t tw,
                              const uint16_t *d_bias, uint16_t *d_out, uint32_t out_stride, void *d_workspace,
-                             size_t workspace_bytes, bool dense, hipStream_t s, const uint16_t *d_plain_w = nullptr,
+                             size_t workspace_bytes, int layout, hipStream_t s, const uint16_t *d_plain_w = nullptr,
                              const void *d_checkpoints = nullptr, uint32_t segments = 1,
                              const void *d_slot_table = nullptr, uint32_t max_window_rows = 0) {
+    const bool dense = layout != kBodyTwo;      // one stream per column: one partial per tile row, no 32-column kernels
+    const bool exact = layout == kExactBytes;   // d_meta0 / d_meta1 are stream_offsets / stream_sizes
     if (M == 0 || N == 0) return CI_OK;
     if (K == 0) return fail(CI_ERR_ARG, "fused linear: K is 0");
     if (!d_x || !d_out) return fail(CI_ERR_ARG, "fused linear: null pointer");
@@ -1103,10 +1106,10 @@ static int fused_linear_impl(const uint16_t *d_x, uint32_t M, uint32_t K, uint32
     a.states = d_states;
     a.tables = d_tables;
     a.slot_map = d_slot_map;
-    a.tile_offsets = dense ? nullptr : d_meta0;
-    a.tile_max_lens = dense ? nullptr : d_meta1;
-    a.stream_offsets = dense ? d_meta0 : nullptr;
-    a.stream_sizes = dense ? d_meta1 : nullptr;
+    a.tile_offsets = exact ? nullptr : d_meta0;
+    a.tile_max_lens = exact ? nullptr : d_meta1;
+    a.stream_offsets = exact ? d_meta0 : nullptr;
+    a.stream_sizes = exact ? d_meta1 : nullptr;
     a.man_tiled = d_man_tiled;
     a.dense_w = d_plain_w;
     a.bias = d_bias;
@@ -1220,10 +1223,12 @@ static int fused_linear_impl(const uint16_t *d_x, uint32_t M, uint32_t K, uint32
         const uint64_t nz = (uint64_t)p.P * M * N;
         hipLaunchKernelGGL(zero_f32_kernel, dim3((uint32_t)((nz + 255) / 256)), dim3(256), 0, s, a.partial, nz);
         CI_LAUNCH_CHECK("zero_f32_kernel");
-        if (dense)
-            hipLaunchKernelGGL(fused_linear_generic_kernel<true>, grid, block, 0, s, a);
+        if (layout == kExactBytes)
+            hipLaunchKernelGGL(fused_linear_generic_kernel<kExactBytes>, grid, block, 0, s, a);
+        else if (layout == kBodyOne)
+            hipLaunchKernelGGL(fused_linear_generic_kernel<kBodyOne>, grid, block, 0, s, a);
         else
-            hipLaunchKernelGGL(fused_linear_generic_kernel<false>, grid, block, 0, s, a);
+            hipLaunchKernelGGL(fused_linear_generic_kernel<kBodyTwo>, grid, block, 0, s, a);
         CI_LAUNCH_CHECK("fused_linear_generic_kernel");
     }
     if (via_workspace) {
@@ -1255,6 +1260,18 @@ extern "C" int ci_fused_linear_dense(const uint16_t *d_x, uint32_t M, uint32_t K
     return fused_linear_impl(d_x, M, K, N, x_stride, d_stream, stream_len, d_states, d_tables, d_slot_map,
                              d_stream_offsets, d_stream_sizes, d_man_tiled, tile_height, tile_width, d_bias, d_out,
                              out_stride, d_workspace, workspace_bytes, true, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int ci_fused_linear_one(const uint16_t *d_x, uint32_t M, uint32_t K, uint32_t N, uint32_t x_stride,
+                                   const uint8_t *d_stream, uint64_t stream_len, const uint32_t *d_states,
+                                   const uint32_t *d_tables, const uint8_t *d_slot_map,
+                                   const uint32_t *d_tile_offsets, const uint32_t *d_tile_max_lens,
+                                   const uint8_t *d_man_tiled, uint32_t tile_height, uint32_t tile_width,
+                                   const uint16_t *d_bias, uint16_t *d_out, uint32_t out_stride,
+                                   void *d_workspace, size_t workspace_bytes, ci_stream_t stream) {
+    return fused_linear_impl(d_x, M, K, N, x_stride, d_stream, stream_len, d_states, d_tables, d_slot_map,
+                             d_tile_offsets, d_tile_max_lens, d_man_tiled, tile_height, tile_width, d_bias, d_out,
+                             out_stride, d_workspace, workspace_bytes, kBodyOne, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int ci_fused_linear_ilp2_segmented(const uint16_t *d_x, uint32_t M, uint32_t K, uint32_t N, uint32_t x_stride,

@@ -351,20 +351,21 @@ __global__ __launch_bounds__(kTrSegWaves *kWave) void trans32_seg_kernel(TransAr
     }
 }
 
-// Any tile width and the dense layout: one thread per (tile, half): it decodes the tile's columns
+// Any tile width, any tiled layout (TileLayout): one thread per (tile, half): it decodes the tile's columns
 // one after the other and accumulates their products into its own rows of the tile's partial, so
 // the summation order is fixed.  Slow; kept for format coverage.
-template <bool kDense>
+template <int kLayout>
 __global__ __launch_bounds__(256) void trans_generic_kernel(TransArgs a) {
     __shared__ uint2 tab[kProbScale];
     build_slot_table(tab, a.tables, a.slot_map, threadIdx.x, 256);
     __syncthreads();
-    const uint32_t spt = kDense ? 1u : 2u;
+    constexpr bool kOne = kLayout != kBodyTwo;  // one stream per column over the whole tile height
+    const uint32_t spt = kOne ? 1u : 2u;
     const uint64_t id = (uint64_t)blockIdx.x * 256 + threadIdx.x;
     if (id >= (uint64_t)a.num_tiles * spt) return;
     const uint32_t tile = (uint32_t)(id / spt), hsel = (uint32_t)(id % spt);
     const uint32_t tk = tile / a.tiles_n, tn = tile % a.tiles_n;
-    const uint32_t span = kDense ? a.th : a.th / 2, v0 = tk * a.th + hsel * span;
+    const uint32_t span = kOne ? a.th : a.th / 2, v0 = tk * a.th + hsel * span;
     if (v0 >= a.V) return;
     const uint32_t rows = min(span, a.V - v0);
     float *dst = a.partial + (size_t)tn * a.M * a.V + v0;
@@ -385,7 +386,7 @@ __global__ __launch_bounds__(256) void trans_generic_kernel(TransArgs a) {
                     dst[(size_t)m * a.V + i] += w * __uint_as_float((uint32_t)a.x[(size_t)m * a.x_stride + h] << 16);
             }
         };
-        if (kDense) {
+        if (kLayout == kExactBytes) {
             const uint32_t sid = tile * a.tw + c;
             x = a.states[sid];
             const uint64_t off = a.stream_offsets[sid];
@@ -395,13 +396,13 @@ __global__ __launch_bounds__(256) void trans_generic_kernel(TransArgs a) {
             src.init(a.stream + off, size);
             run(src);
         } else {
-            const uint32_t q = hsel * a.tw + c;
-            x = a.states[(size_t)tile * 2 * a.tw + q];
+            const uint32_t row_bytes = spt * a.tw, q = hsel * a.tw + c;
+            x = a.states[(size_t)tile * row_bytes + q];
             uint64_t base = a.tile_offsets[tile];
             uint32_t depth = a.tile_max_lens[tile];
-            if (base + (uint64_t)depth * 2 * a.tw > a.stream_len) depth = 0;
+            if (base + (uint64_t)depth * row_bytes > a.stream_len) depth = 0;
             GlobalBytes src;
-            src.init(a.stream + base, depth, 2 * a.tw, q);
+            src.init(a.stream + base, depth, row_bytes, q);
             run(src);
         }
     }
@@ -423,9 +424,11 @@ static int transposed_impl(const uint16_t *d_x, uint32_t M, uint32_t H, uint32_t
                            const uint32_t *d_tables, const uint8_t *d_slot_map, const uint32_t *d_meta0,
                            const uint32_t *d_meta1, const uint8_t *d_man_tiled, uint32_t th, uint32_t tw,
                            const uint16_t *d_bias, uint16_t *d_out, uint32_t out_stride, void *d_workspace,
-                           size_t workspace_bytes, bool dense, ci_stream_t stream,
+                           size_t workspace_bytes, int layout, ci_stream_t stream,
                            const uint16_t *d_plain_w = nullptr, const void *d_checkpoints = nullptr,
                            uint32_t segments = 1, uint32_t max_window_rows = 0, const void *d_slot_table = nullptr) {
+    const bool dense = layout != kBodyTwo;     // one stream per column: one thread per tile in the general kernel
+    const bool exact = layout == kExactBytes;  // d_meta0 / d_meta1 are stream_offsets / stream_sizes
     if (M == 0 || V == 0) return CI_OK;
     if (H == 0) return fail(CI_ERR_ARG, "transposed linear: hidden size is 0");
     if (!d_x || !d_out) return fail(CI_ERR_ARG, "transposed linear: null pointer");
@@ -451,10 +454,10 @@ static int transposed_impl(const uint16_t *d_x, uint32_t M, uint32_t H, uint32_t
     a.states = d_states;
     a.tables = d_tables;
     a.slot_map = d_slot_map;
-    a.tile_offsets = dense ? nullptr : d_meta0;
-    a.tile_max_lens = dense ? nullptr : d_meta1;
-    a.stream_offsets = dense ? d_meta0 : nullptr;
-    a.stream_sizes = dense ? d_meta1 : nullptr;
+    a.tile_offsets = exact ? nullptr : d_meta0;
+    a.tile_max_lens = exact ? nullptr : d_meta1;
+    a.stream_offsets = exact ? d_meta0 : nullptr;
+    a.stream_sizes = exact ? d_meta1 : nullptr;
     a.man_tiled = d_man_tiled;
     a.dense_w = d_plain_w;
     a.partial = static_cast<float *>(d_workspace);
@@ -517,10 +520,12 @@ static int transposed_impl(const uint16_t *d_x, uint32_t M, uint32_t H, uint32_t
         } else {
             const uint64_t threads = (uint64_t)a.num_tiles * (dense ? 1 : 2);
             const dim3 grid((uint32_t)((threads + 255) / 256)), block(256);
-            if (dense)
-                hipLaunchKernelGGL(trans_generic_kernel<true>, grid, block, 0, s, a);
+            if (layout == kExactBytes)
+                hipLaunchKernelGGL(trans_generic_kernel<kExactBytes>, grid, block, 0, s, a);
+            else if (layout == kBodyOne)
+                hipLaunchKernelGGL(trans_generic_kernel<kBodyOne>, grid, block, 0, s, a);
             else
-                hipLaunchKernelGGL(trans_generic_kernel<false>, grid, block, 0, s, a);
+                hipLaunchKernelGGL(trans_generic_kernel<kBodyTwo>, grid, block, 0, s, a);
             CI_LAUNCH_CHECK("trans_generic_kernel");
         }
         int rc = ci_splitk_reduce(a.partial, 0, a.tiles_n, a.M, V, d_bias, d_out + (size_t)m0 * out_stride, out_stride,
@@ -555,6 +560,19 @@ extern "C" int ci_fused_linear_transposed_tiled(const ci_tiled_weight *w, const 
                            w->tile_width, d_bias, d_out, out_stride, d_workspace, workspace_bytes, false, stream, nullptr,
                            w->segments > 1 ? w->d_checkpoints : nullptr, w->segments > 1 ? w->segments : 1,
                            w->max_window_rows, w->d_slot_table);
+}
+
+extern "C" int ci_fused_linear_transposed_one(const uint16_t *d_x, uint32_t M, uint32_t H, uint32_t V,
+                                              uint32_t x_stride, const uint8_t *d_stream, uint64_t stream_len,
+                                              const uint32_t *d_states, const uint32_t *d_tables,
+                                              const uint8_t *d_slot_map, const uint32_t *d_tile_offsets,
+                                              const uint32_t *d_tile_max_lens, const uint8_t *d_man_tiled,
+                                              uint32_t tile_height, uint32_t tile_width, const uint16_t *d_bias,
+                                              uint16_t *d_out, uint32_t out_stride, void *d_workspace,
+                                              size_t workspace_bytes, ci_stream_t stream) {
+    return transposed_impl(d_x, M, H, V, x_stride, d_stream, stream_len, d_states, d_tables, d_slot_map,
+                           d_tile_offsets, d_tile_max_lens, d_man_tiled, tile_height, tile_width, d_bias, d_out,
+                           out_stride, d_workspace, workspace_bytes, kBodyOne, stream);
 }
 
 extern "C" int ci_fused_linear_transposed_dense(const uint16_t *d_x, uint32_t M, uint32_t H, uint32_t V,

@@ -1,7 +1,7 @@
 """Fused decompress + embedding gather on the GPU.
 
-Call signatures follow comp_inference/embedding_triton.py:278-291 (`fused_rans_embedding_triton`)
-and :431-444 (`fused_rans_embedding_triton_uncoalesced`); the kernels are HIP (csrc/embedding.hip).
+Call signatures follow comp_inference/embedding_triton.py:278-291 (`fused_rans_embedding_triton`),
+:431-444 (`fused_rans_embedding_triton_uncoalesced`) and :8-21 (`fused_rans_embedding_triton_2`); the kernels are HIP (csrc/embedding.hip).
 """
 from __future__ import annotations
 
@@ -15,10 +15,10 @@ from .linear_hip import _Scratch
 
 
 def _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, meta0, meta1, tile_k, tile_n,
-         mantissas, out, dense: bool, checkpoints=None, segments: int = 1):
+         mantissas, out, dense: bool, checkpoints=None, segments: int = 1, one: bool = False):
     K, N = int(weight_shape[0]), int(weight_shape[1])  # K = vocabulary, N = hidden
     _lib.require_device(x)
-    _lib.check_tiled_operands(K, N, int(tile_k), int(tile_n), initial_states, tables, slot_map, meta0, meta1, dense)
+    _lib.check_tiled_operands(K, N, int(tile_k), int(tile_n), initial_states, tables, slot_map, meta0, meta1, dense, one)
     dev = x.device
     ids = x.reshape(-1)
     if ids.dtype != torch.int64:
@@ -39,8 +39,9 @@ def _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, met
     # device copies must stay referenced until the launch has been enqueued
     st, tb, sm = _lib.as_u32(initial_states, dev), _lib.as_u32(tables, dev), _lib.as_u8(slot_map, dev)
     m0, m1 = _lib.as_u32(meta0, dev), _lib.as_u32(meta1, dev)
-    if dense:
-        check(lib().ci_fused_embedding_dense(
+    if dense or one:
+        entry = lib().ci_fused_embedding_one if one else lib().ci_fused_embedding_dense
+        check(entry(
             ptr(ids), n, ptr(stream_t), C.c_uint64(stream_t.numel()), ptr(st), ptr(tb), ptr(sm), ptr(m0), ptr(m1),
             ptr(man), K, N, int(tile_k), int(tile_n), ptr(result), result.stride(0), _lib.stream_handle(dev)))
     else:
@@ -77,6 +78,15 @@ def fused_rans_embedding_uncoalesced(x, compressed_data, initial_states, tables,
                 tile_k, tile_n, mantissas, out, dense=True)
 
 
+def fused_rans_embedding_one_stream(x, compressed_data, initial_states, tables, slot_map, weight_shape,
+                                    tile_offsets, tile_max_lens, tile_k, tile_n, mantissas, out=None):
+    """Same for the first tiled format, one stream per column and tile in tile bodies of `tile_n` bytes a row
+    (`fused_rans_embedding_triton_2`, comp_inference/embedding_triton.py:8-67; kernel :71-167)."""
+    return _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, tile_offsets, tile_max_lens,
+                tile_k, tile_n, mantissas, out, dense=False, one=True)
+
+
 # Names under which the reference exports these ops (comp_inference/__init__.py:49-52).
 fused_rans_embedding_triton = fused_rans_embedding
 fused_rans_embedding_triton_uncoalesced = fused_rans_embedding_uncoalesced
+fused_rans_embedding_triton_2 = fused_rans_embedding_one_stream  # (defined there, not exported by the reference)

@@ -96,10 +96,10 @@ def _pick_workspace(workspace, need: int, dev):
 
 
 def _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, meta0, meta1, tile_k,
-         tile_n, mantissas, bias, out, workspace, dense: bool, checkpoints=None, segments: int = 1):
+         tile_n, mantissas, bias, out, workspace, dense: bool, checkpoints=None, segments: int = 1, one: bool = False):
     K, N = int(weight_shape[0]), int(weight_shape[1])
     _lib.require_device(x)
-    _lib.check_tiled_operands(K, N, int(tile_k), int(tile_n), initial_states, tables, slot_map, meta0, meta1, dense)
+    _lib.check_tiled_operands(K, N, int(tile_k), int(tile_n), initial_states, tables, slot_map, meta0, meta1, dense, one)
     dev = x.device
     x2 = _prep_x(x, K)
     M = x2.shape[0]
@@ -111,7 +111,7 @@ def _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, met
         result = out.view(M, N) if out.is_contiguous() else out
         if result.stride(-1) != 1:
             raise RuntimeError("out must have unit stride in its last dimension")
-    if not dense and DECODE_ONCE_ABOVE_ROWS is not None and M > DECODE_ONCE_ABOVE_ROWS:
+    if not dense and not one and DECODE_ONCE_ABOVE_ROWS is not None and M > DECODE_ONCE_ABOVE_ROWS:
         w = _decode_once_weight(dev, compressed_data, initial_states, tables, slot_map, (K, N), meta0, meta1,
                                 int(tile_k), int(tile_n), mantissas, "weight_kn", checkpoints, segments)
         if result.is_contiguous():
@@ -126,8 +126,8 @@ def _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, met
     need_man = (-(-K // tile_k)) * (-(-N // tile_n)) * tile_k * tile_n
     if man.numel() < need_man:
         man = torch.nn.functional.pad(man, (0, need_man - man.numel()))
-    segments = int(segments) if checkpoints is not None and not dense else 1
-    need = lib().ci_fused_linear_workspace_bytes_segmented(M, K, N, int(tile_k), int(tile_n), int(dense), segments)
+    segments = int(segments) if checkpoints is not None and not dense and not one else 1
+    need = lib().ci_fused_linear_workspace_bytes_segmented(M, K, N, int(tile_k), int(tile_n), int(dense or one), segments)
     ws, ws_bytes = _pick_workspace(workspace, need, dev)
     b = None
     if bias is not None:
@@ -135,7 +135,7 @@ def _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, met
     # device copies must stay referenced until the launch has been enqueued
     st, tb, sm = _lib.as_u32(initial_states, dev), _lib.as_u32(tables, dev), _lib.as_u8(slot_map, dev)
     m0, m1 = _lib.as_u32(meta0, dev), _lib.as_u32(meta1, dev)
-    if not dense:
+    if not dense and not one:
         ck = None
         if segments > 1:
             ck = checkpoints.to(dev).contiguous()
@@ -146,7 +146,8 @@ def _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, met
         check(lib().ci_fused_linear_tiled(C.byref(w), ptr(x2), M, x2.stride(0), ptr(b), ptr(result), result.stride(0),
                                           ptr(ws), C.c_size_t(ws_bytes), _lib.stream_handle(dev)))
     else:
-        check(lib().ci_fused_linear_dense(
+        entry = lib().ci_fused_linear_one if one else lib().ci_fused_linear_dense
+        check(entry(
             ptr(x2), M, K, N, x2.stride(0), ptr(stream_t), C.c_uint64(stream_t.numel()), ptr(st), ptr(tb), ptr(sm),
             ptr(m0), ptr(m1), ptr(man), int(tile_k), int(tile_n), ptr(b), ptr(result), result.stride(0), ptr(ws),
             C.c_size_t(ws_bytes), _lib.stream_handle(dev)))
@@ -259,6 +260,25 @@ def fused_rans_linear_uncoalesced(x, compressed_data, initial_states, tables, sl
                 stream_sizes, tile_k, tile_n, mantissas, bias, out, workspace, dense=True)
 
 
+def fused_rans_linear_one_stream(x, compressed_data, initial_states, tables, slot_map, weight_shape, tile_offsets,
+                                 tile_max_lens, tile_k, tile_n, mantissas, accum_block_size=32, bias=None, out=None,
+                                 SPLIT_K=8, workspace=None):
+    """Same for the first tiled format, one stream per column and tile in tile bodies of `tile_n` bytes a row
+    (`fused_rans_linear_triton_splitk`, comp_inference/linear_triton.py:806-890; kernel :893-1035).  The
+    reference sums bf16 partials of SPLIT_K groups of tile rows with torch.sum; here every tile row has an
+    fp32 partial of its own, summed in order and rounded once."""
+    return _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, tile_offsets,
+                tile_max_lens, tile_k, tile_n, mantissas, bias, out, workspace, dense=False, one=True)
+
+
+def fused_rans_linear_triton_2(x, compressed_data, initial_states, tables, slot_map, weight_shape, tile_offsets,
+                               tile_max_lens, tile_k, tile_n, mantissas, accum_block_size=16, bias=None, out=None):
+    """comp_inference/linear_triton.py:705-803: despite its name it launches the two-streams-per-column kernel
+    (:769), so it is `fused_rans_linear` without the split-K arguments."""
+    return fused_rans_linear(x, compressed_data, initial_states, tables, slot_map, weight_shape, tile_offsets,
+                             tile_max_lens, tile_k, tile_n, mantissas, accum_block_size, bias, out)
+
+
 def splitk_reduce(workspace: torch.Tensor, bias=None, out=None):
     """out = sum over dim 0 of a [SPLIT_K, M, N] workspace (+ bias), fp32 accumulate, one rounding
     to bf16: the reduction the reference performs with torch.sum
@@ -313,6 +333,7 @@ def plain_linear_same_order(x, weight_kn, tile_k=1024, tile_n=32, bias=None, wor
 # Names under which the reference exports these ops (comp_inference/__init__.py:39-42).
 fused_rans_linear_triton = fused_rans_linear
 fused_rans_linear_triton_uncoalesced = fused_rans_linear_uncoalesced
+fused_rans_linear_triton_splitk = fused_rans_linear_one_stream  # (defined there, not exported by the reference)
 
 
 def dense_matmul(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:

@@ -187,6 +187,40 @@ def rans_decomp_tiled_uncoalesced(compressed_streams, initial_states, tables, sl
     return out
 
 
+def rans_decomp_tiled_one_stream(compressed_streams, initial_states, tables, slot_map, output_shape,
+                                 tile_offsets, tile_max_lens, tile_k=1024, tile_n=32, mantissas=None):
+    """Decode the first tiled format -- one stream per column and tile, tile bodies of `tile_n` bytes a row --
+    into u8[K,N] (`rans_decomp_triton_tiled_splitk`, comp_inference/rans_triton.py:468-516, and
+    `rans_decomp_triton_tiled2`, :355-395, which runs the same kernel: the second definition at :399
+    replaces the first of that name at :275), or into the bf16 weight with `mantissas`."""
+    _lib.require_device(compressed_streams)
+    dev = compressed_streams.device
+    K, N = int(output_shape[0]), int(output_shape[1])
+    # comp_inference/rans_triton.py:482-487, extended to the other per-tile operands
+    _lib.check_tiled_operands(K, N, int(tile_k), int(tile_n), initial_states, tables, slot_map, tile_offsets,
+                              tile_max_lens, False, True)
+    stream_t = _lib.as_u8(compressed_streams, dev)
+    merge = mantissas is not None
+    man = None
+    if merge:
+        man = _lib.as_u8(mantissas, dev).view(-1)
+        num_tiles_n, num_tiles_k = _tiles(K, N, tile_k, tile_n)
+        need = num_tiles_k * num_tiles_n * tile_k * tile_n
+        if man.numel() < need:  # a truncated tail reads as zero padding, as in rans_decomp_tiled
+            man = torch.nn.functional.pad(man, (0, need - man.numel()))
+    out = torch.empty((K, N), device=dev, dtype=torch.bfloat16 if merge else torch.uint8)
+    st, tb, sm = _lib.as_u32(initial_states, dev), _lib.as_u32(tables, dev), _lib.as_u8(slot_map, dev)
+    to, tl = _lib.as_u32(tile_offsets, dev), _lib.as_u32(tile_max_lens, dev)
+    check(lib().ci_decode_tiled_one(
+        ptr(stream_t), C.c_uint64(stream_t.numel()), ptr(st), ptr(tb), ptr(sm), ptr(to), ptr(tl),
+        K, N, int(tile_k), int(tile_n), None if merge else ptr(out), ptr(man) if merge else None,
+        ptr(out) if merge else None, _lib.stream_handle(dev)))
+    return out
+
+
 # Names under which the reference exports these ops (comp_inference/__init__.py:34-37).
 rans_decomp_triton_tiled = rans_decomp_tiled
 rans_decomp_triton = rans_decomp_flat
+# (defined in comp_inference/rans_triton.py, not exported by the reference's package)
+rans_decomp_triton_tiled_splitk = rans_decomp_tiled_one_stream
+rans_decomp_triton_tiled2 = rans_decomp_tiled_one_stream

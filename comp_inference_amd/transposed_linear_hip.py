@@ -22,10 +22,10 @@ DECODE_ONCE_ABOVE_ROWS = 4
 
 def _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, meta0, meta1, tile_k, tile_n,
          mantissas, bias, out, dense: bool, checkpoints=None, segments: int = 1, max_window_rows: int = 0,
-         slot_table=None):
+         slot_table=None, one: bool = False):
     V, H = int(weight_shape[0]), int(weight_shape[1])  # weight is [vocab, hidden]
     _lib.require_device(x)
-    _lib.check_tiled_operands(V, H, int(tile_k), int(tile_n), initial_states, tables, slot_map, meta0, meta1, dense)
+    _lib.check_tiled_operands(V, H, int(tile_k), int(tile_n), initial_states, tables, slot_map, meta0, meta1, dense, one)
     dev = x.device
     x2 = _prep_x(x, H)
     M = x2.shape[0]
@@ -35,7 +35,7 @@ def _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, met
         if out.dtype != torch.bfloat16 or not out.is_cuda:
             raise RuntimeError("out must be a bfloat16 GPU tensor")
         result = out.view(M, V)
-    if not dense and DECODE_ONCE_ABOVE_ROWS is not None and M > DECODE_ONCE_ABOVE_ROWS:
+    if not dense and not one and DECODE_ONCE_ABOVE_ROWS is not None and M > DECODE_ONCE_ABOVE_ROWS:
         w = linear_hip._decode_once_weight(dev, compressed_data, initial_states, tables, slot_map, (V, H), meta0, meta1,
                                            int(tile_k), int(tile_n), mantissas, "weight_vh")
         if result.is_contiguous():
@@ -56,8 +56,9 @@ def _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, met
     # device copies must stay referenced until the launch has been enqueued
     st, tb, sm = _lib.as_u32(initial_states, dev), _lib.as_u32(tables, dev), _lib.as_u8(slot_map, dev)
     m0, m1 = _lib.as_u32(meta0, dev), _lib.as_u32(meta1, dev)
-    if dense:
-        check(lib().ci_fused_linear_transposed_dense(
+    if dense or one:
+        entry = lib().ci_fused_linear_transposed_one if one else lib().ci_fused_linear_transposed_dense
+        check(entry(
             ptr(x2), M, H, V, x2.stride(0), ptr(stream_t), C.c_uint64(stream_t.numel()), ptr(st), ptr(tb), ptr(sm),
             ptr(m0), ptr(m1), ptr(man), int(tile_k), int(tile_n), ptr(b), ptr(result), result.stride(0), ptr(ws),
             C.c_size_t(ws.numel()), _lib.stream_handle(dev)))
@@ -100,6 +101,17 @@ def fused_rans_linear_transposed_uncoalesced(x, compressed_data, initial_states,
                 tile_k, tile_n, mantissas, bias, out, dense=True)
 
 
+def fused_rans_linear_transposed_one_stream(x, compressed_data, initial_states, tables, slot_map, weight_shape,
+                                            tile_offsets, tile_max_lens, tile_k, tile_n, mantissas, bias=None, out=None):
+    """Same for the first tiled format, one stream per column and tile in tile bodies of `tile_n` bytes a row:
+    what `fused_rans_linear_transposed_triton_2` (comp_inference/transposed_linear_triton.py:438-500) is
+    written for.  The reference's function cannot run -- the kernel it launches,
+    `fused_rans_matmul_transposed_kernel` (:469), is defined nowhere -- so the result is pinned by the
+    decoded weight and a matmul, not by that function."""
+    return _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, tile_offsets, tile_max_lens,
+                tile_k, tile_n, mantissas, bias, out, dense=False, one=True)
+
+
 def plain_linear_transposed_same_order(x, weight_vh, tile_k=1024, tile_n=32, bias=None):
     """x[..., H] @ weight_vh[V, H]^T (+ bias) for an uncompressed bf16 weight, through the fused
     kernel's own products and reductions: bit-identical to `fused_rans_linear_transposed` on the
@@ -133,3 +145,4 @@ def plain_linear_transposed_same_order(x, weight_vh, tile_k=1024, tile_n=32, bia
 # Names under which the reference exports these ops (comp_inference/__init__.py:44-47).
 fused_rans_linear_transposed_triton = fused_rans_linear_transposed
 fused_rans_linear_transposed_triton_uncoalesced = fused_rans_linear_transposed_uncoalesced
+fused_rans_linear_transposed_triton_2 = fused_rans_linear_transposed_one_stream  # (defined there, not exported)

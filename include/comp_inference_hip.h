@@ -125,6 +125,70 @@ int ci_pack_tiled_dense(const uint8_t *d_scratch, const ci_tiling *t, const uint
                         ci_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------
+ * The first tiled format: one stream per (tile, column) over the full tile height, packed into
+ * tile bodies like the default format -- tile_max_lens[t] rows of tile_width bytes, stream q in
+ * byte column q, bottom-aligned under a zero prefix, tile_offsets = scan of depth * tile_width.
+ * ci_encode_tiled_one / ci_pack_tiled_one replace RansManager::compress_tiled
+ * (src/cuda/rans_ops.cu:412-600) = kernel rans_compress_kernel_tiled
+ * (src/cuda/rans_kernels.cuh:316-391) + the host packing loop (src/cuda/rans_ops.cu:522-566);
+ * same two-step protocol and arguments as ci_encode_tiled_ilp2 / ci_pack_tiled_ilp2, with a tiling
+ * from ci_tiling_init(..., ilp2 = 0).  The reference's Python module does not bind this encoder
+ * (src/python_bindings.cpp:302-347 binds the two-stream one under the name compress_tiled), but
+ * its Triton files still hold the consumers:
+ *   ci_decode_tiled_one            rans_decomp_triton_tiled2 / rans_decomp_triton_tiled_splitk
+ *                                  (comp_inference/rans_triton.py:355-516)
+ *   ci_fused_linear_one            fused_rans_linear_triton_splitk / fused_rans_matmul_kernel_splitk
+ *                                  (comp_inference/linear_triton.py:806-1035); workspace:
+ *                                  ci_fused_linear_workspace_bytes(M, K, N, th, tw, dense = 1)
+ *   ci_fused_embedding_one         fused_rans_embedding_triton_2 / fused_rans_embedding_kernel
+ *                                  (comp_inference/embedding_triton.py:8-167)
+ *   ci_fused_linear_transposed_one what fused_rans_linear_transposed_triton_2
+ *                                  (comp_inference/transposed_linear_triton.py:438-500) is written for;
+ *                                  the kernel that function launches is defined nowhere in the reference
+ * Arguments as the _ilp2 entry points of the same operator (d_states: tile_width entries a tile).
+ * Any tile width; one thread per stream, as for the dense format: format coverage, not a fast path.
+ * ------------------------------------------------------------------------------------- */
+int ci_encode_tiled_one(const uint8_t *d_symbols, const ci_tiling *t, const uint16_t *h_freqs,
+                        const uint16_t *h_cdf, uint8_t *d_scratch, size_t scratch_bytes,
+                        uint32_t *d_states, uint32_t *d_sizes, uint32_t *d_tile_offsets,
+                        uint32_t *d_tile_max_lens, uint64_t *h_stream_len, ci_stream_t stream);
+
+int ci_pack_tiled_one(const uint8_t *d_scratch, const ci_tiling *t, const uint32_t *d_sizes,
+                      const uint32_t *d_tile_offsets, const uint32_t *d_tile_max_lens,
+                      uint8_t *d_stream, uint64_t stream_len, ci_stream_t stream);
+
+int ci_decode_tiled_one(const uint8_t *d_stream, uint64_t stream_len, const uint32_t *d_states,
+                        const uint32_t *d_tables, const uint8_t *d_slot_map,
+                        const uint32_t *d_tile_offsets, const uint32_t *d_tile_max_lens,
+                        uint32_t K, uint32_t N, uint32_t tile_height, uint32_t tile_width,
+                        uint8_t *d_out_exp, const uint8_t *d_man_tiled, uint16_t *d_out_bf16,
+                        ci_stream_t stream);
+
+int ci_fused_linear_one(const uint16_t *d_x, uint32_t M, uint32_t K, uint32_t N, uint32_t x_stride,
+                        const uint8_t *d_stream, uint64_t stream_len, const uint32_t *d_states,
+                        const uint32_t *d_tables, const uint8_t *d_slot_map,
+                        const uint32_t *d_tile_offsets, const uint32_t *d_tile_max_lens,
+                        const uint8_t *d_man_tiled, uint32_t tile_height, uint32_t tile_width,
+                        const uint16_t *d_bias, uint16_t *d_out, uint32_t out_stride,
+                        void *d_workspace, size_t workspace_bytes, ci_stream_t stream);
+
+int ci_fused_embedding_one(const int64_t *d_ids, uint32_t n_ids, const uint8_t *d_stream,
+                           uint64_t stream_len, const uint32_t *d_states, const uint32_t *d_tables,
+                           const uint8_t *d_slot_map, const uint32_t *d_tile_offsets,
+                           const uint32_t *d_tile_max_lens, const uint8_t *d_man_tiled, uint32_t K,
+                           uint32_t N, uint32_t tile_height, uint32_t tile_width, uint16_t *d_out,
+                           uint32_t out_stride, ci_stream_t stream);
+
+int ci_fused_linear_transposed_one(const uint16_t *d_x, uint32_t M, uint32_t H, uint32_t V,
+                                   uint32_t x_stride, const uint8_t *d_stream, uint64_t stream_len,
+                                   const uint32_t *d_states, const uint32_t *d_tables,
+                                   const uint8_t *d_slot_map, const uint32_t *d_tile_offsets,
+                                   const uint32_t *d_tile_max_lens, const uint8_t *d_man_tiled,
+                                   uint32_t tile_height, uint32_t tile_width, const uint16_t *d_bias,
+                                   uint16_t *d_out, uint32_t out_stride, void *d_workspace,
+                                   size_t workspace_bytes, ci_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------
  * Encoder, flat (legacy) format.  Replaces RansManager::compress (src/cuda/rans_ops.cu:16-72)
  * = StreamConfigurator::suggest (src/cuda/rans_host.cuh:161-183) + kernel rans_compress_kernel
  * (src/cuda/rans_kernels.cuh:393-509).  num_streams = ceil(K / min_block_size) * N; stream g
