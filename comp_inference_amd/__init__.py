@@ -37,6 +37,7 @@ from .linear_hip import (
 )
 from .rans_hip import (
     build_checkpoints,
+    build_slot_table,
     rans_decomp_flat,
     rans_decomp_tiled,
     rans_decomp_tiled_batch,

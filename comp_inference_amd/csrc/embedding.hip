@@ -360,6 +360,7 @@ __device__ __forceinline__ uint32_t sort_chunk_rows(uint32_t row, uint32_t n, ui
 // streams once, to the chunk's deepest row, and writes every requested row on the way as one
 // 128-byte store.
 // rec = the chunk's record {first request, its key}, hi = the first request of the next chunk.
+// kStride = 0: no staging area of that kind; the item takes the guarded path.
 template <uint32_t kStride>
 __device__ __forceinline__ void embed_one_item(const EmbedArgs &a, uint2 rec, uint32_t hi, uint32_t pair,
                                                const uint2 *tab, uint8_t *stage, int lane) {
@@ -410,8 +411,8 @@ __device__ __forceinline__ void embed_one_item(const EmbedArgs &a, uint2 rec, ui
     const int32_t w_lo = max(wave_min_i32(row_end) - 1, 0), w_hi = wave_max_i32(row);
     const uint32_t win_a = (uint32_t)max(min(w_hi + 1, (int32_t)depth_a) - w_lo, 0),
                    win_b = (uint32_t)max(min(w_hi + 1, (int32_t)depth_b) - w_lo, 0);
-    const bool fast = __builtin_amdgcn_ballot_w64(!col_ok) == 0 && win_a >= 2 && win_b >= 2 && win_a < kStride &&
-                      win_b < kStride && (uint32_t)(uintptr_t)tab == 0;
+    const bool fast = kStride != 0 && __builtin_amdgcn_ballot_w64(!col_ok) == 0 && win_a >= 2 && win_b >= 2 &&
+                      win_a < kStride && win_b < kStride && (uint32_t)(uintptr_t)tab == 0;
     // the chunk's requests in row order, one per lane: row inside the bucket and output position
     const uint32_t nb = hi - lo;
     const uint32_t raw_row = (uint32_t)lane < nb ? min(a.keys[lo + lane] - bucket_row0, rows_b - 1) : 0u;
@@ -419,7 +420,7 @@ __device__ __forceinline__ void embed_one_item(const EmbedArgs &a, uint2 rec, ui
     const uint32_t sorted = sort_chunk_rows(raw_row, nb, (uint32_t)lane);
     const uint32_t my_row = (uint32_t)lane < nb ? sorted >> 6 : 0u;
     const uint32_t my_pos = (uint32_t)__shfl((int)raw_pos, (int)(sorted & 63u), 64);
-    if (fast) {
+    if constexpr (kStride != 0) if (fast) {
         StageRegs body;
         const uint32_t deepest = max(win_a, win_b), my_depth = (lane & 4) ? win_b : win_a;
         const uint8_t *src_a = a.stream + base_a + (size_t)w_lo * 64, *src_b = a.stream + base_b + (size_t)w_lo * 64;
@@ -558,6 +559,271 @@ __global__ __launch_bounds__(kPersistWaves *kWave) void embed_gather32_kernel(Em
         embed_wave_items<10, kDepthMedium>(a, tab, lds, wave, lane);
 }
 
+// ---- sixteen wavefronts per CU ------------------------------------------------------------------------
+// With decoder checkpoints an item is short (a walk of at most bucket_rows steps) and what it costs is the
+// chain of dependent loads in front of the walk: chunk record -> tile metadata, checkpoints and the chunk's
+// requests -> body rows.  Sixteen wavefronts per CU (128 VGPRs, 7 KB of LDS each: stage_window_pair) walk
+// their items with that chain taken apart: the record of the item three ahead, the metadata of the item two
+// ahead and the window of the next item are on their way while the current item is decoded.  Items that do
+// not qualify (ids outside the table, ragged columns, a window larger than the area) take embed_one_item's
+// guarded path.
+constexpr uint32_t kEmbSegBucketRows = 128;  // buckets up to this many rows go to this kernel
+
+struct EmbRec {  // a chunk record as loaded (the same in every lane)
+    uint32_t lo, key0, hi;
+};
+struct EmbRaw {  // what an item reads before its window is known
+    uint32_t state, row, row_end;             // per lane, as stored (row: 0x7fffffff = from the body's last row)
+    uint32_t off_a, depth_a, off_b, depth_b;  // the two tile bodies
+    uint32_t key, pos;                        // this lane's request of the chunk
+    uint32_t b, tile_a, tile_row0;            // the chunk's bucket (n_buckets: it touches no tile), its first tile,
+                                              // the bucket's first row inside the tile
+};
+struct EmbItem {  // an item ready to be staged
+    EmbRec rec;
+    uint32_t pair;
+    uint32_t nb, tile_a, tile_row0, bucket_row0;  // requests; first tile; first row of the bucket in its tile / in the table
+    uint32_t state;
+    int32_t row;
+    uint32_t w_lo, rows, win_a, win_b;  // first body row of the window, rows in it (both bodies / each)
+    uint32_t base_a, base_b;
+    uint32_t my_row, my_pos;  // the chunk's requests in row order, one per lane
+    bool fast;
+};
+
+__device__ __forceinline__ uint32_t uniform_u32(uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); }
+
+__device__ __forceinline__ void emb_rec_load(const EmbedArgs &a, uint32_t chunk, EmbRec &r) {
+    const uint2 v = a.chunk_rec[chunk];
+    r.lo = v.x;
+    r.key0 = v.y;
+    r.hi = a.chunk_rec[chunk + 1].x;
+}
+
+// The chunk's bucket, or n_buckets for a chunk that touches no tile (no requests, ids outside the table).
+__device__ __forceinline__ uint32_t emb_bucket(const EmbedArgs &a, const EmbRec &r) {
+    const uint32_t lo = uniform_u32(r.lo), hi = uniform_u32(r.hi), key0 = uniform_u32(r.key0);
+    if (lo >= hi || hi > a.n_ids || key0 == 0xFFFFFFFFu) return a.n_buckets;
+    return min(key0 / a.bucket_rows, a.n_buckets - 1);
+}
+
+__device__ __forceinline__ void emb_request(const EmbedArgs &a, const EmbRec &r, uint32_t pair, int lane, EmbRaw &m) {
+    const uint32_t b = emb_bucket(a, r);
+    m.state = m.row = m.row_end = m.off_a = m.depth_a = m.off_b = m.depth_b = m.key = m.pos = 0;
+    m.b = b;
+    m.tile_a = m.tile_row0 = 0;
+    if (b == a.n_buckets) return;
+    const uint32_t lo = uniform_u32(r.lo), nb = min(uniform_u32(r.hi) - lo, kEmbRun);
+    const uint32_t bs = b / a.segs, seg = b - bs * a.segs, hsel = bs & 1, tk = bs / 2;
+    const uint32_t side = lane / 32, c = lane % 32;
+    const bool have_b = pair * 2 + 1 < a.tiles_n;
+    const uint32_t tile_a = tk * a.tiles_n + pair * 2, tile_b = have_b ? tile_a + 1 : tile_a;
+    m.tile_a = tile_a;
+    m.tile_row0 = hsel * (a.th / 2) + seg * a.bucket_rows;
+    m.off_a = a.tile_offsets[tile_a];
+    m.depth_a = a.tile_max_lens[tile_a];
+    m.off_b = a.tile_offsets[tile_b];
+    m.depth_b = a.tile_max_lens[tile_b];
+    const uint32_t tile = side ? tile_b : tile_a, q = hsel * 32 + c;
+    const uint2 *ck = a.ckpt + ((size_t)tile * (a.segs - 1)) * 64 + q;
+    if (seg == 0) {
+        m.state = a.states[(size_t)tile * 64 + q];
+        m.row = 0x7fffffffu;
+    } else {
+        const uint2 v = ck[(size_t)(seg - 1) * 64];
+        m.state = v.x;
+        m.row = v.y;
+    }
+    m.row_end = seg + 1 < a.segs ? ck[(size_t)seg * 64].y : 0xffffffffu;
+    if ((uint32_t)lane < nb) {
+        m.key = a.keys[lo + lane];
+        m.pos = a.pos[lo + lane];
+    }
+}
+
+// Same window and the same conditions as embed_one_item's, for the as-is staging area.
+__device__ __forceinline__ void emb_resolve(const EmbedArgs &a, const EmbRec &r, uint32_t pair, int lane, const EmbRaw &m,
+                                            EmbItem &it) {
+    it.rec = r;
+    it.pair = pair;
+    it.fast = false;
+    const uint32_t b = m.b;
+    if (b == a.n_buckets) return;
+    const uint32_t rows_b = a.bucket_rows;
+    const uint32_t side = lane / 32, c = lane % 32, tn = pair * 2 + side, col = tn * 32 + c;
+    it.nb = min(uniform_u32(r.hi) - uniform_u32(r.lo), kEmbRun);
+    it.tile_a = m.tile_a;
+    it.tile_row0 = m.tile_row0;
+    it.bucket_row0 = b * rows_b;
+    it.base_a = uniform_u32(m.off_a);
+    it.base_b = uniform_u32(m.off_b);
+    uint32_t depth_a = uniform_u32(m.depth_a), depth_b = uniform_u32(m.depth_b);
+    if ((uint64_t)it.base_a + (uint64_t)depth_a * 64 > a.stream_len) depth_a = 0;
+    if ((uint64_t)it.base_b + (uint64_t)depth_b * 64 > a.stream_len) depth_b = 0;
+    const uint32_t depth = side ? depth_b : depth_a;
+    it.state = m.state;
+    it.row = min((int32_t)m.row, (int32_t)depth - 1);
+    const int32_t row_end = min((int32_t)m.row_end, it.row);
+    const bool col_ok = tn < a.tiles_n && col < a.N;
+    const int32_t w_lo = max(wave_min_i32(row_end) - 1, 0), w_hi = wave_max_i32(it.row);
+    it.w_lo = (uint32_t)w_lo;
+    it.win_a = (uint32_t)max(min(w_hi + 1, (int32_t)depth_a) - w_lo, 0);
+    it.win_b = (uint32_t)max(min(w_hi + 1, (int32_t)depth_b) - w_lo, 0);
+    it.rows = max(it.win_a, it.win_b);
+    it.fast = __builtin_amdgcn_ballot_w64(!col_ok) == 0 && it.win_a >= 2 && it.win_b >= 2 && it.rows <= kPairWinRows;
+    // the chunk's requests in row order, one per lane: row inside the bucket and output position
+    const uint32_t raw_row = (uint32_t)lane < it.nb ? min(m.key - it.bucket_row0, rows_b - 1) : 0u;
+    const uint32_t sorted = sort_chunk_rows(raw_row, it.nb, (uint32_t)lane);
+    it.my_row = (uint32_t)lane < it.nb ? sorted >> 6 : 0u;
+    it.my_pos = (uint32_t)__shfl((int)m.pos, (int)(sorted & 63u), 64);
+}
+
+// Touches the cache lines of the item's two windows (a 128-byte line per lane and body); the values are not
+// used, the caller keeps them alive until the current item has been decoded.
+__device__ __forceinline__ void emb_touch(const EmbedArgs &a, const EmbItem &it, int lane, uint32_t &t, uint32_t &t2) {
+    t = t2 = 0;
+    if (!it.fast) return;
+    if ((uint32_t)lane * 128 < it.win_a * 64)
+        t = *reinterpret_cast<const uint32_t *>(a.stream + it.base_a + (size_t)it.w_lo * 64 + lane * 128);
+    if ((uint32_t)lane * 128 < it.win_b * 64)
+        t2 = *reinterpret_cast<const uint32_t *>(a.stream + it.base_b + (size_t)it.w_lo * 64 + lane * 128);
+}
+
+// A resolved, fast item: its window into the wavefront's area, then the walk to the chunk's deepest row; every
+// requested row leaves as one 128-byte store (see embed_one_item).
+__device__ __forceinline__ void emb_run(const EmbedArgs &a, const EmbItem &it, uint8_t *stage, int lane) {
+    const uint32_t side = lane / 32, c = lane % 32, rows_b = a.bucket_rows, nb = it.nb;
+    const uint32_t col = (it.pair * 2 + side) * 32 + c;
+    const uint8_t *man = a.man_tiled + (size_t)(it.tile_a + side) * a.th * 32 + (size_t)it.tile_row0 * 32 + c;
+    FastLane st;
+    const int32_t rel = it.row - (int32_t)it.w_lo;  // this lane's next byte, in rows of the window (< 0: none left)
+    st.X = it.state << 3;
+    st.q = (uint32_t)(uintptr_t)stage + (uint32_t)(rel * 64 + lane);
+    st.n1 = rel >= 0 ? stage[rel * 64 + lane] : 0;  // (a wavefront's LDS operations complete in order)
+    const uint32_t my_row = it.my_row, my_pos = it.my_pos;
+    uint32_t done = 0, sym = 0;  // rows decoded so far, symbol of row done - 1
+    constexpr int kG = 8;
+    uint32_t row_cur[kG] = {}, row_next[kG] = {};
+    uint8_t man_cur[kG] = {}, man_next[kG] = {};
+    auto fetch = [&](uint32_t first, uint32_t(&rows)[kG], uint8_t(&mans)[kG]) {
+#pragma unroll
+        for (int u = 0; u < kG; ++u) {
+            const uint32_t idx = min(first + u, nb - 1);  // wave uniform
+            rows[u] = min((uint32_t)__builtin_amdgcn_readlane((int)my_row, (int)idx), rows_b - 1);
+            mans[u] = man[(size_t)rows[u] * 32];
+        }
+    };
+    fetch(0, row_cur, man_cur);
+    for (uint32_t s0 = 0; s0 < nb; s0 += kG) {
+        if (s0 + kG < nb) fetch(s0 + kG, row_next, man_next);
+#pragma unroll
+        for (int u = 0; u < kG; ++u)
+            if (s0 + u < nb) {
+                const uint32_t want = row_cur[u];
+                if (want + 1 > done) {  // wave uniform; requests in row order make the step count >= 1
+                    sym = advance_asm(st, want + 1 - done, 64) >> 24;
+                    done = want + 1;
+                }
+                const uint32_t p = (uint32_t)__builtin_amdgcn_readlane((int)my_pos, (int)(s0 + u));
+                a.out[(size_t)p * a.out_stride + col] = (uint16_t)assemble_bf16(sym, man_cur[u]);
+            }
+#pragma unroll
+        for (int u = 0; u < kG; ++u) {
+            row_cur[u] = row_next[u];
+            man_cur[u] = man_next[u];
+        }
+    }
+}
+
+// grid: at most one workgroup per CU; wavefront w of workgroup j takes the items j + (w + 16 i) * gridDim.x,
+// chunk-major like embed_gather32_kernel.  The host launches it only when items number fewer than 2^31.
+__global__ __launch_bounds__(kPairSegWaves *kWave) void embed_gather32_seg_kernel(EmbedArgs a, const uint2 *slot_table) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    const uint2 *tab = reinterpret_cast<const uint2 *>(lds);
+    const int tid = threadIdx.x, lane = tid % kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const uint32_t pairs = (a.tiles_n + 1) / 2;
+    const uint32_t n_chunks = min(*a.chunk_count, emb_max_chunks(a.n_ids, a.n_buckets));
+    uint8_t *stage = lds + kSlotTableBytes + (size_t)wave * kPairWinBytes;
+    // (chunk, pair) of this wavefront's items, stepped without a division per item
+    const uint32_t step = (uint32_t)kPairSegWaves * gridDim.x, step_q = step / pairs, step_r = step % pairs;
+    const uint32_t first = (uint32_t)wave * gridDim.x + blockIdx.x;
+    uint32_t ch2 = first / pairs, pr2 = first % pairs;  // the item whose record is asked for next
+    auto advance = [&]() {
+        ch2 += step_q;
+        pr2 += step_r;
+        if (pr2 >= pairs) {
+            pr2 -= pairs;
+            ++ch2;
+        }
+    };
+    EmbRec r0 = {0, 0, 0}, r1 = r0, r2 = r0;
+    uint32_t pr0 = 0, pr1 = 0;
+    bool h0 = false, h1 = false, h2 = false;
+    // the first three records, then the first item's metadata: on their way while the table arrives
+    h0 = ch2 < n_chunks;
+    if (h0) emb_rec_load(a, ch2, r0);
+    pr0 = pr2;
+    advance();
+    h1 = h0 && ch2 < n_chunks;
+    if (h1) emb_rec_load(a, ch2, r1);
+    pr1 = pr2;
+    advance();
+    h2 = h1 && ch2 < n_chunks;
+    if (h2) emb_rec_load(a, ch2, r2);
+    EmbRaw raw;
+    EmbItem nxt;
+    nxt.fast = false;
+    const bool tab_ok = (uint32_t)(uintptr_t)tab == 0;  // the hand-scheduled step reads the table at LDS address 0
+    if (h0) emb_request(a, r0, pr0, lane, raw);
+    if (slot_table) {
+        const u32x4 *src = reinterpret_cast<const u32x4 *>(slot_table);
+        u32x4 *dst = reinterpret_cast<u32x4 *>(lds);
+        const u32x4 e0 = src[tid * 2], e1 = src[tid * 2 + 1];  // 1024 threads x 32 bytes = the 32 KB table
+        dst[tid * 2] = e0;
+        dst[tid * 2 + 1] = e1;
+    } else {
+        build_slot_table_x8(reinterpret_cast<uint2 *>(lds), a.tables, a.slot_map, tid, kPairSegWaves * kWave);
+    }
+    if (h0) {
+        emb_resolve(a, r0, pr0, lane, raw, nxt);
+        nxt.fast = nxt.fast && tab_ok;
+        if (h1) emb_request(a, r1, pr1, lane, raw);
+    }
+    __syncthreads();
+    while (h0) {
+        const EmbItem cur = nxt;
+        if (cur.fast)
+            stage_window_pair(stage, a.stream + cur.base_a + (size_t)cur.w_lo * 64, cur.win_a,
+                              a.stream + cur.base_b + (size_t)cur.w_lo * 64, cur.win_b, cur.tile_row0 >= a.th / 2 ? 1u : 0u,
+                              cur.rows, lane);
+        uint32_t touched = 0, touched2 = 0;
+        h0 = h1;
+        r0 = r1;
+        pr0 = pr1;
+        h1 = h2;
+        r1 = r2;
+        pr1 = pr2;
+        if (h0) {
+            emb_resolve(a, r0, pr0, lane, raw, nxt);
+            nxt.fast = nxt.fast && tab_ok;
+            emb_touch(a, nxt, lane, touched, touched2);
+            if (h1) emb_request(a, r1, pr1, lane, raw);
+        }
+        if (h2) {
+            advance();
+            h2 = ch2 < n_chunks;
+            if (h2) emb_rec_load(a, ch2, r2);
+        }
+        if (cur.fast)
+            emb_run(a, cur, stage, lane);
+        else
+            embed_one_item<0>(a, make_uint2(uniform_u32(cur.rec.lo), uniform_u32(cur.rec.key0)), uniform_u32(cur.rec.hi),
+                              cur.pair, tab, stage, lane);
+        asm volatile("" ::"v"(touched), "v"(touched2));  // the touching loads end here
+    }
+}
+
 // Any tile width, any tiled layout (TileLayout): one thread per (token, column), discarding the rows above
 // the requested one exactly as the reference does (comp_inference/embedding_triton.py:239-257; one stream per column: :124-144).
 template <int kLayout>
@@ -637,7 +903,7 @@ static int embedding_impl(const int64_t *d_ids, uint32_t n_ids, const uint8_t *d
                           const uint32_t *d_meta0, const uint32_t *d_meta1, const uint8_t *d_man_tiled, uint32_t K,
                           uint32_t N, uint32_t th, uint32_t tw, uint16_t *d_out, uint32_t out_stride,
                           void *d_workspace, size_t workspace_bytes, int layout, hipStream_t s,
-                          const void *d_checkpoints = nullptr, uint32_t segments = 1) {
+                          const void *d_checkpoints = nullptr, uint32_t segments = 1, const void *d_slot_table = nullptr) {
     const bool dense = layout != kBodyTwo;     // one stream per column: the one-thread-per-column kernel
     const bool exact = layout == kExactBytes;  // d_meta0 / d_meta1 are stream_offsets / stream_sizes
     if (n_ids == 0 || N == 0) return CI_OK;
@@ -709,6 +975,7 @@ static int embedding_impl(const int64_t *d_ids, uint32_t n_ids, const uint8_t *d
         a.chunk_rec = reinterpret_cast<uint2 *>((at + 7) & ~(uintptr_t)7);
     }
     CI_ALLOW_FULL_LDS(embed_gather32_kernel);
+    CI_ALLOW_FULL_LDS(embed_gather32_seg_kernel);
     CI_ALLOW_FULL_LDS(embed_sort_kernel<true>);
     CI_ALLOW_FULL_LDS(embed_sort_kernel<false>);
     CI_ALLOW_FULL_LDS(embed_group_kernel);
@@ -741,6 +1008,16 @@ static int embedding_impl(const int64_t *d_ids, uint32_t n_ids, const uint8_t *d
         }
         const uint64_t most = (uint64_t)emb_max_chunks(a.n_ids, a.n_buckets) * ceil_div(a.tiles_n, 2u);
         const uint32_t gather_grid = (uint32_t)(most < (uint64_t)cus ? most : (uint64_t)cus);
+        // Short buckets (decoder checkpoints) whose table the caller keeps beside the weight: sixteen wavefronts per
+        // CU, every load of an item asked for ahead of it.
+        if (segments > 1 && a.bucket_rows <= kEmbSegBucketRows && d_slot_table && aligned(d_slot_table, 16) &&
+            most < (1ull << 31)) {
+            hipLaunchKernelGGL(embed_gather32_seg_kernel, dim3(gather_grid), dim3(kPairSegWaves * kWave),
+                               kSlotTableBytes + kPairSegWaves * kPairWinBytes, s, a,
+                               static_cast<const uint2 *>(d_slot_table));
+            CI_LAUNCH_CHECK("embed_gather32_seg_kernel");
+            continue;
+        }
         hipLaunchKernelGGL(embed_gather32_kernel, dim3(gather_grid), dim3(kPersistWaves * kWave), kLdsLimit, s, a);
         CI_LAUNCH_CHECK("embed_gather32_kernel");
     }
@@ -783,7 +1060,8 @@ extern "C" int ci_fused_embedding_tiled(const ci_tiled_weight *w, const int64_t 
     return embedding_impl(d_ids, n_ids, w->d_stream, w->stream_len, w->d_states, w->d_tables, w->d_slot_map,
                           w->d_tile_offsets, w->d_tile_max_lens, w->d_man_tiled, w->K, w->N, w->tile_height,
                           w->tile_width, d_out, out_stride, d_workspace, workspace_bytes, false,
-                          static_cast<hipStream_t>(stream), segments > 1 ? w->d_checkpoints : nullptr, segments);
+                          static_cast<hipStream_t>(stream), segments > 1 ? w->d_checkpoints : nullptr, segments,
+                          w->d_slot_table);
 }
 
 extern "C" int ci_fused_embedding_one(const int64_t *d_ids, uint32_t n_ids, const uint8_t *d_stream,

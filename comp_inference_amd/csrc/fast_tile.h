@@ -192,6 +192,39 @@ __device__ __forceinline__ void stage_body(uint8_t *stage, const uint8_t *__rest
         }
 }
 
+// ---- windows of tile pairs for sixteen wavefronts per CU -----------------------------------------
+// Sixteen wavefronts leave each, next to the slot table, 7 KB of LDS: the window of a short item on a pair of
+// neighbouring column tiles (one half of each: 32 + 32 streams), staged as the rows lie in memory -- LDS row r
+// of the window = the item's 32 bytes of row r of body A, then those of body B, so lane l finds its bytes at
+// 64 r + l and its pointer moves by 64 per byte (qdec = 64).
+constexpr int kPairSegWaves = 16;
+constexpr uint32_t kPairWinRows = 112;
+constexpr uint32_t kPairWinBytes = kPairWinRows * 64;
+constexpr int kPairWinPieces = (int)(kPairWinRows / 16);  // one 16-byte load per lane covers 16 rows
+static_assert(kPairWinRows % 16 == 0 && kSlotTableBytes + kPairSegWaves * kPairWinBytes <= kLdsLimit, "windows exceed the LDS");
+
+// Rows [0, rows) of the window: lane l loads 16 bytes of row 16 g + l / 4 -- body A for l % 4 < 2, body B
+// otherwise, columns hsel * 32 + 16 * (l % 2) on -- and writes them where they belong.  A body shorter than
+// the window (win_x < rows) repeats its last row: those bytes belong to no lane.
+__device__ __forceinline__ void stage_window_pair(uint8_t *stage, const uint8_t *__restrict__ src_a, uint32_t win_a,
+                                                  const uint8_t *__restrict__ src_b, uint32_t win_b, uint32_t hsel,
+                                                  uint32_t rows, int lane) {
+    const uint32_t r0 = lane / 4, side = (lane % 4) / 2, part = lane % 2;
+    const uint8_t *src = (side ? src_b : src_a) + hsel * 32 + part * 16;
+    const uint32_t win = side ? win_b : win_a;  // >= 1
+    u32x4 w[kPairWinPieces];
+#pragma unroll
+    for (int g = 0; g < kPairWinPieces; ++g) {
+        const uint32_t r = min((uint32_t)g * 16 + r0, win - 1);
+        w[g] = *reinterpret_cast<const u32x4 *>(src + (size_t)r * 64);
+    }
+#pragma unroll
+    for (int g = 0; g < kPairWinPieces; ++g) {
+        const uint32_t r = (uint32_t)g * 16 + r0;
+        if (r < rows) *reinterpret_cast<u32x4 *>(stage + r * 64 + side * 32 + part * 16) = w[g];
+    }
+}
+
 // ---- assembly building blocks ----------------------------------------------------------------
 // Fixed temporaries (declared as clobbers by every user):
 //   v[72:73], v[74:75]  slot-table entries of the even / odd step of a pair

@@ -15,7 +15,7 @@ from .linear_hip import _Scratch
 
 
 def _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, meta0, meta1, tile_k, tile_n,
-         mantissas, out, dense: bool, checkpoints=None, segments: int = 1, one: bool = False):
+         mantissas, out, dense: bool, checkpoints=None, segments: int = 1, one: bool = False, slot_table=None):
     K, N = int(weight_shape[0]), int(weight_shape[1])  # K = vocabulary, N = hidden
     _lib.require_device(x)
     _lib.check_tiled_operands(K, N, int(tile_k), int(tile_n), initial_states, tables, slot_map, meta0, meta1, dense, one)
@@ -53,7 +53,7 @@ def _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, met
         need = lib().ci_fused_embedding_workspace_bytes_segmented(n, K, int(tile_k), segments)
         ws = _Scratch.get(need, ("emb", dev))
         # the lengths of every operand travel with it and are checked by the library before the launch
-        w = _lib.tiled_weight(K, N, tile_k, tile_n, stream_t, st, tb, sm, m0, m1, man, ck, segments)
+        w = _lib.tiled_weight(K, N, tile_k, tile_n, stream_t, st, tb, sm, m0, m1, man, ck, segments, slot_table)
         check(lib().ci_fused_embedding_tiled(C.byref(w), ptr(ids), n, ptr(result), result.stride(0), ptr(ws),
                                              C.c_size_t(ws.numel() if ws is not None else 0), _lib.stream_handle(dev)))
     if out is not None:
@@ -62,13 +62,17 @@ def _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, met
 
 
 def fused_rans_embedding(x, compressed_data, initial_states, tables, slot_map, weight_shape, tile_offsets,
-                         tile_max_lens, tile_k, tile_n, mantissas, out=None, checkpoints=None, segments=1):
+                         tile_max_lens, tile_k, tile_n, mantissas, out=None, checkpoints=None, segments=1,
+                         slot_table=None):
     """table[x] for a table in the tiled two-streams-per-column format; ids outside the table give
     zero rows (comp_inference/embedding_triton.py:204-210, :278-330).  `checkpoints`, `segments` (not in
     the reference): the index made by `rans_hip.build_checkpoints`; a row then costs at most
-    tile_k / (2 segments) decode steps instead of tile_k / 2."""
+    tile_k / (2 segments) decode steps instead of tile_k / 2.  `slot_table` (not in the reference):
+    the table made by `rans_hip.build_slot_table`; with it and checkpoints that cut buckets of at most 128 rows
+    the gather runs on sixteen wavefronts per CU with every load of an item asked for ahead of it."""
     return _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, tile_offsets, tile_max_lens,
-                tile_k, tile_n, mantissas, out, dense=False, checkpoints=checkpoints, segments=segments)
+                tile_k, tile_n, mantissas, out, dense=False, checkpoints=checkpoints, segments=segments,
+                slot_table=slot_table)
 
 
 def fused_rans_embedding_uncoalesced(x, compressed_data, initial_states, tables, slot_map, weight_shape,

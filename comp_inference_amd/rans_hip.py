@@ -101,6 +101,23 @@ def build_checkpoints(compressed_streams, initial_states, tables, slot_map, weig
     return out
 
 
+def build_slot_table(tables, slot_map, device=None) -> torch.Tensor:
+    """The decoder's lookup table in the form the kernels keep in LDS (32 KB, uint8 tensor on the GPU): one
+    8-byte entry per 12-bit slot, the reference's `slot_map` and `tables` folded into one read
+    (src/cuda/rans_kernels.cuh:677-690).  Derived data kept beside a weight like the checkpoints: an operator
+    given it copies the table instead of building it in every workgroup."""
+    dev = torch.device(device) if device is not None else tables.device
+    tb, sm = _lib.as_u32(tables, dev), _lib.as_u8(slot_map, dev)
+    _lib.require_device(tb)
+    if tb.numel() != 256 or sm.numel() != 4096:
+        raise ValueError("tables must hold 256 entries and slot_map 4096")
+    out = torch.empty(_lib.SLOT_TABLE_BYTES, dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        check(lib().ci_build_slot_table(ptr(tb), ptr(sm), ptr(out), C.c_size_t(_lib.SLOT_TABLE_BYTES),
+                                        _lib.stream_handle(dev)))
+    return out
+
+
 class _DecodeItem(C.Structure):
     _fields_ = [("d_stream", C.c_void_p), ("stream_len", C.c_uint64), ("d_states", C.c_void_p),
                 ("d_tables", C.c_void_p), ("d_slot_map", C.c_void_p), ("d_tile_offsets", C.c_void_p),
