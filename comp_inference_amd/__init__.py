@@ -26,6 +26,7 @@ from .embedding_hip import (
 from .linear_hip import (
     dense_matmul,
     fused_rans_linear,
+    fused_wide_rows,
     fused_rans_linear_one_stream,
     fused_rans_linear_triton,
     fused_rans_linear_triton_uncoalesced,

@@ -281,6 +281,153 @@ __global__ __launch_bounds__(kLinMaxWaves *kWave) void fused_linear32_kernel(Lin
     }
 }
 
+// ---- more than 64 rows of x in one pass over the weight ---------------------------------------------------
+// The same decomposition as fused_linear32_kernel (a wavefront per tile, kw k-tiles of nw column tiles per
+// workgroup, the kw accumulators of a column tile added through LDS in k order), with MB = 4 or 8 groups of 32
+// rows of x per pass: a tile is decoded once, its eight-row weight fragments stay in registers, and every
+// fragment goes into MB matrix instructions, one per group of rows, against the x fragments of the copy in
+// fragment order (LinearArgs::xf, which this kernel needs).  The decode cost is then paid once per 128 or 256
+// rows instead of once per 64.  Every row of x still sees the same sequence of matrix instructions and the same
+// sums as in fused_linear32_kernel, so the results are bit-identical to it.
+// grid: (ceil(tiles_n / nw), P, ceil(M / (32 * MB)))   block: kw * nw waves
+template <int MB>
+__device__ __forceinline__ void linear_tile_wide(FastLane &st, f32x16 (&acc)[MB], const uint32_t *__restrict__ mrow,
+                                                 const u32x4 *__restrict__ xrow, uint32_t group_stride,
+                                                 uint32_t man_sel, uint32_t nblk) {
+    // mrow: the aligned dword holding this lane's sign|mantissa byte of the tile half's first row (+ 8 dwords per
+    // row); xrow: this lane's 16 bytes of the first block's fragment of the pass's first group (+ 32 per block,
+    // + group_stride per group).  The next block's operands are loaded while this one decodes.
+    uint32_t mcur[8], mnext[8];
+    u32x4 xcur[MB], xnext[MB];
+#pragma unroll
+    for (int r = 0; r < 8; ++r) mcur[r] = mrow[r * 8];
+#pragma unroll
+    for (int g = 0; g < MB; ++g) xcur[g] = xrow[(size_t)g * group_stride];
+    for (uint32_t blk = 0; blk < nblk; ++blk) {
+        const uint32_t nb = blk + 1 < nblk ? blk + 1 : blk;  // (the last block re-reads its own: stays inside the tile)
+#pragma unroll
+        for (int r = 0; r < 8; ++r) mnext[r] = mrow[(size_t)nb * 64 + r * 8];
+#pragma unroll
+        for (int g = 0; g < MB; ++g) xnext[g] = xrow[(size_t)nb * 32 + (size_t)g * group_stride];
+        uint32_t w[4];
+        decode8_weights_asm(st, mcur, man_sel, w);
+        // (the statement's last instruction but one writes w[3]: a matrix instruction may read a register a vector
+        // instruction wrote no sooner than two wait states later, and the compiler does not see inside the
+        // statement; w[3] passes through the wait, so whatever reads it comes after)
+        asm volatile("s_nop 1" : "+v"(w[3]));
+        const u32x4 wv = {w[0], w[1], w[2], w[3]};
+#pragma unroll
+        for (int g = 0; g < MB; ++g)
+            acc[g] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, wv),
+                                                             __builtin_bit_cast(bf16x8, xcur[g]), acc[g], 0, 0, 0);
+#pragma unroll
+        for (int r = 0; r < 8; ++r) mcur[r] = mnext[r];
+#pragma unroll
+        for (int g = 0; g < MB; ++g) xcur[g] = xnext[g];
+    }
+}
+
+template <int MB>
+__global__ __launch_bounds__(kLinMaxWaves *kWave) void fused_linear32_wide_kernel(LinearArgs a) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    uint2 *tab = reinterpret_cast<uint2 *>(lds);
+    const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
+    const int nthreads = blockDim.x;
+    uint8_t *stage = lds + kSlotTableBytes + (size_t)wave * kFastStageBytes;
+
+    const uint32_t kidx = wave % a.kw, nidx = wave / a.kw;
+    const uint32_t tk = blockIdx.y * a.kw + kidx, tn = blockIdx.x * a.nw + nidx;
+    const bool have_tile = tk < a.tiles_k && tn < a.tiles_n;
+    const uint32_t tile = tk * a.tiles_n + tn;
+    const uint32_t half = a.th / 2, hsel = lane / 32, c = lane % 32;
+    const uint32_t col0 = tn * 32, k0 = tk * a.th + hsel * half;
+    uint32_t depth = 0, my_steps = 0, state = 0;
+    uint64_t base = 0;
+    bool fast = false;
+    StageRegs body;
+    if (have_tile) {
+        base = a.tile_offsets[tile];
+        depth = a.tile_max_lens[tile];
+        state = a.states[(size_t)tile * 64 + lane];
+        if (base + (uint64_t)depth * 64 > a.stream_len) depth = 0;
+        if (col0 + c < a.N && k0 < a.K) my_steps = min(half, a.K - k0);
+        const bool full = __builtin_amdgcn_ballot_w64(my_steps != half) == 0;
+        // the same conditions as fused_linear32_kernel's hand-scheduled loop (a tile takes the same path in both)
+        fast = full && a.fast_ok && depth >= 2 && depth < kFastStride && half % 16 == 0 && (uint32_t)(uintptr_t)tab == 0;
+        if (fast) stage_fetch(body, a.stream + base, 0, depth, lane);
+    }
+    build_slot_table_x8(tab, a.tables, a.slot_map, tid, nthreads);  // runs under the body loads
+    if (fast) {
+        stage_commit(body, stage, 0, depth, lane);
+        for (int grp = 1; grp < kStageGroups; ++grp)
+            if ((uint32_t)grp * 128 < depth) {
+                stage_fetch(body, a.stream + base, grp * 128, depth, lane);
+                stage_commit(body, stage, grp * 128, depth, lane);
+            }
+    }
+    __syncthreads();
+
+    const uint32_t g0 = blockIdx.z * MB;  // first 32-row group of this pass
+    f32x16 acc[MB];
+#pragma unroll
+    for (int g = 0; g < MB; ++g)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[g][v] = 0.f;
+
+    if (have_tile) {
+        const size_t man_tile = (size_t)tile * a.th * 32;
+        if (fast) {
+            FastLane st;
+            st.init(stage, depth, lane, state);
+            // (the fragment copy holds whole passes: its groups past the last row of x are zero)
+            const uint32_t kbs = a.K / 8;
+            const u32x4 *xrow = reinterpret_cast<const u32x4 *>(a.xf) + ((size_t)g0 * kbs + k0 / 8) * 32 + c;
+            const uint32_t *mrow =
+                reinterpret_cast<const uint32_t *>(a.man_tiled + man_tile + (size_t)hsel * half * 32 + (c & ~3u));
+            const uint32_t man_sel = 0x04040000u + (c & 3u) * 0x01010101u;
+            linear_tile_wide<MB>(st, acc, mrow, xrow, kbs * 32, man_sel, half / 8);
+        } else {
+            const uint8_t *man = a.man_tiled + man_tile + (size_t)hsel * half * 32 + c;
+#pragma unroll
+            for (int g = 0; g < MB; ++g) {  // the guarded path walks the tile again for every group of rows
+                const uint32_t m = (g0 + g) * 32 + c;
+                const bool m_ok = m < a.M;
+                GlobalBytes src;
+                src.init(a.stream + base, depth, 64, lane);
+                linear_tile_guarded(src, state << 3, tab, a.K, half, my_steps, man,
+                                    a.x + (size_t)(m_ok ? m : 0) * a.x_stride + k0, m_ok, k0, acc[g]);
+            }
+        }
+    }
+
+    // Sum the kw accumulators of each column tile in k order (as in fused_linear32_kernel).
+    __syncthreads();
+    float *red = reinterpret_cast<float *>(lds + kSlotTableBytes);
+    const uint32_t frag = 16 * kWave;
+#pragma unroll
+    for (int g = 0; g < MB; ++g) {
+        const uint32_t mg = (g0 + g) * 32 + c;
+        if (g) __syncthreads();
+#pragma unroll
+        for (int v = 0; v < 16; ++v) red[(size_t)wave * frag + v * kWave + lane] = acc[g][v];
+        __syncthreads();
+        if (kidx == 0 && tn < a.tiles_n) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                float s = 0.f;
+                for (uint32_t kk = 0; kk < a.kw; ++kk) s += red[(size_t)(nidx * a.kw + kk) * frag + v * kWave + lane];
+                const uint32_t n = tn * 32 + (v / 4) * 8 + hsel * 4 + (v % 4);
+                if (mg < a.M && n < a.N) {
+                    if (a.P == 1)
+                        a.out[(size_t)mg * a.out_stride + n] = finish_bf16(s, a.bias, n);
+                    else
+                        a.partial[((size_t)blockIdx.y * a.M + mg) * a.N + n] = s;
+                }
+            }
+        }
+    }
+}
+
 // The same tile work with workgroups resident for the launch (fast_tile.h): wavefront w of workgroup j
 // takes the items j + (w + n i) * gridDim.x and writes its 32-column partial product to the fp32 workspace
 // [tiles_k * segs][M][N], which the reduction kernel sums in k order.  For weights with more tiles than
@@ -958,9 +1105,19 @@ static void launch_splitk_reduce(const float *partial, uint32_t P, uint32_t M, u
     }
 }
 
+// Groups of 32 rows per pass of fused_linear32_wide_kernel for M rows of x (0: not its case).
+static uint32_t wide_groups(uint32_t M) { return M <= 64 ? 0u : M <= 128 ? 4u : 8u; }
+
+// Groups of 32 rows in the fragment copy: whole passes where the wide kernel may run (the groups past the last
+// row of x are zero), else the groups x has.
+static uint32_t x_fragment_groups(uint32_t M) {
+    const uint32_t groups = ceil_div(M, 32u), per_pass = wide_groups(M);
+    return per_pass ? ceil_div(groups, per_pass) * per_pass : groups;
+}
+
 static size_t x_fragment_bytes(uint32_t M, uint32_t K, bool fast_plan) {
     if (!fast_plan || M < kFragMinRows || K % 8) return 0;
-    return (size_t)ceil_div(M, 32u) * 32 * K * 2;
+    return (size_t)x_fragment_groups(M) * 32 * K * 2;
 }
 
 struct LinearPlan {
@@ -1072,6 +1229,12 @@ extern "C" uint32_t ci_suggest_segments(uint32_t K, uint32_t N, uint32_t tile_he
     }
     return best;
 }
+
+// Whether more than 64 rows of x go through fused_linear32_wide_kernel (one decode per 128 or 256 rows) instead
+// of fused_linear32_kernel<2> once per 64 rows.  Same results bit for bit; off until it has been measured.
+static std::atomic<int> g_wide_rows{0};
+
+extern "C" int ci_fused_linear_wide_rows(int enable) { return g_wide_rows.exchange(enable ? 1 : 0); }
 
 static int fused_linear_impl(const uint16_t *d_x, uint32_t M, uint32_t K, uint32_t N, uint32_t x_stride,
                              const uint8_t *d_stream, uint64_t stream_len, const uint32_t *d_states,
@@ -1209,8 +1372,18 @@ static int fused_linear_impl(const uint16_t *d_x, uint32_t M, uint32_t K, uint32
         const uint32_t lds_bytes = kSlotTableBytes + waves * kFastStageBytes;
         CI_ALLOW_FULL_LDS(fused_linear32_kernel<1>);
         CI_ALLOW_FULL_LDS(fused_linear32_kernel<2>);
+        CI_ALLOW_FULL_LDS(fused_linear32_wide_kernel<4>);
+        CI_ALLOW_FULL_LDS(fused_linear32_wide_kernel<8>);
         const dim3 block(waves * kWave);
-        if (M > 32)
+        const uint32_t per_pass = wide_groups(M);
+        if (per_pass && a.xf && !d_plain_w && g_wide_rows.load(std::memory_order_relaxed)) {
+            const dim3 grid(ceil_div(a.tiles_n, p.nw), p.P, ceil_div(M, 32 * per_pass));
+            if (per_pass == 4)
+                hipLaunchKernelGGL(fused_linear32_wide_kernel<4>, grid, block, lds_bytes, s, a);
+            else
+                hipLaunchKernelGGL(fused_linear32_wide_kernel<8>, grid, block, lds_bytes, s, a);
+            CI_LAUNCH_CHECK("fused_linear32_wide_kernel");
+        } else if (M > 32)
             hipLaunchKernelGGL(fused_linear32_kernel<2>, dim3(ceil_div(a.tiles_n, p.nw), p.P, ceil_div(M, 64)), block,
                                lds_bytes, s, a);
         else

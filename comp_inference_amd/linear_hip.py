@@ -59,6 +59,13 @@ def release_scratch() -> int:
 DECODE_ONCE_ABOVE_ROWS = 64
 
 
+def fused_wide_rows(enable: bool) -> bool:
+    """More than 64 rows of x inside the fused kernel (reached with DECODE_ONCE_ABOVE_ROWS = None, or from C):
+    with `enable` a tile is decoded once per 128 or 256 rows of x instead of once per 64.  Bit-identical results.
+    Process-wide, off by default; returns the previous setting."""
+    return bool(lib().ci_fused_linear_wide_rows(1 if enable else 0))
+
+
 def _decode_once_weight(dev, compressed_data, initial_states, tables, slot_map, shape, tile_offsets, tile_max_lens,
                         tile_k, tile_n, mantissas, tag, checkpoints=None, segments=1):
     """The bf16 weight, decoded into a grow-only scratch of its own (valid until the next such call).  With

@@ -514,6 +514,13 @@ int ci_fused_linear_tiled_noalloc(const ci_tiled_weight *w, const uint16_t *d_x,
                                   const uint16_t *d_bias, uint16_t *d_out, uint32_t out_stride,
                                   ci_stream_t stream);
 
+/* More than 64 rows of x: with `enable` non-zero the fused linears of the default format decode a tile once per
+ * 128 (65..128 rows) or 256 rows of x and feed every eight-row weight fragment to one matrix instruction per
+ * group of 32 rows, instead of decoding the weight again for every 64 rows.  Results are bit-identical either
+ * way.  Process-wide, off by default; returns the previous setting.  No counterpart in the reference, which
+ * decodes once per 16 rows (comp_inference/linear_triton.py:250-266). */
+int ci_fused_linear_wide_rows(int enable);
+
 /* ---------------------------------------------------------------------------------------
  * Verification aids: the contraction of the fused kernels applied to a plain (uncompressed) bf16
  * weight.  No counterpart in the reference, whose tests compare the fused kernels with
