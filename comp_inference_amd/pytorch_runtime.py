@@ -232,12 +232,28 @@ class RansEmbedding(nn.Module):
             (max(1, half // 64) if self.tile_n == 32 and half % 64 == 0 else 1)
         return _cached_checkpoints(self, device, (self.num_embeddings, self.embedding_dim), segs)
 
+    # The gather on sixteen wavefronts per CU (needs checkpoints and the slot table kept beside the table, built on
+    # first use).  Off until that kernel has been measured.
+    sixteen_wavefronts = False
+
+    def _slot_table(self, device):
+        from .rans_hip import build_slot_table
+
+        t, m = self.rans_exp_tables, self.rans_exp_slot_map
+        key = (str(device), t.data_ptr(), t._version, m.data_ptr(), m._version)
+        cached = getattr(self, "_slot_table_cache", None)
+        if cached is None or cached[0] != key:
+            cached = (key, build_slot_table(t, m, device))
+            self._slot_table_cache = cached
+        return cached[1]
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         device = x.device
         checkpoints, segments = self._checkpoints(device)
         return fused_rans_embedding(
             x=x,
             checkpoints=checkpoints, segments=segments,
+            slot_table=self._slot_table(device) if self.sixteen_wavefronts and segments > 1 else None,
             compressed_data=self.rans_exp_stream.to(device, non_blocking=True),
             initial_states=self.rans_exp_states.to(device, non_blocking=True),
             tables=self.rans_exp_tables.to(device, non_blocking=True),

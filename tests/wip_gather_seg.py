@@ -84,3 +84,22 @@ def test_every_row_of_a_tile_row(oracle):
     t = _Table(oracle, K, N, th, 8, seed=2)
     _check(t, torch.arange(1024, 2048, dtype=torch.int64))
     _check(t, torch.arange(2047, -1, -1, dtype=torch.int64))
+
+
+def test_the_module_takes_the_kernel_when_switched_on(oracle):
+    import comp_inference_amd as ci
+
+    V, H = 2048, 128
+    emb = torch.nn.Embedding(V, H).to(torch.bfloat16)
+    with torch.no_grad():
+        emb.weight.copy_(make_weight_kn(H, V, seed=6))
+    table = emb.weight.detach().clone()
+    src = emb.cuda()
+    ci.rans_compress_module_weight(src, tile_height=1024, tile_width=32)
+    mod = ci.RansEmbedding.from_compressed(src).cuda()
+    ids = torch.randint(0, V, (3, 50), generator=torch.Generator().manual_seed(1))
+    want = table[ids].view(torch.int16)
+    assert torch.equal(mod(ids.cuda()).cpu().view(torch.int16), want)
+    mod.sixteen_wavefronts = True
+    assert torch.equal(mod(ids.cuda()).cpu().view(torch.int16), want)
+    assert mod._slot_table_cache[1].numel() == 32768
