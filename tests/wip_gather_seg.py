@@ -94,9 +94,8 @@ def test_the_module_takes_the_kernel_when_switched_on(oracle):
     with torch.no_grad():
         emb.weight.copy_(make_weight_kn(H, V, seed=6))
     table = emb.weight.detach().clone()
-    src = emb.cuda()
-    ci.rans_compress_module_weight(src, tile_height=1024, tile_width=32)
-    mod = ci.RansEmbedding.from_compressed(src).cuda()
+    ci.rans_compress_module_weight(emb, tile_height=1024, tile_width=32, transpose_weight=False)
+    mod = ci.RansEmbedding.from_compressed(emb)
     ids = torch.randint(0, V, (3, 50), generator=torch.Generator().manual_seed(1))
     want = table[ids].view(torch.int16)
     assert torch.equal(mod(ids.cuda()).cpu().view(torch.int16), want)
