@@ -261,6 +261,9 @@ def main() -> int:
     ap.add_argument("--no-gemv", action="store_true")
     ap.add_argument("--no-embedding", action="store_true")
     ap.add_argument("--no-model", action="store_true", help="skip the 32-layer decoder (about a minute)")
+    ap.add_argument("--new-kernels", action="store_true",
+                    help="also time the kernels that are off by default (more than 64 rows of x in one pass, the "
+                         "gather on sixteen wavefronts), each checked against the default path first")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three 64 MiB device-to-device copies, so that a counter run has a "
                          "kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
@@ -394,6 +397,35 @@ def main() -> int:
                          "torch_matmul_bf16_us": round(us_ref, 2),
                          "torch_matmul_weight_GBs": round(2 * gate.K * gate.N / (us_ref * 1e-6) / 1e9, 1)})
         out["fused_gemv"] = {"layer": "gate K=4096 N=14336", "bytes_M1": gate.linear_bytes(1), "rows": rows}
+        if a.new_kernels:
+            # more than 64 rows of x: the fused kernel that decodes once per 64 rows, the one that decodes once per
+            # 128 / 256 rows (must give the same bits), and the default policy (decode once to HBM + library GEMM)
+            import comp_inference_amd.linear_hip as lh
+
+            wide_rows = []
+            for M in (128, 256, 512, 2048):
+                xm = torch.randn(M, gate.K, generator=g, dtype=torch.float32).to(torch.bfloat16).to(dev)
+                policy = lh.DECODE_ONCE_ABOVE_ROWS
+                t_default = batched_time_us(lambda: gate.linear(xm), 5, 20)
+                lh.DECODE_ONCE_ABOVE_ROWS = None
+                try:
+                    lh.fused_wide_rows(False)
+                    narrow = gate.linear(xm)
+                    t_narrow = batched_time_us(lambda: gate.linear(xm), 5, 20)
+                    lh.fused_wide_rows(True)
+                    wide = gate.linear(xm)
+                    t_wide = batched_time_us(lambda: gate.linear(xm), 5, 20)
+                finally:
+                    lh.fused_wide_rows(False)
+                    lh.DECODE_ONCE_ABOVE_ROWS = policy
+                t_ref = batched_time_us(lambda: torch.matmul(xm, w_dense), 5, 20)
+                flops = 2.0 * M * gate.K * gate.N
+                wide_rows.append({"M": M, "us_one_decode_per_64_rows": round(t_narrow, 1),
+                                  "us_one_decode_per_pass": round(t_wide, 1), "bit_identical": bool(torch.equal(narrow, wide)),
+                                  "us_decode_once_plus_library_gemm": round(t_default, 1),
+                                  "mfma_util_vs_2500_TFLOPs": round(flops / (t_wide * 1e-6) / 1e12 / 2500.0, 4),
+                                  "torch_matmul_bf16_us": round(t_ref, 1)})
+            out["fused_gemm_rows"] = {"layer": "gate K=4096 N=14336", "rows": wide_rows}
 
     # --- the four GEMVs of a decoder layer at M = 1 (q/k/v and gate/up fused along the outputs, as the
     # runtime modules hold them), with decoder checkpoints where the library suggests them
@@ -460,6 +492,18 @@ def main() -> int:
         # useful bytes of the gather: the rows written and, per distinct (half tile of rows, pair of column
         # tiles) touched, nothing less than the rows themselves in compressed form -- counted as output only
         record("embed_gather32_kernel (+ grouping)", f"{V}x{H} table, {T} Zipf ids, 8 segments", T * H * 2 + T * 8, us)
+        if a.new_kernels:
+            slot_table = ci.build_slot_table(emb.tables, emb.slot_map)
+
+            def gather16():
+                return ci.fused_rans_embedding(ids, emb.stream, emb.states, emb.tables, emb.slot_map, (V, H),
+                                               emb.tile_offsets, emb.tile_max_lens, emb.th, emb.tw, emb.man,
+                                               checkpoints=ck, segments=emb_segments, slot_table=slot_table)
+
+            exact16 = bool(torch.equal(gather16().cpu().view(torch.int16), want_rows))
+            us16 = batched_time_us(gather16, 10, 50)
+            out["fused_embedding"]["sixteen_wavefronts"] = {"bit_exact": exact16, "us": round(us16, 1)}
+            record("embed_gather32_seg_kernel (+ grouping)", f"{V}x{H} table, {T} Zipf ids, 8 segments", T * H * 2 + T * 8, us16)
 
         # --- the same table as a tied LM head: logits = x W^T, M = 1
         xh = torch.randn(1, H, generator=torch.Generator("cpu").manual_seed(2), dtype=torch.float32).to(torch.bfloat16).to(dev)
