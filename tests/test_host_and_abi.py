@@ -316,3 +316,88 @@ def test_a_descriptor_with_a_short_array_is_refused_on_the_host():
     assert lib.ci_fused_embedding_tiled(bare, fake, 3, fake, N, fake, sz(1 << 20), None) == 1
     assert lib.ci_fused_linear_transposed_tiled(bare, fake, 1, N, None, fake, K, fake, sz(1 << 20), None) == 1
     assert lib.ci_decode_tiled(bare, None, fake, None) == 1
+
+
+def test_one_stream_layout_host_checks():
+    """The first tiled format (one stream per column and tile in tile bodies): operand lengths in Python, tiling
+    and pointer checks of the entry points, all before any HIP call."""
+    from comp_inference_amd import _lib
+    from comp_inference_amd._lib import check_tiled_operands as chk
+
+    z = lambda n: torch.zeros(n, dtype=torch.int32)  # noqa: E731
+    chk(1300, 80, 1024, 32, z(2 * 3 * 32), z(256), z(4096), z(6), z(6), False, True)      # 2 x 3 tiles, 32 streams each
+    for bad in (lambda: chk(1300, 80, 1024, 32, z(2 * 3 * 64), z(256), z(4096), z(6), z(6), False, True),
+                lambda: chk(1300, 80, 1024, 32, z(192), z(256), z(4096), z(192), z(192), False, True),
+                lambda: chk(1300, 80, 1024, 32, z(192), z(256), z(4095), z(6), z(6), False, True)):
+        with pytest.raises(ValueError):
+            bad()
+
+    lib = _lib.lib()
+    P = ctypes.c_void_p
+    fake, null = P(0x1000), P(0)
+    u64, sz = ctypes.c_uint64, ctypes.c_size_t
+    two, one = _lib.Tiling(), _lib.Tiling()
+    assert lib.ci_tiling_init(ctypes.byref(two), 2048, 64, 1024, 32, 1) == 0
+    assert lib.ci_tiling_init(ctypes.byref(one), 2048, 64, 1024, 32, 0) == 0
+    assert (one.streams_per_tile, one.num_streams, two.num_streams) == (32, 128, 256)
+    total = u64(0)
+    f = np.full(256, 16, np.uint16)
+    c = (np.arange(256) * 16).astype(np.uint16)
+    fp, cp = f.ctypes.data_as(P), c.ctypes.data_as(P)
+    # a tiling made for the other layout is refused by both encoders and both packers
+    assert lib.ci_encode_tiled_one(fake, ctypes.byref(two), fp, cp, fake, sz(1 << 30), fake, fake, fake, fake,
+                                   ctypes.byref(total), None) == 1 and b"one stream" in lib.ci_last_error()
+    assert lib.ci_encode_tiled_ilp2(fake, ctypes.byref(one), fp, cp, fake, sz(1 << 30), fake, fake, fake, fake,
+                                    ctypes.byref(total), None) == 1 and b"two streams" in lib.ci_last_error()
+    assert lib.ci_pack_tiled_one(fake, ctypes.byref(two), fake, fake, fake, fake, u64(64), None) == 1
+    assert lib.ci_pack_tiled_ilp2(fake, ctypes.byref(one), fake, fake, fake, fake, u64(64), None) == 1
+    assert lib.ci_pack_tiled_one(fake, ctypes.byref(one), fake, fake, fake, null, u64(64), None) == 1    # no stream buffer
+    assert lib.ci_pack_tiled_one(fake, ctypes.byref(one), fake, fake, fake, null, u64(0), None) == 0     # nothing to pack
+    # scratch too small: refused before the encode kernel (CI_ERR_CAPACITY)
+    assert lib.ci_encode_tiled_one(fake, ctypes.byref(one), fp, cp, fake, sz(16), fake, fake, fake, fake,
+                                   ctypes.byref(total), None) == 3
+
+    def dec(out, states=fake, th=1024, man=None, out16=None):
+        return lib.ci_decode_tiled_one(fake, u64(64), states, fake, fake, fake, fake, 2048, 64, th, 32, out, man, out16, None)
+
+    assert dec(null) == 1 and dec(fake, states=null) == 1 and dec(fake, th=0) == 1
+    assert dec(null, man=fake, out16=null) == 1                                  # merge asked without bf16 output
+    assert lib.ci_decode_tiled_one(fake, u64(64), fake, fake, fake, fake, fake, 0, 64, 1024, 32, null, None, None, None) == 0
+
+    M, K, N = 2, 2048, 64
+    need = lib.ci_fused_linear_workspace_bytes(M, K, N, 1024, 32, 1)
+    assert need >= 2 * M * N * 4                                                  # one partial per tile row
+
+    def lin(ws, ws_bytes, x_stride=K, states=fake):
+        return lib.ci_fused_linear_one(fake, M, K, N, x_stride, fake, u64(64), states, fake, fake, fake, fake, fake, 1024, 32,
+                                       None, fake, N, ws, sz(ws_bytes), None)
+
+    assert lin(null, 0) == 3 and lin(fake, need - 1) == 3 and lin(fake, need, x_stride=K - 1) == 1
+    assert lin(fake, need, states=null) == 1
+    assert lib.ci_fused_embedding_one(fake, 5, fake, u64(64), fake, fake, fake, fake, fake, fake, 2048, 64, 1024, 32, fake,
+                                      63, None) == 1                              # row stride shorter than the row
+    assert lib.ci_fused_embedding_one(fake, 5, fake, u64(64), null, fake, fake, fake, fake, fake, 2048, 64, 1024, 32, fake,
+                                      64, None) == 1
+    tneed = lib.ci_fused_linear_transposed_workspace_bytes(M, 64, 2048, 32)
+    assert lib.ci_fused_linear_transposed_one(fake, M, 64, 2048, 64, fake, u64(64), fake, fake, fake, fake, fake, fake, 1024,
+                                              32, None, fake, 2048, fake, sz(tneed - 1), None) == 3
+    assert lib.ci_fused_linear_transposed_one(fake, M, 64, 2048, 63, fake, u64(64), fake, fake, fake, fake, fake, fake, 1024,
+                                              32, None, fake, 2048, fake, sz(tneed), None) == 1
+
+
+def test_wide_rows_switch_and_fragment_sizes():
+    """ci_fused_linear_wide_rows returns the previous setting; the workspace of more than 64 rows holds the fragment
+    copy of x padded to whole passes (4 groups of 32 rows up to 128 rows, 8 above), whichever kernel then runs."""
+    from comp_inference_amd import _lib
+
+    lib = _lib.lib()
+    assert lib.ci_fused_linear_wide_rows(1) == 0 and lib.ci_fused_linear_wide_rows(0) == 1
+    assert lib.ci_fused_linear_wide_rows(0) == 0
+    K, N = 4096, 256
+    size = lambda M: lib.ci_fused_linear_workspace_bytes(M, K, N, 1024, 32, 0)  # noqa: E731
+    # (sized for the one-thread-per-stream plan too: 8 partial sums per output, then the fragment copy)
+    want = lambda M, groups: 8 * M * N * 4 + groups * 32 * K * 2  # noqa: E731
+    assert size(64) == want(64, 2)
+    assert size(65) == want(65, 4) and size(128) == want(128, 4)
+    assert size(129) == want(129, 8) and size(256) == want(256, 8)
+    assert size(257) == want(257, 16)
