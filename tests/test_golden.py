@@ -29,6 +29,10 @@ def test_oracle_reproduces_fixture(oracle):
     assert np.array_equal(t.stream, G["ilp2_stream"]) and np.array_equal(t.states, G["ilp2_states"])
     assert np.array_equal(t.sizes, G["ilp2_sizes"]) and np.array_equal(t.tile_offsets, G["ilp2_tile_offsets"])
     assert np.array_equal(t.tile_max_lens, G["ilp2_tile_max_lens"])
+    o = oracle.encode_tiled_one(exp, freq, cdf, TH, TW)
+    assert np.array_equal(o.stream, G["one_stream"]) and np.array_equal(o.states, G["one_states"])
+    assert np.array_equal(o.sizes, G["one_sizes"]) and np.array_equal(o.tile_offsets, G["one_tile_offsets"])
+    assert np.array_equal(o.tile_max_lens, G["one_tile_max_lens"])
     d = oracle.encode_tiled_dense(exp, freq, cdf, TH, TW)
     assert np.array_equal(d.stream, G["dense_stream"]) and np.array_equal(d.states, G["dense_states"])
     assert np.array_equal(d.stream_offsets, G["dense_stream_offsets"])
@@ -44,6 +48,13 @@ def test_decoders_read_fixture(oracle):
                                                    G["ilp2_tile_offsets"], G["ilp2_tile_max_lens"], K, N, TH, TW), exp)
     assert np.array_equal(pyref.decode_tiled(G["ilp2_stream"], G["ilp2_states"], G["tables"], G["slot_map"],
                                              G["ilp2_tile_offsets"], G["ilp2_tile_max_lens"], K, N, TH, TW), exp)
+    one = (G["one_stream"], G["one_states"], G["tables"], G["slot_map"], G["one_tile_offsets"], G["one_tile_max_lens"])
+    assert np.array_equal(oracle.decode_tiled_one(*one, K, N, TH, TW), exp)
+    assert np.array_equal(pyref.decode_tiled(*one, K, N, TH, TW, halves=1), exp)
+    # the same streams as the dense layout holds, at other addresses: states and lengths agree stream for stream
+    assert np.array_equal(G["one_states"], G["dense_states"])
+    assert np.array_equal(G["one_sizes"],
+                          np.diff(np.concatenate([G["dense_stream_offsets"], [G["dense_stream"].size]])))
     sizes = np.diff(np.concatenate([G["dense_stream_offsets"], [G["dense_stream"].size]])).astype(np.uint32)
     assert np.array_equal(oracle.decode_tiled_dense(G["dense_stream"], G["dense_states"], G["tables"], G["slot_map"],
                                                     G["dense_stream_offsets"], sizes, K, N, TH, TW), exp)
