@@ -151,3 +151,25 @@ def test_one_stream_transposed_linear(oracle):
                                                            _t32(dense.stream_offsets).to(dev), _t32(dense.sizes).to(dev),
                                                            th, tw, man, workspace=None)
     assert torch.equal(got, same)
+
+
+def test_one_stream_encoder_and_decoder_on_the_committed_fixture():
+    import os
+
+    from comp_inference_amd import ccore, get_rans_lut, rans_decomp_tiled_one_stream
+
+    G = np.load(os.path.join(os.path.dirname(__file__), "golden", "small_formats.npz"))
+    K, N, TH, TW = (int(v) for v in G["shape"])
+    exp = torch.from_numpy(G["exp"])
+    f, c = get_rans_lut(exp)
+    t = ccore.RansManager(exp.numel()).compress_tiled_one_stream(exp, f, c, TH, TW)
+    assert np.array_equal(t.stream.numpy(), G["one_stream"])
+    assert np.array_equal(_np32(t.states), G["one_states"]) and np.array_equal(_np32(t.output_sizes), G["one_sizes"])
+    assert np.array_equal(_np32(t.tile_offsets), G["one_tile_offsets"])
+    assert np.array_equal(_np32(t.tile_max_lens), G["one_tile_max_lens"])
+    dev = "cuda"
+    out = rans_decomp_tiled_one_stream(torch.from_numpy(G["one_stream"]).to(dev), _t32(G["one_states"]).to(dev),
+                                       _t32(G["tables"]).to(dev), torch.from_numpy(G["slot_map"]).to(dev), (K, N),
+                                       _t32(G["one_tile_offsets"]).to(dev), _t32(G["one_tile_max_lens"]).to(dev),
+                                       tile_k=TH, tile_n=TW, mantissas=torch.from_numpy(G["man_tiled"]).to(dev))
+    assert np.array_equal(out.cpu().view(torch.int16).numpy().view(np.uint16), G["w_bits"])
