@@ -48,3 +48,27 @@ def test_one_row_of_x_on_sixteen_wavefronts(oracle, V, H, segments):
     assert torch.equal(ci.fused_rans_linear_transposed(x3, *args, checkpoints=ck, segments=segments, max_window_rows=max_rows),
                        ci.fused_rans_linear_transposed(x3, *args))
     assert torch.equal(ci.fused_rans_linear_transposed(x, *args, checkpoints=ck, segments=segments), whole)
+
+
+def test_the_module_takes_the_kernel_when_segments_are_switched_on():
+    import comp_inference_amd as ci
+
+    V, H = 4096, 128
+    emb = torch.nn.Embedding(V, H).to(torch.bfloat16)
+    table = emb.weight.detach().clone()
+    ci.rans_compress_module_weight(emb, tile_height=1024, tile_width=32, transpose_weight=False)
+    re = ci.RansEmbedding.from_compressed(emb)
+    head = ci.RansLMHead(H, V)
+    head.tie_to(re)
+    h = make_x(1, H, seed=3)
+    whole = head(h.cuda())
+    assert torch.allclose(whole.float().cpu(), h.float() @ table.float().t(), atol=ATOL, rtol=RTOL)
+    head.segments = "auto"
+    ck, segs, max_rows, slot_table = head._derived(torch.device("cuda", 0))
+    assert segs > 1 and 0 < max_rows <= 112 and slot_table.numel() == 32768
+    assert torch.equal(head(h.cuda()), whole)
+    h3 = make_x(3, H, seed=4)
+    head.segments = 1
+    whole3 = head(h3.cuda())
+    head.segments = "auto"
+    assert torch.equal(head(h3.cuda()), whole3)
