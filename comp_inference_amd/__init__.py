@@ -50,6 +50,7 @@ from .rans_hip import (
 )
 from .transposed_linear_hip import (
     fused_rans_linear_transposed,
+    head_matrix_sums,
     fused_rans_linear_transposed_one_stream,
     fused_rans_linear_transposed_triton,
     fused_rans_linear_transposed_triton_uncoalesced,

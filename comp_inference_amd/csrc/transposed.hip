@@ -256,6 +256,20 @@ constexpr uint32_t kTrWinBytes = kTrWinRows * 64;
 constexpr int kTrWinPieces = (int)(kTrWinBytes / 1024);  // 16 bytes per lane each
 static_assert(kTrWinBytes % 1024 == 0 && kSlotTableBytes + kTrSegWaves * kTrWinBytes <= kLdsLimit, "windows exceed the LDS");
 
+// kMatrix: the sums across the 32 lanes of a half go through the matrix pipe instead of lane exchanges.  A
+// block's weight fragment A[h][k] (k = the block's eight rows of the top half, then of the bottom half) times a
+// one-hot B[k][n] is that fragment transposed into the accumulator: after the blocks 2p and 2p + 1,
+// D[h][n] = W[row][h] with n < 16 the top half's rows 16 p + n and n >= 16 the bottom half's rows 16 p + n - 16,
+// h down the registers (register r of lane l: h = 8 (r / 4) + 4 (l / 32) + r % 4, n = l % 32).  Sixteen
+// multiply-adds against the lane's sixteen values of x give half a row sum per lane, the other half sits 32
+// lanes away: one v_permlane32_swap and an add over two such pairs of blocks leave 32 consecutive rows of each
+// half in the 64 lanes, stored as whole lines.  11 instead of 15 vector instructions per symbol and no chain of
+// lane exchanges; the order of the sum over h differs from the other kernels' (not bit-identical to them), and
+// 0 x Inf = NaN: a weight with exponent 255 spoils the 31 other rows of its group, so this is for finite weights.
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x16v __attribute__((ext_vector_type(16)));
+
+template <bool kMatrix>
 __device__ __forceinline__ void trans_one_segment(const TransArgs &a, uint32_t tile, uint32_t seg, uint8_t *stage, int lane) {
     const uint32_t tk = tile / a.tiles_n, tn = tile - tk * a.tiles_n;
     const uint32_t half = a.th / 2, seglen = a.seglen, hsel = lane / 32, c = lane % 32;
@@ -304,50 +318,100 @@ __device__ __forceinline__ void trans_one_segment(const TransArgs &a, uint32_t t
     st.q = (uint32_t)(uintptr_t)stage + (uint32_t)(rel * 64 + lane);
     st.n1 = rel >= 0 ? stage[rel * 64 + lane] : 0;  // (a wavefront's LDS operations complete in order)
 
-    uint32_t xb[1] = {a.x[h]};  // bf16 bits of x[0, h]
     const uint8_t *man_seg = a.man_tiled + (size_t)tile * a.th * 32 + (size_t)(hsel * half + seg * seglen) * 32;
-    float *dst = a.partial + (size_t)tn * a.V + v0;  // (M = 1)
     const uint32_t man_sel = 0x04040000u + (c & 3u) * 0x01010101u;
     const uint32_t *mrow = reinterpret_cast<const uint32_t *>(man_seg + (c & ~3u));  // + 8 dwords per row
     const uint32_t nblk = seglen / 8;
     uint32_t mcur[8], mnext[8];
-    float keep[1] = {0.f};
 #pragma unroll
     for (int r = 0; r < 8; ++r) mcur[r] = mrow[r * 8];
-    for (uint32_t blk = 0; blk < nblk; ++blk) {
-        // rows of the next block (the last block re-reads its own: stays inside the segment)
-        const uint32_t *nrow = mrow + (size_t)(blk + 1 < nblk ? blk + 1 : blk) * 64;
+    if constexpr (kMatrix) {
+        // this lane's sixteen values of x (the h of its accumulator registers) and its one-hot operands
+        float xv[16];
 #pragma unroll
-        for (int r = 0; r < 8; ++r) mnext[r] = nrow[r * 8];
-        uint32_t w[4];
-        decode8_weights_asm(st, mcur, man_sel, w, 64);
-        trans_emit8_lines<1>(w, xb, 1, a.V, dst, blk, keep, lane);
+        for (int r = 0; r < 16; ++r)
+            xv[r] = __uint_as_float((uint32_t)a.x[tn * 32 + 8 * (r / 4) + 4 * hsel + r % 4] << 16);
+        const uint32_t n = c, jstar = n % 8;
+        const u32x4 one = {jstar / 2 == 0 ? (jstar & 1 ? 0x3F800000u : 0x3F80u) : 0u,
+                           jstar / 2 == 1 ? (jstar & 1 ? 0x3F800000u : 0x3F80u) : 0u,
+                           jstar / 2 == 2 ? (jstar & 1 ? 0x3F800000u : 0x3F80u) : 0u,
+                           jstar / 2 == 3 ? (jstar & 1 ? 0x3F800000u : 0x3F80u) : 0u};
+        const u32x4 none = {0u, 0u, 0u, 0u};
+        const bool mine = n / 16 == hsel;  // this lane's column n takes rows of this lane's half k = 8 hsel + j
+        const u32x4 hot0 = mine && (n % 16) / 8 == 0 ? one : none, hot1 = mine && (n % 16) / 8 == 1 ? one : none;
+        // rows [16 P + L % 16] of half L / 16 (L = lane % 32, P = lane / 32) of every group of 32 rows
+        float *dst = a.partial + (size_t)tn * a.V + tk * a.th + (c / 16) * half + seg * seglen + 16 * hsel + c % 16;
+        // one block: the next block's sign|mantissa dwords on their way, eight steps, the weights as one operand
+        auto block = [&](uint32_t blk) {
+            const uint32_t *nrow = mrow + (size_t)(blk + 1 < nblk ? blk + 1 : blk) * 64;
 #pragma unroll
-        for (int r = 0; r < 8; ++r) mcur[r] = mnext[r];
+            for (int r = 0; r < 8; ++r) mnext[r] = nrow[r * 8];
+            uint32_t w[4];
+            decode8_weights_asm(st, mcur, man_sel, w, 64);
+            // (w[3] is written two instructions before the statement ends: a matrix instruction may read it no sooner
+            // than two wait states later, and the compiler does not see inside the statement)
+            asm volatile("s_nop 1" : "+v"(w[3]));
+#pragma unroll
+            for (int r = 0; r < 8; ++r) mcur[r] = mnext[r];
+            const u32x4 wv = {w[0], w[1], w[2], w[3]};
+            return __builtin_bit_cast(bf16x8_t, wv);
+        };
+        // two blocks: 16 rows of each half transposed into the accumulator, then this lane's half of their sums
+        auto pair_sums = [&](uint32_t blk) {
+            const f32x16v zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            f32x16v acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(block(blk), __builtin_bit_cast(bf16x8_t, hot0), zero, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(block(blk + 1), __builtin_bit_cast(bf16x8_t, hot1), acc, 0, 0, 0);
+            float sum = acc[0] * xv[0];
+#pragma unroll
+            for (int r = 1; r < 16; ++r) sum = __builtin_fmaf(acc[r], xv[r], sum);
+            return sum;
+        };
+        for (uint32_t g = 0; g < nblk / 4; ++g) {  // (seglen is a multiple of 32: whole groups of four blocks)
+            const float first = pair_sums(4 * g), second = pair_sums(4 * g + 2);
+            const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(first), __float_as_uint(second), false, false);
+            dst[g * 32] = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
+        }
+    } else {
+        uint32_t xb[1] = {a.x[h]};  // bf16 bits of x[0, h]
+        float *dst = a.partial + (size_t)tn * a.V + v0;  // (M = 1)
+        float keep[1] = {0.f};
+        for (uint32_t blk = 0; blk < nblk; ++blk) {
+            // rows of the next block (the last block re-reads its own: stays inside the segment)
+            const uint32_t *nrow = mrow + (size_t)(blk + 1 < nblk ? blk + 1 : blk) * 64;
+#pragma unroll
+            for (int r = 0; r < 8; ++r) mnext[r] = nrow[r * 8];
+            uint32_t w[4];
+            decode8_weights_asm(st, mcur, man_sel, w, 64);
+            trans_emit8_lines<1>(w, xb, 1, a.V, dst, blk, keep, lane);
+#pragma unroll
+            for (int r = 0; r < 8; ++r) mcur[r] = mnext[r];
+        }
     }
 }
 
-// grid: at most one workgroup per CU; workgroup j's wavefront w takes the items w * gridDim + j, + 16 gridDim, ...
-// of the tiles below a.first_tile (item = tile * segs + segment).
-__global__ __launch_bounds__(kTrSegWaves *kWave) void trans32_seg_kernel(TransArgs a) {
+// grid: at most one workgroup per CU; workgroup j's wavefront w takes the items w * gridDim + j, + waves * gridDim, ...
+// of the tiles below a.first_tile (item = tile * segs + segment).  kMatrix: see trans_one_segment (the accumulator
+// and the lane's values of x fit the 128 registers of sixteen wavefronts too).
+constexpr int kTrMatWaves = 16;
+template <bool kMatrix>
+__global__ __launch_bounds__((kMatrix ? kTrMatWaves : kTrSegWaves) * kWave) void trans32_seg_kernel(TransArgs a) {
+    constexpr int kWaves = kMatrix ? kTrMatWaves : kTrSegWaves;
     extern __shared__ __align__(16) uint8_t lds[];
     const int lane = threadIdx.x % kWave;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWave));
     if (a.slot_table) {
         const u32x4 *src = reinterpret_cast<const u32x4 *>(a.slot_table);
         u32x4 *dst = reinterpret_cast<u32x4 *>(lds);
-        const u32x4 e0 = src[threadIdx.x * 2], e1 = src[threadIdx.x * 2 + 1];
-        dst[threadIdx.x * 2] = e0;
-        dst[threadIdx.x * 2 + 1] = e1;
+        for (uint32_t e = threadIdx.x; e < kSlotTableBytes / 16; e += kWaves * kWave) dst[e] = src[e];
     } else {
-        build_slot_table_x8(reinterpret_cast<uint2 *>(lds), a.tables, a.slot_map, threadIdx.x, kTrSegWaves * kWave);
+        build_slot_table_x8(reinterpret_cast<uint2 *>(lds), a.tables, a.slot_map, threadIdx.x, kWaves * kWave);
     }
     __syncthreads();
     uint8_t *stage = lds + kSlotTableBytes + (size_t)wave * kTrWinBytes;
     const uint64_t n_items = (uint64_t)a.first_tile * a.segs;
-    for (uint64_t item = (uint64_t)wave * gridDim.x + blockIdx.x; item < n_items; item += (uint64_t)kTrSegWaves * gridDim.x) {
+    for (uint64_t item = (uint64_t)wave * gridDim.x + blockIdx.x; item < n_items; item += (uint64_t)kWaves * gridDim.x) {
         const uint32_t tile = (uint32_t)(item / a.segs), seg = (uint32_t)(item - (uint64_t)tile * a.segs);
-        trans_one_segment(a, tile, seg, stage, lane);
+        trans_one_segment<kMatrix>(a, tile, seg, stage, lane);
     }
 }
 
@@ -418,6 +482,13 @@ extern "C" size_t ci_fused_linear_transposed_workspace_bytes(uint32_t M, uint32_
     const uint32_t rows = M < (uint32_t)kTrRows ? M : (uint32_t)kTrRows;
     return (size_t)ceil_div(H, tile_width) * rows * V * sizeof(float);
 }
+
+// Whether the sixteen-wavefront kernel for one row of x sums across lanes on the matrix pipe (trans_one_segment).
+// Another order of the sum over the hidden dimension (not bit-identical to the other kernels), finite weights only;
+// off until it has been measured.
+static std::atomic<int> g_matrix_sums{0};
+
+extern "C" int ci_fused_linear_transposed_matrix_sums(int enable) { return g_matrix_sums.exchange(enable ? 1 : 0); }
 
 static int transposed_impl(const uint16_t *d_x, uint32_t M, uint32_t H, uint32_t V, uint32_t x_stride,
                            const uint8_t *d_stream, uint64_t stream_len, const uint32_t *d_states,
@@ -494,9 +565,15 @@ static int transposed_impl(const uint16_t *d_x, uint32_t M, uint32_t H, uint32_t
             a.seglen = th / 2 / segments;
             a.first_tile = whole_rows * a.tiles_n;
             const uint64_t items = (uint64_t)a.first_tile * segments;
-            CI_ALLOW_FULL_LDS(trans32_seg_kernel);
-            const dim3 grid((uint32_t)(items < cus ? items : cus)), block(kTrSegWaves * kWave);
-            hipLaunchKernelGGL(trans32_seg_kernel, grid, block, kSlotTableBytes + kTrSegWaves * kTrWinBytes, s, a);
+            CI_ALLOW_FULL_LDS(trans32_seg_kernel<false>);
+            CI_ALLOW_FULL_LDS(trans32_seg_kernel<true>);
+            const dim3 grid((uint32_t)(items < cus ? items : cus));
+            if (g_matrix_sums.load(std::memory_order_relaxed))
+                hipLaunchKernelGGL(trans32_seg_kernel<true>, grid, dim3(kTrMatWaves * kWave),
+                                   kSlotTableBytes + kTrMatWaves * kTrWinBytes, s, a);
+            else
+                hipLaunchKernelGGL(trans32_seg_kernel<false>, grid, dim3(kTrSegWaves * kWave),
+                                   kSlotTableBytes + kTrSegWaves * kTrWinBytes, s, a);
             CI_LAUNCH_CHECK("trans32_seg_kernel");
             a.ckpt = nullptr;
             a.segs = 1;

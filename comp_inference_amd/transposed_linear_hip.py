@@ -20,6 +20,15 @@ from .linear_hip import _Scratch, _prep_x
 DECODE_ONCE_ABOVE_ROWS = 4
 
 
+def head_matrix_sums(enable: bool) -> bool:
+    """One row of x on a weight with decoder checkpoints (the sixteen-wavefront kernel): with `enable` the sums over
+    the hidden dimension are formed on the matrix pipe instead of by lane exchanges -- fewer vector instructions per
+    symbol, another order of the sum (same tolerance, not bit-identical to the other kernels), finite weights only
+    (0 x Inf = NaN would spoil the other rows of a group of 32).  Process-wide, off by default; returns the previous
+    setting."""
+    return bool(lib().ci_fused_linear_transposed_matrix_sums(1 if enable else 0))
+
+
 def _run(x, compressed_data, initial_states, tables, slot_map, weight_shape, meta0, meta1, tile_k, tile_n,
          mantissas, bias, out, dense: bool, checkpoints=None, segments: int = 1, max_window_rows: int = 0,
          slot_table=None, one: bool = False):

@@ -521,6 +521,15 @@ int ci_fused_linear_tiled_noalloc(const ci_tiled_weight *w, const uint16_t *d_x,
  * decodes once per 16 rows (comp_inference/linear_triton.py:250-266). */
 int ci_fused_linear_wide_rows(int enable);
 
+/* One row of x against a weight with decoder checkpoints (the sixteen-wavefront kernel of
+ * ci_fused_linear_transposed_tiled): with `enable` non-zero the sums over the hidden dimension are formed on the
+ * matrix pipe -- a block's weights transposed by a matrix instruction against a one-hot operand, then multiply-adds
+ * inside a lane -- instead of by lane exchanges.  The sum runs in another order (results within the same
+ * tolerance, not bit-identical to the other kernels) and 0 x Inf = NaN: a weight with exponent 255 spoils the
+ * other rows of its group of 32, so this is for finite weights.  Process-wide, off by default; returns the
+ * previous setting.  No counterpart in the reference. */
+int ci_fused_linear_transposed_matrix_sums(int enable);
+
 /* ---------------------------------------------------------------------------------------
  * Verification aids: the contraction of the fused kernels applied to a plain (uncompressed) bf16
  * weight.  No counterpart in the reference, whose tests compare the fused kernels with

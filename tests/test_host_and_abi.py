@@ -393,6 +393,8 @@ def test_wide_rows_switch_and_fragment_sizes():
     lib = _lib.lib()
     assert lib.ci_fused_linear_wide_rows(1) == 0 and lib.ci_fused_linear_wide_rows(0) == 1
     assert lib.ci_fused_linear_wide_rows(0) == 0
+    assert lib.ci_fused_linear_transposed_matrix_sums(1) == 0 and lib.ci_fused_linear_transposed_matrix_sums(0) == 1
+    assert lib.ci_fused_linear_transposed_matrix_sums(0) == 0
     K, N = 4096, 256
     size = lambda M: lib.ci_fused_linear_workspace_bytes(M, K, N, 1024, 32, 0)  # noqa: E731
     # (sized for the one-thread-per-stream plan too: 8 partial sums per output, then the fragment copy)

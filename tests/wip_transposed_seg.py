@@ -72,3 +72,41 @@ def test_the_module_takes_the_kernel_when_segments_are_switched_on():
     whole3 = head(h3.cuda())
     head.segments = "auto"
     assert torch.equal(head(h3.cuda()), whole3)
+
+
+@pytest.mark.parametrize("V,H,segments", [(2304, 128, 2), (4096, 64, 4), (1024, 96, 8), (8192, 256, 2)])
+def test_sums_on_the_matrix_pipe(oracle, V, H, segments):
+    """`head_matrix_sums`: another order of the sum over the hidden dimension, so the bar is the operator's tolerance
+    against torch.matmul, a tight bound against the float64 product (every output is 16 + 16 fp32 multiply-adds of
+    exact bf16 products), the same bits on a second call, and the other kernel's answer back once switched off."""
+    import comp_inference_amd as ci
+    from comp_inference_amd import _lib
+
+    th = 1024
+    w = make_weight_kn(H, V, seed=V + H + 1)
+    enc, man = oracle.compress_bf16(bf16_bits(w), th, 32)
+    dev = torch.device("cuda", 0)
+    t = [torch.from_numpy(enc.stream).to(dev), _t32(enc.states).to(dev), _t32(enc.tables).to(dev),
+         torch.from_numpy(enc.slot_map).to(dev), _t32(enc.tile_offsets).to(dev), _t32(enc.tile_max_lens).to(dev),
+         torch.from_numpy(man).to(dev)]
+    args = (t[0], t[1], t[2], t[3], (V, H), t[4], t[5], th, 32, t[6])
+    x = make_x(1, H, seed=9).to(dev)
+    ck = ci.build_checkpoints(t[0], t[1], t[2], t[3], (V, H), t[4], t[5], th, 32, segments)
+    rows = torch.zeros(1, dtype=torch.int32, device=dev)
+    desc = _lib.tiled_weight(V, H, th, 32, t[0], t[1], t[2], t[3], t[4], t[5], None, ck, segments)
+    _lib.check(_lib.lib().ci_max_window_rows(C.byref(desc), _lib.ptr(rows), _lib.stream_handle(dev)))
+    kw = dict(checkpoints=ck, segments=segments, max_window_rows=int(rows.item()))
+    lanes = ci.fused_rans_linear_transposed(x, *args, **kw)
+    assert ci.head_matrix_sums(True) is False
+    try:
+        got = ci.fused_rans_linear_transposed(x, *args, **kw)
+        again = ci.fused_rans_linear_transposed(x, *args, **kw)
+    finally:
+        assert ci.head_matrix_sums(False) is True
+    assert torch.equal(got, again)
+    want64 = (x.double().cpu() @ w.double().t())
+    assert torch.allclose(got.float().cpu(), want64.float(), atol=ATOL, rtol=RTOL)
+    # fp32 sums of at most H exact products, rounded once to bf16: within a bf16 step of the exact value
+    scale = (x.double().cpu().abs() @ w.double().abs().t())
+    assert ((got.double().cpu() - want64).abs() <= scale * 2.0 ** -8 + 1e-30).all()
+    assert torch.equal(ci.fused_rans_linear_transposed(x, *args, **kw), lanes)
