@@ -74,6 +74,23 @@ def test_every_layout_round_trips(oracle, case):
                                                     den.stream_offsets, den.sizes, K, N, th, tw), sym)
     assert den.stream.size == int(den.sizes.astype(np.int64).sum())
 
+    # one stream per column in tile bodies: the dense layout's streams (same states, same lengths) packed like
+    # the default layout's (bottom-aligned rows of tw bytes, offsets = scan of depth * tw)
+    one = _encode(oracle.encode_tiled_one, sym, f, c, th, tw)
+    if one is not None:
+        assert np.array_equal(one.states, den.states) and np.array_equal(one.sizes, den.sizes)
+        depth = one.tile_max_lens.astype(np.int64)
+        assert np.array_equal(depth, one.sizes.reshape(-1, tw).max(1))
+        assert np.array_equal(one.tile_offsets.astype(np.int64), np.concatenate(([0], np.cumsum(depth * tw)[:-1])))
+        assert one.stream.size == int((depth * tw).sum())
+        dec1, end1, left1 = oracle.decode_tiled_one(one.stream, one.states, one.tables, one.slot_map, one.tile_offsets,
+                                                    one.tile_max_lens, K, N, th, tw, want_end=True)
+        assert np.array_equal(dec1, sym) and (end1 == L).all()
+        assert np.array_equal(left1.astype(np.int64), np.repeat(depth, tw) - one.sizes - 1)
+        if K * N <= 2048:
+            assert np.array_equal(pyref.decode_tiled(one.stream, one.states, one.tables, one.slot_map, one.tile_offsets,
+                                                     one.tile_max_lens, K, N, th, tw, halves=1), sym)
+
     assert np.array_equal(oracle.decode_flat_segmented(flat.stream, flat.states, flat.sizes, flat.tables,
                                                        flat.slot_map, K, N), sym)
 
