@@ -67,19 +67,5 @@ def build(force: bool = False, verbose: bool = False) -> str:
     return LIB_PATH
 
 
-MICROBENCH_SRC = os.path.join(CSRC, "microbench", "step_rate.hip")
-MICROBENCH_BIN = os.path.join(PKG_DIR, "step_rate_bench")
-
-
-def build_microbench() -> str:
-    """The step-rate microbenchmark (csrc/microbench/step_rate.hip): a stand-alone program, not part of the library."""
-    subprocess.check_call([HIPCC, "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
-                           "-packed-fp32-ops", MICROBENCH_SRC, "-o", MICROBENCH_BIN], stderr=subprocess.DEVNULL)
-    return MICROBENCH_BIN
-
-
 if __name__ == "__main__":
-    if "--microbench" in sys.argv:
-        print(build_microbench())
-    else:
-        print(build(force="--force" in sys.argv, verbose=True))
+    print(build(force="--force" in sys.argv, verbose=True))
