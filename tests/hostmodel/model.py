@@ -1,0 +1,225 @@
+"""Python side of the host model: loads libci_hostmodel.so (the library's own sources compiled for the CPU model
+of a gfx950 workgroup, tests/hostmodel/sim.h), hands it arrays that end at an inaccessible page, and reports what
+the model saw.  numpy only.  Test infrastructure.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import pickle
+import sys
+import traceback
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(os.path.dirname(HERE))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+CI_SLOT_TABLE_BYTES = 32768
+
+
+class TiledWeight(C.Structure):
+    """ci_tiled_weight (include/comp_inference_hip.h)."""
+    _fields_ = [("K", C.c_uint32), ("N", C.c_uint32), ("tile_height", C.c_uint32), ("tile_width", C.c_uint32),
+                ("d_stream", C.c_void_p), ("stream_len", C.c_uint64),
+                ("d_states", C.c_void_p), ("n_states", C.c_uint64),
+                ("d_tables", C.c_void_p), ("d_slot_map", C.c_void_p),
+                ("d_tile_offsets", C.c_void_p), ("d_tile_max_lens", C.c_void_p), ("n_tiles", C.c_uint64),
+                ("d_man_tiled", C.c_void_p), ("man_len", C.c_uint64),
+                ("d_checkpoints", C.c_void_p), ("checkpoint_bytes", C.c_uint64), ("segments", C.c_uint32),
+                ("d_slot_table", C.c_void_p), ("slot_table_bytes", C.c_uint64), ("max_window_rows", C.c_uint32)]
+
+
+class DecodeItem(C.Structure):
+    """ci_decode_item."""
+    _fields_ = [("d_stream", C.c_void_p), ("stream_len", C.c_uint64), ("d_states", C.c_void_p),
+                ("d_tables", C.c_void_p), ("d_slot_map", C.c_void_p), ("d_tile_offsets", C.c_void_p),
+                ("d_tile_max_lens", C.c_void_p), ("K", C.c_uint32), ("N", C.c_uint32), ("tile_height", C.c_uint32),
+                ("tile_width", C.c_uint32), ("d_out_exp", C.c_void_p), ("d_checkpoints", C.c_void_p),
+                ("segments", C.c_uint32)]
+
+
+class Dev:
+    """An array in the model's checked memory."""
+
+    def __init__(self, ptr: int, shape, dtype):
+        self.ptr, self.shape, self.dtype = ptr, tuple(shape), np.dtype(dtype)
+
+    @property
+    def nbytes(self) -> int:
+        return int(np.prod(self.shape, dtype=np.int64)) * self.dtype.itemsize
+
+    @property
+    def p(self) -> C.c_void_p:
+        return C.c_void_p(self.ptr if self.nbytes else 0)
+
+    def get(self) -> np.ndarray:
+        out = np.empty(self.shape, self.dtype)
+        if self.nbytes:
+            C.memmove(out.ctypes.data, self.ptr, self.nbytes)
+        return out
+
+
+class ModelError(AssertionError):
+    pass
+
+
+class Model:
+    def __init__(self, cus: int = 8, end_at_guard: bool = True):
+        from tests.hostmodel import build
+
+        self.lib = C.CDLL(build.build())
+        L = self.lib
+        L.sim_alloc.restype = C.c_void_p
+        L.sim_alloc.argtypes = [C.c_size_t, C.c_int]
+        L.sim_violation.restype = C.c_char_p
+        L.sim_launch_name.restype = C.c_char_p
+        L.sim_asm_instructions.restype = C.c_uint64
+        L.ci_last_error.restype = C.c_char_p
+        for f in ("ci_encode_scratch_bytes", "ci_fused_linear_workspace_bytes", "ci_fused_embedding_workspace_bytes",
+                  "ci_fused_linear_transposed_workspace_bytes", "ci_fused_linear_workspace_bytes_segmented",
+                  "ci_checkpoint_bytes", "ci_fused_embedding_workspace_bytes_segmented"):
+            getattr(L, f).restype = C.c_size_t
+        L.ci_suggest_segments.restype = C.c_uint32
+        L.sim_init()
+        L.sim_set_cus(cus)
+        self.end_at_guard = 1 if end_at_guard else 0
+        L.sim_free_all()
+        L.sim_clear()
+
+    # ---- memory
+    def dev(self, a: np.ndarray) -> Dev:
+        a = np.ascontiguousarray(a)
+        d = self.empty(a.shape, a.dtype)
+        if a.nbytes:
+            C.memmove(d.ptr, a.ctypes.data, a.nbytes)
+        return d
+
+    def empty(self, shape, dtype) -> Dev:
+        shape = (shape,) if np.isscalar(shape) else tuple(shape)
+        n = int(np.prod(shape, dtype=np.int64)) * np.dtype(dtype).itemsize
+        ptr = self.lib.sim_alloc(n, self.end_at_guard)
+        assert ptr, "sim_alloc failed"
+        return Dev(ptr, shape, dtype)
+
+    def free_all(self) -> None:
+        self.lib.sim_free_all()
+
+    # ---- calls
+    def call(self, name: str, *args) -> None:
+        """Run an entry point; raise if it reports an error or the model saw a violation."""
+        rc = getattr(self.lib, name)(*args)
+        viol = self.violations()
+        if viol:
+            self.lib.sim_clear()
+            raise ModelError(f"{name}: " + "\n  ".join(viol[:8]))
+        if rc != 0:
+            raise RuntimeError(f"{name}: rc {rc}: {self.lib.ci_last_error().decode()}")
+
+    def violations(self) -> list[str]:
+        return [self.lib.sim_violation(i).decode() for i in range(self.lib.sim_violation_count())]
+
+    def launches(self) -> list[str]:
+        return [self.lib.sim_launch_name(i).decode() for i in range(self.lib.sim_launch_count())]
+
+    def clear(self) -> None:
+        self.lib.sim_clear()
+
+    # ---- a compressed weight as the entry points take it
+    def weight(self, enc, man_tiled, K: int, N: int, segments: int = 1, slot_table: bool = False,
+               window_rows: bool = False):
+        """ci_tiled_weight over copies of the oracle's arrays (and what keeps them alive).  `segments` > 1 builds
+        the decoder checkpoints with the library, `slot_table` the 32 KB table, `window_rows` the largest window."""
+        keep = dict(stream=self.dev(enc.stream), states=self.dev(enc.states), tables=self.dev(enc.tables),
+                    slot_map=self.dev(enc.slot_map), offs=self.dev(enc.tile_offsets), lens=self.dev(enc.tile_max_lens))
+        w = TiledWeight()
+        w.K, w.N, w.tile_height, w.tile_width = K, N, enc.tile_height, enc.tile_width
+        w.d_stream, w.stream_len = keep["stream"].p, enc.stream.size
+        w.d_states, w.n_states = keep["states"].p, enc.states.size
+        w.d_tables, w.d_slot_map = keep["tables"].p, keep["slot_map"].p
+        w.d_tile_offsets, w.d_tile_max_lens, w.n_tiles = keep["offs"].p, keep["lens"].p, enc.tile_offsets.size
+        if man_tiled is not None:
+            keep["man"] = self.dev(man_tiled)
+            w.d_man_tiled, w.man_len = keep["man"].p, man_tiled.size
+        w.segments = 1
+        if segments > 1:
+            nb = self.lib.ci_checkpoint_bytes(K, N, enc.tile_height, enc.tile_width, segments)
+            keep["ckpt"] = self.empty(nb // 8 * 2, np.uint32)
+            # (pointers go in as c_void_p objects: a plain int would be passed as a 32-bit C int)
+            self.call("ci_build_checkpoints_ilp2", keep["stream"].p, C.c_uint64(w.stream_len), keep["states"].p,
+                      keep["tables"].p, keep["slot_map"].p, keep["offs"].p, keep["lens"].p, K, N, enc.tile_height,
+                      enc.tile_width, segments, keep["ckpt"].p, C.c_size_t(nb), None)
+            w.d_checkpoints, w.checkpoint_bytes, w.segments = keep["ckpt"].p, nb, segments
+        if slot_table:
+            keep["slot_table"] = self.empty(CI_SLOT_TABLE_BYTES // 4, np.uint32)
+            self.call("ci_build_slot_table", keep["tables"].p, keep["slot_map"].p, keep["slot_table"].p, C.c_size_t(CI_SLOT_TABLE_BYTES), None)
+            w.d_slot_table, w.slot_table_bytes = keep["slot_table"].p, CI_SLOT_TABLE_BYTES
+        if window_rows:
+            keep["rows"] = self.empty(1, np.uint32)
+            self.call("ci_max_window_rows", C.byref(w), keep["rows"].p, None)
+            w.max_window_rows = int(keep["rows"].get()[0])
+        return w, keep
+
+
+# ---- synthetic inputs (the recipes of tests/helpers.py without torch) ---------------------------------------------
+def f32_to_bf16_bits(a: np.ndarray) -> np.ndarray:
+    u = np.ascontiguousarray(a, np.float32).view(np.uint32).astype(np.uint64)
+    return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+
+
+def bf16_bits_to_f32(b: np.ndarray) -> np.ndarray:
+    return (np.ascontiguousarray(b, np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def weight_bits(K: int, N: int, seed: int, std: float = 0.02) -> np.ndarray:
+    rng = np.random.default_rng(seed)
+    return f32_to_bf16_bits((rng.standard_normal((K, N), dtype=np.float32) * std))
+
+
+def x_bits(M: int, K: int, seed: int) -> np.ndarray:
+    rng = np.random.default_rng(seed)
+    return f32_to_bf16_bits(rng.standard_normal((M, K), dtype=np.float32))
+
+
+# ---- running a test body in a child process -----------------------------------------------------------------------
+def in_child(fn):
+    """Decorator: the test body runs in a forked child, so that a memory fault inside the model (which ends the
+    process with a message naming kernel, workgroup, thread and address) fails one test and not the test run."""
+    import functools
+
+    @functools.wraps(fn)
+    def wrapper(*args, **kwargs):
+        r, w = os.pipe()
+        sys.stdout.flush()
+        sys.stderr.flush()
+        pid = os.fork()
+        if pid == 0:
+            os.close(r)
+            code = 0
+            try:
+                fn(*args, **kwargs)
+                payload = pickle.dumps(None)
+            except BaseException:  # noqa: BLE001
+                payload = pickle.dumps(traceback.format_exc())
+                code = 1
+            with os.fdopen(w, "wb") as f:
+                f.write(payload)
+            sys.stdout.flush()
+            sys.stderr.flush()
+            os._exit(code)
+        os.close(w)
+        with os.fdopen(r, "rb") as f:
+            data = f.read()
+        _, status = os.waitpid(pid, 0)
+        if os.WIFSIGNALED(status):
+            raise AssertionError(f"the host-model child died of signal {os.WTERMSIG(status)}")
+        code = os.WEXITSTATUS(status)
+        if code == 70:
+            raise AssertionError("memory fault inside the host model (see the message on stderr)")
+        err = pickle.loads(data) if data else f"child exited with {code} and no report"
+        if err is not None:
+            raise AssertionError(err)
+
+    return wrapper
