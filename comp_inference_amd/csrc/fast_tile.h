@@ -225,6 +225,27 @@ __device__ __forceinline__ void stage_window_pair(uint8_t *stage, const uint8_t 
     }
 }
 
+// The window of ONE tile body for the sixteen-wavefront kernels that take both halves of a tile (fused linear, LM
+// head): rows [0, rows) of `src` (64 bytes a row) -> LDS as they lie, piece g = bytes [1024 g + 16 lane, + 16).  Every
+// lane loads every piece, from the window's first bytes where its own lie outside: loads without conditions can all
+// be in flight together.  rows <= kPairWinRows; nothing is read when rows == 0 (an empty body may end the stream).
+constexpr int kWinPieces = (int)(kPairWinRows * 64 / 1024);  // 16 bytes per lane each
+__device__ __forceinline__ void stage_window(uint8_t *stage, const uint8_t *__restrict__ src, uint32_t rows, int lane) {
+    const uint32_t bytes = rows * 64;
+    if (bytes == 0) return;
+    u32x4 w[kWinPieces];
+#pragma unroll
+    for (int g = 0; g < kWinPieces; ++g) {
+        const uint32_t o = (uint32_t)g * 1024 + lane * 16;
+        w[g] = *reinterpret_cast<const u32x4 *>(src + (o < bytes ? o : 0u));
+    }
+#pragma unroll
+    for (int g = 0; g < kWinPieces; ++g) {
+        const uint32_t o = (uint32_t)g * 1024 + lane * 16;
+        if (o < bytes) *reinterpret_cast<u32x4 *>(stage + o) = w[g];
+    }
+}
+
 // ---- assembly building blocks ----------------------------------------------------------------
 // Fixed temporaries (declared as clobbers by every user):
 //   v[72:73], v[74:75]  slot-table entries of the even / odd step of a pair

@@ -592,8 +592,7 @@ __global__ __launch_bounds__(kPersistWaves *kWave) void fused_linear32_resident_
 // cache lines of the next item's window and first sign|mantissa rows are touched, before the current
 // item's loop starts, so that between two items a wavefront waits for cache hits, not for HBM.
 constexpr int kSegWaves = 16;
-constexpr uint32_t kWinRows = 112;
-constexpr int kWinPieces = (int)(kWinRows * 64 / 1024);  // 16 bytes per lane each
+constexpr uint32_t kWinRows = kPairWinRows;
 constexpr uint32_t kWinBytes = kWinRows * 64;
 // Behind the windows: for up to kSmallM rows of x, the sums a wavefront hands over at the end of a job (32
 // tile columns per row of x), and two words of bookkeeping (wavefronts arrived, jobs added up).
@@ -677,24 +676,9 @@ __device__ __forceinline__ void seg_touch(const LinearArgs &a, const SegItem &it
                                                  (size_t)(hsel * half + seg * seglen + line * 4) * 32);
 }
 
-// The item's window, memory -> LDS as it lies (piece g = bytes [1024 g + 16 lane, + 16) of the window).
-// Every lane loads every piece, from the window's first bytes where its own lie outside: loads without
-// conditions can all be in flight together.
+// The item's window, memory -> LDS as it lies (stage_window).
 __device__ __forceinline__ void seg_stage(const LinearArgs &a, const SegItem &it, uint8_t *stage, int lane) {
-    const uint32_t bytes = it.rows * 64;
-    if (bytes == 0) return;
-    const uint8_t *src = a.stream + it.base + (size_t)it.lo * 64;
-    u32x4 w[kWinPieces];
-#pragma unroll
-    for (int g = 0; g < kWinPieces; ++g) {
-        const uint32_t o = (uint32_t)g * 1024 + lane * 16;
-        w[g] = *reinterpret_cast<const u32x4 *>(src + (o < bytes ? o : 0u));
-    }
-#pragma unroll
-    for (int g = 0; g < kWinPieces; ++g) {
-        const uint32_t o = (uint32_t)g * 1024 + lane * 16;
-        if (o < bytes) *reinterpret_cast<u32x4 *>(stage + o) = w[g];
-    }
+    stage_window(stage, a.stream + it.base + (size_t)it.lo * 64, it.rows, lane);
 }
 
 // One staged item through the hand-scheduled loop, accumulating into acc (and acc2 for x rows 32..63).

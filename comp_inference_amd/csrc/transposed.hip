@@ -251,9 +251,8 @@ __global__ __launch_bounds__(kPersistWaves *kWave) void trans32_kernel(TransArgs
 // item that does not qualify after all is left out rather than staged beyond its area.  Tiles of a short last
 // tile row go to trans32_kernel (first_tile).
 constexpr int kTrSegWaves = 16;
-constexpr uint32_t kTrWinRows = 112;
+constexpr uint32_t kTrWinRows = kPairWinRows;
 constexpr uint32_t kTrWinBytes = kTrWinRows * 64;
-constexpr int kTrWinPieces = (int)(kTrWinBytes / 1024);  // 16 bytes per lane each
 static_assert(kTrWinBytes % 1024 == 0 && kSlotTableBytes + kTrSegWaves * kTrWinBytes <= kLdsLimit, "windows exceed the LDS");
 
 // kMatrix: the sums across the 32 lanes of a half go through the matrix pipe instead of lane exchanges.  A
@@ -294,24 +293,18 @@ __device__ __forceinline__ void trans_one_segment(const TransArgs &a, uint32_t t
     const bool whole = __builtin_amdgcn_ballot_w64(v0 >= a.V || a.V - v0 < seglen || h >= a.H) == 0;
     const int32_t lo = max(wave_min_i32(row_end), 0), hi = wave_max_i32(row);
     const uint32_t rows = hi >= lo ? (uint32_t)(hi - lo + 1) : 0u;
-    if (!whole || rows == 0 || rows > kTrWinRows || seglen % 32 != 0) return;  // (promised not to happen)
-
-    // the window, memory -> LDS as it lies; every lane loads every piece (from the window's first bytes where its
-    // own lie outside), so that the loads are all in flight together
-    const uint8_t *src = a.stream + base + (size_t)lo * 64;
-    {
-        u32x4 w[kTrWinPieces];
-#pragma unroll
-        for (int g = 0; g < kTrWinPieces; ++g) {
-            const uint32_t o = (uint32_t)g * 1024 + lane * 16;
-            w[g] = *reinterpret_cast<const u32x4 *>(src + (o < rows * 64 ? o : 0u));
-        }
-#pragma unroll
-        for (int g = 0; g < kTrWinPieces; ++g) {
-            const uint32_t o = (uint32_t)g * 1024 + lane * 16;
-            if (o < rows * 64) *reinterpret_cast<u32x4 *>(stage + o) = w[g];
-        }
+    if (!whole || rows > kTrWinRows || seglen % 32 != 0) {
+        // Promised not to happen (the host sends whole tile rows of a weight whose largest window is known to fit).
+        // A descriptor that promised too much gets zeros for this item's rows -- wrong sums, as documented for an
+        // understated window, but never whatever an earlier launch left in the workspace, and nothing staged beyond
+        // the window area.
+        if (h < a.H && v0 < a.V)
+            for (uint32_t i = c; i < min(seglen, a.V - v0); i += 32) a.partial[(size_t)tn * a.V + v0 + i] = 0.f;
+        return;
     }
+    // the window, memory -> LDS as it lies (rows == 0: a body without bytes, e.g. a constant plane; nothing to stage,
+    // and the steps below never ask for a byte)
+    stage_window(stage, a.stream + base + (size_t)lo * 64, rows, lane);
     FastLane st;
     const int32_t rel = row - lo;  // this lane's next byte, in rows of the window (< 0: none left)
     st.X = state << 3;

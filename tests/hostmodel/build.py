@@ -29,10 +29,10 @@ LIB_PATH = os.path.join(HERE, "libci_hostmodel.so")
 CXX = os.environ.get("CI_HOSTMODEL_CXX", "/opt/rocm/llvm/bin/clang++")
 SOURCES = ["api.hip", "encode.hip", "decode.hip", "linear.hip", "embedding.hip", "transposed.hip", "legacy.hip"]
 CXXFLAGS = ["-std=c++17", "-O1", "-g", "-fPIC", "-fno-strict-aliasing", "-Wno-unused-value", "-Wno-unknown-attributes",
-            "-Wno-ignored-attributes", "-Wno-pass-failed"]
+            "-Wno-ignored-attributes", "-Wno-pass-failed", "-Wno-psabi"]
 
 # Functions after (and before) which the lanes of a wavefront read LDS bytes that other lanes wrote.
-LDS_HANDOVER = ["stage_commit", "stage_window_pair", "seg_stage", "trans_stage_window", "emb_stage"]
+LDS_HANDOVER = ["stage_commit", "stage_window_pair", "stage_window"]
 
 
 def _balanced(text: str, i: int, open_c: str = "(", close_c: str = ")") -> int:
@@ -164,7 +164,7 @@ def needs_build() -> bool:
     if not os.path.exists(LIB_PATH):
         return True
     built = os.path.getmtime(LIB_PATH)
-    deps = [os.path.join(CSRC, f) for f in os.listdir(CSRC)] + [os.path.join(HERE, f) for f in ("sim.cpp", "sim.h", "build.py")]
+    deps = [os.path.join(CSRC, f) for f in os.listdir(CSRC)] + [os.path.join(HERE, f) for f in ("sim.cpp", "sim.h", "build.py", "selftest.hip")]
     deps += [os.path.join(HERE, "hip", "hip_runtime.h"), os.path.join(ROOT, "include", "comp_inference_hip.h")]
     return any(os.path.getmtime(d) > built for d in deps)
 
@@ -174,8 +174,9 @@ def build(force: bool = False, verbose: bool = False) -> str:
         return LIB_PATH
     os.makedirs(OUT_DIR, exist_ok=True)
     procs, objs = [], []
-    for src in SOURCES:
-        pre = subprocess.run([CXX, "-E", "-x", "c++", "-std=c++17", "-I", HERE, "-I", CSRC, os.path.join(CSRC, src), "-o", "-"],
+    for src in SOURCES + ["selftest.hip"]:
+        path = os.path.join(HERE if src == "selftest.hip" else CSRC, src)
+        pre = subprocess.run([CXX, "-E", "-x", "c++", "-std=c++17", "-I", HERE, "-I", CSRC, path, "-o", "-"],
                              check=True, capture_output=True, text=True).stdout
         ii = os.path.join(OUT_DIR, src + ".ii")
         with open(ii, "w") as f:

@@ -67,7 +67,7 @@ class ModelError(AssertionError):
 
 
 class Model:
-    def __init__(self, cus: int = 8, end_at_guard: bool = True):
+    def __init__(self, cus: int = 8, end_at_guard: bool = True, schedule: int = 0):
         from tests.hostmodel import build
 
         self.lib = C.CDLL(build.build())
@@ -85,6 +85,8 @@ class Model:
         L.ci_suggest_segments.restype = C.c_uint32
         L.sim_init()
         L.sim_set_cus(cus)
+        L.sim_set_schedule.argtypes = [C.c_uint64]
+        L.sim_set_schedule(schedule)
         self.end_at_guard = 1 if end_at_guard else 0
         L.sim_free_all()
         L.sim_clear()

@@ -25,6 +25,7 @@ static int g_cus = 8;
 static const char *g_kernel = "(no kernel)";
 static uint64_t g_asm_instructions = 0;
 static bool g_abort_launch = false;
+static uint64_t g_schedule = 0;  // 0: wavefronts run in index order; else the seed of a new order every round
 
 struct Fiber;
 static Fiber *g_cur = nullptr;
@@ -1068,10 +1069,22 @@ static bool run_workgroup(uint32_t nthreads, const LaneCtx &proto) {
     }
     memset(g_lds, 0xCD, kLdsBytes);
     const uint32_t n_waves = (nthreads + 63) / 64;
+    uint32_t order[kMaxThreads / 64];
+    for (uint32_t i = 0; i < n_waves; ++i) order[i] = i;
     for (;;) {
         bool progress = false;
         uint32_t live = 0, at_wg = 0;
-        for (uint32_t wv = 0; wv < n_waves; ++wv) {
+        if (g_schedule)  // another order of the wavefronts every round: the kernels must not depend on it
+            for (uint32_t i = n_waves; i > 1; --i) {
+                g_schedule ^= g_schedule << 13;
+                g_schedule ^= g_schedule >> 7;
+                g_schedule ^= g_schedule << 17;
+                const uint32_t j = (uint32_t)(g_schedule % i), t = order[i - 1];
+                order[i - 1] = order[j];
+                order[j] = t;
+            }
+        for (uint32_t wi = 0; wi < n_waves; ++wi) {
+            const uint32_t wv = order[wi];
             const uint32_t lo = wv * 64, hi = lo + 64 < nthreads ? lo + 64 : nthreads;
             uint32_t live_w = 0, wait_wave = 0, wait_wg = 0;
             for (uint32_t t = lo; t < hi; ++t) {
@@ -1208,6 +1221,7 @@ extern "C" void sim_free_all(void) {
 }
 
 extern "C" void sim_set_cus(int n) { g_cus = n > 0 ? n : 1; }
+extern "C" void sim_set_schedule(uint64_t seed) { g_schedule = seed; }
 extern "C" int sim_violation_count(void) { return (int)g_viol.size(); }
 extern "C" const char *sim_violation(int i) { return i >= 0 && i < (int)g_viol.size() ? g_viol[i].c_str() : ""; }
 extern "C" void sim_clear(void) {
