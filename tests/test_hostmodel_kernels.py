@@ -1,0 +1,220 @@
+"""Every kernel of the library on the host model (tests/hostmodel): the library's own sources compiled for the CPU,
+the assembly statements interpreted, every address the interpreter forms checked against the exact extent of the
+arrays and every array ending at an inaccessible page.  Results are compared with the oracle (bit-exact decode,
+encode and gather; fused linears within 1e-2 of the fp32 product and bit for bit with the same contraction on the
+plain weight), and each case names the kernel it must have run.
+
+The kernels that have run on the GPU (decode, the fused linear's plans, the gather, the LM head) give the oracle's
+results here too, which is what ties the model to the hardware; the kernels that have not yet run on a GPU
+(embed_gather32_seg_kernel, fused_linear32_wide_kernel, trans32_seg_kernel with both kinds of sums, the entry points of
+the one-stream-per-column layout) are held to the same checks before their first launch."""
+import numpy as np
+import pytest
+
+from tests.hostmodel import cases
+from tests.hostmodel.model import Model, in_child, weight_bits, x_bits
+
+
+# ---- stand-alone decode -----------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("K,N,th,segs,merge,kernel", [
+    (2048, 128, 1024, 1, False, "decode_tiled32_persist_kernel<false>"),
+    (2048, 128, 1024, 1, True, "decode_tiled32_persist_kernel<true>"),
+    (2048, 128, 1024, 2, False, "decode_tiled32_seg_kernel<false>"),
+    (2048, 128, 1024, 4, True, "decode_tiled32_seg_kernel<true>"),
+    (1024, 96, 512, 1, False, "decode_tiled32_seg_kernel<false>"),   # low tiles: whole streams on sixteen wavefronts
+    (2048 + 300, 100, 1024, 2, False, "decode_tiled32_seg_kernel<false>"),  # ragged rows and columns, odd last tile
+    (3000, 70, 2048, 1, True, "decode_tiled32_persist_kernel<true>"),
+])
+@in_child
+def test_decode(K, N, th, segs, merge, kernel):
+    cases.decode(Model(cus=4), weight_bits(K, N, 1), th, segs, merge, expect_kernel=kernel)
+
+
+@pytest.mark.parametrize("kind", cases.KINDS)
+@in_child
+def test_decode_of_unusual_planes(kind):
+    rng = np.random.default_rng(11)
+    for segs in (1, 2, 8):
+        cases.decode(Model(cus=3), cases.weight_kind(rng, 2048, 96, kind), 1024, segs)
+
+
+@in_child
+def test_decode_batch_of_a_layer_in_one_launch():
+    """ci_decode_tiled_ilp2_batch: several tensors, with and without checkpoints, CUs divided among them."""
+    import ctypes as C
+
+    from oracle import rans_oracle as ro
+    from tests.hostmodel.model import DecodeItem
+
+    m = Model(cus=6)
+    shapes = [(1024, 128, 1), (2048, 64, 2), (1024, 256, 4), (1500, 40, 2)]
+    items = (DecodeItem * len(shapes))()
+    keep, outs, refs = [], [], []
+    for i, (K, N, segs) in enumerate(shapes):
+        bits = weight_bits(K, N, 20 + i)
+        enc, man = cases.compress(bits, 1024)
+        w, kp = m.weight(enc, None, K, N, segments=segs)
+        out = m.empty((K, N), np.uint8)
+        keep.append((w, kp))
+        outs.append(out)
+        refs.append(ro.split_bf16(bits)[0])
+        it = items[i]
+        it.d_stream, it.stream_len, it.d_states, it.d_tables, it.d_slot_map = w.d_stream, w.stream_len, w.d_states, w.d_tables, w.d_slot_map
+        it.d_tile_offsets, it.d_tile_max_lens, it.K, it.N, it.tile_height, it.tile_width = w.d_tile_offsets, w.d_tile_max_lens, K, N, 1024, 32
+        it.d_out_exp, it.d_checkpoints, it.segments = out.p, w.d_checkpoints, segs
+    m.clear()
+    m.call("ci_decode_tiled_ilp2_batch", items, len(shapes), None)
+    # one tensor has whole streams of 512 rows: the whole batch runs on the whole-stream kernel
+    assert m.launches() == ["decode_tiled32_persist_kernel<false>"], m.launches()
+    for out, ref in zip(outs, refs):
+        assert np.array_equal(out.get(), ref)
+
+
+# ---- fused linear -----------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("K,N,M,th,segs,prep,kernel", [
+    (2048, 128, 1, 1024, 1, False, "fused_linear32_kernel<1>"),
+    (2048, 128, 40, 1024, 1, False, "fused_linear32_kernel<2>"),
+    (2048, 128, 3, 1024, 2, False, "fused_linear32_seg_kernel<1, true>"),
+    (2048, 128, 3, 1024, 2, True, "fused_linear32_seg_kernel<1, false>"),    # M <= 4: sums handed over without a barrier
+    (2048, 128, 9, 1024, 4, True, "fused_linear32_seg_kernel<1, false>"),
+    (2048, 128, 64, 1024, 2, True, "fused_linear32_seg_kernel<2, false>"),
+    (4096, 64, 2, 1024, 8, True, "fused_linear32_seg_kernel<1, false>"),     # 64 items per column tile: several rounds per job
+    (1024, 320, 4, 256, 1, False, "fused_linear32_seg_kernel<1, true>"),     # low tiles, several column tiles per job
+    (2048 + 100, 100, 5, 1024, 2, False, "fused_linear32_seg_kernel<1, true>"),  # ragged: guarded path inside the kernel
+    (3072, 96, 7, 2048, 1, False, "fused_linear32_kernel<1>"),
+])
+@in_child
+def test_fused_linear(K, N, M, th, segs, prep, kernel):
+    cases.linear(Model(cus=4), weight_bits(K, N, 1), x_bits(M, K, 2), th, segs, slot_table=prep, window_rows=prep,
+                 expect_kernel=kernel)
+
+
+@pytest.mark.parametrize("M,kernel", [(2, "fused_linear32_resident_kernel<1>"), (40, "fused_linear32_resident_kernel<2>")])
+@in_child
+def test_fused_linear_resident_kernel(M, kernel):
+    # segments of 512 rows: too long for the sixteen-wavefront kernel's windows, so every (tile, segment) is an item
+    # of the twelve-wavefront resident kernel, whole bodies' windows transposed
+    cases.linear(Model(cus=4), weight_bits(4096, 64, 1), x_bits(M, 4096, 2), 2048, 2, expect_kernel=kernel)
+
+
+@pytest.mark.parametrize("M,kernel", [(65, "fused_linear32_wide_kernel<4>"), (128, "fused_linear32_wide_kernel<4>"),
+                                      (129, "fused_linear32_wide_kernel<8>"), (300, "fused_linear32_wide_kernel<8>")])
+@in_child
+def test_fused_linear_above_64_rows_in_one_pass(M, kernel):
+    """fused_linear32_wide_kernel: bit-identical to the 64-rows-a-pass kernel, which the twin check implies (the
+    plain-weight twin always runs the 64-row kernel) and which is asserted directly as well."""
+    import ctypes as C
+
+    m = Model(cus=4)
+    K, N, th = 2048, 96, 1024
+    bits, xb = weight_bits(K, N, 1), x_bits(M, K, 2)
+    cases.linear(m, bits, xb, th, wide=True, expect_kernel=kernel)
+    cases.linear(m, bits, xb, th, wide=False, expect_kernel="fused_linear32_kernel<2>")
+    # ragged weight: every tile of the last row and column takes the guarded path of the wide kernel
+    cases.linear(m, weight_bits(K + 40, N - 6, 3), x_bits(M, K + 40, 2), th, wide=True, expect_kernel=kernel)
+
+
+@in_child
+def test_fused_linear_bias_row_stride_and_the_entry_point_without_allocation():
+    m = Model(cus=4)
+    K, N, th = 2048, 128, 1024
+    bits, bias = weight_bits(K, N, 1), x_bits(1, N, 9)[0]
+    for M, segs in ((1, 2), (33, 1), (5, 4)):
+        cases.linear(m, bits, x_bits(M, K, 2), th, segs, bias=bias, x_pad=24, window_rows=True)
+        cases.linear(m, bits, x_bits(M, K, 2), th, segs, bias=bias, noalloc=True, window_rows=True)
+
+
+@pytest.mark.parametrize("kind", cases.KINDS)
+@in_child
+def test_fused_linear_on_unusual_planes(kind):
+    rng = np.random.default_rng(12)
+    bits = cases.weight_kind(rng, 2048, 96, kind)
+    m = Model(cus=3)
+    for M, segs, prep in ((1, 1, False), (2, 2, True), (40, 4, False), (100, 1, False)):
+        cases.linear(m, bits, x_bits(M, 2048, 2), 1024, segs, slot_table=prep, window_rows=prep, wide=M > 64)
+
+
+# ---- fused gather -----------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("K,N,n,th,segs,slot,kernel", [
+    (4096, 128, 300, 1024, 1, False, "embed_gather32_kernel"),
+    (4096, 128, 300, 1024, 8, False, "embed_gather32_kernel"),
+    (4096, 128, 300, 1024, 8, True, "embed_gather32_seg_kernel"),
+    (4096, 128, 300, 1024, 4, True, "embed_gather32_seg_kernel"),
+    (5000, 100, 257, 1024, 8, True, "embed_gather32_seg_kernel"),   # ragged rows and columns, odd last column tile
+    (3000, 96, 1, 512, 4, True, "embed_gather32_seg_kernel"),
+    (70000, 64, 2048, 1024, 8, True, "embed_gather32_seg_kernel"),
+    (270000, 32, 500, 32, 1, False, "embed_sort_kernel"),            # more buckets than counting slots: the sort
+])
+@in_child
+def test_fused_gather(K, N, n, th, segs, slot, kernel):
+    rng = np.random.default_rng(4)
+    ids = cases.zipf_ids(rng, K, n)
+    if n > 8:
+        ids[1], ids[5], ids[7] = -3, K, K + 12345678901  # outside the table: zero rows
+        ids[2] = ids[3] = ids[4]                          # duplicates
+    cases.gather(Model(cus=4), weight_bits(K, N, 3), ids, th, segs, slot, expect_kernel=kernel)
+
+
+@pytest.mark.parametrize("kind", cases.KINDS)
+@in_child
+def test_fused_gather_on_unusual_planes(kind):
+    rng = np.random.default_rng(13)
+    bits = cases.weight_kind(rng, 6000, 96, kind)
+    m = Model(cus=3)
+    for segs, slot in ((1, False), (8, True), (4, True)):
+        cases.gather(m, bits, rng.integers(0, 6000, 400), 1024, segs, slot)
+        cases.gather(m, bits, np.full(70, 4095), 1024, segs, slot)  # one row asked for seventy times, the last of its tile
+
+
+# ---- LM head ----------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("V,H,M,th,segs,prep,matrix,kernel", [
+    (2048, 128, 1, 1024, 1, False, False, "trans32_kernel<1>"),
+    (2048, 128, 3, 1024, 1, False, False, "trans32_kernel<kTrRows>"),
+    (2048, 96, 6, 1024, 1, False, False, "trans32_kernel<kTrRows>"),
+    (2048, 128, 1, 1024, 2, True, False, "trans32_seg_kernel<false>"),
+    (2048, 128, 1, 1024, 4, True, False, "trans32_seg_kernel<false>"),
+    (2048 + 300, 128, 1, 1024, 2, True, False, "trans32_seg_kernel<false>"),   # short last tile row: trans32_kernel takes it
+    (2048, 128, 1, 1024, 2, True, True, "trans32_seg_kernel<true>"),
+    (2048 + 300, 256, 1, 1024, 4, True, True, "trans32_seg_kernel<true>"),
+    (2000, 100, 2, 512, 1, False, False, "trans32_kernel<kTrRows>"),
+])
+@in_child
+def test_lm_head(V, H, M, th, segs, prep, matrix, kernel):
+    cases.lm_head(Model(cus=4), weight_bits(V, H, 3), x_bits(M, H, 2), th, segs, slot_table=prep, window_rows=prep,
+                  matrix_sums=matrix, expect_kernel=kernel, check_twin=not matrix)
+
+
+@pytest.mark.parametrize("kind", cases.KINDS)
+@in_child
+def test_lm_head_on_unusual_planes(kind):
+    rng = np.random.default_rng(14)
+    bits = cases.weight_kind(rng, 2048, 64, kind)
+    m = Model(cus=3)
+    cases.lm_head(m, bits, x_bits(1, 64, 2), 1024)
+    cases.lm_head(m, bits, x_bits(1, 64, 2), 1024, 2, window_rows=True)
+    cases.lm_head(m, bits, x_bits(1, 64, 2), 1024, 4, window_rows=True, slot_table=True, matrix_sums=True, check_twin=False)
+
+
+# ---- encoders and the other layouts --------------------------------------------------------------------------------------
+@pytest.mark.parametrize("layout,th,tw", [("ilp2", 1024, 32), ("ilp2", 64, 16), ("one", 256, 32), ("one", 128, 64),
+                                          ("dense", 512, 32)])
+@in_child
+def test_encoders(layout, th, tw):
+    from oracle import rans_oracle as ro
+
+    m = Model(cus=4)
+    for K, N, seed in ((1500, 100, 1), (th, tw, 2), (2 * th + 1, 3 * tw + 5, 3)):
+        cases.encode(m, ro.split_bf16(weight_bits(K, N, seed))[0], th, tw, layout)
+
+
+@pytest.mark.parametrize("layout,th,tw", [("one", 256, 32), ("one", 64, 16), ("one", 1024, 128), ("dense", 512, 32),
+                                          ("ilp2", 128, 64), ("ilp2", 32, 16)])
+@in_child
+def test_operators_of_the_other_layouts(layout, th, tw):
+    """a7 (one stream per column in tile bodies), the dense layout and other tile widths of the default layout: decode,
+    fused linear, gather and LM head through the one-thread-per-stream kernels."""
+    rng = np.random.default_rng(15)
+    K, N = 2 * th + th // 2, 3 * tw + 7
+    ids = rng.integers(-2, K + 2, 37)
+    launches = cases.other_layout_ops(Model(cus=4), weight_bits(K, N, 5), x_bits(3, max(K, N), 2)[:, :K], ids, th, tw, layout)
+    assert any("generic_kernel" in k for k in launches), launches
