@@ -187,8 +187,19 @@ def encode(m: Model, exp_plane, th, tw, layout="ilp2"):
     fp, cp = f16.ctypes.data_as(C.c_void_p), c16.ctypes.data_as(C.c_void_p)
     n = C.c_uint64(0)
     m.clear()
+    oracle_encoder = {"ilp2": ro.encode_tiled_ilp2, "one": ro.encode_tiled_one, "dense": ro.encode_tiled_dense}[layout]
+    try:
+        want = oracle_encoder(exp_plane, f, c, th, tw)
+    except RuntimeError as e:
+        if "outgrew" not in str(e):
+            raise
+        # a stream longer than the capacity the reference reserves: the library must refuse the input too
+        meta = [m.empty(max(t.num_streams, t.num_tiles), np.uint32).p for _ in range(2 if layout != "dense" else 1)]
+        rc = getattr(m.lib, f"ci_encode_tiled_{layout}")(sym.p, C.byref(t), fp, cp, scratch.p, C.c_size_t(nb), states.p, sizes.p,
+                                                         *meta, C.byref(n), None)
+        assert rc != 0 and m.violations() == [], "the oracle refuses this input (capacity), the library encoded it"
+        raise
     if layout == "dense":
-        want = ro.encode_tiled_dense(exp_plane, f, c, th, tw)
         offs = m.empty(t.num_streams, np.uint32)
         m.call("ci_encode_tiled_dense", sym.p, C.byref(t), fp, cp, scratch.p, C.c_size_t(nb), states.p, sizes.p, offs.p,
                C.byref(n), None)
@@ -196,7 +207,6 @@ def encode(m: Model, exp_plane, th, tw, layout="ilp2"):
         m.call("ci_pack_tiled_dense", scratch.p, C.byref(t), sizes.p, offs.p, stream.p, n, None)
         assert np.array_equal(offs.get(), want.stream_offsets)
     else:
-        want = (ro.encode_tiled_ilp2 if layout == "ilp2" else ro.encode_tiled_one)(exp_plane, f, c, th, tw)
         offs, lens = m.empty(t.num_tiles, np.uint32), m.empty(t.num_tiles, np.uint32)
         m.call(f"ci_encode_tiled_{layout}", sym.p, C.byref(t), fp, cp, scratch.p, C.c_size_t(nb), states.p, sizes.p, offs.p,
                lens.p, C.byref(n), None)

@@ -98,8 +98,13 @@ static inline T atomicOr(T *p, T v) {
 }
 #define __HIP_MEMORY_SCOPE_WORKGROUP 0
 #define __hip_atomic_load(p, order, scope) (*(volatile __typeof__(*(p)) *)(p))
-#define __hip_atomic_store(p, v, order, scope) ((void)(*(volatile __typeof__(*(p)) *)(p) = (v)))
-#define __hip_atomic_fetch_add(p, v, order, scope) atomicAdd((p), (__typeof__(*(p)))(v))
+// (an operation that publishes -- release semantics -- comes after what the other lanes of the wavefront did earlier
+// in the program: sim::wave_catch_up)
+#define CI_SIM_RELEASES(order) ((order) == __ATOMIC_RELEASE || (order) == __ATOMIC_ACQ_REL || (order) == __ATOMIC_SEQ_CST)
+#define __hip_atomic_store(p, v, order, scope) \
+    ((void)(CI_SIM_RELEASES(order) ? sim::wave_catch_up() : (void)0), (void)(*(volatile __typeof__(*(p)) *)(p) = (v)))
+#define __hip_atomic_fetch_add(p, v, order, scope) \
+    ((void)(CI_SIM_RELEASES(order) ? sim::wave_catch_up() : (void)0), atomicAdd((p), (__typeof__(*(p)))(v)))
 
 // ---- host API -------------------------------------------------------------------------------------------------
 typedef int hipError_t;

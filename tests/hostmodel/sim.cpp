@@ -108,7 +108,7 @@ static void map_lds() {
 
 // ---- fibres ---------------------------------------------------------------------------------------------------
 enum St : uint8_t { RUN, WAIT_WAVE, WAIT_WG, DONE };
-enum Op : int { OP_SYNC = 1, OP_BALLOT, OP_READLANE, OP_READFIRST, OP_DPP, OP_PERMSWAP, OP_SHFL, OP_SHFL_UP, OP_MFMA, OP_ASM };
+enum Op : int { OP_CATCHUP = 100, OP_SYNC = 1, OP_BALLOT, OP_READLANE, OP_READFIRST, OP_DPP, OP_PERMSWAP, OP_SHFL, OP_SHFL_UP, OP_MFMA, OP_ASM };
 
 struct Fiber {
     void *sp;
@@ -272,6 +272,10 @@ __attribute__((noinline)) int shfl_up(int v, unsigned delta, int width) {
     return a.out;
 }
 __attribute__((noinline)) void wave_sync() { meet(OP_SYNC, nullptr, __builtin_return_address(0)); }
+// A lane about to publish something (a store or read-modify-write with release semantics) waits until every other
+// lane of its wavefront has run up to its next meeting point: on the GPU the lanes of a wavefront run in step, so
+// what the other lanes did earlier in the program has happened before one lane's later store.
+void wave_catch_up() { meet(OP_CATCHUP, nullptr, nullptr); }
 __attribute__((noinline)) void mfma_impl(const void *a, const void *b, void *c) {
     MfmaArgs m{a, b, c};
     meet(OP_MFMA, &m, __builtin_return_address(0));
@@ -1086,7 +1090,7 @@ static bool run_workgroup(uint32_t nthreads, const LaneCtx &proto) {
         for (uint32_t wi = 0; wi < n_waves; ++wi) {
             const uint32_t wv = order[wi];
             const uint32_t lo = wv * 64, hi = lo + 64 < nthreads ? lo + 64 : nthreads;
-            uint32_t live_w = 0, wait_wave = 0, wait_wg = 0;
+            uint32_t live_w = 0, wait_wave = 0, wait_wg = 0, catching_up = 0, spinning = 0;
             for (uint32_t t = lo; t < hi; ++t) {
                 Fiber &f = g_fib[t];
                 if (f.st == RUN) {
@@ -1098,10 +1102,19 @@ static bool run_workgroup(uint32_t nthreads, const LaneCtx &proto) {
                     if (g_abort_launch) return false;
                 }
                 if (f.st != DONE) ++live_w;
-                if (f.st == WAIT_WAVE) ++wait_wave;
+                if (f.st == WAIT_WAVE && f.op == OP_CATCHUP)
+                    ++catching_up;
+                else if (f.st == WAIT_WAVE)
+                    ++wait_wave;
                 if (f.st == WAIT_WG) ++wait_wg;
+                if (f.st == RUN && f.yielded) ++spinning;  // (in a wait loop: it has got as far as it can, too)
             }
-            if (wait_wave && wait_wave + wait_wg == live_w) {
+            if (catching_up && catching_up + wait_wave + wait_wg + spinning == live_w) {
+                // everybody else of the wavefront has got as far as it can: the lanes that waited for that go on
+                for (uint32_t t = lo; t < hi; ++t)
+                    if (g_fib[t].st == WAIT_WAVE && g_fib[t].op == OP_CATCHUP) g_fib[t].st = RUN;
+                progress = true;
+            } else if (wait_wave && wait_wave + wait_wg == live_w) {
                 exec_collective(&g_fib[lo], (int)(hi - lo));
                 g_cur = nullptr;
                 if (g_abort_launch) return false;

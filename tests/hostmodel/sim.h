@@ -41,6 +41,7 @@ u32x2v permlane_swap(uint32_t a, uint32_t b, int rows);
 int shfl(int v, int src, int width);
 int shfl_up(int v, unsigned delta, int width);
 void wave_sync();
+void wave_catch_up();  // this lane waits until the other lanes of its wavefront have reached their next meeting point
 void syncthreads();
 void yield();
 void mfma_impl(const void *a, const void *b, void *c);

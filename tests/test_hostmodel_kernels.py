@@ -218,3 +218,71 @@ def test_operators_of_the_other_layouts(layout, th, tw):
     ids = rng.integers(-2, K + 2, 37)
     launches = cases.other_layout_ops(Model(cus=4), weight_bits(K, N, 5), x_bits(3, max(K, N), 2)[:, :K], ids, th, tw, layout)
     assert any("generic_kernel" in k for k in launches), launches
+
+
+# ---- descriptors that promise too much ------------------------------------------------------------------------------------
+@in_child
+def test_an_understated_window_leaves_items_out_and_reads_nothing_out_of_bounds():
+    """max_window_rows smaller than the truth selects the kernel instances without guarded path; an item whose window
+    does not fit is then left out (fused linear) or gets zeros (LM head): wrong sums, as the header says, and no
+    access outside the arrays or the window areas."""
+    import ctypes as C
+
+    m = Model(cus=4)
+    rng = np.random.default_rng(3)
+    K, N, th, segs = 2048, 64, 1024, 2
+    bits = cases.weight_kind(rng, K, N, "wide")  # deep bodies: windows of more than 112 rows
+    enc, man = cases.compress(bits, th)
+    w, keep = m.weight(enc, man, K, N, segments=segs, slot_table=True, window_rows=True)
+    assert w.max_window_rows > 112, w.max_window_rows
+    w.max_window_rows = 7  # the lie
+    x, y = m.dev(x_bits(1, K, 2)), m.empty((1, N), np.uint16)
+    nb = m.lib.ci_fused_linear_workspace_bytes_segmented(1, K, N, th, 32, 0, segs)
+    ws = m.empty(max(nb, 16), np.uint8)
+    m.clear()
+    m.call("ci_fused_linear_tiled", C.byref(w), x.p, 1, K, None, y.p, N, ws.p, C.c_size_t(nb), None)
+    assert m.launches() == ["(fused_linear32_seg_kernel<1, false>)"], m.launches()
+    # the LM head on the same arrays read as a [V = 2048, H = 64] table
+    xh, z = m.dev(x_bits(1, N, 2)), m.empty((1, K), np.uint16)
+    nbt = m.lib.ci_fused_linear_transposed_workspace_bytes(1, N, K, 32)
+    wst = m.dev(np.full(nbt // 4, np.float32(np.nan)))  # what an earlier launch might have left in the workspace
+    m.clear()
+    m.call("ci_fused_linear_transposed_tiled", C.byref(w), xh.p, 1, N, None, z.p, K, wst.p, C.c_size_t(nbt), None)
+    assert "trans32_seg_kernel<false>" in m.launches()
+    from tests.hostmodel.model import bf16_bits_to_f32
+
+    assert np.isfinite(bf16_bits_to_f32(z.get())).all(), "rows of a refused item surfaced as stale workspace contents"
+
+
+@in_child
+def test_tile_metadata_that_points_past_the_stream_is_not_followed():
+    """Every kernel treats a tile body that would run past stream_len as empty instead of reading it."""
+    import ctypes as C
+
+    m = Model(cus=4)
+    K, N, th = 2048, 96, 1024
+    bits = weight_bits(K, N, 1)
+    enc, man = cases.compress(bits, th)
+    bad = enc.tile_offsets.copy()
+    bad[-1] = enc.stream.size - 64      # the last body now ends beyond the stream
+    bad[2] = 0xFFFFFF00                  # and one starts far outside it
+    enc.tile_offsets = bad
+    for segs, slot in ((1, False), (2, True)):
+        w, keep = m.weight(enc, man, K, N, segments=segs, slot_table=slot)
+        out, x, y = m.empty((K, N), np.uint8), m.dev(x_bits(2, K, 2)), m.empty((2, N), np.uint16)
+        nb = m.lib.ci_fused_linear_workspace_bytes_segmented(2, K, N, th, 32, 0, segs)
+        ws = m.empty(max(nb, 16), np.uint8)
+        ids = m.dev(np.arange(0, K, 37, dtype=np.int64))
+        n_ids = ids.shape[0]
+        g = m.empty((n_ids, N), np.uint16)
+        nbe = m.lib.ci_fused_embedding_workspace_bytes_segmented(n_ids, K, th, segs)
+        wse = m.empty(nbe, np.uint8)
+        z = m.empty((1, K), np.uint16)
+        nbt = m.lib.ci_fused_linear_transposed_workspace_bytes(1, N, K, 32)
+        wst = m.empty(nbt, np.uint8)
+        m.clear()
+        m.call("ci_decode_tiled", C.byref(w), out.p, None, None)
+        m.call("ci_fused_linear_tiled", C.byref(w), x.p, 2, K, None, y.p, N, ws.p, C.c_size_t(nb), None)
+        m.call("ci_fused_embedding_tiled", C.byref(w), ids.p, n_ids, g.p, N, wse.p, C.c_size_t(nbe), None)
+        m.call("ci_fused_linear_transposed_tiled", C.byref(w), m.dev(x_bits(1, N, 2)).p, 1, N, None, z.p, K, wst.p, C.c_size_t(nbt), None)
+        m.free_all()

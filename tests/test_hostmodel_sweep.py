@@ -1,0 +1,189 @@
+"""Random ragged shapes through the host model (tests/hostmodel): some 3,000 seeded cases over the operators, with the
+weights' statistics, tile heights, segment counts, row counts, CU counts, the side of the arrays that touches the
+inaccessible page and the order in which the model runs the wavefronts all drawn per case.  Every case checks the
+result against the oracle and that the model saw no address outside an array, no LDS address outside the launch's
+LDS, no register used before its load was waited for.  A failing case prints its seed and parameters."""
+import numpy as np
+import pytest
+
+from tests.hostmodel import cases
+from tests.hostmodel.model import Model, in_child, x_bits
+
+TILE_HEIGHTS = (32, 64, 128, 256, 512, 1024)
+BLOCKS = 12          # child processes per family
+PER_BLOCK = 44       # cases per child: 6 families x 12 x 44 = 3,168 cases, of which a few per cent are refused by the oracle
+
+
+def _draw(rng, need_blocks_of_16=True):
+    th = int(rng.choice(TILE_HEIGHTS))
+    half = th // 2
+    segs_ok = [s for s in (1, 2, 4, 8, 16) if half % ((16 if need_blocks_of_16 else 1) * s) == 0 and half // s >= 8]
+    segs = int(rng.choice(segs_ok)) if segs_ok else 1
+    tiles_k = int(rng.integers(1, 4))
+    K = int(rng.integers(max(1, (tiles_k - 1) * th + 1), tiles_k * th + 1))
+    if rng.random() < 0.4:
+        K = tiles_k * th  # whole tiles: the hand-scheduled paths
+    N = int(rng.integers(1, 140)) if rng.random() < 0.6 else 32 * int(rng.integers(1, 5))
+    kind = cases.KINDS[int(rng.integers(0, len(cases.KINDS)))] if rng.random() < 0.5 else "normal"
+    return th, segs, K, N, kind
+
+
+def _model(rng):
+    return Model(cus=int(rng.integers(1, 9)), end_at_guard=bool(rng.random() < 0.7), schedule=int(rng.integers(0, 1 << 30)) * int(rng.random() < 0.5))
+
+
+FAMILY = {"decode": 1, "linear": 2, "gather": 3, "lm_head": 4, "layouts": 5}
+
+
+def _run(family, block, body):
+    ran = 0
+    for i in range(PER_BLOCK):
+        seed = FAMILY[family] * 100000 + block * 1000 + i
+        rng = np.random.default_rng(seed)
+        m = _model(rng)
+        try:
+            body(rng, m)
+            ran += 1
+        except RuntimeError as e:
+            # an incompressible plane on a ragged shape can outgrow the per-stream capacity the reference reserves
+            # (src/cuda/rans_host.cuh:470-471): the oracle refuses such an input, and the case is not counted
+            if "outgrew" not in str(e):
+                raise AssertionError(f"{family} case seed {seed}: {e}") from e
+        except BaseException as e:  # noqa: BLE001
+            raise AssertionError(f"{family} case seed {seed}: {e}") from e
+        finally:
+            m.free_all()
+    assert ran >= PER_BLOCK * 3 // 4, f"{family}: only {ran} of {PER_BLOCK} cases could be encoded"
+
+
+@pytest.mark.parametrize("block", range(BLOCKS))
+@in_child
+def test_decode_sweep(block):
+    def body(rng, m):
+        th, segs, K, N, kind = _draw(rng)
+        bits = cases.weight_kind(rng, K, N, kind)
+        return cases.decode(m, bits, th, segs, merge=bool(rng.random() < 0.4))
+
+    _run("decode", block, body)
+
+
+@pytest.mark.parametrize("block", range(BLOCKS))
+@in_child
+def test_fused_linear_sweep(block):
+    def body(rng, m):
+        th, segs, K, N, kind = _draw(rng)
+        M = int(rng.choice((1, 1, 2, 3, 4, 5, 8, 17, 32, 33, 64, 65, 100, 128, 129, 200)))
+        if M > 64:
+            segs = 1
+        prep = bool(rng.random() < 0.5)
+        bits = cases.weight_kind(rng, K, N, kind)
+        return cases.linear(m, bits, x_bits(M, K, int(rng.integers(1 << 30))), th, segs, slot_table=prep, window_rows=prep,
+                            wide=M > 64 and bool(rng.random() < 0.7), noalloc=bool(rng.random() < 0.15),
+                            x_pad=8 * int(rng.integers(0, 3)))
+
+    _run("linear", block, body)
+
+
+@pytest.mark.parametrize("block", range(BLOCKS))
+@in_child
+def test_fused_gather_sweep(block):
+    def body(rng, m):
+        th, segs, K, N, kind = _draw(rng, need_blocks_of_16=False)
+        n = int(rng.choice((1, 2, 7, 64, 65, 200, 700)))
+        ids = rng.integers(0, K, n) if rng.random() < 0.5 else cases.zipf_ids(rng, K, n)
+        if n > 4:
+            ids[rng.integers(0, n, 2)] = (-1, K + int(rng.integers(0, 5)))
+        bits = cases.weight_kind(rng, K, N, kind)
+        return cases.gather(m, bits, ids, th, segs, slot_table=bool(rng.random() < 0.7))
+
+    _run("gather", block, body)
+
+
+@pytest.mark.parametrize("block", range(BLOCKS))
+@in_child
+def test_lm_head_sweep(block):
+    def body(rng, m):
+        th, segs, V, H, kind = _draw(rng)
+        if rng.random() < 0.6:
+            H = 32 * int(rng.integers(1, 4))  # whole column tiles: what the sixteen-wavefront kernel takes
+        M = int(rng.choice((1, 1, 1, 2, 4, 5, 9)))
+        prep = bool(rng.random() < 0.7)
+        matrix = prep and M == 1 and kind != "wide" and bool(rng.random() < 0.5)
+        bits = cases.weight_kind(rng, V, H, kind)
+        return cases.lm_head(m, bits, x_bits(M, H, int(rng.integers(1 << 30))), th, segs, slot_table=prep, window_rows=prep,
+                             matrix_sums=matrix, check_twin=not matrix)
+
+    _run("lm_head", block, body)
+
+
+@pytest.mark.parametrize("block", range(BLOCKS))
+@in_child
+def test_other_layouts_and_encoders_sweep(block):
+    from oracle import rans_oracle as ro
+
+    def body(rng, m):
+        th = int(rng.choice((16, 32, 64, 128, 256)))
+        tw = int(rng.choice((8, 16, 32, 64, 128)))
+        layout = ("one", "dense", "ilp2")[int(rng.integers(0, 3))]
+        K, N = int(rng.integers(1, 3 * th)), int(rng.integers(1, 2 * tw + 9))
+        kind = cases.KINDS[int(rng.integers(0, len(cases.KINDS)))]
+        bits = cases.weight_kind(rng, K, N, kind)
+        cases.encode(m, ro.split_bf16(bits)[0], th, tw, layout)
+        if layout == "ilp2" and tw == 32:
+            return None  # (the 32-column kernels of the default layout have their own sweeps)
+        M = int(rng.integers(1, 10))
+        return cases.other_layout_ops(m, bits, x_bits(M, max(K, N), 3)[:, :K], rng.integers(-1, K + 1, 9), th, tw, layout)
+
+    _run("layouts", block, body)
+
+
+FAMILY["hot"] = 6
+
+
+@pytest.mark.parametrize("block", range(BLOCKS))
+@in_child
+def test_hand_scheduled_paths_sweep(block):
+    """Shapes drawn so that the hand-scheduled paths are the ones taken: the one-pass kernel above 64 rows, the
+    sixteen-wavefront kernels of the fused linear (the instance without guarded path) and of the LM head (both kinds
+    of sums), the whole-tile kernels."""
+    def body(rng, m):
+        target = ("wide", "lm_seg", "lm_matrix", "lin_hot", "lin_tile", "dec_persist")[int(rng.integers(0, 6))]
+        kind = cases.KINDS[int(rng.integers(0, len(cases.KINDS)))] if rng.random() < 0.4 else "normal"
+        ragged = int(rng.integers(1, 60)) if rng.random() < 0.3 else 0
+        if target == "wide":
+            th = int(rng.choice((64, 256, 1024)))
+            K, N = th * int(rng.integers(1, 3)) + (ragged & ~7 if rng.random() < 0.7 else ragged), 32 * int(rng.integers(1, 4)) - (ragged % 7)
+            M = int(rng.choice((65, 96, 128, 129, 200, 256, 300)))
+            la = cases.linear(m, cases.weight_kind(rng, K, N, kind), x_bits(M, K, 5), th, wide=True)
+            # (the one-pass kernel reads x from its fragment copy, which exists for K a multiple of 8)
+            assert any("fused_linear32_wide_kernel" in k for k in la) or K % 8, la
+        elif target in ("lm_seg", "lm_matrix"):
+            th = int(rng.choice((128, 256, 512, 1024)))
+            segs = int(rng.choice([s for s in (2, 4, 8, 16) if (th // 2) % (32 * s) == 0]))
+            V, H = th * int(rng.integers(1, 3)) + ragged, 32 * int(rng.integers(1, 4))
+            matrix = target == "lm_matrix"
+            if matrix and kind == "wide":
+                kind = "normal"
+            la = cases.lm_head(m, cases.weight_kind(rng, V, H, kind), x_bits(1, H, 5), th, segs, slot_table=bool(rng.random() < 0.5),
+                               window_rows=True, matrix_sums=matrix, check_twin=not matrix)
+            # (a window above 112 rows -- deep bodies of the wide kinds -- sends the weight to the whole-tile kernel)
+            assert any("trans32_seg_kernel<%s>" % ("true" if matrix else "false") in k for k in la) or kind != "normal", la
+        elif target == "lin_hot":
+            th = int(rng.choice((64, 128, 256, 512, 1024)))
+            segs = int(rng.choice([s for s in (1, 2, 4, 8) if (th // 2) % (16 * s) == 0 and th // 2 // s <= 256]))
+            K, N = th * int(rng.integers(1, 4)), 32 * int(rng.integers(1, 5))
+            M = int(rng.choice((1, 2, 4, 5, 16, 32, 33, 64)))
+            la = cases.linear(m, cases.weight_kind(rng, K, N, kind), x_bits(M, K, 5), th, segs, slot_table=True, window_rows=True)
+            assert any("fused_linear32_seg_kernel" in k for k in la), la
+        elif target == "lin_tile":
+            th = int(rng.choice((1024, 2048)))
+            K, N = th * int(rng.integers(1, 3)) + ragged, 32 * int(rng.integers(1, 3))
+            la = cases.linear(m, cases.weight_kind(rng, K, N, kind), x_bits(int(rng.choice((1, 3, 32, 40, 64))), K, 5), th)
+            assert any("fused_linear32_kernel" in k for k in la), la
+        else:
+            th = int(rng.choice((1024, 2048)))
+            K, N = th * int(rng.integers(1, 3)) + ragged, int(rng.integers(1, 100))
+            la = cases.decode(m, cases.weight_kind(rng, K, N, kind), th, 1, merge=bool(rng.random() < 0.5))
+            assert any("decode_tiled32_persist_kernel" in k for k in la), la
+
+    _run("hot", block, body)
