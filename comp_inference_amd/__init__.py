@@ -24,7 +24,9 @@ from .embedding_hip import (
     fused_rans_embedding_uncoalesced,
 )
 from .linear_hip import (
+    debug_wait_limit,
     dense_matmul,
+    device_status,
     fused_rans_linear,
     fused_wide_rows,
     fused_rans_linear_one_stream,

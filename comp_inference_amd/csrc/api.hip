@@ -19,5 +19,6 @@ extern "C" int ci_check_device(void) {
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return ci::fail(CI_ERR_DEVICE, "device %d is %s; this library holds gfx950 code only", dev,
                         prop.gcnArchName);
-    return CI_OK;
+    // per-device set-up that must not happen for the first time inside a graph capture
+    return ci_fused_linear_noalloc_init();
 }

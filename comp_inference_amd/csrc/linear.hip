@@ -63,7 +63,14 @@ struct LinearArgs {
     const uint2 *slot_table;
     uint32_t rounds;  // fused_linear32_seg_kernel: items of a job per wavefront
     bool all_fast;    // every item of the weight takes the hand-scheduled loop (known from the descriptor)
+    uint32_t wait_limit;  // looks a wavefront takes at another wavefront's flag before it gives up (see g_device_status)
 };
+
+// What a kernel could not do and did not hang over, one bit per kind (ci_device_status reads and clears it):
+// a wavefront that waits for another one inside a kernel looks at the flag at most LinearArgs::wait_limit times, then
+// records CI_STATUS_WAIT_GAVE_UP here and goes on, so that a slip in a hand-over shows as an error code and wrong
+// sums, never as a kernel that does not end.
+static __device__ uint32_t g_device_status;
 
 // x [M, K] -> the fragment order described at LinearArgs::xf.  In a plain row-major x the 64 lanes of
 // one operand load touch 64 different cache lines (16 bytes of each); with many rows that traffic, not
@@ -874,8 +881,14 @@ __global__ __launch_bounds__(kSegWaves *kWave) void fused_linear32_seg_kernel(Li
             float *buf = reinterpret_cast<float *>(lds + kSmallBufOff);
             uint32_t *flags = reinterpret_cast<uint32_t *>(lds + kSmallFlagsOff);
             const uint32_t jn = sl / jb.R;  // which of this workgroup's jobs
-            while (__hip_atomic_load(&flags[1], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) != jn)
-                __builtin_amdgcn_s_sleep(2);  // (the wavefront adding up the job before this one is not waiting for us)
+            // (the wavefront adding up the job before this one is not waiting for us; the wait is bounded all the same)
+            for (uint32_t looks = 0; __hip_atomic_load(&flags[1], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) != jn; ++looks) {
+                if (looks >= a.wait_limit) {
+                    if (lane == 0) atomicOr(&g_device_status, (uint32_t)CI_STATUS_WAIT_GAVE_UP);
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(2);
+            }
             if (c < a.M) {
 #pragma unroll
                 for (int v = 0; v < 16; ++v)
@@ -1092,16 +1105,19 @@ static void launch_splitk_reduce(const float *partial, uint32_t P, uint32_t M, u
 // Groups of 32 rows per pass of fused_linear32_wide_kernel for M rows of x (0: not its case).
 static uint32_t wide_groups(uint32_t M) { return M <= 64 ? 0u : M <= 128 ? 4u : 8u; }
 
-// Groups of 32 rows in the fragment copy: whole passes where the wide kernel may run (the groups past the last
-// row of x are zero), else the groups x has.
-static uint32_t x_fragment_groups(uint32_t M) {
-    const uint32_t groups = ceil_div(M, 32u), per_pass = wide_groups(M);
-    return per_pass ? ceil_div(groups, per_pass) * per_pass : groups;
+// Groups of 32 rows in the fragment copy (the groups past the last row of x are zero): whole passes of the kernel
+// that will read it -- four or eight groups where the one-pass kernel may run (`whole_passes`), else the pairs of
+// groups that fused_linear32_kernel<2> reads per 64 rows, or the single group of up to 32 rows.
+static uint32_t x_fragment_groups(uint32_t M, bool whole_passes) {
+    const uint32_t groups = ceil_div(M, 32u), per_pass = whole_passes ? wide_groups(M) : 0u;
+    if (per_pass) return ceil_div(groups, per_pass) * per_pass;
+    return M > 32 ? 2 * ceil_div(M, 64u) : 1u;
 }
 
-static size_t x_fragment_bytes(uint32_t M, uint32_t K, bool fast_plan) {
+// whole_passes = true gives the larger figure: what the size queries answer, whichever kernel then runs.
+static size_t x_fragment_bytes(uint32_t M, uint32_t K, bool fast_plan, bool whole_passes = true) {
     if (!fast_plan || M < kFragMinRows || K % 8) return 0;
-    return (size_t)x_fragment_groups(M) * 32 * K * 2;
+    return (size_t)x_fragment_groups(M, whole_passes) * 32 * K * 2;
 }
 
 struct LinearPlan {
@@ -1214,6 +1230,24 @@ extern "C" uint32_t ci_suggest_segments(uint32_t K, uint32_t N, uint32_t tile_he
     return best;
 }
 
+// Looks of a bounded wait inside a kernel (a look every 128 clocks or so: the default is a fifth of a second, against
+// the microsecond a hand-over takes).  ci_debug_wait_limit sets it, for tests that force the give-up path.
+static std::atomic<uint32_t> g_wait_limit{1u << 22};
+
+extern "C" uint32_t ci_debug_wait_limit(uint32_t looks) { return g_wait_limit.exchange(looks); }
+
+extern "C" int ci_device_status(uint32_t *h_status, ci_stream_t stream) {
+    if (!h_status) return fail(CI_ERR_ARG, "ci_device_status: null result pointer");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    void *word = nullptr;
+    CI_HIP(hipGetSymbolAddress(&word, HIP_SYMBOL(g_device_status)));
+    CI_HIP(hipMemcpyAsync(h_status, word, sizeof(uint32_t), hipMemcpyDeviceToHost, s));
+    CI_HIP(hipMemsetAsync(word, 0, sizeof(uint32_t), s));
+    CI_HIP(hipStreamSynchronize(s));
+    if (*h_status) return fail(CI_ERR_HIP, "a kernel gave up a bounded wait (device status 0x%x): results since the last check are not to be used", *h_status);
+    return CI_OK;
+}
+
 // Whether more than 64 rows of x go through fused_linear32_wide_kernel (one decode per 128 or 256 rows) instead
 // of fused_linear32_kernel<2> once per 64 rows.  Same results bit for bit; off until it has been measured.
 static std::atomic<int> g_wide_rows{0};
@@ -1286,6 +1320,7 @@ static int fused_linear_impl(const uint16_t *d_x, uint32_t M, uint32_t K, uint32
     a.all_fast = !d_plain_w && a.fast_ok && K % th == 0 && N % tw == 0 && max_window_rows != 0 &&
                  max_window_rows <= kWinRows;
     a.rounds = p.rounds;
+    a.wait_limit = g_wait_limit.load(std::memory_order_relaxed);
     a.segs = p.segs;
     a.kw = p.kw;
     a.nw = p.nw;
@@ -1312,7 +1347,9 @@ static int fused_linear_impl(const uint16_t *d_x, uint32_t M, uint32_t K, uint32
     }
     // the fragment copy of x goes behind the partials when the caller's workspace has room for it
     a.xf = nullptr;
-    const size_t frag_bytes = d_plain_w ? 0 : x_fragment_bytes(M, K, p.fast && a.fast_ok);  // (the guarded path reads x in place)
+    // (the guarded path reads x in place; whole passes of four or eight groups only where the one-pass kernel is on)
+    const bool wide_on = g_wide_rows.load(std::memory_order_relaxed) != 0;
+    const size_t frag_bytes = d_plain_w ? 0 : x_fragment_bytes(M, K, p.fast && a.fast_ok, wide_on);
     if (frag_bytes && frag_bytes < (1ull << 31) && d_workspace) {
         uint8_t *at = static_cast<uint8_t *>(d_workspace) + ((partial_bytes + 15) & ~(size_t)15);
         at += (16 - (reinterpret_cast<uintptr_t>(at) & 15)) & 15;
@@ -1360,7 +1397,7 @@ static int fused_linear_impl(const uint16_t *d_x, uint32_t M, uint32_t K, uint32
         CI_ALLOW_FULL_LDS(fused_linear32_wide_kernel<8>);
         const dim3 block(waves * kWave);
         const uint32_t per_pass = wide_groups(M);
-        if (per_pass && a.xf && !d_plain_w && g_wide_rows.load(std::memory_order_relaxed)) {
+        if (per_pass && a.xf && !d_plain_w && wide_on) {
             const dim3 grid(ceil_div(a.tiles_n, p.nw), p.P, ceil_div(M, 32 * per_pass));
             if (per_pass == 4)
                 hipLaunchKernelGGL(fused_linear32_wide_kernel<4>, grid, block, lds_bytes, s, a);
@@ -1586,6 +1623,13 @@ static int scratch_address(void **out) {
     return CI_OK;
 }
 }  // namespace ci
+
+// The set-up of the entry point below for the current device (the address of the scratch array), outside any graph
+// capture: ci_check_device does it too, so a process that has checked its device is ready.
+extern "C" int ci_fused_linear_noalloc_init(void) {
+    void *ws = nullptr;
+    return scratch_address(&ws);
+}
 
 extern "C" int ci_fused_linear_tiled_noalloc(const ci_tiled_weight *w, const uint16_t *d_x, uint32_t M,
                                              uint32_t x_stride, const uint16_t *d_bias, uint16_t *d_out,

@@ -11,7 +11,7 @@ import ctypes as C
 import torch
 
 from . import _lib
-from ._lib import check, lib, ptr
+from ._lib import check, lib, ptr, stream_handle
 
 
 class _Scratch:
@@ -64,6 +64,23 @@ def fused_wide_rows(enable: bool) -> bool:
     with `enable` a tile is decoded once per 128 or 256 rows of x instead of once per 64.  Bit-identical results.
     Process-wide, off by default; returns the previous setting."""
     return bool(lib().ci_fused_linear_wide_rows(1 if enable else 0))
+
+
+def device_status(device=None) -> int:
+    """What the kernels could not do and did not hang over since the last call, as CI_STATUS_* bits (0: nothing);
+    raises RuntimeError if a bit is set.  Waits for the device's current stream: for health checks, not the token loop."""
+    dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    word = C.c_uint32(0)
+    with torch.cuda.device(dev):
+        check(lib().ci_device_status(C.byref(word), stream_handle(dev)))
+    return word.value
+
+
+def debug_wait_limit(looks: int) -> int:
+    """Looks a wavefront takes at another wavefront's flag before it gives up (ci_debug_wait_limit); returns the
+    previous value.  0 forces the give-up path: for tests."""
+    lib().ci_debug_wait_limit.restype = C.c_uint32
+    return int(lib().ci_debug_wait_limit(C.c_uint32(int(looks))))
 
 
 def _decode_once_weight(dev, compressed_data, initial_states, tables, slot_map, shape, tile_offsets, tile_max_lens,

@@ -56,12 +56,18 @@ def _load_from_compressed(mod: nn.Module, src: nn.Module) -> None:
     mod.tile_k, mod.tile_n = int(src.exponent_tile_height), int(src.exponent_tile_width)
 
 
+def _version_of(t: torch.Tensor) -> int:
+    """Version counter of a tensor for the cache keys below; tensors made under torch.inference_mode() (a model
+    loaded or moved inside it) do not track one and cannot be updated in place either: 0."""
+    return 0 if t.is_inference() else t._version
+
+
 def _cached_checkpoints(mod: nn.Module, device, shape, segments: int):
     """(checkpoints, segments) of `mod`'s compressed weight as it lies on `device`: built on first use from
     the stream (one pass of the decoder) and kept beside it; derived data, not part of the saved state."""
     cached = getattr(mod, "_ckpt_cache", None)
     st = mod.rans_exp_stream
-    key = ((st.data_ptr(), st.numel(), st._version), device, segments)  # (a reload swaps the storage, not the tensor)
+    key = ((st.data_ptr(), st.numel(), _version_of(st)), device, segments)  # (a reload swaps the storage, not the tensor)
     if cached is not None and cached[0] == key:
         return cached[1], cached[2]
     ck = None
@@ -112,7 +118,7 @@ class RansLinear(nn.Module):
         that swaps `tensor.data` under an unchanged tensor object (the loader's own idiom) or an in-place update
         is noticed."""
         ts = (self.rans_exp_stream, self.rans_exp_states, self.rans_man_raw, self.bias)  # (a reload replaces them all)
-        return tuple((t.data_ptr(), t.numel(), t._version) if t is not None else None for t in ts)
+        return tuple((t.data_ptr(), t.numel(), _version_of(t)) if t is not None else None for t in ts)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         device = x.device
@@ -240,7 +246,7 @@ class RansEmbedding(nn.Module):
         from .rans_hip import build_slot_table
 
         t, m = self.rans_exp_tables, self.rans_exp_slot_map
-        key = (str(device), t.data_ptr(), t._version, m.data_ptr(), m._version)
+        key = (str(device), t.data_ptr(), _version_of(t), m.data_ptr(), _version_of(m))
         cached = getattr(self, "_slot_table_cache", None)
         if cached is None or cached[0] != key:
             cached = (key, build_slot_table(t, m, device))

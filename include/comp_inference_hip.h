@@ -510,6 +510,12 @@ int ci_fused_linear_transposed_tiled(const ci_tiled_weight *w, const uint16_t *d
  * time on one GPU (two streams, two threads) race; calls queued on one stream do not.  Results are
  * bit-identical to ci_fused_linear_tiled. */
 #define CI_NOALLOC_SCRATCH_BYTES (16u << 20)
+/* Set-up: the address of the array is asked for once per device (hipGetSymbolAddress), which is not a call to make
+ * for the first time while a stream is being captured.  ci_fused_linear_noalloc_init does it for the current device;
+ * ci_check_device calls it, so a process that has checked its device is ready, and otherwise the first
+ * ci_fused_linear_tiled_noalloc on a device does it -- then that first call must come before any capture.  The
+ * current device must be the device of `stream` in every call (the array used is the current device's). */
+int ci_fused_linear_noalloc_init(void);
 int ci_fused_linear_tiled_noalloc(const ci_tiled_weight *w, const uint16_t *d_x, uint32_t M, uint32_t x_stride,
                                   const uint16_t *d_bias, uint16_t *d_out, uint32_t out_stride,
                                   ci_stream_t stream);
@@ -529,6 +535,23 @@ int ci_fused_linear_wide_rows(int enable);
  * other rows of its group of 32, so this is for finite weights.  Process-wide, off by default; returns the
  * previous setting.  No counterpart in the reference. */
 int ci_fused_linear_transposed_matrix_sums(int enable);
+
+/* ---------------------------------------------------------------------------------------
+ * Bounded waits.  One kernel lets a wavefront wait for another inside a workgroup (the fused linear for up to four
+ * rows of x hands its column sums to the last wavefront to arrive through LDS).  Such a wait looks at the flag a
+ * bounded number of times; a wavefront that gives up records it in a status word in device memory and goes on, so
+ * a defect there ends as wrong sums and an error code, never as a kernel that does not finish.  The reference's
+ * Triton kernels have no such wait and nothing to report (their split-K sum is a second launch,
+ * comp_inference/linear_triton.py:303-314).
+ *   ci_device_status     copies the status word of the current device to *h_status, clears it, waits for `stream`,
+ *                        and returns CI_ERR_HIP if a bit was set (CI_STATUS_*).  Synchronises: for health checks
+ *                        and tests, not for the token loop.
+ *   ci_debug_wait_limit  sets the number of looks (default 2^22, about a fifth of a second); returns the previous
+ *                        value.  0 makes every such wait give up at once: the give-up path under test.
+ * ------------------------------------------------------------------------------------- */
+#define CI_STATUS_WAIT_GAVE_UP 1u
+int ci_device_status(uint32_t *h_status, ci_stream_t stream);
+uint32_t ci_debug_wait_limit(uint32_t looks);
 
 /* ---------------------------------------------------------------------------------------
  * Verification aids: the contraction of the fused kernels applied to a plain (uncompressed) bf16

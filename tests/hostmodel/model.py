@@ -200,6 +200,12 @@ def in_child(fn):
         if pid == 0:
             os.close(r)
             code = 0
+            # The oracle is OpenMP code, and a process forked from one whose OpenMP runtime already has its worker
+            # threads (an earlier test used the oracle) would wait for those threads for ever: teams of one here.
+            try:
+                C.CDLL("libgomp.so.1").omp_set_num_threads(1)
+            except OSError:
+                pass
             try:
                 fn(*args, **kwargs)
                 payload = pickle.dumps(None)
@@ -223,5 +229,27 @@ def in_child(fn):
         err = pickle.loads(data) if data else f"child exited with {code} and no report"
         if err is not None:
             raise AssertionError(err)
+
+    return wrapper
+
+
+def in_fresh_process(fn):
+    """Like in_child, but the body runs in a new interpreter (the oracle keeps all its threads there): for the few
+    tests whose inputs take the oracle tens of seconds to encode.  The test function must be a module-level one
+    whose arguments have a repr that evaluates to them."""
+    import functools
+    import subprocess
+
+    @functools.wraps(fn)
+    def wrapper(*args, **kwargs):
+        code = (f"import sys; sys.path[:0] = [{ROOT!r}, {os.path.join(ROOT, 'tests')!r}]; import importlib; "
+                f"f = getattr(importlib.import_module({fn.__module__.split('.')[-1]!r}), {fn.__name__!r}); "
+                f"f.__wrapped__(*{args!r}, **{kwargs!r})")
+        p = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True)
+        sys.stderr.write(p.stderr[-4000:])
+        if p.returncode == 70:
+            raise AssertionError("memory fault inside the host model:\n" + p.stderr[-2000:])
+        if p.returncode != 0:
+            raise AssertionError(p.stderr[-6000:] or f"child exited with {p.returncode}")
 
     return wrapper

@@ -6,12 +6,12 @@ against the oracle, every address against the arrays, 256 CUs as on the chip."""
 import numpy as np
 
 from tests.hostmodel import cases
-from tests.hostmodel.model import Model, in_child, weight_bits, x_bits
+from tests.hostmodel.model import Model, in_fresh_process, weight_bits, x_bits
 
 CUS = 256
 
 
-@in_child
+@in_fresh_process
 def test_gate_projection_decode_and_gemv_at_full_size():
     """Configurations 1 and 2: the gate projection decoded in one launch (decoder checkpoints at the middle of every
     stream, as bench.py runs it) and the fused GEMV for one row of x on the prepared weight."""
@@ -43,7 +43,7 @@ def test_gate_projection_decode_and_gemv_at_full_size():
     assert np.allclose(bf16_bits_to_f32(y.get()), want, atol=1e-2, rtol=1e-2)
 
 
-@in_child
+@in_fresh_process
 def test_k_projection_every_operator():
     """1024 x 4096 stored [K = 4096, N = 1024]: decode with and without checkpoints, GEMV / GEMM at the rows of
     configuration 2 and above 64 rows."""
@@ -57,7 +57,7 @@ def test_k_projection_every_operator():
     cases.linear(m, bits, x_bits(128, 4096, 2), 1024, wide=True, expect_kernel="fused_linear32_wide_kernel<4>")
 
 
-@in_child
+@in_fresh_process
 def test_embedding_table_rows_gather_and_lm_head():
     """Configuration 3's 128,256 rows (last tile row 256 rows: its bottom-half streams are empty) and 2048 Zipf(1.1)
     ids from numpy's default_rng(4), on 256 of the 4096 columns: the gather with 8 segments per stream through the

@@ -286,3 +286,33 @@ def test_tile_metadata_that_points_past_the_stream_is_not_followed():
         m.call("ci_fused_embedding_tiled", C.byref(w), ids.p, n_ids, g.p, N, wse.p, C.c_size_t(nbe), None)
         m.call("ci_fused_linear_transposed_tiled", C.byref(w), m.dev(x_bits(1, N, 2)).p, 1, N, None, z.p, K, wst.p, C.c_size_t(nbt), None)
         m.free_all()
+
+
+@in_child
+def test_the_bounded_wait_gives_up_and_says_so():
+    """fused_linear32_seg_kernel for up to four rows of x: a wavefront waits for the one adding up the previous job.
+    With the number of looks forced to zero (ci_debug_wait_limit) every such wait that would have had to wait gives
+    up: the kernel still ends, the device status word says so, ci_device_status returns an error once and is clear
+    after.  With the default limit the word stays clear."""
+    import ctypes as C
+
+    m = Model(cus=1)  # one workgroup takes every job in turn: waits between jobs
+    m.lib.ci_debug_wait_limit.restype = C.c_uint32
+    K, N, th, segs = 768, 200, 256, 2
+    bits = weight_bits(K, N, 1)
+    st = C.c_uint32(7)
+    cases.linear(m, bits, x_bits(2, K, 2), th, segs)
+    assert m.lib.ci_device_status(C.byref(st), None) == 0 and st.value == 0
+    before = m.lib.ci_debug_wait_limit(0)
+    assert before == 1 << 22
+    try:
+        try:
+            cases.linear(m, bits, x_bits(2, K, 2), th, segs)  # the sums may or may not survive: not the point
+        except AssertionError as e:
+            assert "differs" in str(e) or "max error" in str(e), e
+        assert m.violations() == []
+        rc = m.lib.ci_device_status(C.byref(st), None)
+        assert rc == 2 and st.value == 1 and b"bounded wait" in m.lib.ci_last_error(), (rc, st.value)
+        assert m.lib.ci_device_status(C.byref(st), None) == 0 and st.value == 0
+    finally:
+        m.lib.ci_debug_wait_limit(before)

@@ -1,4 +1,4 @@
-"""Random ragged shapes through the host model (tests/hostmodel): some 3,000 seeded cases over the operators, with the
+"""Random ragged shapes through the host model (tests/hostmodel): some 2,500 seeded cases over the operators, with the
 weights' statistics, tile heights, segment counts, row counts, CU counts, the side of the arrays that touches the
 inaccessible page and the order in which the model runs the wavefronts all drawn per case.  Every case checks the
 result against the oracle and that the model saw no address outside an array, no LDS address outside the launch's
@@ -11,7 +11,7 @@ from tests.hostmodel.model import Model, in_child, x_bits
 
 TILE_HEIGHTS = (32, 64, 128, 256, 512, 1024)
 BLOCKS = 12          # child processes per family
-PER_BLOCK = 44       # cases per child: 6 families x 12 x 44 = 3,168 cases, of which a few per cent are refused by the oracle
+PER_BLOCK = 36       # cases per child: 6 families x 12 x 36 = 2,592 cases, of which a few per cent are refused by the oracle
 
 
 def _draw(rng, need_blocks_of_16=True):
