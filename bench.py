@@ -49,11 +49,79 @@ def step_bound_us(wave_steps: int, chain: int) -> dict:
     """Lower bounds from the step rate: throughput (all CUs busy) and latency (one chain)."""
     return {"throughput_us": round(wave_steps * STEP_NS_PER_CU / NUM_CUS * 1e-3, 1),
             "latency_us": round(chain * STEP_NS_LATENCY * 1e-3, 1)}
-# HBM bytes of one batched decode launch on this workload.  Not measured by this program: taken from
-# offline rocprofv3 FETCH_SIZE and WRITE_SIZE passes over this same command, scaled by what the same
-# counters read for a plain copy of known size: 72735.3 KiB x 1.9988 fetched + 212992.0 KiB x 1.0 written.
-MEASURED_TRAFFIC_BYTES = 366_978_000
-TRAFFIC_SOURCE = "profiles/decode_tiled32_seg_kernel_llama8b_layer.md (offline counter passes, not this run)"
+# HBM bytes of one batched decode launch on this workload are not measured by this program: they come from two
+# rocprofv3 counter passes over this same command (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what
+# the same counter reads for a plain copy of known size (--copy-calibration).  `bench.py --record-traffic FETCH.csv
+# WRITE.csv` turns the two counter files into profiles/traffic.json, which also holds a digest of the kernel sources
+# it was taken on; a run reports the figure only while the sources are still those, and null otherwise.
+TRAFFIC_JSON = os.path.join(ROOT, "profiles", "traffic.json")
+TRAFFIC_KERNEL = "decode_tiled32_seg_kernel"
+COPY_KERNEL, COPY_BYTES = "__amd_rocclr_copyBuffer", 64 << 20  # what --copy-calibration launches
+
+
+def sources_digest() -> str:
+    """sha256 over the kernel sources (names and contents): what a counter figure was measured on."""
+    import hashlib
+
+    h = hashlib.sha256()
+    csrc = os.path.join(ROOT, "comp_inference_amd", "csrc")
+    for name in sorted(os.listdir(csrc)):
+        if name.endswith((".hip", ".h")):
+            h.update(name.encode())
+            with open(os.path.join(csrc, name), "rb") as f:
+                h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def _counter_kib(csv_path: str, counter: str, kernel: str, first: int = 0) -> float:
+    """Mean of `counter` over the dispatches of the kernels whose name contains `kernel` (rocprofv3 --pmc, csv);
+    `first` > 0: over the first so many of them only."""
+    import csv
+
+    vals = []
+    with open(csv_path, newline="") as f:
+        for row in csv.DictReader(f):
+            if row["Counter_Name"] == counter and kernel in row["Kernel_Name"]:
+                vals.append((int(row["Dispatch_Id"]), float(row["Counter_Value"])))
+    if not vals:
+        raise SystemExit(f"{csv_path}: no {counter} reading for a kernel named *{kernel}*")
+    vals = [v for _, v in sorted(vals)][:first or None]
+    return sum(vals) / len(vals)
+
+
+def record_traffic(fetch_csv: str, write_csv: str) -> int:
+    """profiles/traffic.json from the two counter files (no GPU needed)."""
+    fetch, write = _counter_kib(fetch_csv, "FETCH_SIZE", TRAFFIC_KERNEL), _counter_kib(write_csv, "WRITE_SIZE", TRAFFIC_KERNEL)
+    # (the calibration copies are the first three copies of the run: --copy-calibration runs before anything is uploaded)
+    f_scale = COPY_BYTES / 1024 / _counter_kib(fetch_csv, "FETCH_SIZE", COPY_KERNEL, first=3)
+    w_scale = COPY_BYTES / 1024 / _counter_kib(write_csv, "WRITE_SIZE", COPY_KERNEL, first=3)
+    rec = {"kernel": TRAFFIC_KERNEL, "workload": "llama3-8b layer, seven tensors, one launch, 2 segments per stream",
+           "fetch_kib": round(fetch, 1), "fetch_scale": round(f_scale, 4), "write_kib": round(write, 1),
+           "write_scale": round(w_scale, 4), "bytes": int(round((fetch * f_scale + write * w_scale) * 1024)),
+           "sources": sources_digest(),
+           "command": "rocprofv3 --pmc FETCH_SIZE (then WRITE_SIZE) --output-format csv -- python3 bench.py --steps 3 --warmup 1 "
+                      "--no-cpu-baseline --no-gemv --no-embedding --no-model --copy-calibration"}
+    with open(TRAFFIC_JSON, "w") as f:
+        json.dump(rec, f, indent=1)
+        f.write("\n")
+    print(json.dumps(rec))
+    return 0
+
+
+def measured_traffic():
+    """(bytes or None, where the answer comes from)."""
+    try:
+        with open(TRAFFIC_JSON) as f:
+            rec = json.load(f)
+    except (OSError, ValueError):
+        return None, "no counter record (profiles/traffic.json)"
+    now = sources_digest()
+    if rec.get("sources") != now or rec.get("kernel") != TRAFFIC_KERNEL:
+        return None, (f"profiles/traffic.json holds {rec.get('bytes')} bytes measured on kernel sources {rec.get('sources')}; "
+                      f"the sources are now {now}: not carried over")
+    return int(rec["bytes"]), "profiles/traffic.json (offline rocprofv3 counter passes over this command on these sources)"
+
+
 LAYER = [("q", 4096, 4096), ("k", 1024, 4096), ("v", 1024, 4096), ("o", 4096, 4096),
          ("gate", 14336, 4096), ("up", 14336, 4096), ("down", 4096, 14336)]  # (name, out, in)
 
@@ -267,7 +335,12 @@ def main() -> int:
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three 64 MiB device-to-device copies, so that a counter run has a "
                          "kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
+    ap.add_argument("--record-traffic", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
+                    help="no benchmark: write profiles/traffic.json from the counter_collection.csv files of a FETCH_SIZE "
+                         "and a WRITE_SIZE pass of rocprofv3 over `bench.py --copy-calibration`")
     a = ap.parse_args()
+    if a.record_traffic:
+        return record_traffic(*a.record_traffic)
     if a.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU part (run with --gpus 1)", file=sys.stderr)
         return 2
@@ -344,9 +417,10 @@ def main() -> int:
     for o, c in zip(ci.rans_decomp_tiled_batch(plain_items, tile_k=th, tile_n=tw), layer):
         assert np.array_equal(o.cpu().numpy(), c.exp_host), f"decode without checkpoints: mismatch on {c.name}"
     us_whole_streams = batched_time_us(lambda: ci.rans_decomp_tiled_batch(plain_items, tile_k=th, tile_n=tw), 5, 20)
+    traffic_bytes, traffic_source = measured_traffic()
     roofline = {"bound": "hbm", "kernel": "decode_tiled32_seg_kernel", "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                "traffic": MEASURED_TRAFFIC_BYTES, "traffic_source": TRAFFIC_SOURCE,
+                "traffic": traffic_bytes, "traffic_source": traffic_source,
                 "bytes_per_launch": int(algo_bytes), "cus": int(NUM_CUS),
                 "launch_us": round(launch_us, 2), "single_tensor_launch_us": per_kernel,
                 "decoder_checkpoint_segments": DECODE_SEGMENTS, "checkpoint_bytes": checkpoint_bytes,

@@ -16,9 +16,10 @@
  *   - LUT: exact-integer floor cross-check, sum/positivity/scan invariants, uniform and
  *     single-symbol closed forms, argmax tie order.
  *   - coder: decode(encode(x)) == x for every layout; state interval invariant
- *     [2^16, 2^24); decoder ends on 2^16 with every byte consumed; agreement with an
- *     independent big-integer ANS on short inputs; closed form for a one-symbol input;
- *     layout invariants of the packed stream (offset scan, zero prefix rows, length).
+ *     [2^16, 2^24); decoder ends on 2^16 with every byte consumed; decode_step(encode_step(x, s))
+ *     == (x, s); an independent plain-integer encoder and decoder (tests/pyref.py) byte for byte;
+ *     closed forms for power-of-two frequencies and a one-symbol input; layout invariants of
+ *     the packed stream (offset scan, zero prefix rows, length).
  *   - mantissa interleave: explicit index formula + inverse.
  *   - fused GEMM numerics restatement: compared with float64 matmul within the
  *     reference's own 1e-2/1e-2 tolerance.
