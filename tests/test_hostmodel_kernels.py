@@ -316,3 +316,21 @@ def test_the_bounded_wait_gives_up_and_says_so():
         assert m.lib.ci_device_status(C.byref(st), None) == 0 and st.value == 0
     finally:
         m.lib.ci_debug_wait_limit(before)
+
+
+@in_child
+def test_tile_bodies_without_a_byte():
+    """A constant exponent plane in low tiles: no stream emits a byte, every tile body has depth 0, every window is
+    empty.  The sixteen-wavefront kernels decode such items like any other (nothing to stage, no byte ever asked for)."""
+    rng = np.random.default_rng(1)
+    V, H, th = 384, 64, 128
+    bits = cases.weight_kind(rng, V, H, "constant")
+    enc, _ = cases.compress(bits, th)
+    assert not enc.tile_max_lens.any() and enc.stream.size == 0
+    m = Model(cus=2)
+    cases.lm_head(m, bits, x_bits(1, H, 2), th, 2, window_rows=True, expect_kernel="trans32_seg_kernel<false>")
+    cases.lm_head(m, bits, x_bits(1, H, 2), th, 2, window_rows=True, matrix_sums=True, check_twin=False,
+                  expect_kernel="trans32_seg_kernel<true>")
+    cases.linear(m, bits, x_bits(1, V, 2), th, 2, window_rows=True, slot_table=True, expect_kernel="fused_linear32_seg_kernel<1, false>")
+    cases.decode(m, bits, th, 2, expect_kernel="decode_tiled32_seg_kernel<false>")
+    cases.gather(m, bits, np.arange(0, V, 5), th, 2, slot_table=True, expect_kernel="embed_gather32_seg_kernel")

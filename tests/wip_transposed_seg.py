@@ -50,6 +50,30 @@ def test_one_row_of_x_on_sixteen_wavefronts(oracle, V, H, segments):
     assert torch.equal(ci.fused_rans_linear_transposed(x, *args, checkpoints=ck, segments=segments), whole)
 
 
+def test_tile_bodies_without_a_byte(oracle):
+    """A constant exponent plane in low tiles: no stream emits a byte, every body has depth 0 and every window is
+    empty; the items are decoded all the same (their rows once surfaced as whatever the workspace held)."""
+    import comp_inference_amd as ci
+
+    V, H, th, segments = 384, 64, 128, 2
+    g = torch.Generator("cpu").manual_seed(1)
+    w = ((1.0 + torch.rand(V, H, generator=g) * 0.99) * torch.where(torch.rand(V, H, generator=g) < 0.5, -1.0, 1.0)).to(torch.bfloat16)
+    enc, man = oracle.compress_bf16(bf16_bits(w), th, 32)
+    assert not enc.tile_max_lens.any()
+    dev = torch.device("cuda", 0)
+    t = [torch.from_numpy(enc.stream).to(dev), _t32(enc.states).to(dev), _t32(enc.tables).to(dev),
+         torch.from_numpy(enc.slot_map).to(dev), _t32(enc.tile_offsets).to(dev), _t32(enc.tile_max_lens).to(dev),
+         torch.from_numpy(man).to(dev)]
+    args = (t[0], t[1], t[2], t[3], (V, H), t[4], t[5], th, 32, t[6])
+    x = make_x(1, H, seed=7).to(dev)
+    whole = ci.fused_rans_linear_transposed(x, *args)
+    ck = ci.build_checkpoints(t[0], t[1], t[2], t[3], (V, H), t[4], t[5], th, 32, segments)
+    torch.full((1 << 20,), float("nan"), device=dev)  # (what a recycled workspace may hold)
+    got = ci.fused_rans_linear_transposed(x, *args, checkpoints=ck, segments=segments, max_window_rows=1)
+    assert torch.equal(got.view(torch.int16), whole.view(torch.int16))
+    assert torch.allclose(got.float().cpu(), x.float().cpu() @ w.float().t(), atol=ATOL, rtol=RTOL)
+
+
 def test_the_module_takes_the_kernel_when_segments_are_switched_on():
     import comp_inference_amd as ci
 
