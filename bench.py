@@ -477,7 +477,7 @@ def main() -> int:
             import comp_inference_amd.linear_hip as lh
 
             wide_rows = []
-            for M in (128, 256, 512, 2048):
+            for M in (16, 64, 128, 256, 512, 2048, 8192):
                 xm = torch.randn(M, gate.K, generator=g, dtype=torch.float32).to(torch.bfloat16).to(dev)
                 policy = lh.DECODE_ONCE_ABOVE_ROWS
                 t_default = batched_time_us(lambda: gate.linear(xm), 5, 20)
@@ -595,6 +595,40 @@ def main() -> int:
                           "hbm_frac_compressed_bytes": round(record("trans32_kernel (+ reduction)", f"{V}x{H} head M=1", head_bytes, us_h), 4),
                           "effective_weight_GBs": round(2 * V * H / (us_h * 1e-6) / 1e9, 1),
                           "torch_matmul_bf16_us": round(us_h_ref, 1)}
+        if a.new_kernels:
+            # the head's sixteen-wavefront kernel for one row of x (decoder checkpoints, largest window from the library),
+            # with the sums by lane exchanges (bit-identical to the default) and on the matrix pipe (within tolerance)
+            import ctypes as C
+
+            from comp_inference_amd import _lib
+
+            variants = []
+            for segs in (2, 4):
+                ck_h = ci.build_checkpoints(emb.stream, emb.states, emb.tables, emb.slot_map, (V, H), emb.tile_offsets,
+                                            emb.tile_max_lens, emb.th, emb.tw, segs)
+                rows_t = torch.zeros(1, dtype=torch.int32, device=dev)
+                desc = _lib.tiled_weight(V, H, emb.th, emb.tw, emb.stream, emb.states, emb.tables, emb.slot_map,
+                                         emb.tile_offsets, emb.tile_max_lens, None, ck_h, segs)
+                _lib.check(_lib.lib().ci_max_window_rows(C.byref(desc), _lib.ptr(rows_t), _lib.stream_handle(dev)))
+                kw = dict(checkpoints=ck_h, segments=segs, max_window_rows=int(rows_t.item()),
+                          slot_table=ci.build_slot_table(emb.tables, emb.slot_map))
+
+                def head_seg():
+                    return ci.fused_rans_linear_transposed(xh, emb.stream, emb.states, emb.tables, emb.slot_map, (V, H),
+                                                           emb.tile_offsets, emb.tile_max_lens, emb.th, emb.tw, emb.man, **kw)
+
+                same = bool(torch.equal(head_seg(), head()))
+                us_seg = batched_time_us(head_seg, 5, 20)
+                ci.head_matrix_sums(True)
+                try:
+                    close = bool(torch.allclose(head_seg().float(), want_logits, atol=1e-2, rtol=1e-2))
+                    us_mat = batched_time_us(head_seg, 5, 20)
+                finally:
+                    ci.head_matrix_sums(False)
+                variants.append({"segments": segs, "max_window_rows": kw["max_window_rows"], "us_lane_exchange_sums": round(us_seg, 1),
+                                 "bit_identical_to_default": same, "us_matrix_pipe_sums": round(us_mat, 1), "allclose_1e-2": close})
+                del ck_h
+            out["lm_head"]["sixteen_wavefronts"] = variants
         del emb, table_dev, table, ck
 
     roofline["kernels"] = kernels
