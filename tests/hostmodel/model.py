@@ -253,3 +253,56 @@ def in_fresh_process(fn):
             raise AssertionError(p.stderr[-6000:] or f"child exited with {p.returncode}")
 
     return wrapper
+
+
+def fork_all(fn, arg_list, jobs: int | None = None):
+    """fn(arg) for every arg, each in a forked child (see in_child), up to `jobs` at a time; raises AssertionError with
+    every failure's report.  The children write nothing but their report."""
+    jobs = jobs or max(1, (os.cpu_count() or 2) - 1)
+    pending, running, failures = list(arg_list), {}, []
+
+    def start(arg):
+        r, w = os.pipe()
+        sys.stdout.flush()
+        sys.stderr.flush()
+        pid = os.fork()
+        if pid == 0:
+            os.close(r)
+            code = 0
+            try:
+                C.CDLL("libgomp.so.1").omp_set_num_threads(1)  # (see in_child)
+            except OSError:
+                pass
+            try:
+                fn(arg)
+                payload = pickle.dumps(None)
+            except BaseException:  # noqa: BLE001
+                payload = pickle.dumps(traceback.format_exc())
+                code = 1
+            with os.fdopen(w, "wb") as f:
+                f.write(payload)
+            sys.stdout.flush()
+            sys.stderr.flush()
+            os._exit(code)
+        os.close(w)
+        running[pid] = (arg, r)
+
+    while pending or running:
+        while pending and len(running) < jobs:
+            start(pending.pop(0))
+        pid, status = os.wait()
+        if pid not in running:
+            continue
+        arg, r = running.pop(pid)
+        with os.fdopen(r, "rb") as f:
+            data = f.read()
+        if os.WIFSIGNALED(status):
+            failures.append(f"[{arg!r}] the child died of signal {os.WTERMSIG(status)}")
+        elif os.WEXITSTATUS(status) == 70:
+            failures.append(f"[{arg!r}] memory fault inside the host model (see the message on stderr)")
+        else:
+            err = pickle.loads(data) if data else f"child exited with {os.WEXITSTATUS(status)} and no report"
+            if err is not None:
+                failures.append(f"[{arg!r}] {err}")
+    if failures:
+        raise AssertionError("\n".join(failures))

@@ -25,6 +25,7 @@ static int g_cus = 8;
 static const char *g_kernel = "(no kernel)";
 static uint64_t g_asm_instructions = 0;
 static bool g_abort_launch = false;
+static bool g_any_memory = false;  // addresses outside the model's own arrays are taken on trust (arrays of the caller's)
 static uint64_t g_schedule = 0;  // 0: wavefronts run in index order; else the seed of a new order every round
 
 struct Fiber;
@@ -51,7 +52,10 @@ struct Alloc {
 static std::vector<Alloc> g_allocs;
 static std::vector<Alloc> g_symbols;  // (no mapping of their own)
 
+static const Alloc g_trusted = {nullptr, 0, nullptr, 0};
+
 static const Alloc *find_alloc(uint64_t addr, size_t n) {
+    if (g_any_memory && addr >= 4096) return &g_trusted;
     for (const Alloc &a : g_allocs)
         if (addr >= (uint64_t)a.ptr && addr + n <= (uint64_t)a.ptr + a.bytes) return &a;
     for (const Alloc &a : g_symbols)
@@ -323,11 +327,17 @@ static inline float bf16_f32(uint16_t h) { return __builtin_bit_cast(float, (uin
 // column l % 32, the same k; C / D: register v of lane l is row 8 (v / 4) + 4 (l / 32) + v % 4, column l % 32.
 // Products are exact in fp32; they are added to the accumulator in ascending k (the hardware's order is its own).
 static void mfma_compute(const uint16_t (*a)[8], const uint16_t (*b)[8], float (*c)[16]) {
+    float af[32][16], bf[32][16];  // [row i][k], [column j][k]
+    for (int l = 0; l < 64; ++l)
+        for (int t = 0; t < 8; ++t) {
+            af[l % 32][8 * (l / 32) + t] = bf16_f32(a[l][t]);
+            bf[l % 32][8 * (l / 32) + t] = bf16_f32(b[l][t]);
+        }
     for (int l = 0; l < 64; ++l)
         for (int v = 0; v < 16; ++v) {
             const int i = 8 * (v / 4) + 4 * (l / 32) + v % 4, j = l % 32;
             float s = c[l][v];
-            for (int k = 0; k < 16; ++k) s += bf16_f32(a[i + 32 * (k / 8)][k % 8]) * bf16_f32(b[j + 32 * (k / 8)][k % 8]);
+            for (int k = 0; k < 16; ++k) s += af[i][k] * bf[j][k];
             c[l][v] = s;
         }
 }
@@ -719,24 +729,38 @@ static void exec_asm(Fiber **lanes, int n_lanes_total, uint64_t part) {
                     violation("`%s`: destination is not a vector register", in.text.c_str());
                     break;
                 }
-                for (int l = 0; l < 64; ++l) {
-                    if (!(w.exec >> l & 1)) continue;
-                    const uint32_t a = vsrc(o[1], l), b = in.nops > 2 ? vsrc(o[2], l) : 0, c = in.nops > 3 ? vsrc(o[3], l) : 0;
-                    uint32_t r = 0;
-                    switch (in.c) {
-                        case I_V_AND: r = a & b; break;
-                        case I_V_LSHRREV: r = b >> (a & 31); break;
-                        case I_V_LSHLREV: r = b << (a & 31); break;
-                        case I_V_SUBREV: r = b - a; break;
-                        case I_V_ADD: r = a + b; break;
-                        case I_V_MOV: r = a; break;
-                        case I_V_MAD_U24: r = (a & 0xFFFFFFu) * (b & 0xFFFFFFu) + c; break;
-                        case I_V_LSHL_OR: r = (a << (b & 31)) | c; break;
-                        case I_V_PERM: r = v_perm(a, b, c); break;
-                        case I_V_AND_OR: r = (a & b) | c; break;
-                        default: break;
+                // sources as arrays of 64 (scalars and literals broadcast), then one plain loop per operation
+                uint32_t bc[3][64];
+                const uint32_t *src[3] = {bc[0], bc[1], bc[2]};
+                for (int k = 1; k <= 3; ++k) {
+                    if (k < in.nops && o[k].k == K_V) {
+                        src[k - 1] = w.v[o[k].reg];
+                    } else {
+                        const uint32_t val = k < in.nops ? vsrc(o[k], 0) : 0u;
+                        for (int l = 0; l < 64; ++l) bc[k - 1][l] = val;
                     }
-                    w.v[o[0].reg][l] = r;
+                }
+                const uint32_t *A = src[0], *B = src[1], *Cs = src[2];
+                uint32_t r[64];
+                switch (in.c) {
+                    case I_V_AND: for (int l = 0; l < 64; ++l) r[l] = A[l] & B[l]; break;
+                    case I_V_LSHRREV: for (int l = 0; l < 64; ++l) r[l] = B[l] >> (A[l] & 31); break;
+                    case I_V_LSHLREV: for (int l = 0; l < 64; ++l) r[l] = B[l] << (A[l] & 31); break;
+                    case I_V_SUBREV: for (int l = 0; l < 64; ++l) r[l] = B[l] - A[l]; break;
+                    case I_V_ADD: for (int l = 0; l < 64; ++l) r[l] = A[l] + B[l]; break;
+                    case I_V_MOV: for (int l = 0; l < 64; ++l) r[l] = A[l]; break;
+                    case I_V_MAD_U24: for (int l = 0; l < 64; ++l) r[l] = (A[l] & 0xFFFFFFu) * (B[l] & 0xFFFFFFu) + Cs[l]; break;
+                    case I_V_LSHL_OR: for (int l = 0; l < 64; ++l) r[l] = (A[l] << (B[l] & 31)) | Cs[l]; break;
+                    case I_V_PERM: for (int l = 0; l < 64; ++l) r[l] = v_perm(A[l], B[l], Cs[l]); break;
+                    case I_V_AND_OR: for (int l = 0; l < 64; ++l) r[l] = (A[l] & B[l]) | Cs[l]; break;
+                    default: break;
+                }
+                uint32_t *D = w.v[o[0].reg];
+                if (w.exec == ~0ull) {
+                    memcpy(D, r, sizeof r);
+                } else {
+                    for (int l = 0; l < 64; ++l)
+                        if (w.exec >> l & 1) D[l] = r[l];
                 }
                 break;
             }
@@ -1235,6 +1259,7 @@ extern "C" void sim_free_all(void) {
 
 extern "C" void sim_set_cus(int n) { g_cus = n > 0 ? n : 1; }
 extern "C" void sim_set_schedule(uint64_t seed) { g_schedule = seed; }
+extern "C" void sim_trust_foreign_memory(int on) { g_any_memory = on != 0; }
 extern "C" int sim_violation_count(void) { return (int)g_viol.size(); }
 extern "C" const char *sim_violation(int i) { return i >= 0 && i < (int)g_viol.size() ? g_viol[i].c_str() : ""; }
 extern "C" void sim_clear(void) {

@@ -77,6 +77,7 @@ void *sim_alloc(size_t bytes, int end_at_guard);  // end_at_guard: 1 = the byte 
 void sim_free_all(void);
 void sim_set_cus(int n);
 void sim_set_schedule(uint64_t seed);  // 0: wavefronts of a workgroup run in index order; else the seed of a new order every round
+void sim_trust_foreign_memory(int on);  // 1: the interpreter also accepts addresses outside sim_alloc's arrays (a caller's own memory)
 int sim_violation_count(void);
 const char *sim_violation(int i);
 void sim_clear(void);  // violations and the launch log

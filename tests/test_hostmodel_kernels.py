@@ -334,3 +334,24 @@ def test_tile_bodies_without_a_byte():
     cases.linear(m, bits, x_bits(1, V, 2), th, 2, window_rows=True, slot_table=True, expect_kernel="fused_linear32_seg_kernel<1, false>")
     cases.decode(m, bits, th, 2, expect_kernel="decode_tiled32_seg_kernel<false>")
     cases.gather(m, bits, np.arange(0, V, 5), th, 2, slot_table=True, expect_kernel="embed_gather32_seg_kernel")
+
+
+# ---- the reference's own parity sweep ---------------------------------------------------------------------------------------
+@pytest.mark.parametrize("th", [32, 64, 128, 256, 512, 1024])
+@in_child
+def test_reference_tile_sweep(th):
+    """tests/test_mat_mul.py:108-264 of the reference: K = 3072 (a multiple of every height), tile heights 32..1024 x
+    widths 16..128, fused result and decode-then-matmul against the product on the decompressed weight within
+    allclose(1e-2, 1e-2).  Here with a quarter of the columns and 24 rows of x instead of 8192 (the CPU model's pace)."""
+    from oracle import rans_oracle as ro
+
+    m = Model(cus=8)
+    K, N, M = 3072, 256, 24
+    bits, xb = weight_bits(K, N, th), x_bits(M, K, 2)
+    for tw in (16, 32, 64, 128):
+        if tw == 32:
+            cases.decode(m, bits, th, merge=True)
+            cases.linear(m, bits, xb, th)
+        else:
+            cases.other_layout_ops(m, bits, xb, np.arange(0, K, 97), th, tw, "ilp2")
+        m.free_all()

@@ -1,4 +1,4 @@
-"""Random ragged shapes through the host model (tests/hostmodel): some 2,500 seeded cases over the operators, with the
+"""Random ragged shapes through the host model (tests/hostmodel): some 4,000 seeded cases over the operators, with the
 weights' statistics, tile heights, segment counts, row counts, CU counts, the side of the arrays that touches the
 inaccessible page and the order in which the model runs the wavefronts all drawn per case.  Every case checks the
 result against the oracle and that the model saw no address outside an array, no LDS address outside the launch's
@@ -7,11 +7,11 @@ import numpy as np
 import pytest
 
 from tests.hostmodel import cases
-from tests.hostmodel.model import Model, in_child, x_bits
+from tests.hostmodel.model import Model, fork_all, x_bits
 
 TILE_HEIGHTS = (32, 64, 128, 256, 512, 1024)
-BLOCKS = 12          # child processes per family
-PER_BLOCK = 36       # cases per child: 6 families x 12 x 36 = 2,592 cases, of which a few per cent are refused by the oracle
+BLOCKS = 12          # child processes per family, run side by side
+PER_BLOCK = 56       # cases per child: 6 families x 12 x 56 = 4,032 cases, of which a few per cent are refused by the oracle
 
 
 def _draw(rng, need_blocks_of_16=True):
@@ -56,9 +56,7 @@ def _run(family, block, body):
     assert ran >= PER_BLOCK * 3 // 4, f"{family}: only {ran} of {PER_BLOCK} cases could be encoded"
 
 
-@pytest.mark.parametrize("block", range(BLOCKS))
-@in_child
-def test_decode_sweep(block):
+def _blocks_of_test_decode_sweep(block):
     def body(rng, m):
         th, segs, K, N, kind = _draw(rng)
         bits = cases.weight_kind(rng, K, N, kind)
@@ -67,9 +65,7 @@ def test_decode_sweep(block):
     _run("decode", block, body)
 
 
-@pytest.mark.parametrize("block", range(BLOCKS))
-@in_child
-def test_fused_linear_sweep(block):
+def _blocks_of_test_fused_linear_sweep(block):
     def body(rng, m):
         th, segs, K, N, kind = _draw(rng)
         M = int(rng.choice((1, 1, 2, 3, 4, 5, 8, 17, 32, 33, 64, 65, 100, 128, 129, 200)))
@@ -84,9 +80,7 @@ def test_fused_linear_sweep(block):
     _run("linear", block, body)
 
 
-@pytest.mark.parametrize("block", range(BLOCKS))
-@in_child
-def test_fused_gather_sweep(block):
+def _blocks_of_test_fused_gather_sweep(block):
     def body(rng, m):
         th, segs, K, N, kind = _draw(rng, need_blocks_of_16=False)
         n = int(rng.choice((1, 2, 7, 64, 65, 200, 700)))
@@ -99,9 +93,7 @@ def test_fused_gather_sweep(block):
     _run("gather", block, body)
 
 
-@pytest.mark.parametrize("block", range(BLOCKS))
-@in_child
-def test_lm_head_sweep(block):
+def _blocks_of_test_lm_head_sweep(block):
     def body(rng, m):
         th, segs, V, H, kind = _draw(rng)
         if rng.random() < 0.6:
@@ -116,9 +108,7 @@ def test_lm_head_sweep(block):
     _run("lm_head", block, body)
 
 
-@pytest.mark.parametrize("block", range(BLOCKS))
-@in_child
-def test_other_layouts_and_encoders_sweep(block):
+def _blocks_of_test_other_layouts_and_encoders_sweep(block):
     from oracle import rans_oracle as ro
 
     def body(rng, m):
@@ -140,9 +130,7 @@ def test_other_layouts_and_encoders_sweep(block):
 FAMILY["hot"] = 6
 
 
-@pytest.mark.parametrize("block", range(BLOCKS))
-@in_child
-def test_hand_scheduled_paths_sweep(block):
+def _blocks_of_test_hand_scheduled_paths_sweep(block):
     """Shapes drawn so that the hand-scheduled paths are the ones taken: the one-pass kernel above 64 rows, the
     sixteen-wavefront kernels of the fused linear (the instance without guarded path) and of the LM head (both kinds
     of sums), the whole-tile kernels."""
@@ -187,3 +175,27 @@ def test_hand_scheduled_paths_sweep(block):
             assert any("decode_tiled32_persist_kernel" in k for k in la), la
 
     _run("hot", block, body)
+
+
+def test_decode_sweep():
+    fork_all(_blocks_of_test_decode_sweep, range(BLOCKS))
+
+
+def test_fused_linear_sweep():
+    fork_all(_blocks_of_test_fused_linear_sweep, range(BLOCKS))
+
+
+def test_fused_gather_sweep():
+    fork_all(_blocks_of_test_fused_gather_sweep, range(BLOCKS))
+
+
+def test_lm_head_sweep():
+    fork_all(_blocks_of_test_lm_head_sweep, range(BLOCKS))
+
+
+def test_other_layouts_and_encoders_sweep():
+    fork_all(_blocks_of_test_other_layouts_and_encoders_sweep, range(BLOCKS))
+
+
+def test_hand_scheduled_paths_sweep():
+    fork_all(_blocks_of_test_hand_scheduled_paths_sweep, range(BLOCKS))
