@@ -120,8 +120,24 @@ class RansLinear(nn.Module):
         ts = (self.rans_exp_stream, self.rans_exp_states, self.rans_man_raw, self.bias)  # (a reload replaces them all)
         return tuple((t.data_ptr(), t.numel(), _version_of(t)) if t is not None else None for t in ts)
 
+    # True: the buffers are converted once per device and the result is kept (PreparedLinear; a module whose buffers
+    # live on the host then holds a device copy for good).  False: the reference's way -- every call moves the buffers
+    # to the input's device and lets go of them afterwards (comp_inference/pytorch_runtime.py:440-459), so a model
+    # larger than the GPU can stay on the host; no decoder checkpoints then (they would be resident derived data).
+    resident = True
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         device = x.device
+        if not self.resident:
+            from .linear_hip import fused_rans_linear
+
+            to = lambda t: t.to(device, non_blocking=True)  # noqa: E731
+            return fused_rans_linear(
+                x=x, compressed_data=to(self.rans_exp_stream), initial_states=to(self.rans_exp_states),
+                tables=to(self.rans_exp_tables), slot_map=to(self.rans_exp_slot_map),
+                weight_shape=(self.in_features, self.out_features), tile_offsets=to(self.rans_exp_tile_offsets),
+                tile_max_lens=to(self.rans_exp_tile_max_lens), tile_k=self.tile_k, tile_n=self.tile_n,
+                mantissas=to(self.rans_man_raw), bias=None if self.bias is None else to(self.bias), SPLIT_K=self.split_k)
         prepared = getattr(self, "_prepared", None)
         key = (self._buffers_key(), device, self.segments)
         if prepared is None or prepared[0] != key:

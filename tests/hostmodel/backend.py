@@ -94,6 +94,7 @@ def python_api_on_hostmodel(cus: int = 8):
         mock.patch.object(torch.cuda, "device", lambda d: contextlib.nullcontext()),
         mock.patch.object(torch.cuda, "current_stream", lambda d=None: _Stream()),
         mock.patch.object(torch.cuda, "current_device", lambda: 0),
+        mock.patch.object(torch.cuda, "set_device", lambda d: None),
         mock.patch.object(torch.cuda, "synchronize", lambda device=None: None),
         mock.patch.object(torch.cuda, "Event", _Event),
         mock.patch.object(torch.cuda, "memory_allocated", lambda device=None: 0),

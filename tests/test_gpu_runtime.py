@@ -438,3 +438,33 @@ def test_reloading_buffers_in_place_is_noticed():
     assert torch.allclose(yb, x.float().cpu() @ wb.float().t(), atol=1e-2, rtol=1e-2)
     assert torch.equal(yb, b(x).float().cpu())
     assert ci.release_scratch() >= 0
+
+
+def test_rans_linear_that_keeps_nothing_on_the_device():
+    """RansLinear.resident = False: the reference's forward (comp_inference/pytorch_runtime.py:440-459) -- the
+    buffers stay where they are (here: on the host), every call moves them to the input's device and drops the
+    copies; the result is the entry point's on the same arguments, and nothing is kept on the module."""
+    import comp_inference_amd as ci
+
+    torch.manual_seed(5)
+    K, N = 1024, 96
+    lin = nn.Linear(K, N, bias=True).to(torch.bfloat16)
+    w, bias = lin.weight.detach().clone(), lin.bias.detach().clone()
+    ci.rans_compress_module_weight(lin, tile_height=512, tile_width=32)
+    rl = ci.RansLinear.from_compressed(lin, bias=bias)
+    rl.resident = False
+    for M in (1, 3, 70):
+        x = torch.randn(M, K).to(torch.bfloat16).cuda()
+        got = rl(x)
+        want = ci.fused_rans_linear_triton(
+            x=x, compressed_data=rl.rans_exp_stream.cuda(), initial_states=rl.rans_exp_states.cuda(),
+            tables=rl.rans_exp_tables.cuda(), slot_map=rl.rans_exp_slot_map.cuda(), weight_shape=(K, N),
+            tile_offsets=rl.rans_exp_tile_offsets.cuda(), tile_max_lens=rl.rans_exp_tile_max_lens.cuda(),
+            tile_k=rl.tile_k, tile_n=rl.tile_n, mantissas=rl.rans_man_raw.cuda(), bias=bias.cuda())
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+        ref = x.float().cpu() @ w.float().t() + bias.float()
+        assert torch.allclose(got.float().cpu(), ref, atol=1e-2, rtol=1e-2)
+    assert not hasattr(rl, "_prepared") and not hasattr(rl, "_ckpt_cache")
+    assert rl.rans_exp_stream.device.type == "cpu"
+    rl.resident = True  # back to the prepared call: a device copy and the checkpoint index are kept from here on
+    assert torch.allclose(rl(x).float().cpu(), ref, atol=1e-2, rtol=1e-2) and hasattr(rl, "_prepared")

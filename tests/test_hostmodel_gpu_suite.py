@@ -15,7 +15,7 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 # file -> tests that must at least have passed there (a guard against a run that silently collects nothing)
 FILES = {"test_gpu_codec.py": 43, "test_gpu_linear.py": 65, "test_gpu_embedding.py": 18, "test_gpu_transposed.py": 21,
-         "test_gpu_runtime.py": 8, "test_gpu_errors.py": 4, "test_golden.py": 1, "test_zz_no_alloc.py": 2,
+         "test_gpu_runtime.py": 9, "test_gpu_errors.py": 4, "test_golden.py": 1, "test_zz_no_alloc.py": 2,
          "test_gpu_zy_device_status.py": 1, "wip_one_stream.py": 15, "wip_transposed_seg.py": 10, "wip_linear_wide.py": 10,
          "wip_gather_seg.py": 8}
 
@@ -39,3 +39,12 @@ def test_gpu_tests_on_the_host_model(runs, name):
     assert rc == 0, out[-6000:]
     m = re.search(r"(\d+) passed", out)
     assert m and int(m.group(1)) >= FILES[name], out[-2000:]
+
+
+def test_smoke_on_the_host_model():
+    """__graft_entry__.smoke() -- encode, decode, fused linear against the oracle, on "cuda:0" -- on the host model."""
+    code = ("import sys; sys.path.insert(0, %r); import __graft_entry__; "
+            "from tests.hostmodel.backend import python_api_on_hostmodel\n"
+            "with python_api_on_hostmodel():\n    __graft_entry__.smoke()\n") % ROOT
+    p = subprocess.run([sys.executable, "-c", code], cwd=ROOT, capture_output=True, text=True)
+    assert p.returncode == 0 and "smoke ok" in p.stdout, (p.stdout + p.stderr)[-3000:]
