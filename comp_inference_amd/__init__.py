@@ -9,12 +9,14 @@ from .comp_inference import (
     extract_exp_and_mantissa,
     get_rans_lut,
     interleave_mantissas,
+    interleave_mantissas_ilp2,
     rans_compress_gate_up_fused,
     rans_compress_module_weight,
     rans_compress_qkv_fused,
     rans_decompress_module_weight,
     reconstruct_from_exp_and_mantissa,
     uninterleave_mantissas,
+    uninterleave_mantissas_ilp2,
 )
 from .embedding_hip import (
     fused_rans_embedding,

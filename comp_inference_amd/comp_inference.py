@@ -63,6 +63,21 @@ def uninterleave_mantissas(interleaved_mantissas, K, N, TILE_K=1024, TILE_N=32):
     return tiled.view(tiles_k * TILE_K, tiles_n * TILE_N)[:K, :N]
 
 
+def interleave_mantissas_ilp2(mantissas: torch.Tensor, TILE_K=128, TILE_N=64):
+    """[K,N] -> flat tile-major plane with each tile stored as its top half (rows 0 .. TILE_K/2) followed by its
+    bottom half   [comp_inference.py:96-129].  Element-for-element the same bytes as `interleave_mantissas` (a tile's
+    halves already follow each other there); the reference keeps the name but calls it nowhere (its two call sites
+    are comments, comp_inference.py:453, :463).  Defaults as the reference's: 128 x 64."""
+    assert TILE_K % 2 == 0, "a tile has two halves"
+    return interleave_mantissas(mantissas.contiguous(), TILE_K=TILE_K, TILE_N=TILE_N)
+
+
+def uninterleave_mantissas_ilp2(interleaved, K, N, TILE_K=128, TILE_N=64):
+    """Inverse of interleave_mantissas_ilp2   [comp_inference.py:132-153]."""
+    assert TILE_K % 2 == 0, "a tile has two halves"
+    return uninterleave_mantissas(interleaved, K, N, TILE_K=TILE_K, TILE_N=TILE_N)
+
+
 def get_rans_lut(data: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     """12-bit frequency and exclusive-cdf tables of a u8 tensor   [comp_inference.py:183-239]
     floor(count/total*4096) in float64, zero -> 1, then the surplus goes to the first maximum or
@@ -190,7 +205,11 @@ def rans_compress_module_weight_bf16(module: nn.Module, skip_mantissa=True, tile
 
 def rans_compress_module_weight(module: nn.Module, tile_height=1024, tile_width=32,
                                 transpose_weight=True, uncoalesced_interleaving=False) -> None:
-    """Dispatcher   [comp_inference.py:548-570]; only bf16 weights are compressed."""
+    """Dispatcher   [comp_inference.py:548-570]; only bf16 weights are compressed.  The reference also names a
+    branch for uint8 / int8 weights (`rans_compress_module_weight_int8`, comp_inference.py:505-545, and its
+    decompressor :716-752); neither can run there (the flat `compress` is called without its required
+    `min_block_size`, src/python_bindings.cpp:225-228, and the decompressor asks for the `weight` the compressor
+    deleted), so there is no behaviour to reproduce and such weights are skipped with the same message."""
     if not hasattr(module, "weight"):
         return
     if module.weight.dtype == torch.bfloat16:

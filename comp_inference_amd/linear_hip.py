@@ -375,3 +375,6 @@ def dense_matmul(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
 
 
 triton_matmul = dense_matmul
+# its two halves take the rows of `a` already flattened to [M, K] (comp_inference/triton_gemm.py:196-321); one library
+# call serves both here
+triton_gemv = triton_gemm = dense_matmul

@@ -131,3 +131,26 @@ def test_interleave_index_formula_and_inverse(oracle, K, N, th, tw):
     assert np.array_equal(ht.numpy(), tiled)
     assert np.array_equal(uninterleave_mantissas(ht, K, N, TILE_K=th, TILE_N=tw).numpy(), plane)
     assert np.array_equal(uninterleave_mantissas(ht[: ht.numel() // 2], K, N, TILE_K=th, TILE_N=tw).numpy(), cut)
+
+
+@pytest.mark.parametrize("K,N,th,tw", [(256, 128, 128, 64), (300, 70, 128, 64), (96, 40, 32, 16)])
+def test_halves_first_layout_of_the_sign_mantissa_plane(K, N, th, tw):
+    """interleave_mantissas_ilp2 (comp_inference.py:96-153): per tile the top half's rows, then the bottom half's --
+    element (tile row tk, tile column tn, half h, row r of the half, column c) at
+    ((((tk * tiles_n + tn) * 2 + h) * th/2 + r) * tw + c, stated here from the reference's stack/view."""
+    from comp_inference_amd import interleave_mantissas_ilp2, uninterleave_mantissas_ilp2
+
+    rng = np.random.default_rng(K + N)
+    plane = rng.integers(1, 256, size=(K, N), dtype=np.uint8)
+    tiled = interleave_mantissas_ilp2(torch.from_numpy(plane), TILE_K=th, TILE_N=tw).numpy()
+    tiles_n, half = -(-N // tw), th // 2
+    assert tiled.size == -(-K // th) * tiles_n * th * tw
+    for _ in range(300):
+        r, c = int(rng.integers(K)), int(rng.integers(N))
+        tk, tn, h, rr = r // th, c // tw, (r % th) // half, (r % th) % half
+        assert tiled[((((tk * tiles_n + tn) * 2 + h) * half + rr) * tw) + c % tw] == plane[r, c]
+    assert int((tiled != 0).sum()) == K * N
+    assert np.array_equal(uninterleave_mantissas_ilp2(torch.from_numpy(tiled), K, N, TILE_K=th, TILE_N=tw).numpy(), plane)
+    # the reference's defaults are 128 x 64
+    assert np.array_equal(interleave_mantissas_ilp2(torch.from_numpy(plane)).numpy(),
+                          interleave_mantissas_ilp2(torch.from_numpy(plane), 128, 64).numpy())
