@@ -126,6 +126,12 @@ LAYER = [("q", 4096, 4096), ("k", 1024, 4096), ("v", 1024, 4096), ("o", 4096, 40
          ("gate", 14336, 4096), ("up", 14336, 4096), ("down", 4096, 14336)]  # (name, out, in)
 
 
+# the other workloads of the line (module constants so that a rehearsal of this file can run them small)
+GEMV_ROWS = (1, 4, 16, 64)
+GEMM_ROWS = (16, 64, 128, 256, 512, 2048, 8192)
+EMBED_SHAPE = (128256, 4096, 2048)  # table rows, columns, ids
+
+
 def log(msg: str) -> None:
     print(msg, file=sys.stderr, flush=True)
 
@@ -447,11 +453,11 @@ def main() -> int:
     if not a.no_gemv:
         gate = next(c for c in layer if c.name == "gate")
         g = torch.Generator("cpu").manual_seed(2)
-        x_all = torch.randn(64, gate.K, generator=g, dtype=torch.float32).to(torch.bfloat16).to(dev)
+        x_all = torch.randn(max(GEMV_ROWS), gate.K, generator=g, dtype=torch.float32).to(torch.bfloat16).to(dev)
         w_dense = ci.rans_decomp_tiled(gate.stream, gate.states, gate.tables, gate.slot_map, (gate.K, gate.N),
                                        gate.tile_offsets, gate.tile_max_lens, mantissas=gate.man)
         rows = []
-        for M in (1, 4, 16, 64):
+        for M in GEMV_ROWS:
             x = x_all[:M].contiguous()
             got = gate.linear_segmented(x).float()
             want = torch.matmul(x, w_dense).float()
@@ -460,7 +466,7 @@ def main() -> int:
             us_plain = batched_time_us(lambda: gate.linear(x), 25, 100)
             us_ref = batched_time_us(lambda: torch.matmul(x, w_dense), 25, 100)
             nbytes = gate.linear_bytes(M)
-            record("fused linear (checkpoints)", f"gate K=4096 N=14336 M={M}", nbytes, us)
+            record("fused linear (checkpoints)", f"gate K={gate.K} N={gate.N} M={M}", nbytes, us)
             sb = step_bound_us(gate.wave_steps(), gate.th // 2 // int(gate.segments))
             rows.append({"M": M, "us": round(us, 2), "us_without_checkpoints": round(us_plain, 2), "allclose_1e-2": ok,
                          "step_rate_bound_us": max(sb["throughput_us"], sb["latency_us"]),
@@ -470,14 +476,14 @@ def main() -> int:
                          "mfma_util_vs_2500_TFLOPs": round(2 * M * gate.K * gate.N / (us * 1e-6) / 1e12 / 2500.0, 5),
                          "torch_matmul_bf16_us": round(us_ref, 2),
                          "torch_matmul_weight_GBs": round(2 * gate.K * gate.N / (us_ref * 1e-6) / 1e9, 1)})
-        out["fused_gemv"] = {"layer": "gate K=4096 N=14336", "bytes_M1": gate.linear_bytes(1), "rows": rows}
+        out["fused_gemv"] = {"layer": f"gate K={gate.K} N={gate.N}", "bytes_M1": gate.linear_bytes(1), "rows": rows}
         if a.new_kernels:
             # more than 64 rows of x: the fused kernel that decodes once per 64 rows, the one that decodes once per
             # 128 / 256 rows (must give the same bits), and the default policy (decode once to HBM + library GEMM)
             import comp_inference_amd.linear_hip as lh
 
             wide_rows = []
-            for M in (16, 64, 128, 256, 512, 2048, 8192):
+            for M in GEMM_ROWS:
                 xm = torch.randn(M, gate.K, generator=g, dtype=torch.float32).to(torch.bfloat16).to(dev)
                 policy = lh.DECODE_ONCE_ABOVE_ROWS
                 t_default = batched_time_us(lambda: gate.linear(xm), 5, 20)
@@ -499,7 +505,7 @@ def main() -> int:
                                   "us_decode_once_plus_library_gemm": round(t_default, 1),
                                   "mfma_util_vs_2500_TFLOPs": round(flops / (t_wide * 1e-6) / 1e12 / 2500.0, 4),
                                   "torch_matmul_bf16_us": round(t_ref, 1)})
-            out["fused_gemm_rows"] = {"layer": "gate K=4096 N=14336", "rows": wide_rows}
+            out["fused_gemm_rows"] = {"layer": f"gate K={gate.K} N={gate.N}", "rows": wide_rows}
 
     # --- the four GEMVs of a decoder layer at M = 1 (q/k/v and gate/up fused along the outputs, as the
     # runtime modules hold them), with decoder checkpoints where the library suggests them
@@ -531,7 +537,7 @@ def main() -> int:
     # --- fused decompress-gather on a 128256 x 4096 table, 2048 Zipf(1.1) ids
     if not a.no_embedding:
         log("generating and compressing the embedding table (seed 3) ...")
-        V, H, T = 128256, 4096, 2048
+        V, H, T = EMBED_SHAPE
         g = torch.Generator("cpu").manual_seed(3)
         table = (torch.randn(V, H, generator=g, dtype=torch.float32) * 0.02).to(torch.bfloat16)
         emb = Compressed("embed", table, dev, transpose=False)

@@ -31,6 +31,15 @@ class _Event:
         return 1e-3
 
 
+class _Properties:
+    """torch.cuda.get_device_properties for code that asks for the CU count."""
+
+    name, gcnArchName, total_memory = "host model", "gfx950:host-model", 288 << 30
+
+    def __init__(self, cus):
+        self.multi_processor_count = cus
+
+
 _CPU = torch.device("cpu")
 
 
@@ -99,6 +108,8 @@ def python_api_on_hostmodel(cus: int = 8):
         mock.patch.object(torch.cuda, "Event", _Event),
         mock.patch.object(torch.cuda, "memory_allocated", lambda device=None: 0),
         mock.patch.object(torch.cuda, "is_available", lambda: True),
+        mock.patch.object(torch.cuda, "get_device_properties", lambda d=None: _Properties(cus)),
+        mock.patch.object(torch.cuda, "empty_cache", lambda: None),
         # operands are "on the GPU" wherever the package asks (the host model is the GPU here)
         mock.patch.object(torch.Tensor, "is_cuda", property(lambda self: True)),
     ]
