@@ -122,7 +122,7 @@ __device__ __forceinline__ void decode_one_item(const DecodeArgs &a, uint32_t it
             st.init_at<kStride>(stage, row - w_lo + 1, lane, state);
         } else {
             stage_window_pair(stage, src_a, win_a, src_b, win_b, hsel, deepest, lane);
-            const int32_t rel = row - w_lo;  // this lane's next byte, in rows of the window (< 0: none left)
+            const int32_t rel = max(row - w_lo, -1);  // this lane's next byte, in rows of the window (-1: none left)
             st.X = state << 3;
             st.q = (uint32_t)(uintptr_t)stage + (uint32_t)(rel * 64 + lane);
             st.n1 = rel >= 0 ? stage[rel * 64 + lane] : 0;
@@ -346,7 +346,7 @@ __device__ __forceinline__ void dec_run(const DecodeArgs &a, const DecItem &it, 
     const uint32_t hsel = it.co.hsel, seg = it.co.seg, p = it.co.p, tk = it.co.tk;
     const uint32_t half = a.th / 2, seglen = a.seglen, row_first = tk * a.th + hsel * half + seg * seglen;
     FastLane st;
-    const int32_t rel = it.row - (int32_t)it.w_lo;  // this lane's next byte, in rows of the window (< 0: none left)
+    const int32_t rel = max(it.row - (int32_t)it.w_lo, -1);  // this lane's next byte, in rows of the window (-1: none left)
     st.X = it.state << 3;
     st.q = (uint32_t)(uintptr_t)stage + (uint32_t)(rel * 64 + lane);
     st.n1 = rel >= 0 ? stage[rel * 64 + lane] : 0;  // (a wavefront's LDS operations complete in order)

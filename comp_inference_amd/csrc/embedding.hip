@@ -696,7 +696,7 @@ __device__ __forceinline__ void emb_run(const EmbedArgs &a, const EmbItem &it, u
     const uint32_t col = (it.pair * 2 + side) * 32 + c;
     const uint8_t *man = a.man_tiled + (size_t)(it.tile_a + side) * a.th * 32 + (size_t)it.tile_row0 * 32 + c;
     FastLane st;
-    const int32_t rel = it.row - (int32_t)it.w_lo;  // this lane's next byte, in rows of the window (< 0: none left)
+    const int32_t rel = max(it.row - (int32_t)it.w_lo, -1);  // this lane's next byte, in rows of the window (-1: none left)
     st.X = it.state << 3;
     st.q = (uint32_t)(uintptr_t)stage + (uint32_t)(rel * 64 + lane);
     st.n1 = rel >= 0 ? stage[rel * 64 + lane] : 0;  // (a wavefront's LDS operations complete in order)

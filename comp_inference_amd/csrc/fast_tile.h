@@ -389,6 +389,7 @@ struct FastLane {
     template <uint32_t kStride = kFastStride>
     __device__ __forceinline__ void init_at(const uint8_t *stage, int32_t have, uint32_t q_lane, uint32_t state) {
         X = state << 3;
+        have = max(have, 0);  // (a checkpoint read from a damaged file may say anything: no address is formed from it unclamped)
         const uint8_t *col = stage + q_lane * kStride;
         q = (uint32_t)(uintptr_t)col + (uint32_t)have - 1;  // low 32 bits of an LDS pointer are its LDS address
         n1 = have >= 1 ? col[have - 1] : 0;

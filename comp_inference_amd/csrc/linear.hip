@@ -697,7 +697,7 @@ __device__ __forceinline__ void seg_run(const LinearArgs &a, const SegItem &it, 
     const uint32_t k0 = tk * a.th + hsel * half + seg * seglen;
     FastLane st;
     st.X = it.state << 3;
-    const int32_t rel = it.row - (int32_t)it.lo;  // this lane's next byte, in rows of the window (< 0: none left)
+    const int32_t rel = max(it.row - (int32_t)it.lo, -1);  // this lane's next byte, in rows of the window (-1: none left)
     st.q = (uint32_t)(uintptr_t)stage + (uint32_t)(rel * 64 + lane);
     st.n1 = rel >= 0 ? stage[rel * 64 + lane] : 0;
     const uint32_t m = c;  // row of x this lane feeds to the (first) MFMA

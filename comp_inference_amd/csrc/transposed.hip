@@ -306,7 +306,7 @@ __device__ __forceinline__ void trans_one_segment(const TransArgs &a, uint32_t t
     // and the steps below never ask for a byte)
     stage_window(stage, a.stream + base + (size_t)lo * 64, rows, lane);
     FastLane st;
-    const int32_t rel = row - lo;  // this lane's next byte, in rows of the window (< 0: none left)
+    const int32_t rel = max(row - lo, -1);  // this lane's next byte, in rows of the window (-1: none left)
     st.X = state << 3;
     st.q = (uint32_t)(uintptr_t)stage + (uint32_t)(rel * 64 + lane);
     st.n1 = rel >= 0 ? stage[rel * 64 + lane] : 0;  // (a wavefront's LDS operations complete in order)

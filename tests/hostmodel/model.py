@@ -61,6 +61,12 @@ class Dev:
             C.memmove(out.ctypes.data, self.ptr, self.nbytes)
         return out
 
+    def put(self, values: np.ndarray) -> None:
+        a = np.ascontiguousarray(values, self.dtype)
+        assert a.size * a.itemsize == self.nbytes, (a.shape, self.shape)
+        if self.nbytes:
+            C.memmove(self.ptr, a.ctypes.data, self.nbytes)
+
 
 class ModelError(AssertionError):
     pass
@@ -260,6 +266,9 @@ def fork_all(fn, arg_list, jobs: int | None = None):
     every failure's report.  The children write nothing but their report."""
     jobs = jobs or max(1, (os.cpu_count() or 2) - 1)
     pending, running, failures = list(arg_list), {}, []
+    from tests.hostmodel import build
+
+    build.build()  # once, here: children that each found the library out of date would all write it at the same time
 
     def start(arg):
         r, w = os.pipe()

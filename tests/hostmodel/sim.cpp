@@ -25,6 +25,7 @@ static int g_cus = 8;
 static const char *g_kernel = "(no kernel)";
 static uint64_t g_asm_instructions = 0;
 static bool g_abort_launch = false;
+static bool g_lds_reads_clamped = false;  // LDS reads beyond the launch's LDS give 0, as on the hardware, instead of a violation
 static bool g_any_memory = false;  // addresses outside the model's own arrays are taken on trust (arrays of the caller's)
 static uint64_t g_schedule = 0;  // 0: wavefronts run in index order; else the seed of a new order every round
 
@@ -835,6 +836,10 @@ static void exec_asm(Fiber **lanes, int n_lanes_total, uint64_t part) {
                 for (int l = 0; l < 64; ++l) {
                     if (!(w.exec >> l & 1)) continue;
                     const uint64_t addr = (uint64_t)w.v[o[1].reg][l] + (uint32_t)in.offset;
+                    if (addr + nb > g_lds_launch && g_lds_reads_clamped) {
+                        for (int j = 0; j < nr; ++j) w.v[o[0].reg + j][l] = 0;
+                        continue;
+                    }
                     if (addr + nb > g_lds_launch) {
                         g_cur = lanes[l] ? lanes[l] : g_cur;
                         violation("`%s`: lane %d reads LDS address 0x%llx, the launch has %zu bytes", in.text.c_str(), l,
@@ -1260,6 +1265,7 @@ extern "C" void sim_free_all(void) {
 extern "C" void sim_set_cus(int n) { g_cus = n > 0 ? n : 1; }
 extern "C" void sim_set_schedule(uint64_t seed) { g_schedule = seed; }
 extern "C" void sim_trust_foreign_memory(int on) { g_any_memory = on != 0; }
+extern "C" void sim_lds_reads_out_of_range_give_zero(int on) { g_lds_reads_clamped = on != 0; }
 extern "C" int sim_violation_count(void) { return (int)g_viol.size(); }
 extern "C" const char *sim_violation(int i) { return i >= 0 && i < (int)g_viol.size() ? g_viol[i].c_str() : ""; }
 extern "C" void sim_clear(void) {

@@ -78,6 +78,10 @@ void sim_free_all(void);
 void sim_set_cus(int n);
 void sim_set_schedule(uint64_t seed);  // 0: wavefronts of a workgroup run in index order; else the seed of a new order every round
 void sim_trust_foreign_memory(int on);  // 1: the interpreter also accepts addresses outside sim_alloc's arrays (a caller's own memory)
+// 1: an LDS read of an assembly statement beyond the launch's LDS gives 0 and is no violation.  That is what the hardware does
+// (out-of-range LDS reads return zero, writes are dropped), and it is the wrong setting for every test but one: on inputs an
+// encoder wrote no kernel forms such an address, and one that does has a defect.  For inputs that are damaged on purpose.
+void sim_lds_reads_out_of_range_give_zero(int on);
 int sim_violation_count(void);
 const char *sim_violation(int i);
 void sim_clear(void);  // violations and the launch log

@@ -177,6 +177,83 @@ def _blocks_of_test_hand_scheduled_paths_sweep(block):
     _run("hot", block, body)
 
 
+FAMILY["corrupt"] = 7
+
+
+def _blocks_of_test_corrupted_contents_sweep(block):
+    """A compressed tensor whose CONTENTS are not what an encoder wrote -- a damaged file, a wrong tensor under the
+    right name: stream bytes, decoder states, tile body offsets and depths, frequency tables, the slot table and the
+    decoder checkpoints replaced by random numbers, one kind or all of them at once, with every array still as long
+    as the shape says (lengths are checked on the host).  Nothing can be said about the results; what is required is
+    that every operator returns, that no kernel reads or writes outside the arrays it was given or outside its LDS,
+    and that no wavefront waits for ever.  Two allowances, both for what the hardware itself tolerates: tile body
+    offsets stay multiples of 16 (a misaligned 16-byte load is legal on the GPU and traps in the x86 build of the
+    kernels), and a decoder fed with noise may take more bytes than its window holds, i.e. read LDS below its window
+    and in rare cases below address 0 -- out-of-range LDS reads return zero on the hardware, and the model is told to
+    do the same for this sweep only."""
+    import ctypes as C
+
+    def body(rng, m):
+        th = int(rng.choice((128, 256, 1024)))
+        K = th * int(rng.integers(1, 3)) + int(rng.integers(0, 40)) * int(rng.random() < 0.4)
+        N = 32 * int(rng.integers(1, 4)) if rng.random() < 0.5 else int(rng.integers(1, 100))
+        from tests.hostmodel.model import weight_bits
+
+        enc, man = cases.compress(weight_bits(K, N, int(rng.integers(1 << 30))), th)
+        what = str(rng.choice(("stream", "states", "offsets", "depths", "tables", "checkpoints", "slot_table", "all")))
+        hit = lambda name: what in (name, "all")  # noqa: E731
+        u32 = lambda n: rng.integers(0, 1 << 32, n, dtype=np.uint64).astype(np.uint32)  # noqa: E731
+        if hit("stream"):
+            enc.stream = rng.integers(0, 256, enc.stream.size, dtype=np.uint8)
+        if hit("states"):
+            enc.states = u32(enc.states.size)
+        if hit("offsets"):
+            enc.tile_offsets = (np.where(rng.random(enc.tile_offsets.size) < 0.5, u32(enc.tile_offsets.size),
+                                         rng.integers(0, enc.stream.size + 200, enc.tile_offsets.size)).astype(np.int64) & ~15).astype(np.uint32)
+        if hit("depths"):
+            enc.tile_max_lens = np.where(rng.random(enc.tile_max_lens.size) < 0.2, u32(enc.tile_max_lens.size),
+                                         rng.integers(0, 600, enc.tile_max_lens.size)).astype(np.uint32)
+        if hit("tables"):
+            enc.tables, enc.slot_map = u32(enc.tables.size), rng.integers(0, 256, enc.slot_map.size, dtype=np.uint8)
+        segs = int(rng.choice([s for s in (1, 2, 4) if (th // 2) % (16 * s) == 0]))
+        slot = bool(rng.random() < 0.6)
+        w, keep = m.weight(enc, man, K, N, segments=segs, slot_table=slot, window_rows=bool(rng.random() < 0.6))
+        if hit("checkpoints") and segs > 1:
+            keep["ckpt"].put(u32(keep["ckpt"].shape[0]))
+        if hit("slot_table") and slot:
+            keep["slot_table"].put(u32(keep["slot_table"].shape[0]))
+        if rng.random() < 0.3:
+            w.max_window_rows = int(rng.integers(1, 113))  # and a promise about the windows that nothing backs
+        M = int(rng.choice((1, 3, 20, 70)))
+        out, x, y = m.empty((K, N), np.uint8), m.dev(x_bits(M, K, 2)), m.empty((M, N), np.uint16)
+        nb = m.lib.ci_fused_linear_workspace_bytes_segmented(M, K, N, th, 32, 0, segs)
+        ws = m.empty(max(nb, 16), np.uint8)
+        ids = m.dev(rng.integers(-2, K + 2, 50).astype(np.int64))
+        g = m.empty((50, N), np.uint16)
+        nbe = m.lib.ci_fused_embedding_workspace_bytes_segmented(50, K, th, segs)
+        wse = m.empty(max(nbe, 16), np.uint8)
+        Mh = int(rng.choice((1, 1, 4)))
+        z, xh = m.empty((Mh, K), np.uint16), m.dev(x_bits(Mh, N, 2))
+        nbt = m.lib.ci_fused_linear_transposed_workspace_bytes(Mh, N, K, 32)
+        wst = m.empty(max(nbt, 16), np.uint8)
+        m.lib.ci_fused_linear_transposed_matrix_sums(int(rng.random() < 0.3))
+        m.lib.sim_lds_reads_out_of_range_give_zero(1)
+        m.clear()
+        try:
+            # (m.call raises on an error code and on anything the model reports)
+            m.call("ci_decode_tiled", C.byref(w), out.p, None, None)
+            m.call("ci_fused_linear_tiled", C.byref(w), x.p, M, K, None, y.p, N, ws.p, C.c_size_t(nb), None)
+            m.call("ci_fused_embedding_tiled", C.byref(w), ids.p, 50, g.p, N, wse.p, C.c_size_t(nbe), None)
+            m.call("ci_fused_linear_transposed_tiled", C.byref(w), xh.p, Mh, N, None, z.p, K, wst.p, C.c_size_t(nbt), None)
+        except BaseException as e:  # noqa: BLE001
+            raise AssertionError(f"{what} damaged, th {th}, K {K}, N {N}, {segs} segments, slot table {slot}: {e}") from e
+        finally:
+            m.lib.ci_fused_linear_transposed_matrix_sums(0)
+            m.lib.sim_lds_reads_out_of_range_give_zero(0)
+
+    _run("corrupt", block, body)
+
+
 def test_decode_sweep():
     fork_all(_blocks_of_test_decode_sweep, range(BLOCKS))
 
@@ -199,3 +276,7 @@ def test_other_layouts_and_encoders_sweep():
 
 def test_hand_scheduled_paths_sweep():
     fork_all(_blocks_of_test_hand_scheduled_paths_sweep, range(BLOCKS))
+
+
+def test_corrupted_contents_sweep():
+    fork_all(_blocks_of_test_corrupted_contents_sweep, range(BLOCKS))
