@@ -429,6 +429,13 @@ int ci_decode_tiled_ilp2_segmented(const uint8_t *d_stream, uint64_t stream_len,
  * those of the reference's fused_rans_linear_triton (comp_inference/linear_triton.py:229-246), which
  * passes torch tensors and checks nothing.  Default format only (two streams per column).
  *
+ * What the arrays CONTAIN is not checked and need not be trusted for memory safety: with every length in
+ * order, no kernel forms a global address from a value it read -- a tile body that would end past
+ * stream_len is taken as empty, a checkpoint's position is clamped to its tile body and to the item's
+ * window, table lookups are masked to the table -- so a damaged file gives wrong numbers, never an access
+ * outside the arrays (d_tile_offsets should be multiples of 16, as an encoder writes them; others cost
+ * unaligned loads).
+ *
  * d_checkpoints / segments: NULL / 0 or 1, or the index made by ci_build_checkpoints_ilp2.
  * d_slot_table: NULL, or the 32 KB made by ci_build_slot_table; a kernel then copies the table
  * instead of building it from d_tables and d_slot_map in every workgroup.
