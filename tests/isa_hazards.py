@@ -207,6 +207,28 @@ def kernels_of(disassembly: str, is_kernel=lambda name: name.startswith("_Z")) -
     return out
 
 
+def labels_of(disassembly: str) -> dict:
+    """{symbol: address} of everything the disassembly names: kernels and the named labels of assembly statements."""
+    return {m.group(2): int(m.group(1), 16) for m in map(SYMBOL.match, disassembly.splitlines()) if m}
+
+
+def kind_of(ins: Ins) -> str:
+    """The issue class of an instruction, for counting what a loop costs."""
+    if ins.mfma:
+        return "mfma"
+    if ins.valu:
+        return "valu"
+    if ins.lds:
+        return "lds"
+    if ins.vmem:
+        return "vmem"
+    if ins.mn in ("s_waitcnt", "s_nop"):
+        return "wait"
+    if ins.mn == "s_branch" or ins.mn.startswith("s_cbranch_"):
+        return "branch"
+    return "salu"
+
+
 def nearest_producer(body: list, start: int, limit: int, is_producer):
     """(wait states, index) of the producer from which `start` is reached with the fewest wait states in between,
     along any path, looking back at most `limit` wait states; None if there is none."""

@@ -107,3 +107,46 @@ def test_the_built_library_leaves_every_wait_state(tmp_path):
     for rule in ("sgpr_vmem", "sgpr_valu", "vgpr_dpp", "vgpr_readlane", "trans_use", "dst_sel", "vgpr_mfma", "vgpr_permlane",
                  "mfma_result"):
         assert closest.get(rule) == CASES[rule][2], (rule, closest.get(rule))
+
+
+# What one pass of each hand-scheduled loop issues, by class, in the built library (steps = decode steps of the
+# 64 streams of a wavefront).  The loops are assembly text, so these are exact; a change to the step shows up here and
+# in the figures the design notes quote per step.  The two-byte renormalisation (about one step in a thousand) runs
+# out of line and is not part of the loop body.
+LOOPS = {
+    # stand-alone decode: a pair of steps and the two exponent bytes they store
+    "ci_dec_loop": dict(steps=2, valu=20, lds=4, salu=6, vmem=2, branch=4, wait=4, mfma=0),
+    # fused linear, up to 32 rows of x: two blocks of eight steps, their sign|mantissa and x loads, two matrix instructions
+    "ci_lin_loop": dict(steps=16, valu=164, lds=32, salu=42, vmem=18, branch=18, wait=36, mfma=2),
+    # the same for 33 to 64 rows: a second x fragment per block and a second matrix instruction
+    "ci_lin2_loop": dict(steps=16, valu=166, lds=32, salu=42, vmem=20, branch=18, wait=36, mfma=4),
+}
+
+
+@pytest.mark.skipif(not (os.path.exists(OBJDUMP) and os.path.exists(LIB)), reason="needs the built library and llvm-objdump")
+def test_what_the_hand_scheduled_loops_issue_per_step(tmp_path):
+    import collections
+    import re
+
+    shutil.copy(LIB, tmp_path / "lib.so")
+    subprocess.run([OBJDUMP, "--offloading", "lib.so"], cwd=tmp_path, check=True, capture_output=True)
+    seen = collections.Counter()
+    for f in sorted(os.listdir(tmp_path)):
+        if "gfx950" not in f:
+            continue
+        text = subprocess.run([OBJDUMP, "-d", str(tmp_path / f)], check=True, capture_output=True, text=True).stdout
+        labels = {a: n for n, a in H.labels_of(text).items() if re.fullmatch(r"ci_(dec|lin|lin2)_loop\d+", n)}
+        for body in H.kernels_of(text).values():
+            for i, ins in enumerate(body):
+                if ins.addr not in labels:
+                    continue
+                family = re.sub(r"\d+$", "", labels[ins.addr])
+                end = next(j for j in range(i, len(body)) if body[j].mn == "s_branch" and body[j].succ == [i])
+                loop = body[i:end + 1]
+                count = collections.Counter(H.kind_of(k) for k in loop)
+                count["steps"] = sum(1 for k in loop if k.mn == "v_mad_u32_u24")
+                want = LOOPS[family]
+                assert {k: count.get(k, 0) for k in want} == want, (labels[ins.addr], dict(count))
+                seen[family] += 1
+    # every kernel that contains a statement has its own copy of the loop
+    assert seen["ci_dec_loop"] >= 2 and seen["ci_lin_loop"] >= 4 and seen["ci_lin2_loop"] >= 4, seen
