@@ -881,12 +881,15 @@ __global__ __launch_bounds__(kSegWaves *kWave) void fused_linear32_seg_kernel(Li
             float *buf = reinterpret_cast<float *>(lds + kSmallBufOff);
             uint32_t *flags = reinterpret_cast<uint32_t *>(lds + kSmallFlagsOff);
             const uint32_t jn = sl / jb.R;  // which of this workgroup's jobs
-            // (the wavefront adding up the job before this one is not waiting for us; the wait is bounded all the same)
-            for (uint32_t looks = 0; __hip_atomic_load(&flags[1], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) != jn; ++looks) {
+            // (the wavefront adding up the job before this one is not waiting for us; the wait is bounded all the same.
+            // The limit is tested before the flag, so that a limit of 0 gives up whatever the flag says: the forced
+            // give-up of the tests does not depend on who got where first)
+            for (uint32_t looks = 0;; ++looks) {
                 if (looks >= a.wait_limit) {
                     if (lane == 0) atomicOr(&g_device_status, (uint32_t)CI_STATUS_WAIT_GAVE_UP);
                     break;
                 }
+                if (__hip_atomic_load(&flags[1], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) == jn) break;
                 __builtin_amdgcn_s_sleep(2);
             }
             if (c < a.M) {

@@ -22,7 +22,8 @@ def _prepared(K, N, th, segs, dev):
 
 
 def test_forced_give_up_ends_the_kernel_and_is_reported():
-    """The number of looks forced to zero from the host: every wait that would have waited gives up.  The kernel
+    """The number of looks forced to zero from the host: every wait gives up without looking at its flag, whoever
+    got where first.  The kernel
     ends all the same, ci_device_status says what happened once and is clear afterwards; with the default limit
     the same launches leave the status word clear and give the usual sums."""
     dev = torch.device("cuda", 0)

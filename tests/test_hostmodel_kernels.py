@@ -291,8 +291,8 @@ def test_tile_metadata_that_points_past_the_stream_is_not_followed():
 @in_child
 def test_the_bounded_wait_gives_up_and_says_so():
     """fused_linear32_seg_kernel for up to four rows of x: a wavefront waits for the one adding up the previous job.
-    With the number of looks forced to zero (ci_debug_wait_limit) every such wait that would have had to wait gives
-    up: the kernel still ends, the device status word says so, ci_device_status returns an error once and is clear
+    With the number of looks forced to zero (ci_debug_wait_limit) every such wait gives up without looking at its
+    flag: the kernel still ends, the device status word says so, ci_device_status returns an error once and is clear
     after.  With the default limit the word stays clear."""
     import ctypes as C
 
