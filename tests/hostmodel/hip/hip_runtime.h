@@ -131,7 +131,10 @@ static inline hipError_t hipGetDeviceProperties(hipDeviceProp_t *p, int) {
     p->multiProcessorCount = sim::cu_count();
     return hipSuccess;
 }
-static inline hipError_t hipFuncSetAttribute(const void *, hipFuncAttribute, int) { return hipSuccess; }
+static inline hipError_t hipFuncSetAttribute(const void *fn, hipFuncAttribute attr, int value) {
+    if (attr == hipFuncAttributeMaxDynamicSharedMemorySize) sim::allow_dynamic_lds(fn, value);
+    return hipSuccess;
+}
 static inline hipError_t hipGetLastError() { return sim::take_launch_error(); }
 static inline const char *hipGetErrorString(hipError_t e) { return e ? "host model: kernel launch failed" : "no error"; }
 static inline hipError_t hipMemsetAsync(void *p, int v, size_t n, hipStream_t) {
@@ -150,4 +153,4 @@ static inline hipError_t hipGetSymbolAddress(void **out, void *sym) {
 }
 
 #define hipLaunchKernelGGL(kernel, grid, block, shmem, stream, ...) \
-    sim::launch(#kernel, (grid), (block), (size_t)(shmem), [=]() { kernel(__VA_ARGS__); })
+    sim::launch(#kernel, reinterpret_cast<const void *>(kernel), (grid), (block), (size_t)(shmem), [=]() { kernel(__VA_ARGS__); })

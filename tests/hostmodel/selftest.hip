@@ -32,6 +32,14 @@ __global__ void st_global_load_kernel(const uint32_t *src, uint32_t n, uint32_t 
     dst[lane] = v;
 }
 
+// the last byte of a large dynamic LDS area, written and read back
+__global__ void st_big_lds_kernel(uint32_t *dst, uint32_t lds_bytes) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    if (threadIdx.x == 0) lds[lds_bytes - 1] = 0x5A;
+    __syncthreads();
+    dst[threadIdx.x] = lds[lds_bytes - 1];
+}
+
 // which: 0 correct; 1 lane 5 reads one byte past the launch's LDS; 2 the statement ends with the read in flight
 __global__ void st_lds_read_kernel(uint32_t *dst, uint32_t lds_bytes, int which) {
     extern __shared__ __align__(16) uint8_t lds[];
@@ -171,6 +179,11 @@ __global__ void st_plain_overrun_kernel(const uint32_t *src, uint32_t n, uint32_
 extern "C" {
 void simtest_global_load(const uint32_t *src, uint32_t n, uint32_t *dst, int which) {
     hipLaunchKernelGGL(st_global_load_kernel, dim3(1), dim3(64), 0, nullptr, src, n, dst, which);
+}
+// allowed: whether hipFuncSetAttribute is called first, as a launch with more than 64 KB of dynamic LDS needs
+void simtest_big_lds(uint32_t *dst, uint32_t lds_bytes, int allowed) {
+    if (allowed) (void)hipFuncSetAttribute(reinterpret_cast<const void *>(st_big_lds_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    hipLaunchKernelGGL(st_big_lds_kernel, dim3(1), dim3(64), lds_bytes, nullptr, dst, lds_bytes);
 }
 void simtest_lds_read(uint32_t *dst, uint32_t lds_bytes, int which) {
     hipLaunchKernelGGL(st_lds_read_kernel, dim3(1), dim3(64), lds_bytes, nullptr, dst, lds_bytes, which);

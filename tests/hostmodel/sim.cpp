@@ -1175,11 +1175,24 @@ static bool run_workgroup(uint32_t nthreads, const LaneCtx &proto) {
     }
 }
 
-void launch(const char *name, Dim3 grid, Dim3 block, size_t shmem, const std::function<void()> &body) {
+static std::map<const void *, int> g_dynamic_lds_allowed;
+void allow_dynamic_lds(const void *fn, int bytes) { g_dynamic_lds_allowed[fn] = bytes; }
+
+void launch(const char *name, const void *fn, Dim3 grid, Dim3 block, size_t shmem, const std::function<void()> &body) {
     sim_init();
     g_launches.push_back(name);
     const uint32_t nthreads = block.x * block.y * block.z;
     g_kernel = name;
+    if (shmem > 65536) {
+        const auto it = g_dynamic_lds_allowed.find(fn);
+        if (it == g_dynamic_lds_allowed.end() || (size_t)it->second < shmem) {
+            violation("launch with %zu bytes of dynamic LDS, and hipFuncSetAttribute(MaxDynamicSharedMemorySize) allowed this kernel %d: "
+                      "the GPU runtime refuses such a launch", shmem, it == g_dynamic_lds_allowed.end() ? 65536 : it->second);
+            g_launch_error = 719;
+            g_kernel = "(no kernel)";
+            return;
+        }
+    }
     if (nthreads == 0 || nthreads > kMaxThreads || block.y != 1 || block.z != 1 || shmem > kLdsBytes ||
         (uint64_t)grid.x * grid.y * grid.z == 0) {
         violation("launch configuration: grid (%u,%u,%u) block (%u,%u,%u) LDS %zu", grid.x, grid.y, grid.z, block.x, block.y, block.z, shmem);

@@ -63,7 +63,10 @@ struct AsmOperand {
 void run_asm(const char *tmpl, AsmOperand *ops, int n_ops);
 
 // launches
-void launch(const char *name, Dim3 grid, Dim3 block, size_t shmem, const std::function<void()> &body);
+// `fn` = the kernel's address, the key under which allow_dynamic_lds recorded what hipFuncSetAttribute was given: a launch
+// that asks for more than 64 KB of dynamic LDS without it fails on the GPU, and is a violation here.
+void launch(const char *name, const void *fn, Dim3 grid, Dim3 block, size_t shmem, const std::function<void()> &body);
+void allow_dynamic_lds(const void *fn, int bytes);
 int take_launch_error();
 int cu_count();
 uint8_t *lds_base();

@@ -58,6 +58,22 @@ def test_lds_reads_of_the_interpreter_are_bounded_by_the_launch():
 
 
 @in_child
+def test_more_than_64_kb_of_dynamic_lds_needs_the_function_attribute():
+    """The GPU runtime refuses a launch with more than 64 KB of dynamic LDS unless hipFuncSetAttribute raised the
+    kernel's limit first; so does the model (every large-LDS launch of the library goes through this check)."""
+    m = Model()
+    dst = _u32(m, 64)
+    m.lib.simtest_big_lds(dst.p, 100 << 10, 0)
+    assert any("bytes of dynamic LDS" in s and "65536" in s for s in m.violations()), m.violations()
+    m.clear()
+    m.lib.simtest_big_lds(dst.p, 64 << 10, 0)  # up to 64 KB need nothing
+    m.lib.simtest_big_lds(dst.p, 100 << 10, 1)
+    assert m.violations() == [] and (dst.get() == 0x5A).all()
+    m.lib.simtest_big_lds(dst.p, 150 << 10, 0)  # allowed 100 KB so far
+    assert any("allowed this kernel 102400" in s for s in m.violations()), m.violations()
+
+
+@in_child
 def test_execution_masks():
     m = Model()
     data = m.dev(np.arange(64, dtype=np.uint32))
