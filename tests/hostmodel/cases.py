@@ -219,14 +219,19 @@ def encode(m: Model, exp_plane, th, tw, layout="ilp2"):
 
 
 # ---- the operators on the other layouts (one thread per stream) ---------------------------------------------------------
-def other_layout_ops(m: Model, bits, xb, ids, th, tw, layout):
+def other_layout_ops(m: Model, bits, xb, ids, th, tw, layout, damage=None):
     """decode, fused linear, gather and LM head of the one-stream-per-column layout ("one") or the dense layout
-    ("dense") or another tile width of the default layout ("ilp2"), against the oracle."""
+    ("dense") or another tile width of the default layout ("ilp2"), against the oracle.  `damage(enc)` may overwrite
+    the encoder's arrays first (same lengths): the operators must then still return without anything the model
+    reports, and their results are not looked at."""
     K, N = bits.shape
     e, man_plane = ro.split_bf16(bits)
     f, c = ro.get_lut(e)
     man = ro.interleave_plane(man_plane, th, tw)
     enc = {"one": ro.encode_tiled_one, "dense": ro.encode_tiled_dense, "ilp2": ro.encode_tiled_ilp2}[layout](e, f, c, th, tw)
+    intact = damage is None
+    if not intact:
+        damage(enc)
     d = dict(stream=m.dev(enc.stream), states=m.dev(enc.states), tables=m.dev(enc.tables), slot_map=m.dev(enc.slot_map), man=m.dev(man))
     if layout == "dense":
         sizes = np.diff(np.append(enc.stream_offsets, enc.stream.size).astype(np.int64)).astype(np.uint32)
@@ -239,10 +244,10 @@ def other_layout_ops(m: Model, bits, xb, ids, th, tw, layout):
     # decode: exponent plane, then merged bf16
     out = m.empty((K, N), np.uint8)
     m.call(f"ci_decode_tiled_{suffix}", *common, K, N, th, tw, out.p, None, None, None)
-    assert np.array_equal(out.get(), e), f"{layout}: decoded plane differs"
+    assert not intact or np.array_equal(out.get(), e), f"{layout}: decoded plane differs"
     outb = m.empty((K, N), np.uint16)
     m.call(f"ci_decode_tiled_{suffix}", *common, K, N, th, tw, None, d["man"].p, outb.p, None)
-    assert np.array_equal(outb.get(), bits), f"{layout}: decoded bf16 differs"
+    assert not intact or np.array_equal(outb.get(), bits), f"{layout}: decoded bf16 differs"
     # fused linear
     M = xb.shape[0]
     x, y = m.dev(xb), m.empty((M, N), np.uint16)
@@ -250,7 +255,7 @@ def other_layout_ops(m: Model, bits, xb, ids, th, tw, layout):
     ws, ws_n = _ws(m, nb)
     m.call(f"ci_fused_linear_{suffix}", x.p, M, K, N, K, *common, d["man"].p, th, tw, None, y.p, N, ws.p, ws_n, None)
     want = ro.linear_f32(xb, bits)
-    assert np.allclose(bf16_bits_to_f32(y.get()), want, atol=1e-2, rtol=1e-2), f"{layout}: fused linear"
+    assert not intact or np.allclose(bf16_bits_to_f32(y.get()), want, atol=1e-2, rtol=1e-2), f"{layout}: fused linear"
     # gather
     ids = np.ascontiguousarray(ids, np.int64)
     g = m.empty((ids.size, N), np.uint16)
@@ -263,7 +268,7 @@ def other_layout_ops(m: Model, bits, xb, ids, th, tw, layout):
     wantg = np.zeros((ids.size, N), np.uint16)
     ok = (ids >= 0) & (ids < K)
     wantg[ok] = bits[ids[ok]]
-    assert np.array_equal(g.get(), wantg), f"{layout}: gathered rows differ"
+    assert not intact or np.array_equal(g.get(), wantg), f"{layout}: gathered rows differ"
     # LM head: the same arrays read as a [V = K, H = N] table
     xh = xb[:, :N] if xb.shape[1] >= N else np.resize(xb, (M, N))
     xh = np.ascontiguousarray(xh)
@@ -273,5 +278,5 @@ def other_layout_ops(m: Model, bits, xb, ids, th, tw, layout):
     m.call(f"ci_fused_linear_transposed_{suffix}", m.dev(xh).p, M, N, K, N, *common, d["man"].p, th, tw, None, z.p, K, wst.p,
            wst_n, None)
     wantz = ro.linear_f32(xh, np.ascontiguousarray(bits.T))
-    assert np.allclose(bf16_bits_to_f32(z.get()), wantz, atol=1e-2, rtol=1e-2), f"{layout}: LM head"
+    assert not intact or np.allclose(bf16_bits_to_f32(z.get()), wantz, atol=1e-2, rtol=1e-2), f"{layout}: LM head"
     return m.launches()

@@ -193,7 +193,43 @@ def _blocks_of_test_corrupted_contents_sweep(block):
     do the same for this sweep only."""
     import ctypes as C
 
+    def other_layouts(rng, m):
+        # the one-stream, dense and other-width layouts (bare-pointer entry points: the lengths are the caller's word)
+        th, tw = int(rng.choice((16, 64, 256))), int(rng.choice((8, 32, 64)))
+        layout = ("one", "dense", "ilp2")[int(rng.integers(0, 3))]
+        if layout == "ilp2" and tw == 32:
+            tw = 16
+        K, N = int(rng.integers(1, 3 * th)), int(rng.integers(1, 2 * tw + 9))
+        what = str(rng.choice(("stream", "states", "meta", "tables", "all")))
+        hit = lambda name: what in (name, "all")  # noqa: E731
+        u32 = lambda n: rng.integers(0, 1 << 32, n, dtype=np.uint64).astype(np.uint32)  # noqa: E731
+
+        def damage(enc):
+            if hit("stream"):
+                enc.stream = rng.integers(0, 256, enc.stream.size, dtype=np.uint8)
+            if hit("states"):
+                enc.states = u32(enc.states.size)
+            if hit("tables"):
+                enc.tables, enc.slot_map = u32(enc.tables.size), rng.integers(0, 256, enc.slot_map.size, dtype=np.uint8)
+            if hit("meta"):
+                noise = lambda a: np.where(rng.random(a.size) < 0.5, u32(a.size),  # noqa: E731
+                                           rng.integers(0, enc.stream.size + 200, a.size)).astype(np.uint32)
+                if layout == "dense":
+                    enc.stream_offsets = noise(enc.stream_offsets)
+                else:
+                    enc.tile_offsets, enc.tile_max_lens = noise(enc.tile_offsets), noise(enc.tile_max_lens)
+
+        from tests.hostmodel.model import weight_bits
+
+        try:
+            cases.other_layout_ops(m, weight_bits(K, N, int(rng.integers(1 << 30))), x_bits(int(rng.integers(1, 6)), max(K, N), 3)[:, :K],
+                                   rng.integers(-1, K + 1, 9), th, tw, layout, damage=damage)
+        except BaseException as e:  # noqa: BLE001
+            raise AssertionError(f"{layout} layout, {what} damaged, tile {th}x{tw}, K {K}, N {N}: {e}") from e
+
     def body(rng, m):
+        if rng.random() < 0.3:
+            return other_layouts(rng, m)
         th = int(rng.choice((128, 256, 1024)))
         K = th * int(rng.integers(1, 3)) + int(rng.integers(0, 40)) * int(rng.random() < 0.4)
         N = 32 * int(rng.integers(1, 4)) if rng.random() < 0.5 else int(rng.integers(1, 100))
