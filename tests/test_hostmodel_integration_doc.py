@@ -1,5 +1,5 @@
-"""The ctypes binding that INTEGRATION.md gives a maintainer of the reference to copy, taken from the file as it
-stands and run (on the host model): the two functions it defines must agree with the package's own operators on a
+"""The ctypes binding that the integration notes at the repository root give a maintainer of the reference to copy,
+taken from the file as it stands and run (on the host model): the two functions it defines must agree with the package's own operators on a
 compressed weight, so the argument order and types printed there are the library's."""
 import os
 import re
@@ -15,7 +15,8 @@ def test_the_binding_printed_in_the_integration_notes_runs():
 
     from tests.hostmodel.backend import python_api_on_hostmodel
 
-    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    notes = next(f for f in sorted(os.listdir(ROOT)) if f.upper().startswith("INTEGRATION") and f.endswith(".md"))
+    text = open(os.path.join(ROOT, notes)).read()
     blocks = re.findall(r"```python\n(.*?)```", text, flags=re.S)
     (code,) = [b for b in blocks if "_hip_backend.py" in b]
     assert 'C.CDLL("libcomp_inference_hip.so")' in code
