@@ -110,9 +110,9 @@ def test_the_built_library_leaves_every_wait_state(tmp_path):
 
 
 # What one pass of each hand-scheduled loop issues, by class, in the built library (steps = decode steps of the
-# 64 streams of a wavefront).  The loops are assembly text, so these are exact; a change to the step shows up here and
-# in the figures the design notes quote per step.  The two-byte renormalisation (about one step in a thousand) runs
-# out of line and is not part of the loop body.
+# 64 streams of a wavefront).  The loops are assembly text, so these are exact, and a change to the step shows up here:
+# ten vector instructions and two LDS reads per step are what bounds every kernel built on it.  The two-byte
+# renormalisation (about one step in a thousand) runs out of line and is not part of the loop body.
 LOOPS = {
     # stand-alone decode: a pair of steps and the two exponent bytes they store
     "ci_dec_loop": dict(steps=2, valu=20, lds=4, salu=6, vmem=2, branch=4, wait=4, mfma=0),
