@@ -225,6 +225,8 @@ def _blocks_of_test_corrupted_contents_sweep(block):
             cases.other_layout_ops(m, weight_bits(K, N, int(rng.integers(1 << 30))), x_bits(int(rng.integers(1, 6)), max(K, N), 3)[:, :K],
                                    rng.integers(-1, K + 1, 9), th, tw, layout, damage=damage)
         except BaseException as e:  # noqa: BLE001
+            if isinstance(e, RuntimeError) and "outgrew" in str(e):
+                raise  # (the oracle could not encode this plane: not a case, see _run)
             raise AssertionError(f"{layout} layout, {what} damaged, tile {th}x{tw}, K {K}, N {N}: {e}") from e
 
     def body(rng, m):
