@@ -45,9 +45,20 @@ STEP_NS_LATENCY = 87.0
 NUM_CUS = 256  # replaced by the device's own count in main()
 
 
+# Two floors no schedule gets under, from what the step is made of: ten VALU instructions of 64 lanes on four 16-lane SIMDs
+# at 2.4 GHz (the chip's 39 T integer lane-operations a second) are 4.17 ns of a CU per wavefront-step, and the LDS
+# pipe needs 2.64 + 1.95 ns for the step's random 8-byte table read and its byte read (the same microbenchmark).
+STEP_VALU_INSTRUCTIONS = 10
+STEP_NS_VALU_FLOOR = STEP_VALU_INSTRUCTIONS * 64 / (4 * 16 * 2.4)  # ns of one CU
+STEP_NS_LDS_FLOOR = 2.64 + 1.95
+
+
 def step_bound_us(wave_steps: int, chain: int) -> dict:
-    """Lower bounds from the step rate: throughput (all CUs busy) and latency (one chain)."""
+    """Lower bounds from the step rate: throughput (all CUs busy) at the measured rate and at the step's VALU-issue and
+    LDS-pipe floors, and latency (one chain)."""
     return {"throughput_us": round(wave_steps * STEP_NS_PER_CU / NUM_CUS * 1e-3, 1),
+            "valu_issue_floor_us": round(wave_steps * STEP_NS_VALU_FLOOR / NUM_CUS * 1e-3, 1),
+            "lds_pipe_floor_us": round(wave_steps * STEP_NS_LDS_FLOOR / NUM_CUS * 1e-3, 1),
             "latency_us": round(chain * STEP_NS_LATENCY * 1e-3, 1)}
 # HBM bytes of one batched decode launch on this workload are not measured by this program: they come from two
 # rocprofv3 counter passes over this same command (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what
