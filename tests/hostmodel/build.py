@@ -203,5 +203,47 @@ def build(force: bool = False, verbose: bool = False) -> str:
     return LIB_PATH
 
 
+def build_mutant(tag: str, edits: list, rebuild: list) -> str:
+    """The host-model library with a deliberate mistake in the kernels: `edits` = [(file under csrc, old text, new text[, occurrences])],
+    the first occurrence of each old text replaced (of one, unless stated); `rebuild` = the .hip sources to compile again from the edited copy (the other
+    objects are the intact build's).  Returns the path of the mutant library, under _build/mutants/<tag>/.  For the
+    tests that show that a mistake of a given kind in the real kernels is noticed."""
+    import shutil
+
+    build()
+    base = os.path.join(OUT_DIR, "mutants", tag)
+    src_dir = os.path.join(base, "csrc")
+    shutil.rmtree(base, ignore_errors=True)
+    shutil.copytree(CSRC, src_dir, ignore=shutil.ignore_patterns("*.o", "*.so"))
+    for name, old_text, new_text, *occurrences in edits:
+        path = os.path.join(src_dir, name)
+        text = open(path).read()
+        want = occurrences[0] if occurrences else 1  # how often the text occurs; the first occurrence is replaced
+        assert text.count(old_text) == want, f"{name}: {text.count(old_text)} occurrences of {old_text!r}"
+        with open(path, "w") as f:
+            f.write(text.replace(old_text, new_text, 1))
+    procs, objs = [], []
+    for src in SOURCES + ["selftest.hip"]:
+        if src not in rebuild:
+            objs.append(os.path.join(OUT_DIR, src + ".o"))
+            continue
+        pre = subprocess.run([CXX, "-E", "-x", "c++", "-std=c++17", "-I", HERE, "-I", src_dir, os.path.join(src_dir, src), "-o", "-"],
+                             check=True, capture_output=True, text=True).stdout
+        ii, obj = os.path.join(base, src + ".ii"), os.path.join(base, src + ".o")
+        with open(ii, "w") as f:
+            f.write(rewrite(pre))
+        procs.append((src, subprocess.Popen([CXX, "-x", "c++-cpp-output", *CXXFLAGS, "-c", ii, "-o", obj],
+                                            stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+        objs.append(obj)
+    objs.append(os.path.join(OUT_DIR, "sim.o"))
+    for src, p in procs:
+        out, _ = p.communicate()
+        if p.returncode != 0:
+            raise RuntimeError(f"mutant {tag}: build failed on {src}:\n{out[-3000:]}")
+    lib = os.path.join(base, "libci_hostmodel.so")
+    subprocess.check_call([CXX, "-shared", "-fPIC", "-o", lib, *objs])
+    return lib
+
+
 if __name__ == "__main__":
     print(build(force="--force" in sys.argv, verbose=True))

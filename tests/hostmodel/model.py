@@ -73,10 +73,10 @@ class ModelError(AssertionError):
 
 
 class Model:
-    def __init__(self, cus: int = 8, end_at_guard: bool = True, schedule: int = 0):
+    def __init__(self, cus: int = 8, end_at_guard: bool = True, schedule: int = 0, lib_path: str | None = None):
         from tests.hostmodel import build
 
-        self.lib = C.CDLL(build.build())
+        self.lib = C.CDLL(lib_path or build.build())  # (lib_path: a build with a deliberate mistake, build.build_mutant)
         L = self.lib
         L.sim_alloc.restype = C.c_void_p
         L.sim_alloc.argtypes = [C.c_size_t, C.c_int]

@@ -92,6 +92,7 @@ void *register_symbol(void *p, size_t bytes) {
 // ---- LDS ------------------------------------------------------------------------------------------------------
 constexpr size_t kLdsBytes = 160 * 1024;
 static uint8_t *g_lds = nullptr;
+static size_t g_lds_open = kLdsBytes;  // bytes of the LDS area that are accessible: the running launch's dynamic LDS, to the page
 static size_t g_lds_launch = 0;  // dynamic LDS the running launch asked for
 
 uint8_t *lds_base() { return g_lds; }
@@ -1100,7 +1101,7 @@ static bool run_workgroup(uint32_t nthreads, const LaneCtx &proto) {
         g_fib[t].ctx = proto;
         g_fib[t].ctx.thread_idx = Dim3(t, 0, 0);
     }
-    memset(g_lds, 0xCD, kLdsBytes);
+    memset(g_lds, 0xCD, g_lds_open);
     const uint32_t n_waves = (nthreads + 63) / 64;
     uint32_t order[kMaxThreads / 64];
     for (uint32_t i = 0; i < n_waves; ++i) order[i] = i;
@@ -1201,6 +1202,9 @@ void launch(const char *name, const void *fn, Dim3 grid, Dim3 block, size_t shme
     g_body = &body;
     // kernels with static LDS arrays get them as ordinary statics; only dynamic LDS is bounded for the interpreter
     g_lds_launch = shmem;
+    // ... and for plain C++ accesses, to the page: what lies behind the launch's dynamic LDS is inaccessible while it runs
+    g_lds_open = (shmem + 4095) & ~(size_t)4095;
+    if (g_lds_open < kLdsBytes) mprotect(g_lds + g_lds_open, kLdsBytes - g_lds_open, PROT_NONE);
     g_abort_launch = false;
     LaneCtx proto;
     proto.block_dim = block;
@@ -1211,6 +1215,8 @@ void launch(const char *name, const void *fn, Dim3 grid, Dim3 block, size_t shme
                 proto.block_idx = Dim3(x, y, z);
                 if (!run_workgroup(nthreads, proto)) g_abort_launch = true;
             }
+    mprotect(g_lds, kLdsBytes, PROT_READ | PROT_WRITE);
+    g_lds_open = kLdsBytes;
     g_cur = nullptr;
     g_body = nullptr;
     g_kernel = "(no kernel)";
@@ -1227,7 +1233,7 @@ static void on_segv(int, siginfo_t *info, void *) {
     // (async-signal-unsafe calls: the process is about to end anyway)
     const uint64_t addr = (uint64_t)info->si_addr;
     fprintf(stderr, "host model: memory fault at %p %s: %s\n", info->si_addr, where().c_str(),
-            addr >= (uint64_t)g_lds && addr < (uint64_t)g_lds + kLdsBytes + 4096 ? "past the end of the LDS" : describe_address(addr).c_str());
+            addr >= (uint64_t)g_lds && addr < (uint64_t)g_lds + kLdsBytes + 4096 ? "in the LDS area, past the end of this launch's dynamic LDS" : describe_address(addr).c_str());
     fflush(stderr);
     _exit(70);
 }

@@ -1,0 +1,102 @@
+"""Does the host model (tests/hostmodel) notice a mistake in the REAL kernels?  Each case builds the library with one
+deliberate slip of a kind that is easy to make in this code -- a wait that covers one load too few, a prefetch that
+does not wrap at the end of its tile, a lane-exchange control in the wrong direction, a row stored one position down,
+a work-space size one group short -- runs the ordinary test case of that operator, and requires that
+it fails, and by which means: the interpreter's load tracking, the exact extents of the arrays, the inaccessible page
+behind an array, or the comparison with the oracle.  (The self-check file shows the same detectors on made-up kernels;
+this one shows that the library's own code paths run through them.)"""
+import numpy as np
+import pytest
+
+from tests.hostmodel import build, cases
+from tests.hostmodel.model import Model, in_child, weight_bits, x_bits
+
+MUTANTS = {
+    # the pack of rows 0/1 waits for all but FIVE of the loads in flight; six lets the row-1 dword be used too early
+    "wait_one_load_short": dict(
+        edits=[("fast_tile.h", '"s_waitcnt vmcnt(5)\\n" CI_PACK("v72", "v74", C0, C1, "v108")',
+                '"s_waitcnt vmcnt(6)\\n" CI_PACK("v72", "v74", C0, C1, "v108")')],
+        rebuild=["linear.hip"], op="linear", expect="before the s_waitcnt"),
+    # the loads of the block after the last wrap to block 0 so that they stay inside the tile
+    "prefetch_runs_off_the_plane": dict(
+        edits=[("fast_tile.h", """                                                uint32_t nblocks, uint32_t qdec = 1) {
+    const uint32_t wrap_m = 0u - (nblocks - 1) * 256u, wrap_x = 0u - (nblocks - 1) * xstep;""",
+                """                                                uint32_t nblocks, uint32_t qdec = 1) {
+    const uint32_t wrap_m = 0x100u, wrap_x = 0u - (nblocks - 1) * xstep;""")],
+        rebuild=["linear.hip"], op="linear", expect="outside every allocation"),
+    # row_shl:4 / row_shr:4 pick the other four-lane group of a row: swapped, every sum takes the wrong partner
+    "lane_exchange_direction": dict(
+        edits=[("transposed.hip", "dpp_add<0x104>(t0), c1 = dpp_add<0x114>(t1)", "dpp_add<0x114>(t0), c1 = dpp_add<0x104>(t1)")],
+        rebuild=["transposed.hip"], op="lm_head", expect="LM head"),
+    # a gathered row goes to the position its id came from
+    "row_stored_one_position_down": dict(
+        edits=[("embedding.hip", "a.out[(size_t)p * a.out_stride + col] = (uint16_t)assemble_bf16(sym, man_cur[u]);",
+                "a.out[(size_t)(p + 1) * a.out_stride + col] = (uint16_t)assemble_bf16(sym, man_cur[u]);", 2)],
+        rebuild=["embedding.hip"], op="gather", expect=("memory fault", "gathered rows differ")),
+    # --- in the kernels that have not run on a GPU yet ---
+    # more than 64 rows in one pass: the last block loads its own operands again instead of the block after the tile's end
+    "one_pass_kernel_prefetches_past_the_tile": dict(
+        edits=[("linear.hip", "const uint32_t nb = blk + 1 < nblk ? blk + 1 : blk;  // (the last block re-reads its own: stays inside the tile)",
+                "const uint32_t nb = blk + 1;")],
+        rebuild=["linear.hip"], op="wide", expect=("memory fault", "outside every allocation")),
+    # the gather on sixteen wavefronts stages windows as they lie: a lane's next byte is 64 bytes down, not 1
+    "gather_window_pointer_step": dict(
+        edits=[("embedding.hip", "sym = advance_asm(st, want + 1 - done, 64) >> 24;", "sym = advance_asm(st, want + 1 - done, 1) >> 24;")],
+        rebuild=["embedding.hip"], op="gather16", expect=("gathered rows differ", "reads LDS address")),
+    # the head's sums on the matrix pipe: the second block of a pair belongs to columns 8..15 / 24..31 of the one-hot operand
+    "one_hot_operands_swapped": dict(
+        edits=[("transposed.hip", "const u32x4 hot0 = mine && (n % 16) / 8 == 0 ? one : none, hot1 = mine && (n % 16) / 8 == 1 ? one : none;",
+                "const u32x4 hot0 = mine && (n % 16) / 8 == 1 ? one : none, hot1 = mine && (n % 16) / 8 == 0 ? one : none;")],
+        rebuild=["transposed.hip"], op="lm_head_matrix", expect="LM head"),
+    # the fragment copy of x holds whole groups of 32 rows
+    "fragment_copy_one_group_short": dict(
+        edits=[("linear.hip", "    return M > 32 ? 2 * ceil_div(M, 64u) : 1u;", "    return M > 32 ? 2 * ceil_div(M, 64u) - 1 : 1u;")],
+        rebuild=["linear.hip"], op="linear64", expect=("outside every allocation", "memory fault", "max error", "differs")),
+}
+
+
+def _run(op: str, lib_path: str):
+    m = Model(cus=2, lib_path=lib_path)
+    if op == "linear":
+        cases.linear(m, weight_bits(2048, 64, 1), x_bits(3, 2048, 2), 1024, 2, slot_table=True, window_rows=True)
+    elif op == "linear64":
+        cases.linear(m, weight_bits(1024, 64, 1), x_bits(40, 1024, 2), 1024)
+    elif op == "lm_head":
+        cases.lm_head(m, weight_bits(2048, 64, 1), x_bits(1, 64, 2), 1024, check_twin=False)
+    elif op == "wide":
+        cases.linear(m, weight_bits(1024, 64, 1), x_bits(129, 1024, 2), 1024, wide=True, expect_kernel="fused_linear32_wide_kernel")
+    elif op == "gather16":
+        ids = np.arange(0, 2048, 3, dtype=np.int64)
+        cases.gather(m, weight_bits(2048, 64, 1), ids, 1024, 8, slot_table=True, expect_kernel="embed_gather32_seg_kernel")
+    elif op == "lm_head_matrix":
+        cases.lm_head(m, weight_bits(2048, 64, 1), x_bits(1, 64, 2), 1024, 2, slot_table=True, window_rows=True,
+                      matrix_sums=True, check_twin=False, expect_kernel="trans32_seg_kernel<true>")
+    elif op == "gather":
+        ids = np.array([0, 5, 2047, 2048, 1024, 7, -1, 2047], np.int64)
+        cases.gather(m, weight_bits(2048, 64, 1), ids, 1024)  # (two column tiles: the hand-scheduled path)
+
+
+@pytest.fixture(scope="module")
+def libraries():
+    # the compilations of all mutants side by side
+    from concurrent.futures import ThreadPoolExecutor
+
+    build.build()
+    with ThreadPoolExecutor(len(MUTANTS)) as pool:
+        futures = {tag: pool.submit(build.build_mutant, tag, mu["edits"], mu["rebuild"]) for tag, mu in MUTANTS.items()}
+        return {tag: f.result() for tag, f in futures.items()}
+
+
+def test_the_cases_pass_on_the_intact_library():
+    for op in sorted({mu["op"] for mu in MUTANTS.values()}):
+        in_child(_run)(op, build.build())
+
+
+@pytest.mark.parametrize("tag", sorted(MUTANTS))
+def test_a_mistake_in_the_kernels_is_noticed(libraries, tag, capfd):
+    mu = MUTANTS[tag]
+    with pytest.raises(AssertionError) as caught:
+        in_child(_run)(mu["op"], libraries[tag])
+    said = str(caught.value) + capfd.readouterr().err
+    expect = mu["expect"] if isinstance(mu["expect"], tuple) else (mu["expect"],)
+    assert any(e in said for e in expect), said[-1500:]
