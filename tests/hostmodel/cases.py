@@ -65,9 +65,11 @@ def decode(m: Model, bits, th, segments=1, merge=False, expect_kernel=None):
 
 # ---- fused linear ---------------------------------------------------------------------------------------------------
 def linear(m: Model, bits, xb, th, segments=1, slot_table=False, window_rows=False, wide=False, bias=None,
-           noalloc=False, expect_kernel=None, x_pad=0, check_twin=True):
+           noalloc=False, expect_kernel=None, x_pad=0, check_twin=True, partials_only=False):
     """out = x W through ci_fused_linear_tiled (or its no-allocation variant): within 1e-2 of the fp32 product on the
-    oracle-decoded weight, and bit for bit the same contraction on the plain weight."""
+    oracle-decoded weight, and bit for bit the same contraction on the plain weight.  partials_only: the workspace has
+    room for the partial sums the plan needs and not for the fragment copy of x (a caller that sized it so): the
+    kernels then read the rows of x where they lie."""
     K, N = bits.shape
     M = xb.shape[0]
     enc, man = compress(bits, th)
@@ -79,6 +81,14 @@ def linear(m: Model, bits, xb, th, segments=1, slot_table=False, window_rows=Fal
     x, out = m.dev(xfull), m.empty((M, N), np.uint16)
     b = m.dev(bias) if bias is not None else None
     nb = m.lib.ci_fused_linear_workspace_bytes_segmented(M, K, N, th, 32, 0, segments)
+    if partials_only:
+        # what the query adds for the fragment copy: whole passes of 4 or 8 groups of 32 rows above 64 rows, else pairs
+        # of groups above 32 rows, else one group (from 17 rows on, K a multiple of 8)
+        groups = -(-M // 32)
+        groups = -(-groups // (4 if M <= 128 else 8)) * (4 if M <= 128 else 8) if M > 64 else (2 * -(-M // 64) if M > 32 else 1)
+        frag = groups * 32 * K * 2 if (M >= 17 and K % 8 == 0) else 0
+        assert nb >= frag
+        nb -= frag
     ws, ws_n = _ws(m, nb)
     m.lib.ci_fused_linear_wide_rows(1 if wide else 0)
     m.clear()

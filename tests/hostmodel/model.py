@@ -76,7 +76,8 @@ class Model:
     def __init__(self, cus: int = 8, end_at_guard: bool = True, schedule: int = 0, lib_path: str | None = None):
         from tests.hostmodel import build
 
-        self.lib = C.CDLL(lib_path or build.build())  # (lib_path: a build with a deliberate mistake, build.build_mutant)
+        # (lib_path, or CI_HOSTMODEL_LIB for a whole test run: a build with a deliberate mistake, build.build_mutant)
+        self.lib = C.CDLL(lib_path or os.environ.get("CI_HOSTMODEL_LIB") or build.build())
         L = self.lib
         L.sim_alloc.restype = C.c_void_p
         L.sim_alloc.argtypes = [C.c_size_t, C.c_int]

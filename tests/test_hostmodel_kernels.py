@@ -124,6 +124,21 @@ def test_fused_linear_bias_row_stride_and_the_entry_point_without_allocation():
         cases.linear(m, bits, x_bits(M, K, 2), th, segs, bias=bias, noalloc=True, window_rows=True)
 
 
+@in_child
+def test_fused_linear_without_room_for_the_fragment_copy():
+    """A workspace that holds the partial sums and nothing more (or no workspace where the plan has none): the
+    kernels read x in place, the rows past the last one masked -- x ends at the inaccessible page."""
+    m = Model(cus=4)
+    bits = weight_bits(2048, 128, 1)
+    for M, segs, prep, kernel in ((40, 2, True, "fused_linear32_seg_kernel<2, false>"), (64, 2, True, "fused_linear32_seg_kernel<2, false>"),
+                                  (33, 4, False, "fused_linear32_seg_kernel<2, true>"), (20, 2, True, "fused_linear32_seg_kernel<1, false>"),
+                                  (50, 1, False, "fused_linear32_kernel<2>"), (100, 1, False, "fused_linear32_kernel<2>")):
+        launches = cases.linear(m, bits, x_bits(M, 2048, 2), 1024, segs, slot_table=prep, window_rows=prep, partials_only=True,
+                                expect_kernel=kernel)
+        assert "x_fragments_kernel" not in launches, launches
+        m.free_all()
+
+
 @pytest.mark.parametrize("kind", cases.KINDS)
 @in_child
 def test_fused_linear_on_unusual_planes(kind):
