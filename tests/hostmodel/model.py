@@ -130,6 +130,10 @@ class Model:
     def violations(self) -> list[str]:
         return [self.lib.sim_violation(i).decode() for i in range(self.lib.sim_violation_count())]
 
+    def asm_instructions(self) -> int:
+        """Instructions of hand-written assembly statements the interpreter has carried out so far (per wavefront)."""
+        return int(self.lib.sim_asm_instructions())
+
     def launches(self) -> list[str]:
         return [self.lib.sim_launch_name(i).decode() for i in range(self.lib.sim_launch_count())]
 

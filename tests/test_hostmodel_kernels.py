@@ -210,6 +210,52 @@ def test_lm_head_on_unusual_planes(kind):
     cases.lm_head(m, bits, x_bits(1, 64, 2), 1024, 4, window_rows=True, slot_table=True, matrix_sums=True, check_twin=False)
 
 
+# ---- which path ran -------------------------------------------------------------------------------------------------
+@in_child
+def test_the_hand_scheduled_loops_are_what_these_tests_run():
+    """Every kernel has a guarded path in C++ that gives the same results as its hand-scheduled loop, so a test that
+    compares results cannot tell which of the two ran -- and the loop is what the GPU will run.  The model counts the
+    assembly instructions it interprets: on whole tiles of ordinary weights, prepared as the runtime prepares them,
+    all decode steps must have gone through the statements (0.95 to 1.1 times the loops' instructions per step: prologues and tails add a few per cent) (decode 20 instructions a step,
+    fused linear 19.5, the eight-step block of the LM head 17, the gather's advance 18)."""
+    m = Model(cus=4)
+    K, N, th = 2048, 128, 1024
+    wave_steps = (K // th) * (N // 32) * (th // 2)
+    bits = weight_bits(K, N, 1)
+
+    def share(per_step, run):
+        run()  # (every case clears the model's records, the instruction count among them, before its call)
+        got = m.asm_instructions() / (wave_steps * per_step)
+        m.free_all()
+        return got
+
+    for segs, kernel in ((1, "decode_tiled32_persist_kernel<false>"), (2, "decode_tiled32_seg_kernel<false>"), (8, "decode_tiled32_seg_kernel<false>")):
+        s = share(20, lambda: cases.decode(m, bits, th, segs, expect_kernel=kernel))
+        assert 0.95 <= s <= 1.1, (kernel, segs, s)
+    for M, segs, prep, kernel in ((1, 1, False, "fused_linear32_kernel<1>"), (40, 1, False, "fused_linear32_kernel<2>"),
+                                  (1, 2, True, "fused_linear32_seg_kernel<1, false>"), (3, 4, False, "fused_linear32_seg_kernel<1, true>"),
+                                  (64, 2, True, "fused_linear32_seg_kernel<2, false>"), (16, 8, True, "fused_linear32_seg_kernel<1, false>")):
+        s = share(19.5, lambda: cases.linear(m, bits, x_bits(M, K, 2), th, segs, slot_table=prep, window_rows=prep,
+                                             expect_kernel=kernel, check_twin=False))
+        assert 0.95 <= s <= 1.15, (kernel, M, segs, s)
+    for M, kernel in ((129, "fused_linear32_wide_kernel<8>"), (70, "fused_linear32_wide_kernel<4>")):
+        s = share(17, lambda: cases.linear(m, bits, x_bits(M, K, 2), th, wide=True, expect_kernel=kernel, check_twin=False))
+        assert 0.95 <= s <= 1.1, (kernel, s)
+    s = share(19.5, lambda: cases.linear(m, weight_bits(4096, 64, 1), x_bits(2, 4096, 2), 2048, 2,
+                                         expect_kernel="fused_linear32_resident_kernel<1>", check_twin=False))
+    assert 0.95 <= s <= 1.15, ("resident", s)   # (4096 x 64 at tile height 2048: the same number of steps)
+    for segs, prep, matrix, kernel in ((1, False, False, "trans32_kernel<1>"), (2, True, False, "trans32_seg_kernel<false>"),
+                                       (4, True, True, "trans32_seg_kernel<true>")):
+        s = share(17, lambda: cases.lm_head(m, bits, x_bits(1, N, 2), th, segs, slot_table=prep, window_rows=prep,
+                                            matrix_sums=matrix, check_twin=False, expect_kernel=kernel))
+        assert 0.95 <= s <= 1.1, (kernel, s)
+    # the gather decodes every bucket it is asked about down to the deepest row asked for: all rows of the table here
+    ids = np.arange(K, dtype=np.int64)
+    for segs, slot, kernel in ((1, False, "embed_gather32_kernel"), (8, False, "embed_gather32_kernel"), (8, True, "embed_gather32_seg_kernel")):
+        s = share(18, lambda: cases.gather(m, bits, ids, th, segs, slot, expect_kernel=kernel))
+        assert s >= 0.95, (kernel, segs, s)
+
+
 # ---- encoders and the other layouts --------------------------------------------------------------------------------------
 @pytest.mark.parametrize("layout,th,tw", [("ilp2", 1024, 32), ("ilp2", 64, 16), ("one", 256, 32), ("one", 128, 64),
                                           ("dense", 512, 32)])
