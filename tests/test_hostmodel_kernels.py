@@ -24,6 +24,10 @@ from tests.hostmodel.model import Model, in_child, weight_bits, x_bits
     (1024, 96, 512, 1, False, "decode_tiled32_seg_kernel<false>"),   # low tiles: whole streams on sixteen wavefronts
     (2048 + 300, 100, 1024, 2, False, "decode_tiled32_seg_kernel<false>"),  # ragged rows and columns, odd last tile
     (3000, 70, 2048, 1, True, "decode_tiled32_persist_kernel<true>"),
+    (2048, 95, 1024, 2, False, "decode_tiled32_seg_kernel<false>"),   # one column short of whole tiles: the 64-byte rows of a pair end one byte early
+    (1024, 63, 1024, 1, False, "decode_tiled32_persist_kernel<false>"),
+    (2048, 63, 1024, 2, False, "decode_tiled32_seg_kernel<false>"),   # ... of a whole pair of tiles
+    (2048, 127, 1024, 4, True, "decode_tiled32_seg_kernel<true>"),
 ])
 @in_child
 def test_decode(K, N, th, segs, merge, kernel):
@@ -70,6 +74,39 @@ def test_decode_batch_of_a_layer_in_one_launch():
         assert np.array_equal(out.get(), ref)
 
 
+@in_child
+def test_decode_batch_on_sixteen_wavefronts():
+    """Several tensors with checkpoints in one launch of decode_tiled32_seg_kernel: every workgroup has to find its
+    tensor in the batch (the CUs are divided among the tensors by their sizes)."""
+    import ctypes as C
+
+    from oracle import rans_oracle as ro
+    from tests.hostmodel.model import DecodeItem
+
+    for cus in (3, 8):
+        m = Model(cus=cus)
+        shapes = [(2048, 64, 2), (1024, 256, 4), (1500, 40, 2), (1024, 96, 8), (3072, 32, 2)]
+        items = (DecodeItem * len(shapes))()
+        keep, outs, refs = [], [], []
+        for i, (K, N, segs) in enumerate(shapes):
+            bits = weight_bits(K, N, 40 + i)
+            enc, man = cases.compress(bits, 1024)
+            w, kp = m.weight(enc, None, K, N, segments=segs)
+            out = m.empty((K, N), np.uint8)
+            keep.append((w, kp))
+            outs.append(out)
+            refs.append(ro.split_bf16(bits)[0])
+            it = items[i]
+            it.d_stream, it.stream_len, it.d_states, it.d_tables, it.d_slot_map = w.d_stream, w.stream_len, w.d_states, w.d_tables, w.d_slot_map
+            it.d_tile_offsets, it.d_tile_max_lens, it.K, it.N, it.tile_height, it.tile_width = w.d_tile_offsets, w.d_tile_max_lens, K, N, 1024, 32
+            it.d_out_exp, it.d_checkpoints, it.segments = out.p, w.d_checkpoints, segs
+        m.clear()
+        m.call("ci_decode_tiled_ilp2_batch", items, len(shapes), None)
+        assert m.launches() == ["decode_tiled32_seg_kernel<false>"], m.launches()
+        for out, ref in zip(outs, refs):
+            assert np.array_equal(out.get(), ref)
+
+
 # ---- fused linear -----------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("K,N,M,th,segs,prep,kernel", [
     (2048, 128, 1, 1024, 1, False, "fused_linear32_kernel<1>"),
@@ -82,6 +119,8 @@ def test_decode_batch_of_a_layer_in_one_launch():
     (1024, 320, 4, 256, 1, False, "fused_linear32_seg_kernel<1, true>"),     # low tiles, several column tiles per job
     (2048 + 100, 100, 5, 1024, 2, False, "fused_linear32_seg_kernel<1, true>"),  # ragged: guarded path inside the kernel
     (3072, 96, 7, 2048, 1, False, "fused_linear32_kernel<1>"),
+    (2048, 95, 2, 1024, 2, True, "fused_linear32_seg_kernel<1, true>"),      # one column short of whole tiles
+    (1024, 31, 40, 1024, 1, False, "fused_linear32_kernel<2>"),
 ])
 @in_child
 def test_fused_linear(K, N, M, th, segs, prep, kernel):
@@ -157,6 +196,10 @@ def test_fused_linear_on_unusual_planes(kind):
     (4096, 128, 300, 1024, 4, True, "embed_gather32_seg_kernel"),
     (5000, 100, 257, 1024, 8, True, "embed_gather32_seg_kernel"),   # ragged rows and columns, odd last column tile
     (3000, 96, 1, 512, 4, True, "embed_gather32_seg_kernel"),
+    (4096, 95, 100, 1024, 8, True, "embed_gather32_seg_kernel"),    # one column short of whole tiles
+    (2048, 63, 100, 1024, 1, False, "embed_gather32_kernel"),
+    (4096, 63, 100, 1024, 8, True, "embed_gather32_seg_kernel"),    # ... of a whole pair of tiles
+    (2048, 127, 64, 1024, 8, False, "embed_gather32_kernel"),
     (70000, 64, 2048, 1024, 8, True, "embed_gather32_seg_kernel"),
     (270000, 32, 500, 32, 1, False, "embed_sort_kernel"),            # more buckets than counting slots: the sort
 ])
