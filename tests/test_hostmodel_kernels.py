@@ -28,6 +28,8 @@ from tests.hostmodel.model import Model, in_child, weight_bits, x_bits
     (1024, 63, 1024, 1, False, "decode_tiled32_persist_kernel<false>"),
     (2048, 63, 1024, 2, False, "decode_tiled32_seg_kernel<false>"),   # ... of a whole pair of tiles
     (2048, 127, 1024, 4, True, "decode_tiled32_seg_kernel<true>"),
+    (512, 63, 256, 2, False, "decode_tiled32_seg_kernel<false>"),     # ... with short items, whose last one ends the array
+    (768, 127, 256, 1, False, "decode_tiled32_seg_kernel<false>"),
 ])
 @in_child
 def test_decode(K, N, th, segs, merge, kernel):
