@@ -255,6 +255,46 @@ def test_lm_head_on_unusual_planes(kind):
     cases.lm_head(m, bits, x_bits(1, 64, 2), 1024, 4, window_rows=True, slot_table=True, matrix_sums=True, check_twin=False)
 
 
+# ---- split-K reduction ------------------------------------------------------------------------------------------------
+@in_child
+def test_splitk_reduction_in_index_order():
+    """ci_splitk_reduce: out = bf16(sum over the planes in index order (+ bias)), fp32 and bf16 partials, through both
+    kernels (one output a thread; four a thread from 65,536 outputs on) and through every stage of their unrolled
+    loops (16 / 4 / 1 planes at a time, 8 / 1): bit for bit the sequential fp32 sum."""
+    import ctypes as C
+
+    from tests.hostmodel.model import bf16_bits_to_f32, f32_to_bf16_bits
+
+    m = Model(cus=4)
+    rng = np.random.default_rng(8)
+    for P, M, N in ((1, 3, 40), (3, 5, 33), (4, 2, 64), (7, 1, 96), (16, 2, 50), (21, 3, 36), (37, 1, 128),
+                    (9, 64, 1024), (16, 128, 512), (23, 33, 2048)):
+        part = (rng.standard_normal((P, M, N), dtype=np.float32) * 3).astype(np.float32)
+        bias = f32_to_bf16_bits(rng.standard_normal(N, dtype=np.float32))
+        want = np.zeros((M, N), np.float32)
+        for p in range(P):
+            want = (want + part[p]).astype(np.float32)
+        for with_bias in (False, True):
+            # (the sum is rounded to bf16 and the bias added in bf16, as torch.sum(...) then `+= bias` do in the reference)
+            w = (bf16_bits_to_f32(f32_to_bf16_bits(want)) + bf16_bits_to_f32(bias)[None, :]).astype(np.float32) if with_bias else want
+            out = m.empty((M, N + 8), np.uint16)
+            b = m.dev(bias)
+            m.clear()
+            m.call("ci_splitk_reduce", m.dev(part).p, 0, P, M, N, b.p if with_bias else None, out.p, N + 8, None)
+            kernel = "splitk_reduce4_kernel" if M * N >= 65536 and N % 4 == 0 else "splitk_reduce_kernel"
+            assert m.launches() == [kernel], (m.launches(), P, M, N)
+            assert np.array_equal(out.get()[:, :N], f32_to_bf16_bits(w)), (P, M, N, with_bias)
+        # the reference's workspace: bf16 partials [S, M, N] (comp_inference/linear_triton.py:303-314)
+        pb = f32_to_bf16_bits(part)
+        want = np.zeros((M, N), np.float32)
+        for p in range(P):
+            want = (want + bf16_bits_to_f32(pb[p])).astype(np.float32)
+        out = m.empty((M, N), np.uint16)
+        m.call("ci_splitk_reduce", m.dev(pb).p, 1, P, M, N, None, out.p, N, None)
+        assert np.array_equal(out.get(), f32_to_bf16_bits(want)), (P, M, N, "bf16 partials")
+        m.free_all()
+
+
 # ---- which path ran -------------------------------------------------------------------------------------------------
 @in_child
 def test_the_hand_scheduled_loops_are_what_these_tests_run():
