@@ -360,8 +360,9 @@ def test_operators_of_the_other_layouts(layout, th, tw):
     """a7 (one stream per column in tile bodies), the dense layout and other tile widths of the default layout: decode,
     fused linear, gather and LM head through the one-thread-per-stream kernels."""
     rng = np.random.default_rng(15)
-    K, N = 2 * th + th // 2, 3 * tw + 7
+    K, N = 2 * th + th // 2 + 3, 3 * tw + 7   # a last tile row of more than half a tile, less than a whole one
     ids = rng.integers(-2, K + 2, 37)
+    ids[:4] = (K, K - 1, -1, K + 1)           # the first row past the table, the last row in it
     launches = cases.other_layout_ops(Model(cus=4), weight_bits(K, N, 5), x_bits(3, max(K, N), 2)[:, :K], ids, th, tw, layout)
     assert any("generic_kernel" in k for k in launches), launches
 
