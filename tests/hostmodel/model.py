@@ -7,6 +7,7 @@ from __future__ import annotations
 import ctypes as C
 import os
 import pickle
+import signal
 import sys
 import traceback
 
@@ -66,6 +67,10 @@ class Dev:
         assert a.size * a.itemsize == self.nbytes, (a.shape, self.shape)
         if self.nbytes:
             C.memmove(self.ptr, a.ctypes.data, self.nbytes)
+
+
+# a test body on the model takes seconds, a sweep block a minute or two
+CHILD_SECONDS = 600
 
 
 class ModelError(AssertionError):
@@ -211,6 +216,7 @@ def in_child(fn):
         if pid == 0:
             os.close(r)
             code = 0
+            signal.alarm(CHILD_SECONDS)  # (a kernel that loops for ever in the model ends its child, not the test run)
             # The oracle is OpenMP code, and a process forked from one whose OpenMP runtime already has its worker
             # threads (an earlier test used the oracle) would wait for those threads for ever: teams of one here.
             try:
@@ -232,6 +238,8 @@ def in_child(fn):
         with os.fdopen(r, "rb") as f:
             data = f.read()
         _, status = os.waitpid(pid, 0)
+        if os.WIFSIGNALED(status) and os.WTERMSIG(status) == signal.SIGALRM:
+            raise AssertionError(f"the host model did not finish within {CHILD_SECONDS} s: a kernel that loops for ever?")
         if os.WIFSIGNALED(status):
             raise AssertionError(f"the host-model child died of signal {os.WTERMSIG(status)}")
         code = os.WEXITSTATUS(status)
@@ -256,7 +264,10 @@ def in_fresh_process(fn):
         code = (f"import sys; sys.path[:0] = [{ROOT!r}, {os.path.join(ROOT, 'tests')!r}]; import importlib; "
                 f"f = getattr(importlib.import_module({fn.__module__.split('.')[-1]!r}), {fn.__name__!r}); "
                 f"f.__wrapped__(*{args!r}, **{kwargs!r})")
-        p = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True)
+        try:
+            p = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=2 * CHILD_SECONDS)
+        except subprocess.TimeoutExpired:
+            raise AssertionError(f"the host model did not finish within {2 * CHILD_SECONDS} s: a kernel that loops for ever?") from None
         sys.stderr.write(p.stderr[-4000:])
         if p.returncode == 70:
             raise AssertionError("memory fault inside the host model:\n" + p.stderr[-2000:])
@@ -283,6 +294,7 @@ def fork_all(fn, arg_list, jobs: int | None = None):
         if pid == 0:
             os.close(r)
             code = 0
+            signal.alarm(2 * CHILD_SECONDS)
             try:
                 C.CDLL("libgomp.so.1").omp_set_num_threads(1)  # (see in_child)
             except OSError:
@@ -310,7 +322,9 @@ def fork_all(fn, arg_list, jobs: int | None = None):
         arg, r = running.pop(pid)
         with os.fdopen(r, "rb") as f:
             data = f.read()
-        if os.WIFSIGNALED(status):
+        if os.WIFSIGNALED(status) and os.WTERMSIG(status) == signal.SIGALRM:
+            failures.append(f"[{arg!r}] the host model did not finish within {2 * CHILD_SECONDS} s: a kernel that loops for ever?")
+        elif os.WIFSIGNALED(status):
             failures.append(f"[{arg!r}] the child died of signal {os.WTERMSIG(status)}")
         elif os.WEXITSTATUS(status) == 70:
             failures.append(f"[{arg!r}] memory fault inside the host model (see the message on stderr)")

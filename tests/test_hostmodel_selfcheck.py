@@ -178,3 +178,17 @@ def test_the_python_descriptor_matches_the_header():
 
     assert [(n, t) for n, t in model.TiledWeight._fields_] == [(n, t) for n, t in _lib.TiledWeight._fields_]
     assert C.sizeof(model.TiledWeight) == C.sizeof(_lib.TiledWeight)
+
+
+def test_a_test_body_that_never_ends_is_ended(monkeypatch):
+    """A kernel that loops for ever inside the model (nothing in it waits, so nothing reports a deadlock) must cost one
+    test, not the test run: the child processes of the helpers have a time limit."""
+    import time
+
+    from tests.hostmodel import model
+
+    monkeypatch.setattr(model, "CHILD_SECONDS", 1)
+    with pytest.raises(AssertionError, match="did not finish within 1 s"):
+        model.in_child(lambda: time.sleep(30))()
+    with pytest.raises(AssertionError, match="did not finish within 2 s"):
+        model.fork_all(lambda arg: time.sleep(30 if arg else 0), [0, 1])
