@@ -229,6 +229,67 @@ def test_entry_points_refuse_bad_arguments_before_any_launch():
     assert lib.ci_last_error() != b""
 
 
+def test_every_required_pointer_and_size_is_checked():
+    """One argument at a time made NULL (or zero, or misaligned) in an otherwise acceptable call of every
+    bare-pointer entry point of the default format: CI_ERR_ARG each time, before any HIP call.  The acceptable
+    call itself gets past the checks (and fails at the first HIP call here, where there is no GPU)."""
+    from comp_inference_amd import _lib
+
+    lib = _lib.lib()
+    P, u64, sz = ctypes.c_void_p, ctypes.c_uint64, ctypes.c_size_t
+    fake, null, odd = P(0x10000), P(0), P(0x10002)
+    big = sz(1 << 30)
+
+    def sweep(name, args, required, zero_is_bad=(), misaligned=()):
+        fn = getattr(lib, name)
+        assert fn(*args) != 1, (name, lib.ci_last_error())  # past the argument checks
+        for i in required:
+            bad = list(args)
+            bad[i] = null
+            assert fn(*bad) == 1, (name, "argument", i, "NULL was accepted")
+            assert lib.ci_last_error() != b""
+        for i in zero_is_bad:
+            bad = list(args)
+            bad[i] = 0
+            assert fn(*bad) == 1, (name, "argument", i, "0 was accepted")
+        for i in misaligned:
+            bad = list(args)
+            bad[i] = odd
+            assert fn(*bad) == 1, (name, "argument", i, "a misaligned pointer was accepted")
+
+    K, N, M, th = 2048, 96, 3, 1024
+    body = (fake, u64(4096), fake, fake, fake, fake, fake)  # stream, its length, states, tables, slot_map, two per-tile arrays
+    # d_x M K N x_stride | body | man th tw bias out out_stride ws ws_bytes stream
+    lin = (fake, M, K, N, K) + body + (fake, th, 32, None, fake, N, fake, big, None)
+    sweep("ci_fused_linear_ilp2", lin, required=(0, 5, 7, 8, 9, 10, 11, 12, 16), zero_is_bad=(2, 13, 14), misaligned=(9,))
+    sweep("ci_fused_linear_dense", lin, required=(0, 5, 7, 8, 9, 10, 11, 12, 16), zero_is_bad=(2, 13, 14), misaligned=(9,))
+    sweep("ci_fused_linear_one", lin, required=(0, 5, 7, 8, 9, 10, 11, 12, 16), zero_is_bad=(2, 13, 14), misaligned=(9,))
+    seg = lin[:15] + (fake, 2) + lin[15:]
+    sweep("ci_fused_linear_ilp2_segmented", seg, required=(0, 5, 7, 8, 9, 10, 11, 12, 15, 18), zero_is_bad=(2, 13, 14), misaligned=(9, 15))
+    # d_x M H V x_stride | body | man th tw bias out out_stride ws ws_bytes stream
+    head = (fake, 1, 96, 2048, 96) + body + (fake, th, 32, None, fake, 2048, fake, big, None)
+    sweep("ci_fused_linear_transposed_ilp2", head, required=(0, 5, 7, 8, 9, 10, 11, 12, 16), zero_is_bad=(2, 13, 14), misaligned=(9,))
+    sweep("ci_fused_linear_transposed_dense", head, required=(0, 5, 7, 8, 9, 10, 11, 12, 16), zero_is_bad=(2, 13, 14), misaligned=(9,))
+    # ids n_ids | body | man K N th tw out out_stride ws ws_bytes stream
+    emb = (fake, 7) + body + (fake, K, N, th, 32, fake, N, fake, big, None)
+    sweep("ci_fused_embedding_ilp2", emb, required=(0, 2, 4, 5, 6, 7, 8, 9, 14), zero_is_bad=(12, 13), misaligned=(6,))
+    embs = emb[:14] + (fake, 8) + emb[14:]
+    sweep("ci_fused_embedding_ilp2_segmented", embs, required=(0, 2, 4, 5, 6, 7, 8, 9, 14, 16), zero_is_bad=(12, 13), misaligned=(6, 14))
+    # body | K N th tw out_exp man out_bf16 stream
+    dec = body + (K, N, th, 32, fake, None, None, None)
+    sweep("ci_decode_tiled_ilp2", dec, required=(0, 2, 3, 4, 5, 6, 11), zero_is_bad=(9, 10), misaligned=(4,))
+    sweep("ci_decode_tiled_one", dec, required=(0, 2, 3, 4, 5, 6, 11), zero_is_bad=(9, 10), misaligned=(4,))
+    decs = body + (K, N, th, 32, fake, 2, fake, None, None, None)
+    sweep("ci_decode_tiled_ilp2_segmented", decs, required=(0, 2, 3, 4, 5, 6, 11, 13), zero_is_bad=(9, 10), misaligned=(4, 11))
+    merged = body + (K, N, th, 32, None, fake, fake, None)  # the bf16 output needs the sign|mantissa plane
+    sweep("ci_decode_tiled_ilp2", merged, required=(12, 13))
+    # body | K N th tw segments ckpt bytes stream
+    ck = body + (K, N, th, 32, 4, fake, big, None)
+    sweep("ci_build_checkpoints_ilp2", ck, required=(0, 2, 3, 4, 5, 6, 12), zero_is_bad=(9, 10), misaligned=(4, 12))
+    # tables slot_map out bytes stream
+    sweep("ci_build_slot_table", (fake, fake, fake, sz(32768), None), required=(0, 1, 2), misaligned=(1, 2))
+
+
 def test_public_header_is_plain_c(tmp_path):
     """The boundary is a C ABI: the header compiles as C99 on its own and a C program links against the
     library's host-only entry points."""
@@ -291,6 +352,11 @@ def test_a_descriptor_with_a_short_array_is_refused_on_the_host():
     assert rc(d_states=None) == 1 and rc(d_tile_offsets=None) == 1 and rc(d_stream=None) == 1
     assert rc(d_slot_map=0x40002) == 1                     # not 4-byte aligned
     assert rc(tile_height=1023) == 1 and rc(K=0) == 1
+    for field in ("N", "tile_height", "tile_width"):
+        assert rc(**{field: 0}) == 1, field
+    for field in ("d_tables", "d_slot_map", "d_tile_max_lens"):
+        assert rc(**{field: None}) == 1, field
+    assert rc(d_slot_table=0x90008, slot_table_bytes=32768) == 1   # not 16-byte aligned
     ck = lib.ci_checkpoint_bytes(K, N, th, tw, 4)
     assert ck == tiles * 3 * 64 * 8
     assert rc(segments=4, d_checkpoints=0x80000, checkpoint_bytes=ck) == 0
