@@ -641,11 +641,18 @@ __device__ __forceinline__ void seg_request(const LinearArgs &a, uint32_t vk, ui
     m.row_end = seg + 1 < a.segs ? ck[(size_t)seg * 64].y : 0xffffffffu;
 }
 
-__device__ __forceinline__ void seg_resolve(const LinearArgs &a, uint32_t vk, uint32_t tn, int lane, const SegRaw &m,
-                                            SegItem &it) {
+// Decode steps this lane's stream has in item vk of column tile tn: the segment's length, less at the ragged
+// end of K, none in a column past N.
+__device__ __forceinline__ uint32_t seg_steps(const LinearArgs &a, uint32_t vk, uint32_t tn, int lane) {
     const uint32_t tk = vk / a.segs, seg = vk % a.segs;
     const uint32_t half = a.th / 2, seglen = half / a.segs, hsel = lane / 32, c = lane % 32;
     const uint32_t k0 = tk * a.th + hsel * half + seg * seglen;
+    return tn * 32 + c < a.N && k0 < a.K ? min(seglen, a.K - k0) : 0u;
+}
+
+__device__ __forceinline__ void seg_resolve(const LinearArgs &a, uint32_t vk, uint32_t tn, int lane, const SegRaw &m,
+                                            SegItem &it) {
+    const uint32_t seglen = a.th / 2 / a.segs;
     it.vk = vk;
     it.tn = tn;
     it.base = m.off;
@@ -654,9 +661,7 @@ __device__ __forceinline__ void seg_resolve(const LinearArgs &a, uint32_t vk, ui
     it.state = m.state;
     it.row = min((int32_t)m.row, (int32_t)depth - 1);
     const int32_t row_end = min((int32_t)m.row_end, it.row);
-    uint32_t my_steps = 0;
-    if (tn * 32 + c < a.N && k0 < a.K) my_steps = min(seglen, a.K - k0);
-    const bool full = __builtin_amdgcn_ballot_w64(my_steps != seglen) == 0;
+    const bool full = __builtin_amdgcn_ballot_w64(seg_steps(a, vk, tn, lane) != seglen) == 0;
     // rows of the body the item can touch: from the lowest row a lane has reached by the item's end (the byte
     // there is fetched ahead, never used) to the highest row a lane starts at
     const int32_t lo = max(wave_min_i32(row_end), 0), hi = wave_max_i32(it.row);
@@ -1507,7 +1512,10 @@ extern "C" int ci_build_slot_table(const uint32_t *d_tables, const uint8_t *d_sl
 
 namespace ci {
 // One wavefront per item (segment of the 64 streams of a tile): the rows of the tile body the item can touch,
-// as the sixteen-wavefront kernel works them out before staging; the maximum over all items, at least 1.
+// as the sixteen-wavefront kernel works them out before staging; the maximum over all items whose 64 streams
+// all run the segment's full length, at least 1.  (An item at a ragged edge of the shape is never staged:
+// every kernel gives it to a path that reads the body in place.  Its window would count for nothing and can
+// be the whole body: the lanes of a stream without symbols stay where they start.)
 __global__ __launch_bounds__(256) void window_rows_kernel(LinearArgs a, uint32_t num_items, uint32_t *out) {
     const uint32_t item = blockIdx.x * 4 + threadIdx.x / kWave;
     const int lane = threadIdx.x % kWave;
@@ -1517,7 +1525,8 @@ __global__ __launch_bounds__(256) void window_rows_kernel(LinearArgs a, uint32_t
     seg_request(a, vk, tn, lane, raw);
     SegItem it;
     seg_resolve(a, vk, tn, lane, raw, it);
-    if (lane == 0) atomicMax(out, it.rows > 1u ? it.rows : 1u);
+    const bool full = __builtin_amdgcn_ballot_w64(seg_steps(a, vk, tn, lane) != a.th / 2 / a.segs) == 0;
+    if (lane == 0) atomicMax(out, full && it.rows > 1u ? it.rows : 1u);
 }
 }  // namespace ci
 

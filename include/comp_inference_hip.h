@@ -475,7 +475,9 @@ int ci_build_slot_table(const uint32_t *d_tables, const uint8_t *d_slot_map, voi
                         size_t slot_table_bytes, ci_stream_t stream);
 
 /* The largest number of rows of a tile body that one item -- a segment of the 64 streams of a tile, or
- * the whole streams without checkpoints -- reads, written to *d_rows (device memory, 4 bytes) on `stream`.
+ * the whole streams without checkpoints -- reads, written to *d_rows (device memory, 4 bytes) on `stream`;
+ * over the items whose 64 streams all have the segment's full length (an item at a ragged edge of the
+ * shape is read in place by every kernel, whatever its window), and at least 1.
  * Derived data like the checkpoints: computed once per weight, copied back by the caller and kept in
  * ci_tiled_weight::max_window_rows.  With it the fused linear knows before the launch that every item
  * fits its staging area and runs a kernel without the guarded path; with 0 there it runs the kernel that

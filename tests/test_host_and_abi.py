@@ -229,6 +229,22 @@ def test_entry_points_refuse_bad_arguments_before_any_launch():
     assert lib.ci_last_error() != b""
 
 
+def test_suggested_segments_for_the_shapes_they_were_chosen_on():
+    """ci_suggest_segments: the fewest segments per stream that make an item 256 rows or less and the items enough to
+    fill a chip of 256 CUs x 16 wavefronts; 1 where the tile shape allows none.  The figures the measurements were
+    taken with (Llama-3-8B projections at tile 1024 x 32)."""
+    from comp_inference_amd import _lib
+
+    lib = _lib.lib()
+    lib.ci_suggest_segments.restype = ctypes.c_uint32
+    for (K, N, th, tw), want in {(4096, 14336, 1024, 32): 2, (4096, 28672, 1024, 32): 2, (14336, 4096, 1024, 32): 2,
+                                 (128256, 4096, 1024, 32): 2, (4096, 6144, 1024, 32): 4, (4096, 4096, 1024, 32): 8,
+                                 (4096, 1024, 1024, 32): 8, (4096, 64, 2048, 32): 16, (4096, 1024, 256, 32): 2,
+                                 (512, 64, 64, 32): 1, (4096, 4096, 1000, 32): 1, (4096, 4096, 1024, 64): 1,
+                                 (4096, 4096, 0, 32): 1}.items():
+        assert lib.ci_suggest_segments(K, N, th, tw) == want, (K, N, th, tw)
+
+
 def test_every_required_pointer_and_size_is_checked():
     """One argument at a time made NULL (or zero, or misaligned) in an otherwise acceptable call of every
     bare-pointer entry point of the default format: CI_ERR_ARG each time, before any HIP call.  The acceptable
@@ -288,6 +304,45 @@ def test_every_required_pointer_and_size_is_checked():
     sweep("ci_build_checkpoints_ilp2", ck, required=(0, 2, 3, 4, 5, 6, 12), zero_is_bad=(9, 10), misaligned=(4, 12))
     # tables slot_map out bytes stream
     sweep("ci_build_slot_table", (fake, fake, fake, sz(32768), None), required=(0, 1, 2), misaligned=(1, 2))
+
+
+def test_segment_counts_a_tile_height_does_not_allow_are_refused():
+    """Checkpoints can cut half a tile into any number of equal runs (the builder and the gather take every divisor);
+    the decode and the fused linear read whole 16-row blocks, so they take the counts whose runs are multiples of 16
+    rows.  Everything else is CI_ERR_ARG before any HIP call; what is accepted gets past the checks."""
+    from comp_inference_amd import _lib
+
+    lib = _lib.lib()
+    P, u64, sz = ctypes.c_void_p, ctypes.c_uint64, ctypes.c_size_t
+    fake, big = P(0x10000), sz(1 << 30)
+    K, N = 4096, 96
+    body = (fake, u64(4096), fake, fake, fake, fake, fake)
+
+    def builder(th, segs):
+        return lib.ci_build_checkpoints_ilp2(*body, K, N, th, 32, segs, fake, big, None)
+
+    def gather(th, segs):
+        return lib.ci_fused_embedding_ilp2_segmented(fake, 7, *body, fake, K, N, th, 32, fake, segs, fake, N, fake, big, None)
+
+    def decode(th, segs):
+        return lib.ci_decode_tiled_ilp2_segmented(*body, K, N, th, 32, fake, segs, fake, None, None, None)
+
+    def linear(th, segs):
+        return lib.ci_fused_linear_ilp2_segmented(fake, 3, K, N, K, *body, fake, th, 32, fake, segs, None, fake, N, fake, big, None)
+
+    any_divisor = {(1024, 2): True, (1024, 64): True, (1024, 512): True, (1024, 3): False, (1024, 1024): False,
+                   (1000, 4): True, (1000, 125): True, (1000, 8): False, (1023, 2): False, (96, 16): True, (96, 32): False}
+    blocks_of_16 = {(1024, 2): True, (1024, 32): True, (1024, 64): False, (1024, 3): False, (1000, 4): False, (1000, 2): False,
+                    (96, 3): True, (96, 2): False, (992, 31): True, (1023, 2): False, (2048, 64): True, (2048, 128): False}
+    for fn, table in ((builder, any_divisor), (gather, any_divisor), (decode, blocks_of_16), (linear, blocks_of_16)):
+        for (th, segs), accepted in table.items():
+            rc = fn(th, segs)
+            assert (rc != 1) == accepted, (fn.__name__, th, segs, rc, lib.ci_last_error())
+    lib.ci_fused_embedding_workspace_bytes_segmented.restype = ctypes.c_size_t
+    for (th, segs), accepted in any_divisor.items():
+        assert (lib.ci_fused_embedding_workspace_bytes_segmented(7, K, th, segs) != 0) == accepted, (th, segs)
+    assert lib.ci_fused_embedding_workspace_bytes_segmented(7, K, 1, 1) == 0
+    assert lib.ci_fused_embedding_workspace_bytes_segmented(7, K, 2, 1) != 0
 
 
 def test_public_header_is_plain_c(tmp_path):

@@ -109,6 +109,47 @@ def test_decode_batch_on_sixteen_wavefronts():
             assert np.array_equal(out.get(), ref)
 
 
+@in_child
+def test_decode_batch_with_an_empty_tensor_and_a_stream_at_an_odd_address():
+    """A batch in which two tensors are empty (skipped) and one has its stream at an address that is no multiple of
+    16: that one goes through the one-thread-per-stream kernel, which reads the stream a byte at a time, the rest
+    through the batched launch."""
+    import ctypes as C
+
+    from oracle import rans_oracle as ro
+    from tests.hostmodel.model import DecodeItem
+
+    m = Model(cus=4)
+    shapes = [(2048, 64, 2), (0, 64, 1), (1024, 96, 1), (1024, 0, 1)]
+    items = (DecodeItem * len(shapes))()
+    keep, outs, refs = [], [], []
+    for i, (K, N, segs) in enumerate(shapes):
+        it = items[i]
+        it.K, it.N, it.tile_height, it.tile_width, it.segments = K, N, 1024, 32, segs
+        if K == 0 or N == 0:
+            continue  # (no pointer of an empty tensor is looked at)
+        bits = weight_bits(K, N, 50 + i)
+        enc, man = cases.compress(bits, 1024)
+        w, kp = m.weight(enc, None, K, N, segments=segs)
+        if i == 2:
+            room = m.empty(enc.stream.size + 16, np.uint8)
+            C.memmove(room.ptr + 8, enc.stream.ctypes.data, enc.stream.size)
+            w.d_stream = room.ptr + 8
+            keep.append(room)
+        out = m.empty((K, N), np.uint8)
+        keep.append((w, kp))
+        outs.append(out)
+        refs.append(ro.split_bf16(bits)[0])
+        it.d_stream, it.stream_len, it.d_states, it.d_tables, it.d_slot_map = w.d_stream, w.stream_len, w.d_states, w.d_tables, w.d_slot_map
+        it.d_tile_offsets, it.d_tile_max_lens = w.d_tile_offsets, w.d_tile_max_lens
+        it.d_out_exp, it.d_checkpoints = out.p, w.d_checkpoints
+    m.clear()
+    m.call("ci_decode_tiled_ilp2_batch", items, len(shapes), None)
+    assert m.launches() == ["(decode_tiled_generic_kernel<false, 2>)", "decode_tiled32_seg_kernel<false>"], m.launches()
+    for out, ref in zip(outs, refs):
+        assert np.array_equal(out.get(), ref)
+
+
 # ---- fused linear -----------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("K,N,M,th,segs,prep,kernel", [
     (2048, 128, 1, 1024, 1, False, "fused_linear32_kernel<1>"),
@@ -123,6 +164,7 @@ def test_decode_batch_on_sixteen_wavefronts():
     (3072, 96, 7, 2048, 1, False, "fused_linear32_kernel<1>"),
     (2048, 95, 2, 1024, 2, True, "fused_linear32_seg_kernel<1, true>"),      # one column short of whole tiles
     (1024, 31, 40, 1024, 1, False, "fused_linear32_kernel<2>"),
+    (2048, 128, 100, 1024, 2, True, "fused_linear32_kernel<2>"),             # above 64 rows the checkpoints are not used
 ])
 @in_child
 def test_fused_linear(K, N, M, th, segs, prep, kernel):
@@ -237,6 +279,10 @@ def test_fused_gather_on_unusual_planes(kind):
     (2048, 128, 1, 1024, 2, True, True, "trans32_seg_kernel<true>"),
     (2048 + 300, 256, 1, 1024, 4, True, True, "trans32_seg_kernel<true>"),
     (2000, 100, 2, 512, 1, False, False, "trans32_kernel<kTrRows>"),
+    (2048, 96, 1, 1024, 2, True, False, "trans32_seg_kernel<false>"),          # three column tiles
+    (2048, 160, 1, 1024, 4, True, True, "trans32_seg_kernel<true>"),
+    (2048 + 500, 64, 1, 1024, 4, True, False, "trans32_seg_kernel<false>"),    # a deep ragged tile row does not count in max_window_rows
+    (500, 64, 1, 1024, 4, True, False, "trans32_kernel<1>"),                   # no whole tile row: nothing for the segment kernel
 ])
 @in_child
 def test_lm_head(V, H, M, th, segs, prep, matrix, kernel):
@@ -253,6 +299,83 @@ def test_lm_head_on_unusual_planes(kind):
     cases.lm_head(m, bits, x_bits(1, 64, 2), 1024)
     cases.lm_head(m, bits, x_bits(1, 64, 2), 1024, 2, window_rows=True)
     cases.lm_head(m, bits, x_bits(1, 64, 2), 1024, 4, window_rows=True, slot_table=True, matrix_sums=True, check_twin=False)
+
+
+# ---- inputs at the edges of what a caller may pass ----------------------------------------------------------------------
+@in_child
+def test_empty_inputs_launch_nothing():
+    """No rows of x, no ids, an empty shape: CI_OK and not one launch (a grid of zero workgroups is an error on the GPU)."""
+    import ctypes as C
+
+    m = Model(cus=4)
+    K, N, th = 2048, 64, 1024
+    enc, man = cases.compress(weight_bits(K, N, 1), th)
+    w, keep = m.weight(enc, man, K, N, segments=2, slot_table=True, window_rows=True)
+    buf = m.empty(4096, np.uint8)
+    big = C.c_size_t(4096)
+    m.clear()
+    m.call("ci_fused_linear_tiled", C.byref(w), buf.p, 0, K, None, buf.p, N, buf.p, big, None)
+    m.call("ci_fused_linear_tiled_noalloc", C.byref(w), buf.p, 0, K, None, buf.p, N, None)
+    m.call("ci_fused_embedding_tiled", C.byref(w), buf.p, 0, buf.p, N, buf.p, big, None)
+    m.call("ci_fused_linear_transposed_tiled", C.byref(w), buf.p, 0, N, None, buf.p, K, buf.p, big, None)
+    m.call("ci_splitk_reduce", buf.p, 0, 3, 0, N, None, buf.p, N, None)
+    m.call("ci_splitk_reduce", buf.p, 0, 3, 5, 0, None, buf.p, 0, None)
+    body = (keep["stream"].p, C.c_uint64(enc.stream.size), keep["states"].p, keep["tables"].p, keep["slot_map"].p,
+            keep["offs"].p, keep["lens"].p)
+    m.call("ci_decode_tiled_ilp2", *body, 0, N, th, 32, buf.p, None, None, None)
+    m.call("ci_decode_tiled_ilp2", *body, K, 0, th, 32, buf.p, None, None, None)
+    m.call("ci_fused_linear_ilp2", buf.p, 3, K, 0, K, *body, keep["man"].p, th, 32, None, buf.p, 0, buf.p, big, None)
+    m.call("ci_build_checkpoints_ilp2", *body, 0, N, th, 32, 2, buf.p, big, None)
+    m.call("ci_build_checkpoints_ilp2", *body, K, 0, th, 32, 2, buf.p, big, None)
+    m.call("ci_fused_embedding_ilp2", buf.p, 3, *body, keep["man"].p, K, 0, th, 32, buf.p, 0, buf.p, big, None)
+    m.call("ci_fused_linear_transposed_ilp2", buf.p, 1, N, 0, N, *body, keep["man"].p, th, 32, None, buf.p, 0, buf.p, big, None)
+    m.call("ci_fused_linear_transposed_ilp2", buf.p, 0, N, K, N, *body, keep["man"].p, th, 32, None, buf.p, K, buf.p, big, None)
+    assert m.launches() == [], m.launches()
+
+
+@in_child
+def test_a_stream_that_is_not_16_byte_aligned():
+    """The whole-tile and sixteen-wavefront kernels load the stream 16 bytes at a time; a stream at another address
+    (a view into a larger buffer) goes through the kernels that read it byte by byte, with the same results."""
+    import ctypes as C
+
+    from oracle import rans_oracle as ro
+    from tests.hostmodel.model import bf16_bits_to_f32
+
+    m = Model(cus=4)
+    K, N, th = 2048, 96, 1024
+    bits = weight_bits(K, N, 1)
+    enc, man = cases.compress(bits, th)
+    w, keep = m.weight(enc, man, K, N)
+    for shift in (8, 4, 1):
+        room = m.empty(enc.stream.size + 16, np.uint8)
+        C.memmove(room.ptr + shift, enc.stream.ctypes.data, enc.stream.size)
+        w.d_stream = room.ptr + shift
+        out = m.empty((K, N), np.uint8)
+        xb = x_bits(3, K, 2)
+        x, y = m.dev(xb), m.empty((3, N), np.uint16)
+        nb = m.lib.ci_fused_linear_workspace_bytes(3, K, N, th, 32, 0)
+        ws = m.empty(max(nb, 16), np.uint8)
+        ids = np.array([0, 7, 2047, 1024, -1], np.int64)
+        g = m.empty((ids.size, N), np.uint16)
+        nbe = m.lib.ci_fused_embedding_workspace_bytes(ids.size, K, th)
+        wse = m.empty(max(nbe, 16), np.uint8)
+        xh = x_bits(1, N, 2)
+        z = m.empty((1, K), np.uint16)
+        nbt = m.lib.ci_fused_linear_transposed_workspace_bytes(1, N, K, 32)
+        wst = m.empty(max(nbt, 16), np.uint8)
+        m.clear()
+        m.call("ci_decode_tiled", C.byref(w), out.p, None, None)
+        m.call("ci_fused_linear_tiled", C.byref(w), x.p, 3, K, None, y.p, N, ws.p, C.c_size_t(nb), None)
+        m.call("ci_fused_embedding_tiled", C.byref(w), m.dev(ids).p, ids.size, g.p, N, wse.p, C.c_size_t(nbe), None)
+        m.call("ci_fused_linear_transposed_tiled", C.byref(w), m.dev(xh).p, 1, N, None, z.p, K, wst.p, C.c_size_t(nbt), None)
+        assert not any(k.startswith(("decode_tiled32", "fused_linear32", "embed_gather32", "trans32")) for k in m.launches()), m.launches()
+        assert np.array_equal(out.get(), ro.split_bf16(bits)[0])
+        assert np.allclose(bf16_bits_to_f32(y.get()), ro.linear_f32(xb, bits), atol=1e-2, rtol=1e-2)
+        want = np.zeros((ids.size, N), np.uint16)
+        want[:4] = bits[ids[:4]]
+        assert np.array_equal(g.get(), want)
+        assert np.allclose(bf16_bits_to_f32(z.get()), ro.linear_f32(xh, np.ascontiguousarray(bits.T)), atol=1e-2, rtol=1e-2)
 
 
 # ---- split-K reduction ------------------------------------------------------------------------------------------------
