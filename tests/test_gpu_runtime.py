@@ -415,6 +415,48 @@ def test_tied_head_package_ties_the_head_to_the_compressed_table(tmp_path):
     assert "lm_head.rans_exp_stream" in tensors and "lm_head.weight" not in tensors
 
 
+def test_transformers_model_from_its_package_directory(tmp_path):
+    """The loader's own path (comp_inference/pytorch_runtime.py:552-642 with a local directory for model_id): the
+    package written from a transformers model holds config.json with the quantization block; the model is built
+    from that config alone, every compressed module is swapped in with the tile shape its layer_configs entry
+    names (none of them the default here), and the logits are those of the model on its decompressed weights."""
+    transformers = pytest.importorskip("transformers")
+    import comp_inference_amd as ci
+
+    cfg = transformers.LlamaConfig(vocab_size=300, hidden_size=64, intermediate_size=128, num_hidden_layers=2,
+                                   num_attention_heads=2, num_key_value_heads=1, max_position_embeddings=64,
+                                   tie_word_embeddings=False)
+    torch.manual_seed(0)
+    ref = transformers.LlamaForCausalLM(cfg).to(torch.bfloat16).eval()
+    ids = torch.tensor([[1, 17, 299, 64, 5]])
+    with torch.no_grad():
+        want = ref(ids).logits.float()
+    comp = transformers.LlamaForCausalLM(cfg).to(torch.bfloat16).eval()
+    comp.load_state_dict(ref.state_dict())
+    for name, mod in list(comp.named_modules()):
+        if isinstance(mod, nn.Embedding) or name == "lm_head":
+            ci.rans_compress_module_weight(mod, tile_height=128, tile_width=32, transpose_weight=False)
+        elif isinstance(mod, nn.Linear):
+            ci.rans_compress_module_weight(mod, tile_height=64, tile_width=32)
+    out_dir = ci.save_rans_model_package(comp, None, str(tmp_path / "llama"))
+    saved = json.load(open(os.path.join(out_dir, "config.json")))
+    assert saved["model_type"] == "llama" and saved["quantization_config"]["quant_method"] == "rans"
+    assert saved["quantization_config"]["layer_configs"]["model.layers.1.mlp.down_proj"]["tile_height"] == 64
+
+    model = ci.load_compressed_model_with_auto_model(out_dir, os.path.join(out_dir, "model.safetensors"))
+    assert isinstance(model.model.embed_tokens, ci.RansEmbedding) and model.model.embed_tokens.tile_k == 128
+    assert isinstance(model.lm_head, ci.RansLMHead) and model.lm_head.tile_k == 128
+    layer = model.model.layers[1]
+    for lin in (layer.self_attn.q_proj, layer.self_attn.k_proj, layer.self_attn.o_proj, layer.mlp.gate_proj, layer.mlp.down_proj):
+        assert isinstance(lin, ci.RansLinear) and lin.tile_k == 64
+    assert torch.equal(model.model.norm.weight.detach().cpu(), ref.model.norm.weight.detach())
+    with torch.no_grad():
+        got = model(ids.cuda()).logits.float().cpu()
+    # (bf16 activations between the layers: a different summation order moves a logit by a bf16 step or two)
+    assert torch.allclose(got, want, atol=5e-2, rtol=5e-2), (got - want).abs().max()
+    assert (got.argmax(-1) == want.argmax(-1)).float().mean() >= 0.8
+
+
 def test_reloading_buffers_in_place_is_noticed():
     """The loader's idiom replaces `tensor.data` under the same tensor objects: a module that has already run
     must drop what it prepared from the old storage (pointers, checkpoints, slot table) and use the new weight."""

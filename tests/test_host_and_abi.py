@@ -306,6 +306,45 @@ def test_every_required_pointer_and_size_is_checked():
     sweep("ci_build_slot_table", (fake, fake, fake, sz(32768), None), required=(0, 1, 2), misaligned=(1, 2))
 
 
+def test_shared_workspace_grows_and_is_reused():
+    """RansWorkspace (comp_inference/pytorch_runtime.py:386-394): one buffer for all layers, twice the first request,
+    handed out again while it is large enough and on the same device, replaced when a request outgrows it."""
+    from comp_inference_amd.pytorch_runtime import RansWorkspace
+
+    RansWorkspace._buffer = None
+    a = RansWorkspace.get_workspace(4, 96, 8, "cpu")
+    assert a.shape == (8, 4, 96) and a.dtype == torch.bfloat16 and RansWorkspace._buffer.numel() == 2 * 8 * 4 * 96
+    first = RansWorkspace._buffer.data_ptr()
+    b = RansWorkspace.get_workspace(8, 96, 8, "cpu")      # exactly what is there
+    c = RansWorkspace.get_workspace(1, 32, 2, torch.device("cpu"))
+    assert b.data_ptr() == c.data_ptr() == first and c.shape == (2, 1, 32)
+    d = RansWorkspace.get_workspace(8, 96, 8 + 1, "cpu")  # one plane more than the buffer holds
+    assert RansWorkspace._buffer.numel() == 2 * 9 * 8 * 96 and d.shape == (9, 8, 96)
+    RansWorkspace._buffer = None
+
+
+def test_size_queries_answer_zero_for_a_tile_shape_that_cannot_be():
+    """A size query has no error code: a tile height or width of zero (and, for checkpoints, fewer than two
+    segments) gives 0, not a division by zero; a usable shape gives a size."""
+    from comp_inference_amd import _lib
+
+    lib = _lib.lib()
+    for name in ("ci_fused_linear_workspace_bytes", "ci_fused_linear_workspace_bytes_segmented", "ci_checkpoint_bytes",
+                 "ci_fused_embedding_workspace_bytes", "ci_fused_embedding_workspace_bytes_segmented",
+                 "ci_fused_linear_transposed_workspace_bytes"):
+        getattr(lib, name).restype = ctypes.c_size_t
+    K, N = 4096, 96
+    for th, tw, ok in ((1024, 32, True), (0, 32, False), (1024, 0, False), (0, 0, False)):
+        assert (lib.ci_fused_linear_workspace_bytes(3, K, N, th, tw, 0) != 0) == ok, (th, tw)
+        assert (lib.ci_fused_linear_workspace_bytes_segmented(3, K, N, th, tw, 0, 2) != 0) == ok, (th, tw)
+        assert (lib.ci_checkpoint_bytes(K, N, th, tw, 2) != 0) == ok, (th, tw)
+    assert lib.ci_checkpoint_bytes(K, N, 1024, 32, 1) == 0 and lib.ci_checkpoint_bytes(K, N, 1024, 32, 0) == 0
+    assert lib.ci_checkpoint_bytes(K, N, 1024, 32, 4) == 4 * 3 * 3 * 64 * 8  # tiles x (segments - 1) x 64 streams x 8 bytes
+    assert lib.ci_fused_embedding_workspace_bytes(7, K, 0) == 0 and lib.ci_fused_embedding_workspace_bytes(7, K, 1024) != 0
+    assert lib.ci_fused_linear_transposed_workspace_bytes(1, N, K, 0) == 0
+    assert lib.ci_fused_linear_transposed_workspace_bytes(1, N, K, 32) != 0
+
+
 def test_segment_counts_a_tile_height_does_not_allow_are_refused():
     """Checkpoints can cut half a tile into any number of equal runs (the builder and the gather take every divisor);
     the decode and the fused linear read whole 16-row blocks, so they take the counts whose runs are multiples of 16

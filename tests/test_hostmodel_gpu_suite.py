@@ -15,7 +15,7 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 # file -> tests that must at least have passed there (a guard against a run that silently collects nothing)
 FILES = {"test_gpu_codec.py": 43, "test_gpu_linear.py": 65, "test_gpu_embedding.py": 18, "test_gpu_transposed.py": 21,
-         "test_gpu_runtime.py": 9, "test_gpu_errors.py": 4, "test_golden.py": 1, "test_zz_no_alloc.py": 2,
+         "test_gpu_runtime.py": 10, "test_gpu_errors.py": 4, "test_golden.py": 1, "test_zz_no_alloc.py": 2,
          "test_gpu_zy_device_status.py": 1, "wip_one_stream.py": 15, "wip_transposed_seg.py": 10, "wip_linear_wide.py": 10,
          "wip_gather_seg.py": 8}
 

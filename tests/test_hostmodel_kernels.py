@@ -246,6 +246,9 @@ def test_fused_linear_on_unusual_planes(kind):
     (2048, 127, 64, 1024, 8, False, "embed_gather32_kernel"),
     (70000, 64, 2048, 1024, 8, True, "embed_gather32_seg_kernel"),
     (270000, 32, 500, 32, 1, False, "embed_sort_kernel"),            # more buckets than counting slots: the sort
+    (2048, 32, 8192, 1024, 4, True, "embed_gather32_seg_kernel"),    # exactly one pass of ids: no second, empty pass
+    (2048, 32, 8192 + 3, 1024, 1, False, "embed_gather32_kernel"),   # a second pass of three ids
+    (300000, 32, 16384, 32, 1, False, "embed_sort_kernel"),          # two whole passes through the sort
 ])
 @in_child
 def test_fused_gather(K, N, n, th, segs, slot, kernel):
