@@ -12,6 +12,12 @@ things are rewritten in the preprocessed text before it is compiled for x86-64:
     wavefront before and after: on the GPU a wavefront's LDS operations complete in order, in the model the lanes are
     fibres that run one after the other between meeting points.
 
+A second library, libci_hostmodel_order.so (`build(order=True)`, `--order`), is the same with the kernel sources
+compiled under the compiler's thread-sanitizer instrumentation and no sanitizer runtime: the model itself (sim.cpp,
+"ordering between wavefronts") takes the calls the instrumentation makes at every plain memory access, and reports
+two wavefronts that touch the same byte with no barrier or release/acquire pair between them -- what fibres that run
+one after the other would never show.
+
 Test infrastructure: nothing of the product is built from, or loads, what this makes.
 """
 from __future__ import annotations
@@ -26,6 +32,8 @@ ROOT = os.path.dirname(os.path.dirname(HERE))
 CSRC = os.path.join(ROOT, "comp_inference_amd", "csrc")
 OUT_DIR = os.path.join(HERE, "_build")
 LIB_PATH = os.path.join(HERE, "libci_hostmodel.so")
+ORDER_LIB_PATH = os.path.join(HERE, "libci_hostmodel_order.so")
+ORDER_FLAGS = ["-fsanitize=thread", "-mllvm", "-tsan-instrument-func-entry-exit=0"]
 CXX = os.environ.get("CI_HOSTMODEL_CXX", "/opt/rocm/llvm/bin/clang++")
 SOURCES = ["api.hip", "encode.hip", "decode.hip", "linear.hip", "embedding.hip", "transposed.hip", "legacy.hip"]
 CXXFLAGS = ["-std=c++17", "-O1", "-g", "-fPIC", "-fno-strict-aliasing", "-Wno-unused-value", "-Wno-unknown-attributes",
@@ -140,6 +148,9 @@ def rewrite_asm(text: str) -> str:
 def rewrite_lds(text: str) -> str:
     text, n = re.subn(r"extern\s+__shared__\s+__attribute__\(\(aligned\(16\)\)\)\s+uint8_t\s+lds\[\]\s*;",
                       "uint8_t *const lds = sim::lds_base();", text)
+    # a `__shared__` array is a static here; the ordering check is told that it is shared memory of the workgroup
+    text = re.sub(r"\b__shared__\s+([\w:]+)\s+(\w+)\s*\[([^\]]+)\]\s*;",
+                  r"static \1 \2[\3]; sim::shared_static(\2, sizeof(\2));", text)
     return re.sub(r"\b__shared__\b", "static", text)
 
 
@@ -160,32 +171,35 @@ def rewrite(text: str) -> str:
     return fence_handover(rewrite_lds(rewrite_asm(text)))
 
 
-def needs_build() -> bool:
-    if not os.path.exists(LIB_PATH):
+def needs_build(lib_path: str = LIB_PATH) -> bool:
+    if not os.path.exists(lib_path):
         return True
-    built = os.path.getmtime(LIB_PATH)
+    built = os.path.getmtime(lib_path)
     deps = [os.path.join(CSRC, f) for f in os.listdir(CSRC)] + [os.path.join(HERE, f) for f in ("sim.cpp", "sim.h", "build.py", "selftest.hip")]
     deps += [os.path.join(HERE, "hip", "hip_runtime.h"), os.path.join(ROOT, "include", "comp_inference_hip.h")]
     return any(os.path.getmtime(d) > built for d in deps)
 
 
-def build(force: bool = False, verbose: bool = False) -> str:
-    if not force and not needs_build():
-        return LIB_PATH
-    os.makedirs(OUT_DIR, exist_ok=True)
+def build(force: bool = False, verbose: bool = False, order: bool = False) -> str:
+    lib_path = ORDER_LIB_PATH if order else LIB_PATH
+    if not force and not needs_build(lib_path):
+        return lib_path
+    out_dir = os.path.join(OUT_DIR, "order") if order else OUT_DIR
+    os.makedirs(out_dir, exist_ok=True)
+    flags = CXXFLAGS + (ORDER_FLAGS if order else [])
     procs, objs = [], []
     for src in SOURCES + ["selftest.hip"]:
         path = os.path.join(HERE if src == "selftest.hip" else CSRC, src)
         pre = subprocess.run([CXX, "-E", "-x", "c++", "-std=c++17", "-I", HERE, "-I", CSRC, path, "-o", "-"],
                              check=True, capture_output=True, text=True).stdout
-        ii = os.path.join(OUT_DIR, src + ".ii")
+        ii = os.path.join(out_dir, src + ".ii")
         with open(ii, "w") as f:
             f.write(rewrite(pre))
-        obj = os.path.join(OUT_DIR, src + ".o")
-        procs.append((src, subprocess.Popen([CXX, "-x", "c++-cpp-output", *CXXFLAGS, "-c", ii, "-o", obj],
+        obj = os.path.join(out_dir, src + ".o")
+        procs.append((src, subprocess.Popen([CXX, "-x", "c++-cpp-output", *flags, "-c", ii, "-o", obj],
                                             stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
         objs.append(obj)
-    obj = os.path.join(OUT_DIR, "sim.o")
+    obj = os.path.join(out_dir, "sim.o")  # (the model itself is never instrumented)
     procs.append(("sim.cpp", subprocess.Popen([CXX, *CXXFLAGS, "-O2", "-c", os.path.join(HERE, "sim.cpp"), "-o", obj],
                                               stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
     objs.append(obj)
@@ -199,19 +213,22 @@ def build(force: bool = False, verbose: bool = False) -> str:
             print(out[-3000:])
     if failed:
         raise RuntimeError("host-model build failed")
-    subprocess.check_call([CXX, "-shared", "-fPIC", "-o", LIB_PATH, *objs])
-    return LIB_PATH
+    subprocess.check_call([CXX, "-shared", "-fPIC", "-o", lib_path, *objs])
+    return lib_path
 
 
-def build_mutant(tag: str, edits: list, rebuild: list) -> str:
+def build_mutant(tag: str, edits: list, rebuild: list, order: bool = False) -> str:
     """The host-model library with a deliberate mistake in the kernels: `edits` = [(file under csrc, old text, new text[, occurrences])],
     the first occurrence of each old text replaced (of one, unless stated); `rebuild` = the .hip sources to compile again from the edited copy (the other
     objects are the intact build's).  Returns the path of the mutant library, under _build/mutants/<tag>/.  For the
-    tests that show that a mistake of a given kind in the real kernels is noticed."""
+    tests that show that a mistake of a given kind in the real kernels is noticed.  `order`: the build that checks the
+    ordering between wavefronts."""
     import shutil
 
-    build()
-    base = os.path.join(OUT_DIR, "mutants", tag)
+    build(order=order)
+    intact = os.path.join(OUT_DIR, "order") if order else OUT_DIR
+    flags = CXXFLAGS + (ORDER_FLAGS if order else [])
+    base = os.path.join(OUT_DIR, "mutants", tag + ("_order" if order else ""))
     src_dir = os.path.join(base, "csrc")
     shutil.rmtree(base, ignore_errors=True)
     shutil.copytree(CSRC, src_dir, ignore=shutil.ignore_patterns("*.o", "*.so"))
@@ -225,17 +242,17 @@ def build_mutant(tag: str, edits: list, rebuild: list) -> str:
     procs, objs = [], []
     for src in SOURCES + ["selftest.hip"]:
         if src not in rebuild:
-            objs.append(os.path.join(OUT_DIR, src + ".o"))
+            objs.append(os.path.join(intact, src + ".o"))
             continue
         pre = subprocess.run([CXX, "-E", "-x", "c++", "-std=c++17", "-I", HERE, "-I", src_dir, os.path.join(src_dir, src), "-o", "-"],
                              check=True, capture_output=True, text=True).stdout
         ii, obj = os.path.join(base, src + ".ii"), os.path.join(base, src + ".o")
         with open(ii, "w") as f:
             f.write(rewrite(pre))
-        procs.append((src, subprocess.Popen([CXX, "-x", "c++-cpp-output", *CXXFLAGS, "-c", ii, "-o", obj],
+        procs.append((src, subprocess.Popen([CXX, "-x", "c++-cpp-output", *flags, "-c", ii, "-o", obj],
                                             stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
         objs.append(obj)
-    objs.append(os.path.join(OUT_DIR, "sim.o"))
+    objs.append(os.path.join(intact, "sim.o"))
     for src, p in procs:
         out, _ = p.communicate()
         if p.returncode != 0:
@@ -246,4 +263,4 @@ def build_mutant(tag: str, edits: list, rebuild: list) -> str:
 
 
 if __name__ == "__main__":
-    print(build(force="--force" in sys.argv, verbose=True))
+    print(build(force="--force" in sys.argv, verbose=True, order="--order" in sys.argv))

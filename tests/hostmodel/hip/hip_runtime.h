@@ -77,34 +77,58 @@ CI_SIM_MINMAX(double)
 #define __shfl(v, src, width) sim::shfl((int)(v), (int)(src), (int)(width))
 #define __shfl_up(v, d, width) sim::shfl_up((int)(v), (unsigned)(d), (int)(width))
 
-// One thread runs at a time: plain reads and writes are atomic.
+// One thread runs at a time: plain reads and writes are atomic.  In the build that checks the ordering between
+// wavefronts these functions are not instrumented: an atomic access is told to the model as such (sim::order_atomic).
+#define CI_SIM_ATOMIC_FN __attribute__((no_sanitize("thread"))) static inline
 template <typename T>
-static inline T atomicAdd(T *p, T v) {
+CI_SIM_ATOMIC_FN T atomicAdd(T *p, T v) {
+    sim::order_atomic(p, true, true);
     T o = *p;
     *p = o + v;
     return o;
 }
 template <typename T>
-static inline T atomicMax(T *p, T v) {
+CI_SIM_ATOMIC_FN T atomicMax(T *p, T v) {
+    sim::order_atomic(p, true, true);
     T o = *p;
     if (v > o) *p = v;
     return o;
 }
 template <typename T>
-static inline T atomicOr(T *p, T v) {
+CI_SIM_ATOMIC_FN T atomicOr(T *p, T v) {
+    sim::order_atomic(p, true, true);
     T o = *p;
     *p = o | v;
     return o;
 }
 #define __HIP_MEMORY_SCOPE_WORKGROUP 0
-#define __hip_atomic_load(p, order, scope) (*(volatile __typeof__(*(p)) *)(p))
 // (an operation that publishes -- release semantics -- comes after what the other lanes of the wavefront did earlier
 // in the program: sim::wave_catch_up)
 #define CI_SIM_RELEASES(order) ((order) == __ATOMIC_RELEASE || (order) == __ATOMIC_ACQ_REL || (order) == __ATOMIC_SEQ_CST)
-#define __hip_atomic_store(p, v, order, scope) \
-    ((void)(CI_SIM_RELEASES(order) ? sim::wave_catch_up() : (void)0), (void)(*(volatile __typeof__(*(p)) *)(p) = (v)))
-#define __hip_atomic_fetch_add(p, v, order, scope) \
-    ((void)(CI_SIM_RELEASES(order) ? sim::wave_catch_up() : (void)0), atomicAdd((p), (__typeof__(*(p)))(v)))
+#define CI_SIM_ACQUIRES(order) ((order) == __ATOMIC_ACQUIRE || (order) == __ATOMIC_ACQ_REL || (order) == __ATOMIC_SEQ_CST)
+template <typename T>
+CI_SIM_ATOMIC_FN T ci_sim_atomic_load(T *p, int order) {
+    const T v = *(volatile T *)p;
+    sim::order_atomic(p, CI_SIM_ACQUIRES(order), false);
+    return v;
+}
+template <typename T, typename V>
+CI_SIM_ATOMIC_FN void ci_sim_atomic_store(T *p, V v, int order) {
+    if (CI_SIM_RELEASES(order)) sim::wave_catch_up();
+    sim::order_atomic(p, false, CI_SIM_RELEASES(order));
+    *(volatile T *)p = (T)v;
+}
+template <typename T, typename V>
+CI_SIM_ATOMIC_FN T ci_sim_atomic_fetch_add(T *p, V v, int order) {
+    if (CI_SIM_RELEASES(order)) sim::wave_catch_up();
+    sim::order_atomic(p, CI_SIM_ACQUIRES(order), CI_SIM_RELEASES(order));
+    const T o = *(volatile T *)p;
+    *(volatile T *)p = o + (T)v;
+    return o;
+}
+#define __hip_atomic_load(p, order, scope) ci_sim_atomic_load((p), (order))
+#define __hip_atomic_store(p, v, order, scope) ci_sim_atomic_store((p), (v), (order))
+#define __hip_atomic_fetch_add(p, v, order, scope) ci_sim_atomic_fetch_add((p), (v), (order))
 
 // ---- host API -------------------------------------------------------------------------------------------------
 typedef int hipError_t;

@@ -174,9 +174,67 @@ __global__ void st_handover_kernel(uint32_t *out) {
 // A plain C++ load past the end of an array: the page behind the array is inaccessible.
 __global__ void st_plain_overrun_kernel(const uint32_t *src, uint32_t n, uint32_t *dst) { dst[threadIdx.x] = src[n + 16 + threadIdx.x]; }
 
+// For the build that checks the ordering between wavefronts.  Four wavefronts each write a row of an LDS array and
+// read their neighbour's; a word goes from one wavefront to another through a flag; two workgroups write the output.
+// which: 0 correct; 1 no barrier between the writes and the neighbour's reads; 2 a second round of writes follows the
+// reads without a barrier (write after read); 3 the flag is written and read without release / acquire; 4 the asm
+// interpreter reads the neighbour's row with no barrier; 5 a `__shared__` array instead of the dynamic LDS, no barrier;
+// 6 every workgroup writes the same output words; 7 workgroup 1 reads what workgroup 0 writes
+__global__ void st_ordering_kernel(uint32_t *out, int which) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    __shared__ uint32_t fixed[256];
+    uint32_t *rows = which == 5 ? fixed : reinterpret_cast<uint32_t *>(lds), *flag = reinterpret_cast<uint32_t *>(lds) + 300,
+             *word = reinterpret_cast<uint32_t *>(lds) + 1000;
+    const uint32_t tid = threadIdx.x, wave = tid / 64, lane = tid % 64, next = ((wave + 1) % 4) * 64 + lane;
+    rows[tid] = tid * 7u;
+    if (tid == 0) *flag = 0;
+    if (which != 1 && which != 4 && which != 5) __syncthreads();
+    uint32_t v;
+    if (which == 4) {
+        __syncthreads();                       // (this one orders the first writes ...)
+        rows[tid] = tid * 7u;                  // ... and these come after it, unordered with the neighbour's read below
+        uint32_t b = 0;
+        const uint32_t addr = (uint32_t)(uintptr_t)lds + next * 4u;
+        asm volatile("ds_read_u8 %[b], %[a]\n"
+                     "s_waitcnt lgkmcnt(0)\n"
+                     : [b] "=&v"(b)
+                     : [a] "v"(addr)
+                     : "memory");
+        v = b;
+    } else {
+        v = rows[next];
+    }
+    if (which == 2) rows[tid] = v;  // the neighbour may not have read this row yet
+    if (which == 0) {
+        __syncthreads();
+        rows[tid] = v;
+    }
+    __syncthreads();
+    // a word handed from wavefront 1 to wavefront 0
+    if (tid == 64) {
+        *word = 4711;
+        if (which == 3)
+            __hip_atomic_store(flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        else
+            __hip_atomic_store(flag, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+    if (tid < 64) {
+        if (which == 3)
+            while (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) == 0) __builtin_amdgcn_s_sleep(2);
+        else
+            while (__hip_atomic_load(flag, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) == 0) __builtin_amdgcn_s_sleep(2);
+        v += *word;
+    }
+    if (which == 7 && blockIdx.x == 1) v += out[tid];
+    out[(which == 6 || which == 7 ? 0u : blockIdx.x) * blockDim.x + tid] = v;
+}
+
 }  // namespace
 
 extern "C" {
+void simtest_ordering(uint32_t *out, int which) {
+    hipLaunchKernelGGL(st_ordering_kernel, dim3(2), dim3(256), 8192, nullptr, out, which);
+}
 void simtest_global_load(const uint32_t *src, uint32_t n, uint32_t *dst, int which) {
     hipLaunchKernelGGL(st_global_load_kernel, dim3(1), dim3(64), 0, nullptr, src, n, dst, which);
 }

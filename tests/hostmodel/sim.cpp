@@ -148,6 +148,221 @@ static std::string where() {
     return buf;
 }
 
+// ---- ordering between wavefronts -------------------------------------------------------------------------------
+// In the build whose kernel sources are compiled with the compiler's thread-sanitizer instrumentation (build.py,
+// `order=True`) every plain memory access of the kernels calls one of the __tsan_* hooks at the end of this file, and
+// the interpreter reports its own accesses here as well.  What is checked is what the fibres cannot show by
+// themselves, since they run one after the other: two wavefronts that touch the same byte, at least one of them
+// writing, with nothing between the two accesses that orders them on the GPU.
+//   * LDS (and `__shared__` arrays): a wavefront counts as one thread -- its lanes run in step, and its LDS
+//     operations complete in order -- with a vector clock over the wavefronts of the workgroup.  A workgroup barrier
+//     joins the clocks of the wavefronts that wait at it; an atomic with release semantics leaves the wavefront's
+//     clock at its address, one with acquire semantics takes what was left there.
+//   * arrays from sim_alloc: the same inside a workgroup; between workgroups of one launch nothing orders anything, so
+//     a byte written by one workgroup and read or written by another is reported.  Launches are ordered by the stream.
+// Atomic accesses themselves are not recorded (they do not race with each other).
+constexpr int kMaxWaves = kMaxThreads / 64;
+static bool g_order_on = false;
+static uint32_t g_vc[kMaxWaves][kMaxWaves];
+static uint8_t *g_sh_wwave = nullptr;   // per LDS byte: the wavefront that wrote it last (0xFF: none in this workgroup)
+static uint32_t *g_sh_wclk = nullptr;   //   ... at this value of its own clock
+static uint32_t *g_sh_rclk = nullptr;   // per LDS byte and wavefront: its clock when it last read the byte (0: never)
+static std::unordered_map<uint64_t, std::vector<uint32_t>> g_sync;  // address of an atomic -> clock left by releases
+struct SharedStatic {  // a `__shared__` array of a kernel, with a shadow of its own (emptied when a new workgroup first touches it)
+    uint64_t ptr;
+    size_t bytes;
+    uint64_t workgroup;
+    std::vector<uint8_t> wwave;
+    std::vector<uint32_t> wclk, rclk;
+};
+static std::vector<SharedStatic> g_shared_statics;
+static uint32_t g_wg_index = 0, g_order_reports = 0;
+static uint64_t g_launch_seq = 0, g_workgroup_seq = 0;
+struct GlobalShadow {
+    uint64_t launch = 0;  // the launch its contents belong to
+    std::vector<uint32_t> w_id, w_clk, r_id, r_clk;  // per byte: (workgroup + 1) << 4 | wavefront, and that wavefront's clock
+};
+static std::unordered_map<uint64_t, GlobalShadow> g_global_shadow;  // by Alloc::ptr
+
+static void order_report(const char *fmt, ...) {
+    if (++g_order_reports > 6) return;  // per launch
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    violation("ordering: %s", buf);
+}
+
+static void order_start_workgroup(uint32_t n_waves, size_t lds_open) {
+    if (!g_order_on) return;
+    ++g_workgroup_seq;
+    if (!g_sh_wwave) {
+        const size_t n = kLdsBytes;
+        g_sh_wwave = (uint8_t *)malloc(n);
+        g_sh_wclk = (uint32_t *)malloc(n * 4);
+        g_sh_rclk = (uint32_t *)malloc(n * 4 * kMaxWaves);
+        if (!g_sh_wwave || !g_sh_wclk || !g_sh_rclk) abort();
+        lds_open = kLdsBytes;
+    }
+    memset(g_sh_wwave, 0xFF, lds_open);
+    memset(g_sh_rclk, 0, lds_open * 4 * kMaxWaves);
+    memset(g_vc, 0, sizeof g_vc);
+    for (uint32_t w = 0; w < n_waves; ++w) g_vc[w][w] = 1;
+    g_sync.clear();
+}
+
+// The wavefronts in `mask` leave a workgroup barrier together.
+static void order_barrier(uint32_t mask) {
+    if (!g_order_on) return;
+    uint32_t joined[kMaxWaves] = {0};
+    for (int w = 0; w < kMaxWaves; ++w)
+        if (mask >> w & 1)
+            for (int k = 0; k < kMaxWaves; ++k) joined[k] = joined[k] > g_vc[w][k] ? joined[k] : g_vc[w][k];
+    for (int w = 0; w < kMaxWaves; ++w)
+        if (mask >> w & 1) {
+            memcpy(g_vc[w], joined, sizeof joined);
+            ++g_vc[w][w];
+        }
+}
+
+static inline uint32_t cur_wave() { return g_cur->ctx.thread_idx.x / 64; }
+
+// The shadow of one area of shared memory.
+struct SharedShadow {
+    uint8_t *wwave;
+    uint32_t *wclk, *rclk;
+};
+
+static void order_shared(const SharedShadow &sh, size_t off, size_t n, bool write, const char *what) {
+    const uint32_t w = cur_wave();
+    for (size_t b = off; b < off + n; ++b) {
+        const uint8_t ww = sh.wwave[b];
+        if (ww != 0xFF && ww != w && sh.wclk[b] > g_vc[w][ww]) {
+            order_report("wavefront %u %s byte 0x%zx of %s (an access of %zu bytes) that wavefront %u wrote, and no barrier or "
+                         "release/acquire pair lies between the two", w, write ? "overwrites" : "reads", b, what, n, ww);
+            return;
+        }
+        if (write) {
+            for (uint32_t r = 0; r < (uint32_t)kMaxWaves; ++r)
+                if (r != w && sh.rclk[b * kMaxWaves + r] > g_vc[w][r]) {
+                    order_report("wavefront %u writes byte 0x%zx of %s (an access of %zu bytes) that wavefront %u read, and no barrier or "
+                                 "release/acquire pair lies between the two", w, b, what, n, r);
+                    return;
+                }
+            sh.wwave[b] = (uint8_t)w;
+            sh.wclk[b] = g_vc[w][w];
+        } else {
+            sh.rclk[b * kMaxWaves + w] = g_vc[w][w];
+        }
+    }
+}
+
+// An access to the LDS or to a `__shared__` array: checked, and true.
+static bool order_shared_access(uint64_t addr, size_t n, bool write) {
+    if (addr - (uint64_t)g_lds < kLdsBytes) {
+        order_shared(SharedShadow{g_sh_wwave, g_sh_wclk, g_sh_rclk}, (size_t)(addr - (uint64_t)g_lds), n, write, "the LDS");
+        return true;
+    }
+    for (SharedStatic &s : g_shared_statics)
+        if (addr - s.ptr < s.bytes) {
+            if (s.workgroup != g_workgroup_seq) {
+                s.workgroup = g_workgroup_seq;
+                s.wwave.assign(s.bytes + 16, 0xFF);
+                s.wclk.assign(s.bytes + 16, 0);
+                s.rclk.assign((s.bytes + 16) * kMaxWaves, 0);
+            }
+            order_shared(SharedShadow{s.wwave.data(), s.wclk.data(), s.rclk.data()}, (size_t)(addr - s.ptr), n, write, "a __shared__ array");
+            return true;
+        }
+    return false;
+}
+
+static bool is_shared(uint64_t addr) {
+    if (addr - (uint64_t)g_lds < kLdsBytes) return true;
+    for (const SharedStatic &s : g_shared_statics)
+        if (addr - s.ptr < s.bytes) return true;
+    return false;
+}
+
+static void order_global(const Alloc &a, uint64_t addr, size_t n, bool write) {
+    GlobalShadow &s = g_global_shadow[(uint64_t)a.ptr];
+    if (s.launch != g_launch_seq || s.w_id.size() != a.bytes) {
+        s.launch = g_launch_seq;
+        s.w_id.assign(a.bytes, 0);
+        s.w_clk.assign(a.bytes, 0);
+        s.r_id.assign(a.bytes, 0);
+        s.r_clk.assign(a.bytes, 0);
+    }
+    const uint32_t w = cur_wave(), me = (g_wg_index + 1) << 4 | w;
+    // did the access `id` at clock `clk` happen before what this wavefront does now?
+    auto before = [&](uint32_t id, uint32_t clk) { return id == 0 || id == me || (id >> 4 == me >> 4 && clk <= g_vc[w][id & 15]); };
+    const size_t o = (size_t)(addr - (uint64_t)a.ptr);
+    for (size_t i = 0; i < n && o + i < a.bytes; ++i) {
+        const size_t b = o + i;
+        if (!before(s.w_id[b], s.w_clk[b])) {
+            order_report("workgroup %u wavefront %u %s byte %zu of allocation #%zu (%zu bytes) that workgroup %u wavefront %u wrote in the "
+                         "same launch, and nothing orders the two", g_wg_index, w, write ? "overwrites" : "reads", b,
+                         (size_t)(&a - g_allocs.data()), a.bytes, (s.w_id[b] >> 4) - 1, s.w_id[b] & 15);
+            return;
+        }
+        if (write) {
+            if (!before(s.r_id[b], s.r_clk[b])) {
+                order_report("workgroup %u wavefront %u writes byte %zu of allocation #%zu (%zu bytes) that workgroup %u wavefront %u read in "
+                             "the same launch, and nothing orders the two", g_wg_index, w, b, (size_t)(&a - g_allocs.data()), a.bytes,
+                             (s.r_id[b] >> 4) - 1, s.r_id[b] & 15);
+                return;
+            }
+            s.w_id[b] = me;
+            s.w_clk[b] = g_vc[w][w];
+        } else {
+            s.r_id[b] = me;
+            s.r_clk[b] = g_vc[w][w];
+        }
+    }
+}
+
+// Every access of kernel code: plain C++ through the compiler's hooks, the interpreter's by its own calls.
+static inline void order_access(uint64_t addr, size_t n, bool write) {
+    if (!g_order_on || !g_cur || n == 0) return;
+    if (addr - (uint64_t)g_stacks < (uint64_t)kMaxThreads * kStackBytes) return;  // a fibre's own stack
+    if (order_shared_access(addr, n, write)) return;
+    static size_t last = 0;
+    if (last < g_allocs.size() && addr - (uint64_t)g_allocs[last].ptr < g_allocs[last].bytes) {
+        order_global(g_allocs[last], addr, n, write);
+        return;
+    }
+    for (size_t k = 0; k < g_allocs.size(); ++k)
+        if (addr - (uint64_t)g_allocs[k].ptr < g_allocs[k].bytes) {
+            last = k;
+            order_global(g_allocs[k], addr, n, write);
+            return;
+        }
+}
+
+// An atomic access of kernel code (the stand-ins of hip_runtime.h call this): no access is recorded; release and
+// acquire move clocks through the address.  Device-scope atomics on arrays order nothing between workgroups here.
+void order_atomic(const void *p, bool acquire, bool release) {
+    if (!g_order_on || !g_cur) return;
+    if (!is_shared((uint64_t)p)) return;
+    const uint32_t w = cur_wave();
+    std::vector<uint32_t> &left = g_sync[(uint64_t)p];
+    if (left.empty()) left.assign(kMaxWaves, 0);
+    if (acquire)
+        for (int k = 0; k < kMaxWaves; ++k) g_vc[w][k] = g_vc[w][k] > left[k] ? g_vc[w][k] : left[k];
+    if (release) {
+        for (int k = 0; k < kMaxWaves; ++k) left[k] = left[k] > g_vc[w][k] ? left[k] : g_vc[w][k];
+        ++g_vc[w][w];
+    }
+}
+
+void shared_static(const void *p, size_t bytes) {
+    if (!g_order_on) return;
+    for (const SharedStatic &s : g_shared_statics)
+        if (s.ptr == (uint64_t)p) return;
+    g_shared_statics.push_back(SharedStatic{(uint64_t)p, bytes, 0, {}, {}, {}});
+}
+
 extern "C" void sim_switch(void **from_sp, void *to_sp);
 asm(R"(
 .text
@@ -849,6 +1064,7 @@ static void exec_asm(Fiber **lanes, int n_lanes_total, uint64_t part) {
                         continue;
                     }
                     if (nb == 8 && (addr & 7)) violation("`%s`: lane %d reads 8 bytes at the unaligned LDS address 0x%llx", in.text.c_str(), l, (unsigned long long)addr);
+                    order_access((uint64_t)g_lds + addr, nb, false);
                     if (nb == 1) {
                         w.v[o[0].reg][l] = g_lds[addr];
                     } else {
@@ -881,6 +1097,7 @@ static void exec_asm(Fiber **lanes, int n_lanes_total, uint64_t part) {
                     }
                     if (addr & (nr == 4 ? 15 : 3))
                         violation("`%s`: lane %d loads %d bytes at the unaligned address 0x%llx", in.text.c_str(), l, 4 * nr, (unsigned long long)addr);
+                    order_access(addr, 4 * nr, false);
                     for (int j = 0; j < nr; ++j) memcpy(&w.v[o[0].reg + j][l], (const void *)(addr + 4 * j), 4);
                 }
                 for (int j = 0; j < nr; ++j) {
@@ -904,6 +1121,7 @@ static void exec_asm(Fiber **lanes, int n_lanes_total, uint64_t part) {
                                   (unsigned long long)addr, describe_address(addr).c_str());
                         continue;
                     }
+                    order_access(addr, 1, true);
                     *(uint8_t *)addr = (uint8_t)w.v[o[1].reg][l];
                 }
                 break;
@@ -1103,6 +1321,8 @@ static bool run_workgroup(uint32_t nthreads, const LaneCtx &proto) {
     }
     memset(g_lds, 0xCD, g_lds_open);
     const uint32_t n_waves = (nthreads + 63) / 64;
+    g_wg_index = (proto.block_idx.z * proto.grid_dim.y + proto.block_idx.y) * proto.grid_dim.x + proto.block_idx.x;
+    order_start_workgroup(n_waves, g_lds_open);
     uint32_t order[kMaxThreads / 64];
     for (uint32_t i = 0; i < n_waves; ++i) order[i] = i;
     for (;;) {
@@ -1155,8 +1375,13 @@ static bool run_workgroup(uint32_t nthreads, const LaneCtx &proto) {
         }
         if (live == 0) return true;
         if (at_wg == live) {
+            uint32_t at_barrier = 0;  // the wavefronts that wait at it (one that has ended takes no part)
             for (uint32_t t = 0; t < nthreads; ++t)
-                if (g_fib[t].st == WAIT_WG) g_fib[t].st = RUN;
+                if (g_fib[t].st == WAIT_WG) {
+                    g_fib[t].st = RUN;
+                    at_barrier |= 1u << (t / 64);
+                }
+            order_barrier(at_barrier);
             progress = true;
         }
         if (!progress) {
@@ -1206,6 +1431,8 @@ void launch(const char *name, const void *fn, Dim3 grid, Dim3 block, size_t shme
     g_lds_open = (shmem + 4095) & ~(size_t)4095;
     if (g_lds_open < kLdsBytes) mprotect(g_lds + g_lds_open, kLdsBytes - g_lds_open, PROT_NONE);
     g_abort_launch = false;
+    ++g_launch_seq;
+    g_order_reports = 0;
     LaneCtx proto;
     proto.block_dim = block;
     proto.grid_dim = grid;
@@ -1296,3 +1523,71 @@ extern "C" void sim_clear(void) {
 extern "C" int sim_launch_count(void) { return (int)g_launches.size(); }
 extern "C" const char *sim_launch_name(int i) { return i >= 0 && i < (int)g_launches.size() ? g_launches[i].c_str() : ""; }
 extern "C" uint64_t sim_asm_instructions(void) { return g_asm_instructions; }
+
+// ---- the compiler's hooks (thread-sanitizer instrumentation of the kernel sources; see "ordering" above) -----------
+// Only the instrumented build calls these; __tsan_init, which every instrumented object calls when the library is
+// loaded, is what switches the ordering check on.
+extern "C" {
+void __tsan_init(void) { g_order_on = true; }
+void __tsan_func_entry(void *) {}
+void __tsan_func_exit(void) {}
+void __tsan_vptr_update(void **, void *) {}
+void __tsan_vptr_read(void **) {}
+#define CI_SIM_HOOK(n)                                                                          \
+    void __tsan_read##n(void *p) { order_access((uint64_t)p, n, false); }                       \
+    void __tsan_write##n(void *p) { order_access((uint64_t)p, n, true); }                       \
+    void __tsan_unaligned_read##n(void *p) { order_access((uint64_t)p, n, false); }             \
+    void __tsan_unaligned_write##n(void *p) { order_access((uint64_t)p, n, true); }             \
+    void __tsan_volatile_read##n(void *p) { order_access((uint64_t)p, n, false); }              \
+    void __tsan_volatile_write##n(void *p) { order_access((uint64_t)p, n, true); }              \
+    void __tsan_unaligned_volatile_read##n(void *p) { order_access((uint64_t)p, n, false); }    \
+    void __tsan_unaligned_volatile_write##n(void *p) { order_access((uint64_t)p, n, true); }    \
+    void __tsan_read_write##n(void *p) { order_access((uint64_t)p, n, true); }                  \
+    void __tsan_unaligned_read_write##n(void *p) { order_access((uint64_t)p, n, true); }
+CI_SIM_HOOK(1)
+CI_SIM_HOOK(2)
+CI_SIM_HOOK(4)
+CI_SIM_HOOK(8)
+CI_SIM_HOOK(16)
+#undef CI_SIM_HOOK
+void __tsan_read_range(void *p, unsigned long n) { order_access((uint64_t)p, n, false); }
+void __tsan_write_range(void *p, unsigned long n) { order_access((uint64_t)p, n, true); }
+void *__tsan_memcpy(void *d, const void *s, unsigned long n) {
+    order_access((uint64_t)s, n, false);
+    order_access((uint64_t)d, n, true);
+    return memcpy(d, s, n);
+}
+void *__tsan_memmove(void *d, const void *s, unsigned long n) {
+    order_access((uint64_t)s, n, false);
+    order_access((uint64_t)d, n, true);
+    return memmove(d, s, n);
+}
+void *__tsan_memset(void *d, int v, unsigned long n) {
+    order_access((uint64_t)d, n, true);
+    return memset(d, v, n);
+}
+// std::atomic in the host code of the sources (process-wide switches): carried out, nothing to check
+#define CI_SIM_ATOMIC(bits, T)                                                                                       \
+    T __tsan_atomic##bits##_load(const volatile T *p, int) { return __atomic_load_n(p, __ATOMIC_SEQ_CST); }          \
+    void __tsan_atomic##bits##_store(volatile T *p, T v, int) { __atomic_store_n(p, v, __ATOMIC_SEQ_CST); }          \
+    T __tsan_atomic##bits##_exchange(volatile T *p, T v, int) { return __atomic_exchange_n(p, v, __ATOMIC_SEQ_CST); } \
+    T __tsan_atomic##bits##_fetch_add(volatile T *p, T v, int) { return __atomic_fetch_add(p, v, __ATOMIC_SEQ_CST); } \
+    T __tsan_atomic##bits##_fetch_sub(volatile T *p, T v, int) { return __atomic_fetch_sub(p, v, __ATOMIC_SEQ_CST); } \
+    T __tsan_atomic##bits##_fetch_and(volatile T *p, T v, int) { return __atomic_fetch_and(p, v, __ATOMIC_SEQ_CST); } \
+    T __tsan_atomic##bits##_fetch_or(volatile T *p, T v, int) { return __atomic_fetch_or(p, v, __ATOMIC_SEQ_CST); }   \
+    T __tsan_atomic##bits##_fetch_xor(volatile T *p, T v, int) { return __atomic_fetch_xor(p, v, __ATOMIC_SEQ_CST); } \
+    int __tsan_atomic##bits##_compare_exchange_strong(volatile T *p, T *e, T v, int, int) {                          \
+        return __atomic_compare_exchange_n(p, e, v, false, __ATOMIC_SEQ_CST, __ATOMIC_SEQ_CST);                      \
+    }                                                                                                                \
+    int __tsan_atomic##bits##_compare_exchange_weak(volatile T *p, T *e, T v, int, int) {                            \
+        return __atomic_compare_exchange_n(p, e, v, false, __ATOMIC_SEQ_CST, __ATOMIC_SEQ_CST);                      \
+    }
+CI_SIM_ATOMIC(8, uint8_t)
+CI_SIM_ATOMIC(16, uint16_t)
+CI_SIM_ATOMIC(32, uint32_t)
+CI_SIM_ATOMIC(64, uint64_t)
+#undef CI_SIM_ATOMIC
+void __tsan_atomic_thread_fence(int) {}
+void __tsan_atomic_signal_fence(int) {}
+int sim_checks_ordering(void) { return g_order_on ? 1 : 0; }
+}

@@ -53,6 +53,11 @@ inline C mfma_32x32x16_bf16(A a, A b, C c) {
 }
 uint32_t v_perm(uint32_t s0, uint32_t s1, uint32_t sel);  // v_perm_b32 (no meeting point)
 
+// The ordering check of the instrumented build (sim.cpp, "ordering between wavefronts"): an atomic access of kernel
+// code, and a `__shared__` array of a kernel (a static in this build) made known as shared memory of the workgroup.
+void order_atomic(const void *p, bool acquire, bool release);
+void shared_static(const void *p, size_t bytes);
+
 // assembly statements
 struct AsmOperand {
     const char *name;        // symbolic name, or "" for a positional operand
@@ -91,4 +96,5 @@ void sim_clear(void);  // violations and the launch log
 int sim_launch_count(void);
 const char *sim_launch_name(int i);
 uint64_t sim_asm_instructions(void);  // instructions the interpreter has run since sim_clear
+int sim_checks_ordering(void);  // 1 in the build with instrumented memory accesses: unordered accesses of two wavefronts are violations
 }

@@ -4,7 +4,11 @@ does not wrap at the end of its tile, a lane-exchange control in the wrong direc
 a work-space size one group short -- runs the ordinary test case of that operator, and requires that
 it fails, and by which means: the interpreter's load tracking, the exact extents of the arrays, the inaccessible page
 behind an array, or the comparison with the oracle.  (The self-check file shows the same detectors on made-up kernels;
-this one shows that the library's own code paths run through them.)"""
+this one shows that the library's own code paths run through them.)
+
+The last group takes barriers and release / acquire pairs out of the real kernels.  Such a kernel still computes the
+right sums in the model, where the wavefronts run one after the other, and nothing of the plain build notices; the
+build that checks the ordering between wavefronts (build.py, `order=True`) must."""
 import numpy as np
 import pytest
 
@@ -55,16 +59,53 @@ MUTANTS = {
 }
 
 
+# Synchronisation taken out: (edits, rebuild, case).  Right results, no violation in the plain build; reported by the
+# build that checks the ordering between wavefronts.
+ORDER_MUTANTS = {
+    # the sums of a job go through the wavefronts' window areas, rows 32..63 of x after rows 0..31: a wavefront that is
+    # ahead writes its second sums while a slower one still reads the first (with one group of rows the barrier orders
+    # nothing that the one at the end of the job before has not ordered: a wavefront writes into its own window area)
+    "sums_overwritten_while_still_read": dict(
+        edits=[("linear.hip", "            __syncthreads();  // the window areas are free: every wavefront has left its loop\n", "")],
+        rebuild=["linear.hip"], op="linear_two_jobs", plain_build_sees_it_too=True),  # (wrong sums in wavefront order as well)
+    # few rows of x: the area of the sums is handed from job to job by a flag; stored without release semantics, the next
+    # job's sums are not ordered after the additions that read the area
+    "handover_flag_without_release": dict(
+        edits=[("linear.hip", "__hip_atomic_store(&flags[1], jn + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);",
+                "__hip_atomic_store(&flags[1], jn + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);")],
+        rebuild=["linear.hip"], op="linear_small_m_two_jobs"),
+    # more than 64 rows in one pass: the groups of rows share one area for their sums
+    "one_pass_kernel_groups_share_the_area": dict(
+        edits=[("linear.hip", "        if (g) __syncthreads();\n#pragma unroll\n        for (int v = 0; v < 16; ++v) red[(size_t)wave * frag + v * kWave + lane] = acc[g][v];",
+                "#pragma unroll\n        for (int v = 0; v < 16; ++v) red[(size_t)wave * frag + v * kWave + lane] = acc[g][v];")],
+        rebuild=["linear.hip"], op="wide_two_k_tiles"),
+    # the gather on sixteen wavefronts decodes with the slot table the whole workgroup has copied into the LDS
+    "slot_table_read_before_it_is_complete": dict(
+        edits=[("embedding.hip", """        if (h1) emb_request(a, r1, pr1, lane, raw);
+    }
+    __syncthreads();
+    while (h0) {""", """        if (h1) emb_request(a, r1, pr1, lane, raw);
+    }
+    while (h0) {""")],
+        rebuild=["embedding.hip"], op="gather16"),
+}
+
+
 def _run(op: str, lib_path: str):
     m = Model(cus=2, lib_path=lib_path)
     if op == "linear":
         cases.linear(m, weight_bits(2048, 64, 1), x_bits(3, 2048, 2), 1024, 2, slot_table=True, window_rows=True)
+    elif op in ("linear_two_jobs", "linear_small_m_two_jobs"):  # four column tiles on two CUs: two jobs a workgroup
+        cases.linear(m, weight_bits(2048, 128, 1), x_bits(40 if op == "linear_two_jobs" else 3, 2048, 2), 256, 2,
+                     slot_table=True, window_rows=True, expect_kernel="fused_linear32_seg_kernel")
     elif op == "linear64":
         cases.linear(m, weight_bits(1024, 64, 1), x_bits(40, 1024, 2), 1024)
     elif op == "lm_head":
         cases.lm_head(m, weight_bits(2048, 64, 1), x_bits(1, 64, 2), 1024, check_twin=False)
     elif op == "wide":
         cases.linear(m, weight_bits(1024, 64, 1), x_bits(129, 1024, 2), 1024, wide=True, expect_kernel="fused_linear32_wide_kernel")
+    elif op == "wide_two_k_tiles":  # two wavefronts add their sums for one column tile
+        cases.linear(m, weight_bits(2048, 64, 1), x_bits(129, 2048, 2), 1024, wide=True, expect_kernel="fused_linear32_wide_kernel")
     elif op == "gather16":
         ids = np.arange(0, 2048, 3, dtype=np.int64)
         cases.gather(m, weight_bits(2048, 64, 1), ids, 1024, 8, slot_table=True, expect_kernel="embed_gather32_seg_kernel")
@@ -100,3 +141,30 @@ def test_a_mistake_in_the_kernels_is_noticed(libraries, tag, capfd):
     said = str(caught.value) + capfd.readouterr().err
     expect = mu["expect"] if isinstance(mu["expect"], tuple) else (mu["expect"],)
     assert any(e in said for e in expect), said[-1500:]
+
+
+@pytest.fixture(scope="module")
+def order_libraries():
+    from concurrent.futures import ThreadPoolExecutor
+
+    build.build()
+    build.build(order=True)
+    with ThreadPoolExecutor(2 * len(ORDER_MUTANTS)) as pool:
+        futures = {(tag, order): pool.submit(build.build_mutant, tag, mu["edits"], mu["rebuild"], order)
+                   for tag, mu in ORDER_MUTANTS.items() for order in (False, True)}
+        return {key: f.result() for key, f in futures.items()}
+
+
+def test_the_cases_pass_on_the_intact_library_that_checks_ordering():
+    for op in sorted({mu["op"] for mu in ORDER_MUTANTS.values()}):
+        in_child(_run)(op, build.build(order=True))
+
+
+@pytest.mark.parametrize("tag", sorted(ORDER_MUTANTS))
+def test_synchronisation_taken_out_is_noticed_by_the_ordering_check(order_libraries, tag):
+    mu = ORDER_MUTANTS[tag]
+    if not mu.get("plain_build_sees_it_too"):
+        in_child(_run)(mu["op"], order_libraries[tag, False])  # right results, nothing reported: the wavefronts run one after the other
+    with pytest.raises(AssertionError) as caught:
+        in_child(_run)(mu["op"], order_libraries[tag, True])
+    assert "ordering:" in str(caught.value), str(caught.value)[-1500:]

@@ -192,3 +192,52 @@ def test_a_test_body_that_never_ends_is_ended(monkeypatch):
         model.in_child(lambda: time.sleep(30))()
     with pytest.raises(AssertionError, match="did not finish within 2 s"):
         model.fork_all(lambda arg: time.sleep(30 if arg else 0), [0, 1])
+
+
+# ---- the ordering check (the build with instrumented memory accesses) ------------------------------------------------
+def _order_model():
+    from tests.hostmodel import build
+
+    m = Model(lib_path=build.build(order=True))
+    assert m.lib.sim_checks_ordering() == 1
+    return m
+
+
+@in_child
+def test_ordered_accesses_of_two_wavefronts_are_no_violation():
+    """Writes, a barrier, the neighbour's reads, a barrier, writes again; a word handed over with release and acquire;
+    every workgroup its own part of the output."""
+    m = _order_model()
+    out = _u32(m, 512)
+    m.lib.simtest_ordering(out.p, 0)
+    assert m.violations() == []
+    tid = np.arange(256)
+    want = ((tid // 64 + 1) % 4 * 64 + tid % 64) * 7 + np.where(tid < 64, 4711, 0)
+    assert np.array_equal(out.get(), np.concatenate([want, want]))
+
+
+@pytest.mark.parametrize("which, said", [
+    (1, "of the LDS"),  # no barrier between the writes and the neighbour's reads
+    (2, "of the LDS"),  # the second writes follow the neighbour's reads without a barrier
+    (3, "of the LDS"),  # a flag without release / acquire orders nothing
+    (4, "of the LDS"),  # a read of the assembly interpreter
+    (5, "a __shared__ array"),
+    (6, "overwrites byte"),  # two workgroups write the same words
+    (7, "in the same launch"),  # a workgroup reads what another one writes
+])
+@in_child
+def test_unordered_accesses_of_two_wavefronts_are_reported(which, said):
+    m = _order_model()
+    out = _u32(m, 512)
+    m.lib.simtest_ordering(out.p, which)
+    v = m.violations()
+    assert v and all("ordering:" in s for s in v) and any(said in s for s in v), v
+
+
+@in_child
+def test_the_plain_build_does_not_check_ordering():
+    m = Model()
+    assert m.lib.sim_checks_ordering() == 0
+    out = _u32(m, 512)
+    m.lib.simtest_ordering(out.p, 1)
+    assert m.violations() == []
