@@ -45,8 +45,8 @@ class DecodeItem(C.Structure):
 class Dev:
     """An array in the model's checked memory."""
 
-    def __init__(self, ptr: int, shape, dtype):
-        self.ptr, self.shape, self.dtype = ptr, tuple(shape), np.dtype(dtype)
+    def __init__(self, ptr: int, shape, dtype, lib=None):
+        self.ptr, self.shape, self.dtype, self.lib = ptr, tuple(shape), np.dtype(dtype), lib
 
     @property
     def nbytes(self) -> int:
@@ -67,6 +67,8 @@ class Dev:
         assert a.size * a.itemsize == self.nbytes, (a.shape, self.shape)
         if self.nbytes:
             C.memmove(self.ptr, a.ctypes.data, self.nbytes)
+            if self.lib is not None:  # (the build that checks it: a kernel may read what an upload wrote)
+                self.lib.sim_mark_written(C.c_void_p(self.ptr), C.c_size_t(self.nbytes))
 
 
 # a test body on the model takes seconds, a sweep block a minute or two
@@ -107,8 +109,7 @@ class Model:
     def dev(self, a: np.ndarray) -> Dev:
         a = np.ascontiguousarray(a)
         d = self.empty(a.shape, a.dtype)
-        if a.nbytes:
-            C.memmove(d.ptr, a.ctypes.data, a.nbytes)
+        d.put(a)
         return d
 
     def empty(self, shape, dtype) -> Dev:
@@ -116,7 +117,7 @@ class Model:
         n = int(np.prod(shape, dtype=np.int64)) * np.dtype(dtype).itemsize
         ptr = self.lib.sim_alloc(n, self.end_at_guard)
         assert ptr, "sim_alloc failed"
-        return Dev(ptr, shape, dtype)
+        return Dev(ptr, shape, dtype, self.lib)
 
     def free_all(self) -> None:
         self.lib.sim_free_all()

@@ -161,6 +161,10 @@ static std::string where() {
 //   * arrays from sim_alloc: the same inside a workgroup; between workgroups of one launch nothing orders anything, so
 //     a byte written by one workgroup and read or written by another is reported.  Launches are ordered by the stream.
 // Atomic accesses themselves are not recorded (they do not race with each other).
+//   * arrays from sim_alloc, second check: a byte that nothing has written -- no upload (sim_mark_written), no host code
+//     of the library (hipMemsetAsync, hipMemcpyAsync), no kernel -- and that a kernel reads.  On the GPU such a byte
+//     holds what an earlier launch left there.  The fill pattern of sim_alloc is a tiny number both as fp32 and as
+//     bf16, so a sum that includes such bytes passes every tolerance; here the read itself is the violation.
 constexpr int kMaxWaves = kMaxThreads / 64;
 static bool g_order_on = false;
 static uint32_t g_vc[kMaxWaves][kMaxWaves];
@@ -181,7 +185,9 @@ static uint64_t g_launch_seq = 0, g_workgroup_seq = 0;
 struct GlobalShadow {
     uint64_t launch = 0;  // the launch its contents belong to
     std::vector<uint32_t> w_id, w_clk, r_id, r_clk;  // per byte: (workgroup + 1) << 4 | wavefront, and that wavefront's clock
+    std::vector<uint8_t> written;  // per byte, for the life of the array: something has written it
 };
+static bool g_check_unwritten = true;
 static std::unordered_map<uint64_t, GlobalShadow> g_global_shadow;  // by Alloc::ptr
 
 static void order_report(const char *fmt, ...) {
@@ -294,6 +300,7 @@ static void order_global(const Alloc &a, uint64_t addr, size_t n, bool write) {
         s.r_id.assign(a.bytes, 0);
         s.r_clk.assign(a.bytes, 0);
     }
+    if (s.written.size() != a.bytes) s.written.assign(a.bytes, 0);
     const uint32_t w = cur_wave(), me = (g_wg_index + 1) << 4 | w;
     // did the access `id` at clock `clk` happen before what this wavefront does now?
     auto before = [&](uint32_t id, uint32_t clk) { return id == 0 || id == me || (id >> 4 == me >> 4 && clk <= g_vc[w][id & 15]); };
@@ -306,7 +313,14 @@ static void order_global(const Alloc &a, uint64_t addr, size_t n, bool write) {
                          (size_t)(&a - g_allocs.data()), a.bytes, (s.w_id[b] >> 4) - 1, s.w_id[b] & 15);
             return;
         }
+        if (!write && !s.written[b] && g_check_unwritten) {
+            order_report("workgroup %u wavefront %u reads byte %zu of allocation #%zu (%zu bytes; an access of %zu bytes at offset %zu), "
+                         "which nothing has written: no upload, no host code of the library, no kernel", g_wg_index, w, b,
+                         (size_t)(&a - g_allocs.data()), a.bytes, n, o);
+            return;
+        }
         if (write) {
+            s.written[b] = 1;
             if (!before(s.r_id[b], s.r_clk[b])) {
                 order_report("workgroup %u wavefront %u writes byte %zu of allocation #%zu (%zu bytes) that workgroup %u wavefront %u read in "
                              "the same launch, and nothing orders the two", g_wg_index, w, b, (size_t)(&a - g_allocs.data()), a.bytes,
@@ -323,8 +337,20 @@ static void order_global(const Alloc &a, uint64_t addr, size_t n, bool write) {
 }
 
 // Every access of kernel code: plain C++ through the compiler's hooks, the interpreter's by its own calls.
+static void mark_written(uint64_t addr, size_t n) {
+    for (const Alloc &a : g_allocs)
+        if (addr - (uint64_t)a.ptr < a.bytes) {
+            GlobalShadow &s = g_global_shadow[(uint64_t)a.ptr];
+            if (s.written.size() != a.bytes) s.written.assign(a.bytes, 0);
+            const size_t o = (size_t)(addr - (uint64_t)a.ptr);
+            memset(s.written.data() + o, 1, n < a.bytes - o ? n : a.bytes - o);
+            return;
+        }
+}
+
 static inline void order_access(uint64_t addr, size_t n, bool write) {
-    if (!g_order_on || !g_cur || n == 0) return;
+    if (!g_order_on || n == 0) return;
+    if (!g_cur) return;  // host code
     if (addr - (uint64_t)g_stacks < (uint64_t)kMaxThreads * kStackBytes) return;  // a fibre's own stack
     if (order_shared_access(addr, n, write)) return;
     static size_t last = 0;
@@ -1506,6 +1532,7 @@ extern "C" void *sim_alloc(size_t bytes, int end_at_guard) {
 extern "C" void sim_free_all(void) {
     for (Alloc &a : g_allocs) munmap(a.map, a.map_bytes);
     g_allocs.clear();
+    g_global_shadow.clear();
 }
 
 extern "C" void sim_set_cus(int n) { g_cus = n > 0 ? n : 1; }
@@ -1552,17 +1579,21 @@ CI_SIM_HOOK(16)
 #undef CI_SIM_HOOK
 void __tsan_read_range(void *p, unsigned long n) { order_access((uint64_t)p, n, false); }
 void __tsan_write_range(void *p, unsigned long n) { order_access((uint64_t)p, n, true); }
+// (called by host code these are the stand-ins of hipMemsetAsync / hipMemcpyAsync: what they write is written)
 void *__tsan_memcpy(void *d, const void *s, unsigned long n) {
+    if (!g_cur && g_order_on && n) mark_written((uint64_t)d, n);
     order_access((uint64_t)s, n, false);
     order_access((uint64_t)d, n, true);
     return memcpy(d, s, n);
 }
 void *__tsan_memmove(void *d, const void *s, unsigned long n) {
+    if (!g_cur && g_order_on && n) mark_written((uint64_t)d, n);
     order_access((uint64_t)s, n, false);
     order_access((uint64_t)d, n, true);
     return memmove(d, s, n);
 }
 void *__tsan_memset(void *d, int v, unsigned long n) {
+    if (!g_cur && g_order_on && n) mark_written((uint64_t)d, n);
     order_access((uint64_t)d, n, true);
     return memset(d, v, n);
 }
@@ -1590,4 +1621,8 @@ CI_SIM_ATOMIC(64, uint64_t)
 void __tsan_atomic_thread_fence(int) {}
 void __tsan_atomic_signal_fence(int) {}
 int sim_checks_ordering(void) { return g_order_on ? 1 : 0; }
+void sim_mark_written(const void *p, size_t n) {
+    if (g_order_on && n) mark_written((uint64_t)p, n);
+}
+void sim_check_unwritten_reads(int on) { g_check_unwritten = on != 0; }
 }

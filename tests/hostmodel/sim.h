@@ -97,4 +97,8 @@ int sim_launch_count(void);
 const char *sim_launch_name(int i);
 uint64_t sim_asm_instructions(void);  // instructions the interpreter has run since sim_clear
 int sim_checks_ordering(void);  // 1 in the build with instrumented memory accesses: unordered accesses of two wavefronts are violations
+// In that build a kernel's read of a byte of a sim_alloc array that nothing has written is a violation too: an upload
+// says what it wrote with sim_mark_written; sim_check_unwritten_reads(0) switches the check off.
+void sim_mark_written(const void *p, size_t n);
+void sim_check_unwritten_reads(int on);
 }

@@ -134,6 +134,7 @@ def test_decode_batch_with_an_empty_tensor_and_a_stream_at_an_odd_address():
         if i == 2:
             room = m.empty(enc.stream.size + 16, np.uint8)
             C.memmove(room.ptr + 8, enc.stream.ctypes.data, enc.stream.size)
+            m.lib.sim_mark_written(C.c_void_p(room.ptr + 8), C.c_size_t(enc.stream.size))  # (the bytes around it stay unwritten)
             w.d_stream = room.ptr + 8
             keep.append(room)
         out = m.empty((K, N), np.uint8)
@@ -353,6 +354,7 @@ def test_a_stream_that_is_not_16_byte_aligned():
     for shift in (8, 4, 1):
         room = m.empty(enc.stream.size + 16, np.uint8)
         C.memmove(room.ptr + shift, enc.stream.ctypes.data, enc.stream.size)
+        m.lib.sim_mark_written(C.c_void_p(room.ptr + shift), C.c_size_t(enc.stream.size))  # (the bytes around it stay unwritten)
         w.d_stream = room.ptr + shift
         out = m.empty((K, N), np.uint8)
         xb = x_bits(3, K, 2)

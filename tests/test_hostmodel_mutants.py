@@ -88,6 +88,13 @@ ORDER_MUTANTS = {
     }
     while (h0) {""")],
         rebuild=["embedding.hip"], op="gather16"),
+    # the LM head on sixteen wavefronts gives an item it must refuse (a descriptor that understates the largest window)
+    # zeros; without them the reduction adds up whatever an earlier launch left in those rows of the workspace -- in
+    # the model the fill pattern of a fresh array, a tiny number as fp32: every tolerance passes
+    "refused_item_leaves_its_rows_of_the_workspace_unwritten": dict(
+        edits=[("transposed.hip", "            for (uint32_t i = c; i < min(seglen, a.V - v0); i += 32) a.partial[(size_t)tn * a.V + v0 + i] = 0.f;\n",
+                "            ;\n")],
+        rebuild=["transposed.hip"], op="lm_head_understated_window", says="nothing has written"),
 }
 
 
@@ -106,6 +113,20 @@ def _run(op: str, lib_path: str):
         cases.linear(m, weight_bits(1024, 64, 1), x_bits(129, 1024, 2), 1024, wide=True, expect_kernel="fused_linear32_wide_kernel")
     elif op == "wide_two_k_tiles":  # two wavefronts add their sums for one column tile
         cases.linear(m, weight_bits(2048, 64, 1), x_bits(129, 2048, 2), 1024, wide=True, expect_kernel="fused_linear32_wide_kernel")
+    elif op == "lm_head_understated_window":
+        import ctypes as C
+
+        rng = np.random.default_rng(3)
+        V, H, th, segs = 2048, 64, 1024, 2
+        enc, man = cases.compress(cases.weight_kind(rng, V, H, "wide"), th)  # deep bodies: windows of more than 112 rows
+        w, keep = m.weight(enc, man, V, H, segments=segs, slot_table=True, window_rows=True)
+        assert w.max_window_rows > 112
+        w.max_window_rows = 7  # the lie: every item is refused
+        x, z = m.dev(x_bits(1, H, 2)), m.empty((1, V), np.uint16)
+        nb = m.lib.ci_fused_linear_transposed_workspace_bytes(1, H, V, 32)
+        ws = m.empty(nb // 4, np.float32)  # (a fresh array: nothing written)
+        m.call("ci_fused_linear_transposed_tiled", C.byref(w), x.p, 1, H, None, z.p, V, ws.p, C.c_size_t(nb), None)
+        assert "trans32_seg_kernel<false>" in m.launches()
     elif op == "gather16":
         ids = np.arange(0, 2048, 3, dtype=np.int64)
         cases.gather(m, weight_bits(2048, 64, 1), ids, 1024, 8, slot_table=True, expect_kernel="embed_gather32_seg_kernel")
@@ -167,4 +188,4 @@ def test_synchronisation_taken_out_is_noticed_by_the_ordering_check(order_librar
         in_child(_run)(mu["op"], order_libraries[tag, False])  # right results, nothing reported: the wavefronts run one after the other
     with pytest.raises(AssertionError) as caught:
         in_child(_run)(mu["op"], order_libraries[tag, True])
-    assert "ordering:" in str(caught.value), str(caught.value)[-1500:]
+    assert "ordering:" in str(caught.value) and mu.get("says", "") in str(caught.value), str(caught.value)[-1500:]

@@ -241,3 +241,27 @@ def test_the_plain_build_does_not_check_ordering():
     out = _u32(m, 512)
     m.lib.simtest_ordering(out.p, 1)
     assert m.violations() == []
+
+
+@in_child
+def test_a_read_of_bytes_that_nothing_has_written_is_reported():
+    """The same build: a kernel that reads an array nobody has filled -- through an assembly statement and through
+    plain C++ -- and the same reads after an upload."""
+    m = _order_model()
+    src, dst = m.empty(100, np.uint32), _u32(m, 64)
+    m.lib.simtest_global_load(src.p, 50, dst.p, 0)
+    v = m.violations()
+    assert v and "nothing has written" in v[0], v
+    m.clear()
+    m.lib.simtest_plain_overrun(src.p, 10, dst.p)  # (words 26 .. 89 of the 100)
+    v = m.violations()
+    assert v and "nothing has written" in v[0], v
+    m.clear()
+    src.put(np.arange(100, dtype=np.uint32))
+    m.lib.simtest_global_load(src.p, 50, dst.p, 0)
+    m.lib.simtest_plain_overrun(src.p, 10, dst.p)
+    assert m.violations() == [] and np.array_equal(dst.get(), 26 + np.arange(64))
+    # what a kernel wrote is written: dst, read by the next launch
+    out = _u32(m, 64)
+    m.lib.simtest_global_load(dst.p, 64, out.p, 0)
+    assert m.violations() == [] and np.array_equal(out.get(), 2 * (26 + np.arange(64)))
