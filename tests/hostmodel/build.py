@@ -16,7 +16,9 @@ A second library, libci_hostmodel_order.so (`build(order=True)`, `--order`), is 
 compiled under the compiler's thread-sanitizer instrumentation and no sanitizer runtime: the model itself (sim.cpp,
 "ordering between wavefronts") takes the calls the instrumentation makes at every plain memory access, and reports
 two wavefronts that touch the same byte with no barrier or release/acquire pair between them -- what fibres that run
-one after the other would never show.
+one after the other would never show.  A third, libci_hostmodel_undefined.so (`build(undefined=True)`, `--undefined`),
+compiles them with the compiler's undefined-behaviour checks (array bounds, shift amounts, alignment, null, signed
+overflow, pointer arithmetic), again without a runtime: the checks' calls become violations of the model.
 
 Test infrastructure: nothing of the product is built from, or loads, what this makes.
 """
@@ -34,6 +36,8 @@ OUT_DIR = os.path.join(HERE, "_build")
 LIB_PATH = os.path.join(HERE, "libci_hostmodel.so")
 ORDER_LIB_PATH = os.path.join(HERE, "libci_hostmodel_order.so")
 ORDER_FLAGS = ["-fsanitize=thread", "-mllvm", "-tsan-instrument-func-entry-exit=0"]
+UNDEFINED_LIB_PATH = os.path.join(HERE, "libci_hostmodel_undefined.so")
+UNDEFINED_FLAGS = ["-fsanitize=bounds,shift,alignment,integer-divide-by-zero,null,unreachable,signed-integer-overflow,pointer-overflow"]
 CXX = os.environ.get("CI_HOSTMODEL_CXX", "/opt/rocm/llvm/bin/clang++")
 SOURCES = ["api.hip", "encode.hip", "decode.hip", "linear.hip", "embedding.hip", "transposed.hip", "legacy.hip"]
 CXXFLAGS = ["-std=c++17", "-O1", "-g", "-fPIC", "-fno-strict-aliasing", "-Wno-unused-value", "-Wno-unknown-attributes",
@@ -180,13 +184,13 @@ def needs_build(lib_path: str = LIB_PATH) -> bool:
     return any(os.path.getmtime(d) > built for d in deps)
 
 
-def build(force: bool = False, verbose: bool = False, order: bool = False) -> str:
-    lib_path = ORDER_LIB_PATH if order else LIB_PATH
+def build(force: bool = False, verbose: bool = False, order: bool = False, undefined: bool = False) -> str:
+    lib_path = ORDER_LIB_PATH if order else UNDEFINED_LIB_PATH if undefined else LIB_PATH
     if not force and not needs_build(lib_path):
         return lib_path
-    out_dir = os.path.join(OUT_DIR, "order") if order else OUT_DIR
+    out_dir = os.path.join(OUT_DIR, "order") if order else os.path.join(OUT_DIR, "undefined") if undefined else OUT_DIR
     os.makedirs(out_dir, exist_ok=True)
-    flags = CXXFLAGS + (ORDER_FLAGS if order else [])
+    flags = CXXFLAGS + (ORDER_FLAGS if order else UNDEFINED_FLAGS if undefined else [])
     procs, objs = [], []
     for src in SOURCES + ["selftest.hip"]:
         path = os.path.join(HERE if src == "selftest.hip" else CSRC, src)
@@ -263,4 +267,4 @@ def build_mutant(tag: str, edits: list, rebuild: list, order: bool = False) -> s
 
 
 if __name__ == "__main__":
-    print(build(force="--force" in sys.argv, verbose=True, order="--order" in sys.argv))
+    print(build(force="--force" in sys.argv, verbose=True, order="--order" in sys.argv, undefined="--undefined" in sys.argv))

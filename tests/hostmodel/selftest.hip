@@ -229,9 +229,30 @@ __global__ void st_ordering_kernel(uint32_t *out, int which) {
     out[(which == 6 || which == 7 ? 0u : blockIdx.x) * blockDim.x + tid] = v;
 }
 
+// For the build with the compiler's undefined-behaviour checks.  which: 0 nothing; 1 a shift by the width of the
+// type; 2 an index one past a fixed-size array; 3 a 16-byte access at an address that is a multiple of 4 only;
+// 4 a signed sum past the largest int
+typedef uint32_t st_u32x4 __attribute__((ext_vector_type(4)));
+__global__ void st_undefined_kernel(uint32_t *out, int which, uint32_t n) {  // n = 32
+    extern __shared__ __align__(16) uint8_t lds[];
+    const uint32_t tid = threadIdx.x;
+    uint32_t regs[4] = {tid, tid + 1, tid + 2, tid + 3};
+    uint32_t v = regs[(tid + n) % 4];
+    if (which == 1) v += 1u << n;
+    static const uint32_t table[4] = {3, 1, 4, 1};  // (in memory: the access past it goes on after the report)
+    if (which == 2) v += table[n / 8];
+    for (uint32_t i = 0; i < 8; ++i) reinterpret_cast<uint32_t *>(lds)[tid * 8 + i] = i;
+    if (which == 3) v += (*reinterpret_cast<const st_u32x4 *>(lds + tid * 32 + n / 8))[1];
+    if (which == 4) v += (uint32_t)((int)(0x7fffffe0u + tid) + (int)n);
+    out[tid] = v;
+}
+
 }  // namespace
 
 extern "C" {
+void simtest_undefined(uint32_t *out, int which, uint32_t n) {
+    hipLaunchKernelGGL(st_undefined_kernel, dim3(1), dim3(64), 4096, nullptr, out, which, n);
+}
 void simtest_ordering(uint32_t *out, int which) {
     hipLaunchKernelGGL(st_ordering_kernel, dim3(2), dim3(256), 8192, nullptr, out, which);
 }

@@ -2,12 +2,14 @@
 // library's assembly statements.  See sim.h.  Test infrastructure only.
 #include "sim.h"
 
+#include <dlfcn.h>
 #include <signal.h>
 #include <stdarg.h>
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
 #include <sys/mman.h>
+#include <ucontext.h>
 #include <unistd.h>
 
 #include <map>
@@ -1482,9 +1484,19 @@ int take_launch_error() {
 }
 int cu_count() { return g_cus; }
 
-static void on_segv(int, siginfo_t *info, void *) {
+static void on_segv(int sig, siginfo_t *info, void *uc) {
     // (async-signal-unsafe calls: the process is about to end anyway)
     const uint64_t addr = (uint64_t)info->si_addr;
+    if (sig == SIGILL) {
+        // a build of the kernel sources with the compiler's undefined-behaviour checks in trap mode ends here
+        Dl_info dl;
+        const void *pc = (const void *)((ucontext_t *)uc)->uc_mcontext.gregs[REG_RIP];
+        const bool known = dladdr(pc, &dl) != 0;
+        fprintf(stderr, "host model: illegal instruction %s at %s+0x%llx (%s)\n", where().c_str(), known ? dl.dli_fname : "?",
+                (unsigned long long)((uint64_t)pc - (known ? (uint64_t)dl.dli_fbase : 0)), known && dl.dli_sname ? dl.dli_sname : "?");
+        fflush(stderr);
+        _exit(71);
+    }
     fprintf(stderr, "host model: memory fault at %p %s: %s\n", info->si_addr, where().c_str(),
             addr >= (uint64_t)g_lds && addr < (uint64_t)g_lds + kLdsBytes + 4096 ? "in the LDS area, past the end of this launch's dynamic LDS" : describe_address(addr).c_str());
     fflush(stderr);
@@ -1515,6 +1527,7 @@ extern "C" void sim_init(void) {
     sa.sa_flags = SA_SIGINFO | SA_ONSTACK;
     sigaction(SIGSEGV, &sa, nullptr);
     sigaction(SIGBUS, &sa, nullptr);
+    sigaction(SIGILL, &sa, nullptr);
 }
 
 extern "C" void *sim_alloc(size_t bytes, int end_at_guard) {
@@ -1625,4 +1638,52 @@ void sim_mark_written(const void *p, size_t n) {
     if (g_order_on && n) mark_written((uint64_t)p, n);
 }
 void sim_check_unwritten_reads(int on) { g_check_unwritten = on != 0; }
+}
+
+// ---- the compiler's undefined-behaviour checks (build.py, `undefined=True`) ----------------------------------------------
+// That build compiles the kernel sources with -fsanitize=bounds,shift,alignment,... and no sanitizer runtime: the
+// calls the checks make come here and become violations with the source position the compiler recorded.  One kind
+// is let through: an offset added to a null pointer (`a.ckpt + ...` where a weight has no checkpoints and the pointer
+// is never read).  It is undefined in C++ and harmless in these kernels: no null test follows that the compiler could
+// drop on the strength of it.
+extern "C" {
+struct CiSimUbLocation {
+    const char *file;
+    uint32_t line, column;
+};
+static void ub_report(const char *kind, const void *data, uint64_t a, uint64_t b) {
+    const CiSimUbLocation *l = (const CiSimUbLocation *)data;
+    violation("undefined behaviour: %s at %s:%u:%u (values 0x%llx, 0x%llx)", kind, l && l->file ? l->file : "?", l ? l->line : 0,
+              l ? l->column : 0, (unsigned long long)a, (unsigned long long)b);
+}
+#define CI_SIM_UB(name)                                                                                 \
+    void __ubsan_handle_##name(void *d, uint64_t a, uint64_t b) { ub_report(#name, d, a, b); }         \
+    void __ubsan_handle_##name##_abort(void *d, uint64_t a, uint64_t b) { ub_report(#name, d, a, b); }
+CI_SIM_UB(type_mismatch_v1)  // (null pointers and misaligned accesses)
+CI_SIM_UB(shift_out_of_bounds)
+CI_SIM_UB(add_overflow)
+CI_SIM_UB(sub_overflow)
+CI_SIM_UB(mul_overflow)
+CI_SIM_UB(negate_overflow)
+CI_SIM_UB(divrem_overflow)
+CI_SIM_UB(builtin_unreachable)
+CI_SIM_UB(missing_return)
+CI_SIM_UB(vla_bound_not_positive)
+CI_SIM_UB(load_invalid_value)
+CI_SIM_UB(invalid_builtin)
+#undef CI_SIM_UB
+// An index past an array of known size: the compiler treats what follows as unreachable, so the process cannot go on.
+void __ubsan_handle_out_of_bounds(void *d, uint64_t index) {
+    const CiSimUbLocation *l = (const CiSimUbLocation *)d;
+    fprintf(stderr, "host model: %sundefined behaviour: out_of_bounds at %s:%u:%u (index %llu)\n", where().c_str(), l->file ? l->file : "?",
+            l->line, l->column, (unsigned long long)index);
+    fflush(stderr);
+    _exit(72);
+}
+void __ubsan_handle_out_of_bounds_abort(void *d, uint64_t index) { __ubsan_handle_out_of_bounds(d, index); }
+void __ubsan_handle_pointer_overflow(void *d, uint64_t base, uint64_t result) {
+    // (base below 4 GB: null, or null plus an earlier offset of the same expression; no array of the model lives there)
+    if (base >> 32) ub_report("pointer_overflow", d, base, result);
+}
+void __ubsan_handle_pointer_overflow_abort(void *d, uint64_t base, uint64_t result) { __ubsan_handle_pointer_overflow(d, base, result); }
 }

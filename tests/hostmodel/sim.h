@@ -10,6 +10,10 @@
 //     LDS address as on the GPU; accesses of the interpreter are checked against the launch's LDS size;
 //   * global memory comes from sim_alloc: each allocation ends (or starts) at an inaccessible page, and the
 //     interpreter checks every address it forms against the exact extent of the allocations.
+//   * two more builds of the same sources take the calls of compiler instrumentation instead of a sanitizer runtime
+//     (build.py): with every plain memory access reported, the model checks that two wavefronts never touch the same
+//     byte without a barrier or a release / acquire pair between them, and that no kernel reads a byte of an array that
+//     nothing has written; with the undefined-behaviour checks compiled in, what they report is a violation.
 //
 // Test infrastructure only.
 #pragma once

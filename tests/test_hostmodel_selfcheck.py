@@ -265,3 +265,29 @@ def test_a_read_of_bytes_that_nothing_has_written_is_reported():
     out = _u32(m, 64)
     m.lib.simtest_global_load(dst.p, 64, out.p, 0)
     assert m.violations() == [] and np.array_equal(out.get(), 2 * (26 + np.arange(64)))
+
+
+# ---- the build with the compiler's undefined-behaviour checks ---------------------------------------------------------
+def _undefined(which):
+    from tests.hostmodel import build
+
+    m = Model(lib_path=build.build(undefined=True))
+    out = _u32(m, 64)
+    m.lib.simtest_undefined(out.p, 0, 32)
+    assert m.violations() == [] and np.array_equal(out.get(), np.arange(64) + np.arange(64) % 4)
+    m.lib.simtest_undefined(out.p, which, 32)
+    return m.violations()
+
+
+@pytest.mark.parametrize("which, said", [(1, "shift_out_of_bounds"), (3, "type_mismatch"), (4, "add_overflow")])
+@in_child
+def test_undefined_behaviour_in_kernel_code_is_reported(which, said):
+    v = _undefined(which)
+    assert v and all("undefined behaviour" in s and "selftest.hip" in s for s in v) and said in v[0], v
+
+
+def test_an_index_past_an_array_ends_the_run_and_says_where(capfd):
+    """(What follows such an index is unreachable for the compiler: the model cannot go on and says so on stderr.)"""
+    with pytest.raises(AssertionError, match="exited with 72"):
+        in_child(_undefined)(2)
+    assert "out_of_bounds at" in capfd.readouterr().err
