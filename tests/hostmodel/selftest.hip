@@ -229,6 +229,25 @@ __global__ void st_ordering_kernel(uint32_t *out, int which) {
     out[(which == 6 || which == 7 ? 0u : blockIdx.x) * blockDim.x + tid] = v;
 }
 
+// A running sum handed from lane to lane through the LDS: right when the lanes run one after the other, as they do in
+// the model, and wrong on the GPU, where they run in step.  which: 0 every lane writes its own word, a wavefront-wide
+// operation, then reads its neighbour's (well defined); 1 lane l adds what lane l - 1 has just stored, with nothing
+// wavefront-wide between the store and the load
+__global__ void st_lane_order_kernel(uint32_t *out, int which) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    uint32_t *word = reinterpret_cast<uint32_t *>(lds);
+    const uint32_t lane = threadIdx.x;
+    if (which == 0) {
+        word[lane] = lane + 1;
+        __builtin_amdgcn_wave_barrier();
+        out[lane] = word[lane] + (lane ? word[lane - 1] : 0u);
+    } else {
+        const uint32_t before = lane ? word[lane - 1] : 0u;
+        word[lane] = before + lane + 1;
+        out[lane] = word[lane];
+    }
+}
+
 // For the build with the compiler's undefined-behaviour checks.  which: 0 nothing; 1 a shift by the width of the
 // type; 2 an index one past a fixed-size array; 3 a 16-byte access at an address that is a multiple of 4 only;
 // 4 a signed sum past the largest int
@@ -250,6 +269,7 @@ __global__ void st_undefined_kernel(uint32_t *out, int which, uint32_t n) {  // 
 }  // namespace
 
 extern "C" {
+void simtest_lane_order(uint32_t *out, int which) { hipLaunchKernelGGL(st_lane_order_kernel, dim3(1), dim3(64), 256, nullptr, out, which); }
 void simtest_undefined(uint32_t *out, int which, uint32_t n) {
     hipLaunchKernelGGL(st_undefined_kernel, dim3(1), dim3(64), 4096, nullptr, out, which, n);
 }

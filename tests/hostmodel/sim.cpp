@@ -163,6 +163,13 @@ static std::string where() {
 //   * arrays from sim_alloc: the same inside a workgroup; between workgroups of one launch nothing orders anything, so
 //     a byte written by one workgroup and read or written by another is reported.  Launches are ordered by the stream.
 // Atomic accesses themselves are not recorded (they do not race with each other).
+//   * inside one wavefront: on the GPU the lanes run in step, so an LDS write that comes earlier in the program than a
+//     read has happened for every lane before any lane reads.  Here the lanes are fibres that run one after the other
+//     between two wavefront-wide operations, so a lane can see a later lane's byte too early or an earlier lane's too
+//     late -- and a result that only comes out right in lane order (a sum handed from lane to lane through the LDS,
+//     say) would pass here and fail on the GPU.  So: two different lanes of a wavefront that touch the same byte, at
+//     least one writing, with no wavefront-wide operation between the two accesses, are reported.  (The interpreter's
+//     accesses are those of the whole wavefront in step and are exempt.)
 //   * arrays from sim_alloc, second check: a byte that nothing has written -- no upload (sim_mark_written), no host code
 //     of the library (hipMemsetAsync, hipMemcpyAsync), no kernel -- and that a kernel reads.  On the GPU such a byte
 //     holds what an earlier launch left there.  The fill pattern of sim_alloc is a tiny number both as fp32 and as
@@ -173,6 +180,12 @@ static uint32_t g_vc[kMaxWaves][kMaxWaves];
 static uint8_t *g_sh_wwave = nullptr;   // per LDS byte: the wavefront that wrote it last (0xFF: none in this workgroup)
 static uint32_t *g_sh_wclk = nullptr;   //   ... at this value of its own clock
 static uint32_t *g_sh_rclk = nullptr;   // per LDS byte and wavefront: its clock when it last read the byte (0: never)
+struct LaneMark {  // per LDS byte: the last plain write and the last plain read, for the check inside a wavefront
+    uint8_t wlane, rwave, rlane;
+    uint32_t wepoch, repoch;
+};
+static LaneMark *g_sh_lane = nullptr;
+static uint32_t g_wave_epoch[kMaxThreads / 64];  // counts the wavefront-wide operations (and barriers) of each wavefront
 static std::unordered_map<uint64_t, std::vector<uint32_t>> g_sync;  // address of an atomic -> clock left by releases
 struct SharedStatic {  // a `__shared__` array of a kernel, with a shadow of its own (emptied when a new workgroup first touches it)
     uint64_t ptr;
@@ -180,6 +193,7 @@ struct SharedStatic {  // a `__shared__` array of a kernel, with a shadow of its
     uint64_t workgroup;
     std::vector<uint8_t> wwave;
     std::vector<uint32_t> wclk, rclk;
+    std::vector<LaneMark> lane;
 };
 static std::vector<SharedStatic> g_shared_statics;
 static uint32_t g_wg_index = 0, g_order_reports = 0;
@@ -210,11 +224,14 @@ static void order_start_workgroup(uint32_t n_waves, size_t lds_open) {
         g_sh_wwave = (uint8_t *)malloc(n);
         g_sh_wclk = (uint32_t *)malloc(n * 4);
         g_sh_rclk = (uint32_t *)malloc(n * 4 * kMaxWaves);
-        if (!g_sh_wwave || !g_sh_wclk || !g_sh_rclk) abort();
+        g_sh_lane = (LaneMark *)malloc(n * sizeof(LaneMark));
+        if (!g_sh_wwave || !g_sh_wclk || !g_sh_rclk || !g_sh_lane) abort();
         lds_open = kLdsBytes;
     }
     memset(g_sh_wwave, 0xFF, lds_open);
     memset(g_sh_rclk, 0, lds_open * 4 * kMaxWaves);
+    memset(g_sh_lane, 0xFF, lds_open * sizeof(LaneMark));
+    memset(g_wave_epoch, 0, sizeof g_wave_epoch);
     memset(g_vc, 0, sizeof g_vc);
     for (uint32_t w = 0; w < n_waves; ++w) g_vc[w][w] = 1;
     g_sync.clear();
@@ -240,12 +257,37 @@ static inline uint32_t cur_wave() { return g_cur->ctx.thread_idx.x / 64; }
 struct SharedShadow {
     uint8_t *wwave;
     uint32_t *wclk, *rclk;
+    LaneMark *lane;
 };
+constexpr uint32_t kWholeWave = 0xFE;  // an access of the interpreter: every lane in step
 
-static void order_shared(const SharedShadow &sh, size_t off, size_t n, bool write, const char *what) {
-    const uint32_t w = cur_wave();
+static void order_shared(const SharedShadow &sh, size_t off, size_t n, bool write, const char *what, uint32_t lane) {
+    const uint32_t w = cur_wave(), epoch = g_wave_epoch[w];
     for (size_t b = off; b < off + n; ++b) {
         const uint8_t ww = sh.wwave[b];
+        LaneMark &lm = sh.lane[b];
+        if (lane != kWholeWave) {
+            if (ww == w && lm.wlane < 64 && lm.wlane != lane && lm.wepoch == epoch) {
+                order_report("lane %u of wavefront %u %s byte 0x%zx of %s (an access of %zu bytes) that lane %u of the same wavefront wrote, and "
+                             "no wavefront-wide operation lies between the two: what this lane sees depends on the order in which the "
+                             "model runs the lanes", lane, w, write ? "overwrites" : "reads", b, what, n, (unsigned)lm.wlane);
+                return;
+            }
+            if (write && lm.rwave == w && lm.rlane < 64 && lm.rlane != lane && lm.repoch == epoch) {
+                order_report("lane %u of wavefront %u writes byte 0x%zx of %s (an access of %zu bytes) that lane %u of the same wavefront read, "
+                             "and no wavefront-wide operation lies between the two: what that lane saw depends on the order in which the "
+                             "model runs the lanes", lane, w, b, what, n, (unsigned)lm.rlane);
+                return;
+            }
+        }
+        if (write) {
+            lm.wlane = (uint8_t)lane;
+            lm.wepoch = epoch;
+        } else {
+            lm.rwave = (uint8_t)w;
+            lm.rlane = (uint8_t)lane;
+            lm.repoch = epoch;
+        }
         if (ww != 0xFF && ww != w && sh.wclk[b] > g_vc[w][ww]) {
             order_report("wavefront %u %s byte 0x%zx of %s (an access of %zu bytes) that wavefront %u wrote, and no barrier or "
                          "release/acquire pair lies between the two", w, write ? "overwrites" : "reads", b, what, n, ww);
@@ -267,9 +309,9 @@ static void order_shared(const SharedShadow &sh, size_t off, size_t n, bool writ
 }
 
 // An access to the LDS or to a `__shared__` array: checked, and true.
-static bool order_shared_access(uint64_t addr, size_t n, bool write) {
+static bool order_shared_access(uint64_t addr, size_t n, bool write, uint32_t lane) {
     if (addr - (uint64_t)g_lds < kLdsBytes) {
-        order_shared(SharedShadow{g_sh_wwave, g_sh_wclk, g_sh_rclk}, (size_t)(addr - (uint64_t)g_lds), n, write, "the LDS");
+        order_shared(SharedShadow{g_sh_wwave, g_sh_wclk, g_sh_rclk, g_sh_lane}, (size_t)(addr - (uint64_t)g_lds), n, write, "the LDS", lane);
         return true;
     }
     for (SharedStatic &s : g_shared_statics)
@@ -279,8 +321,10 @@ static bool order_shared_access(uint64_t addr, size_t n, bool write) {
                 s.wwave.assign(s.bytes + 16, 0xFF);
                 s.wclk.assign(s.bytes + 16, 0);
                 s.rclk.assign((s.bytes + 16) * kMaxWaves, 0);
+                s.lane.assign(s.bytes + 16, LaneMark{0xFF, 0xFF, 0xFF, 0, 0});
             }
-            order_shared(SharedShadow{s.wwave.data(), s.wclk.data(), s.rclk.data()}, (size_t)(addr - s.ptr), n, write, "a __shared__ array");
+            order_shared(SharedShadow{s.wwave.data(), s.wclk.data(), s.rclk.data(), s.lane.data()}, (size_t)(addr - s.ptr), n, write,
+                         "a __shared__ array", lane);
             return true;
         }
     return false;
@@ -350,11 +394,11 @@ static void mark_written(uint64_t addr, size_t n) {
         }
 }
 
-static inline void order_access(uint64_t addr, size_t n, bool write) {
+static inline void order_access(uint64_t addr, size_t n, bool write, bool whole_wave = false) {
     if (!g_order_on || n == 0) return;
     if (!g_cur) return;  // host code
     if (addr - (uint64_t)g_stacks < (uint64_t)kMaxThreads * kStackBytes) return;  // a fibre's own stack
-    if (order_shared_access(addr, n, write)) return;
+    if (order_shared_access(addr, n, write, whole_wave ? kWholeWave : g_cur->ctx.thread_idx.x % 64)) return;
     static size_t last = 0;
     if (last < g_allocs.size() && addr - (uint64_t)g_allocs[last].ptr < g_allocs[last].bytes) {
         order_global(g_allocs[last], addr, n, write);
@@ -388,7 +432,7 @@ void shared_static(const void *p, size_t bytes) {
     if (!g_order_on) return;
     for (const SharedStatic &s : g_shared_statics)
         if (s.ptr == (uint64_t)p) return;
-    g_shared_statics.push_back(SharedStatic{(uint64_t)p, bytes, 0, {}, {}, {}});
+    g_shared_statics.push_back(SharedStatic{(uint64_t)p, bytes, 0, {}, {}, {}, {}});
 }
 
 extern "C" void sim_switch(void **from_sp, void *to_sp);
@@ -1092,7 +1136,7 @@ static void exec_asm(Fiber **lanes, int n_lanes_total, uint64_t part) {
                         continue;
                     }
                     if (nb == 8 && (addr & 7)) violation("`%s`: lane %d reads 8 bytes at the unaligned LDS address 0x%llx", in.text.c_str(), l, (unsigned long long)addr);
-                    order_access((uint64_t)g_lds + addr, nb, false);
+                    order_access((uint64_t)g_lds + addr, nb, false, true);
                     if (nb == 1) {
                         w.v[o[0].reg][l] = g_lds[addr];
                     } else {
@@ -1228,6 +1272,8 @@ static void exec_collective(Fiber *wave0, int n_lanes) {
         part |= 1ull << l;
     }
     g_cur = lanes[__builtin_ctzll(part)];
+    const uint32_t wave_index = (uint32_t)(wave0 - g_fib) / 64;
+    ++g_wave_epoch[wave_index];  // what the lanes did before this operation lies before it for all of them ...
     auto has = [&](int l) { return l >= 0 && l < 64 && (part >> l & 1); };
     switch (op) {
         case OP_SYNC: break;
@@ -1337,6 +1383,7 @@ static void exec_collective(Fiber *wave0, int n_lanes) {
         case OP_ASM: exec_asm(lanes, n_lanes, part); break;
         default: violation("unknown wavefront-wide operation %d", op); break;
     }
+    ++g_wave_epoch[wave_index];  // ... and what they do next after it
     for (int l = 0; l < 64; ++l)
         if (has(l)) lanes[l]->st = RUN;
 }
@@ -1391,6 +1438,7 @@ static bool run_workgroup(uint32_t nthreads, const LaneCtx &proto) {
                 // everybody else of the wavefront has got as far as it can: the lanes that waited for that go on
                 for (uint32_t t = lo; t < hi; ++t)
                     if (g_fib[t].st == WAIT_WAVE && g_fib[t].op == OP_CATCHUP) g_fib[t].st = RUN;
+                ++g_wave_epoch[wv];
                 progress = true;
             } else if (wait_wave && wait_wave + wait_wg == live_w) {
                 exec_collective(&g_fib[lo], (int)(hi - lo));
@@ -1410,6 +1458,7 @@ static bool run_workgroup(uint32_t nthreads, const LaneCtx &proto) {
                     at_barrier |= 1u << (t / 64);
                 }
             order_barrier(at_barrier);
+            for (uint32_t w = 0; w < n_waves; ++w) ++g_wave_epoch[w];
             progress = true;
         }
         if (!progress) {

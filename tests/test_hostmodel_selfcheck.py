@@ -267,6 +267,20 @@ def test_a_read_of_bytes_that_nothing_has_written_is_reported():
     assert m.violations() == [] and np.array_equal(out.get(), 2 * (26 + np.arange(64)))
 
 
+@in_child
+def test_a_result_that_depends_on_the_order_of_the_lanes_is_reported():
+    """A running sum through the LDS comes out right here, where lane l runs after lane l - 1, and would not on the GPU:
+    the same build reports the pair of accesses."""
+    m = _order_model()
+    out = _u32(m, 64)
+    m.lib.simtest_lane_order(out.p, 0)
+    assert m.violations() == [] and np.array_equal(out.get(), 2 * np.arange(64) + 1)
+    m.lib.simtest_lane_order(out.p, 1)
+    v = m.violations()
+    assert np.array_equal(out.get(), np.cumsum(np.arange(64) + 1))  # (lane order: the sum the GPU would not compute)
+    assert v and "of the same wavefront wrote" in v[0] and "order in which the model runs the lanes" in v[0], v
+
+
 # ---- the build with the compiler's undefined-behaviour checks ---------------------------------------------------------
 def _undefined(which):
     from tests.hostmodel import build
