@@ -232,7 +232,7 @@ __global__ void st_ordering_kernel(uint32_t *out, int which) {
 // A running sum handed from lane to lane through the LDS: right when the lanes run one after the other, as they do in
 // the model, and wrong on the GPU, where they run in step.  which: 0 every lane writes its own word, a wavefront-wide
 // operation, then reads its neighbour's (well defined); 1 lane l adds what lane l - 1 has just stored, with nothing
-// wavefront-wide between the store and the load
+// wavefront-wide between the store and the load; 2 the same through the output array instead of the LDS
 __global__ void st_lane_order_kernel(uint32_t *out, int which) {
     extern __shared__ __align__(16) uint8_t lds[];
     uint32_t *word = reinterpret_cast<uint32_t *>(lds);
@@ -241,10 +241,12 @@ __global__ void st_lane_order_kernel(uint32_t *out, int which) {
         word[lane] = lane + 1;
         __builtin_amdgcn_wave_barrier();
         out[lane] = word[lane] + (lane ? word[lane - 1] : 0u);
-    } else {
+    } else if (which == 1) {
         const uint32_t before = lane ? word[lane - 1] : 0u;
         word[lane] = before + lane + 1;
         out[lane] = word[lane];
+    } else {
+        out[lane] = (lane ? out[lane - 1] : 0u) + lane + 1;
     }
 }
 

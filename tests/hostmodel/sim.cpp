@@ -202,6 +202,8 @@ struct GlobalShadow {
     uint64_t launch = 0;  // the launch its contents belong to
     std::vector<uint32_t> w_id, w_clk, r_id, r_clk;  // per byte: (workgroup + 1) << 4 | wavefront, and that wavefront's clock
     std::vector<uint8_t> written;  // per byte, for the life of the array: something has written it
+    std::vector<uint8_t> w_lane, r_lane;  // the lanes of the last plain write and read (the check inside a wavefront) ...
+    std::vector<uint32_t> w_epoch, r_epoch;  // ... and their wavefront's count of wavefront-wide operations then
 };
 static bool g_check_unwritten = true;
 static std::unordered_map<uint64_t, GlobalShadow> g_global_shadow;  // by Alloc::ptr
@@ -337,7 +339,7 @@ static bool is_shared(uint64_t addr) {
     return false;
 }
 
-static void order_global(const Alloc &a, uint64_t addr, size_t n, bool write) {
+static void order_global(const Alloc &a, uint64_t addr, size_t n, bool write, uint32_t lane) {
     GlobalShadow &s = g_global_shadow[(uint64_t)a.ptr];
     if (s.launch != g_launch_seq || s.w_id.size() != a.bytes) {
         s.launch = g_launch_seq;
@@ -345,14 +347,42 @@ static void order_global(const Alloc &a, uint64_t addr, size_t n, bool write) {
         s.w_clk.assign(a.bytes, 0);
         s.r_id.assign(a.bytes, 0);
         s.r_clk.assign(a.bytes, 0);
+        s.w_lane.assign(a.bytes, 0xFF);
+        s.r_lane.assign(a.bytes, 0xFF);
+        s.w_epoch.assign(a.bytes, 0);
+        s.r_epoch.assign(a.bytes, 0);
     }
     if (s.written.size() != a.bytes) s.written.assign(a.bytes, 0);
     const uint32_t w = cur_wave(), me = (g_wg_index + 1) << 4 | w;
     // did the access `id` at clock `clk` happen before what this wavefront does now?
     auto before = [&](uint32_t id, uint32_t clk) { return id == 0 || id == me || (id >> 4 == me >> 4 && clk <= g_vc[w][id & 15]); };
     const size_t o = (size_t)(addr - (uint64_t)a.ptr);
+    const uint32_t epoch = g_wave_epoch[w];
     for (size_t i = 0; i < n && o + i < a.bytes; ++i) {
         const size_t b = o + i;
+        if (lane != kWholeWave) {  // inside the wavefront, as for the LDS
+            if (s.w_id[b] == me && s.w_lane[b] < 64 && s.w_lane[b] != lane && s.w_epoch[b] == epoch) {
+                order_report("lane %u of workgroup %u wavefront %u %s byte %zu of allocation #%zu (%zu bytes) that lane %u of the same "
+                             "wavefront wrote, and no wavefront-wide operation lies between the two: what this lane sees depends on the "
+                             "order in which the model runs the lanes", lane, g_wg_index, w, write ? "overwrites" : "reads", b,
+                             (size_t)(&a - g_allocs.data()), a.bytes, (unsigned)s.w_lane[b]);
+                return;
+            }
+            if (write && s.r_id[b] == me && s.r_lane[b] < 64 && s.r_lane[b] != lane && s.r_epoch[b] == epoch) {
+                order_report("lane %u of workgroup %u wavefront %u writes byte %zu of allocation #%zu (%zu bytes) that lane %u of the same "
+                             "wavefront read, and no wavefront-wide operation lies between the two: what that lane saw depends on the "
+                             "order in which the model runs the lanes", lane, g_wg_index, w, b, (size_t)(&a - g_allocs.data()), a.bytes,
+                             (unsigned)s.r_lane[b]);
+                return;
+            }
+        }
+        if (write) {
+            s.w_lane[b] = (uint8_t)lane;
+            s.w_epoch[b] = epoch;
+        } else {
+            s.r_lane[b] = (uint8_t)lane;
+            s.r_epoch[b] = epoch;
+        }
         if (!before(s.w_id[b], s.w_clk[b])) {
             order_report("workgroup %u wavefront %u %s byte %zu of allocation #%zu (%zu bytes) that workgroup %u wavefront %u wrote in the "
                          "same launch, and nothing orders the two", g_wg_index, w, write ? "overwrites" : "reads", b,
@@ -398,16 +428,17 @@ static inline void order_access(uint64_t addr, size_t n, bool write, bool whole_
     if (!g_order_on || n == 0) return;
     if (!g_cur) return;  // host code
     if (addr - (uint64_t)g_stacks < (uint64_t)kMaxThreads * kStackBytes) return;  // a fibre's own stack
-    if (order_shared_access(addr, n, write, whole_wave ? kWholeWave : g_cur->ctx.thread_idx.x % 64)) return;
+    const uint32_t lane = whole_wave ? kWholeWave : g_cur->ctx.thread_idx.x % 64;
+    if (order_shared_access(addr, n, write, lane)) return;
     static size_t last = 0;
     if (last < g_allocs.size() && addr - (uint64_t)g_allocs[last].ptr < g_allocs[last].bytes) {
-        order_global(g_allocs[last], addr, n, write);
+        order_global(g_allocs[last], addr, n, write, lane);
         return;
     }
     for (size_t k = 0; k < g_allocs.size(); ++k)
         if (addr - (uint64_t)g_allocs[k].ptr < g_allocs[k].bytes) {
             last = k;
-            order_global(g_allocs[k], addr, n, write);
+            order_global(g_allocs[k], addr, n, write, lane);
             return;
         }
 }
@@ -1169,7 +1200,7 @@ static void exec_asm(Fiber **lanes, int n_lanes_total, uint64_t part) {
                     }
                     if (addr & (nr == 4 ? 15 : 3))
                         violation("`%s`: lane %d loads %d bytes at the unaligned address 0x%llx", in.text.c_str(), l, 4 * nr, (unsigned long long)addr);
-                    order_access(addr, 4 * nr, false);
+                    order_access(addr, 4 * nr, false, true);
                     for (int j = 0; j < nr; ++j) memcpy(&w.v[o[0].reg + j][l], (const void *)(addr + 4 * j), 4);
                 }
                 for (int j = 0; j < nr; ++j) {
@@ -1193,7 +1224,7 @@ static void exec_asm(Fiber **lanes, int n_lanes_total, uint64_t part) {
                                   (unsigned long long)addr, describe_address(addr).c_str());
                         continue;
                     }
-                    order_access(addr, 1, true);
+                    order_access(addr, 1, true, true);
                     *(uint8_t *)addr = (uint8_t)w.v[o[1].reg][l];
                 }
                 break;

@@ -279,6 +279,11 @@ def test_a_result_that_depends_on_the_order_of_the_lanes_is_reported():
     v = m.violations()
     assert np.array_equal(out.get(), np.cumsum(np.arange(64) + 1))  # (lane order: the sum the GPU would not compute)
     assert v and "of the same wavefront wrote" in v[0] and "order in which the model runs the lanes" in v[0], v
+    m.clear()
+    m.lib.simtest_lane_order(out.p, 2)  # the same through an array
+    v = m.violations()
+    assert np.array_equal(out.get(), np.cumsum(np.arange(64) + 1))
+    assert v and "of allocation" in v[0] and "of the same wavefront wrote" in v[0], v
 
 
 # ---- the build with the compiler's undefined-behaviour checks ---------------------------------------------------------
