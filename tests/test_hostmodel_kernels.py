@@ -160,6 +160,9 @@ def test_decode_batch_with_an_empty_tensor_and_a_stream_at_an_odd_address():
     (2048, 128, 9, 1024, 4, True, "fused_linear32_seg_kernel<1, false>"),
     (2048, 128, 64, 1024, 2, True, "fused_linear32_seg_kernel<2, false>"),
     (4096, 64, 2, 1024, 8, True, "fused_linear32_seg_kernel<1, false>"),     # 64 items per column tile: several rounds per job
+    (2048, 320, 9, 256, 2, True, "fused_linear32_seg_kernel<1, false>"),     # ten jobs on four CUs: sums through the window areas, job after job
+    (2048, 320, 40, 256, 2, True, "fused_linear32_seg_kernel<2, false>"),
+    (2048, 320, 3, 256, 2, True, "fused_linear32_seg_kernel<1, false>"),     # ... and handed over without a barrier, job after job
     (1024, 320, 4, 256, 1, False, "fused_linear32_seg_kernel<1, true>"),     # low tiles, several column tiles per job
     (2048 + 100, 100, 5, 1024, 2, False, "fused_linear32_seg_kernel<1, true>"),  # ragged: guarded path inside the kernel
     (3072, 96, 7, 2048, 1, False, "fused_linear32_kernel<1>"),
@@ -479,6 +482,49 @@ def test_encoders(layout, th, tw):
     m = Model(cus=4)
     for K, N, seed in ((1500, 100, 1), (th, tw, 2), (2 * th + 1, 3 * tw + 5, 3)):
         cases.encode(m, ro.split_bf16(weight_bits(K, N, seed))[0], th, tw, layout)
+
+
+@pytest.mark.parametrize("K,N,min_block", [(300, 8, 512), (512, 33, 512), (1500, 16, 512), (1024, 5, 256), (1, 1, 512)])
+@in_child
+def test_flat_layout_encoder_and_decoders(K, N, min_block):
+    """a8, the legacy layout (512-row segments, bytes strided by the stream count, a checkpoint every 128 symbols): the
+    library's encoder and packer against the oracle's, every output array compared, and both decoders on the result."""
+    import ctypes as C
+
+    from oracle import rans_oracle as ro
+
+    m = Model(cus=4)
+    exp = ro.split_bf16(weight_bits(K, N, 7))[0]
+    f, c = ro.get_lut(exp)
+    want = ro.encode_flat(exp, f, c, min_block)
+    S, cap = C.c_uint32(0), C.c_uint32(0)
+    m.call("ci_flat_geometry", K, N, min_block, C.byref(S), C.byref(cap))
+    assert S.value == want.num_streams
+    nb = m.lib.ci_encode_scratch_bytes(S.value, cap.value)
+    sym, scratch = m.dev(exp), m.empty(nb, np.uint8)
+    states, sizes, ck = m.empty(S.value, np.uint32), m.empty(S.value, np.uint32), m.empty(S.value * 128, np.uint64)
+    f16, c16 = np.ascontiguousarray(f, np.uint16), np.ascontiguousarray(c, np.uint16)
+    max_len = C.c_uint32(0)
+    m.call("ci_encode_flat", sym.p, K, N, S.value, cap.value, f16.ctypes.data_as(C.c_void_p), c16.ctypes.data_as(C.c_void_p),
+           scratch.p, C.c_size_t(nb), states.p, sizes.p, ck.p, C.byref(max_len), None)
+    assert "max_len_kernel" in m.launches()
+    stream = m.empty(max_len.value * S.value, np.uint8)
+    m.call("ci_pack_flat", scratch.p, S.value, cap.value, sizes.p, max_len.value, stream.p, None)
+    assert np.array_equal(states.get(), want.states) and np.array_equal(sizes.get(), want.sizes)
+    assert np.array_equal(stream.get(), want.stream), "packed stream differs from the oracle's"
+    assert np.array_equal(ck.get(), want.checkpoints), "checkpoints differ from the oracle's"
+    tables, slot_map = m.dev(want.tables), m.dev(want.slot_map)
+    out = m.empty((K, N), np.uint8)
+    m.clear()
+    m.call("ci_decode_flat_segmented", stream.p, C.c_uint64(stream.nbytes), states.p, sizes.p, S.value, tables.p, slot_map.p,
+           K, N, out.p, None)
+    assert any("decode_flat_kernel" in k for k in m.launches()), m.launches()
+    assert np.array_equal(out.get(), exp), "segmented decode differs from the plane"
+    # the extension's decoder: symbol i of stream g at g + i * streams
+    flat = m.empty(K * N, np.uint8)
+    m.call("ci_decode_flat_strided", stream.p, C.c_uint64(stream.nbytes), states.p, sizes.p, S.value, tables.p, slot_map.p,
+           C.c_uint64(K * N), flat.p, None)
+    assert np.array_equal(flat.get(), ro.decode_flat_strided(want.stream, want.states, want.sizes, want.tables, want.slot_map, K * N))
 
 
 @pytest.mark.parametrize("layout,th,tw", [("one", 256, 32), ("one", 64, 16), ("one", 1024, 128), ("dense", 512, 32),
