@@ -1515,6 +1515,12 @@ void allow_dynamic_lds(const void *fn, int bytes) { g_dynamic_lds_allowed[fn] = 
 void launch(const char *name, const void *fn, Dim3 grid, Dim3 block, size_t shmem, const std::function<void()> &body) {
     sim_init();
     g_launches.push_back(name);
+    if (const char *log = getenv("CI_HOSTMODEL_LAUNCH_LOG")) {  // every launch of a test run, for a look at which kernels it reaches
+        if (FILE *f = fopen(log, "a")) {
+            fprintf(f, "%s\n", name);
+            fclose(f);
+        }
+    }
     const uint32_t nthreads = block.x * block.y * block.z;
     g_kernel = name;
     if (shmem > 65536) {

@@ -249,7 +249,8 @@ def test_fused_linear_on_unusual_planes(kind):
     (4096, 63, 100, 1024, 8, True, "embed_gather32_seg_kernel"),    # ... of a whole pair of tiles
     (2048, 127, 64, 1024, 8, False, "embed_gather32_kernel"),
     (70000, 64, 2048, 1024, 8, True, "embed_gather32_seg_kernel"),
-    (270000, 32, 500, 32, 1, False, "embed_sort_kernel"),            # more buckets than counting slots: the sort
+    (270000, 32, 500, 32, 1, False, "embed_sort_kernel<true>"),      # more buckets than counting slots: the sort
+    (530000, 32, 500, 32, 1, False, "embed_sort_kernel<false>"),     # ... of ids that do not fit the packed key (2^19 rows and more)
     (2048, 32, 8192, 1024, 4, True, "embed_gather32_seg_kernel"),    # exactly one pass of ids: no second, empty pass
     (2048, 32, 8192 + 3, 1024, 1, False, "embed_gather32_kernel"),   # a second pass of three ids
     (300000, 32, 16384, 32, 1, False, "embed_sort_kernel"),          # two whole passes through the sort

@@ -35,13 +35,34 @@ def _env():
     return env
 
 
-def test_every_kernel_case_with_ordering_checked():
+def _kernels_the_host_code_can_launch():
+    """Every kernel instance named in a launch of the library's sources."""
+    import glob
+    import re
+
+    names = set()
+    for path in glob.glob(os.path.join(ROOT, "comp_inference_amd", "csrc", "*.hip")):
+        for m in re.finditer(r"hipLaunchKernelGGL\(\s*\(?\s*([a-z0-9_]+(?:<[^>]*>)?)", open(path).read()):
+            names.add(m.group(1).replace(" ", ""))
+    macro = "fused_linear32_seg_kernel<MB_,COLD_>"  # (instantiated for one and two groups of rows, with and without guarded path)
+    assert macro in names
+    names.remove(macro)
+    names |= {f"fused_linear32_seg_kernel<{mb},{cold}>" for mb in (1, 2) for cold in ("true", "false")}
+    return names
+
+
+def test_every_kernel_case_with_ordering_checked(tmp_path):
+    """... and, from the same run's log of launches: the cases reach every kernel instance the host code can launch."""
     cmd = [sys.executable, "-m", "pytest", "tests/test_hostmodel_kernels.py", "-q", "-x", "-p", "no:cacheprovider", "-n", "6"]
     for case in BY_DESIGN:
         cmd += ["--deselect", case]
-    p = subprocess.run(cmd, cwd=ROOT, env=_env(), capture_output=True, text=True, timeout=1500)
+    log = tmp_path / "launches.log"
+    p = subprocess.run(cmd, cwd=ROOT, env=dict(_env(), CI_HOSTMODEL_LAUNCH_LOG=str(log)), capture_output=True, text=True, timeout=1500)
     assert p.returncode == 0, p.stdout[-6000:] + p.stderr[-2000:]
     assert " passed" in p.stdout and "failed" not in p.stdout, p.stdout[-2000:]
+    launched = {line.strip().strip("()").replace(" ", "") for line in log.read_text().splitlines() if not line.startswith("st_")}
+    can = _kernels_the_host_code_can_launch()
+    assert len(can) > 50 and can - launched == set(), f"kernels no case of tests/test_hostmodel_kernels.py launches: {sorted(can - launched)}"
 
 
 def test_the_forced_give_up_is_seen_as_what_it_is():
