@@ -162,7 +162,6 @@ static std::string where() {
 //     clock at its address, one with acquire semantics takes what was left there.
 //   * arrays from sim_alloc: the same inside a workgroup; between workgroups of one launch nothing orders anything, so
 //     a byte written by one workgroup and read or written by another is reported.  Launches are ordered by the stream.
-// Atomic accesses themselves are not recorded (they do not race with each other).
 //   * inside one wavefront: on the GPU the lanes run in step, so an LDS write that comes earlier in the program than a
 //     read has happened for every lane before any lane reads.  Here the lanes are fibres that run one after the other
 //     between two wavefront-wide operations, so a lane can see a later lane's byte too early or an earlier lane's too
@@ -174,6 +173,7 @@ static std::string where() {
 //     of the library (hipMemsetAsync, hipMemcpyAsync), no kernel -- and that a kernel reads.  On the GPU such a byte
 //     holds what an earlier launch left there.  The fill pattern of sim_alloc is a tiny number both as fp32 and as
 //     bf16, so a sum that includes such bytes passes every tolerance; here the read itself is the violation.
+// Atomic accesses themselves are not recorded (they do not race with each other).
 constexpr int kMaxWaves = kMaxThreads / 64;
 static bool g_order_on = false;
 static uint32_t g_vc[kMaxWaves][kMaxWaves];
@@ -222,7 +222,7 @@ static void order_start_workgroup(uint32_t n_waves, size_t lds_open) {
     if (!g_order_on) return;
     ++g_workgroup_seq;
     if (!g_sh_wwave) {
-        const size_t n = kLdsBytes;
+        const size_t n = kLdsBytes + 16;  // (an access that starts at the last byte: it faults, after the check)
         g_sh_wwave = (uint8_t *)malloc(n);
         g_sh_wclk = (uint32_t *)malloc(n * 4);
         g_sh_rclk = (uint32_t *)malloc(n * 4 * kMaxWaves);
