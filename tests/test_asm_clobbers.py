@@ -4,7 +4,8 @@ The sources are preprocessed for the device (`hipcc -E`), every `asm volatile(..
 template, outputs, inputs and clobbers, the template is read instruction by instruction, and every register an
 instruction writes -- a named operand, a literal VGPR / SGPR, `vcc`, `scc`, `exec` -- must be an output operand, a
 listed clobber or, for `exec`, restored from the saved copy inside the statement.  A statement that leaves one
-out lets the compiler keep a live value (a loop compare in SCC, say) across it.
+out lets the compiler keep a live value (a loop compare in SCC, say) across it.  A statement with a memory
+instruction must list "memory": the bytes it reads were stored by C++ code the compiler is otherwise free to move.
 """
 from __future__ import annotations
 
@@ -202,6 +203,11 @@ def check_statement(body: str):
         for name, cons in outs.items():
             if cons.startswith("=") and "&" not in cons:
                 problems.append(f"output %[{name}] of a multi-instruction statement is not early-clobber (\"=&\")")
+    # a statement that reads or writes memory says so: without "memory" among the clobbers the compiler may move the C++
+    # stores that stage bytes in the LDS behind the statement that reads them, or drop them (nothing it can see reads them)
+    touches_memory = any(re.match(r"(ds_|global_|buffer_|flat_|scratch_|s_load|s_buffer_load)", line.split()[0]) for line in lines)
+    if touches_memory and "memory" not in clobbers:
+        problems.append("an instruction reads or writes memory and \"memory\" is not a clobber")
     # loads issued inside the statement are drained before it ends (the compiler knows nothing of them)
     issued_lgkm = issued_vm = False
     for line in lines:
@@ -253,3 +259,7 @@ def test_the_checker_sees_a_missing_scc_clobber():
     assert any("early-clobber" in p for p in check_statement(
         r'"v_mov_b32 %[e], %[n]\n" "v_mov_b32 v3, %[n]\n" : [e] "=v"(e) : [n] "v"(n) : "v3"')[0])
     assert any("in flight" in p for p in check_statement(r'"ds_read_b32 %[e], %[n]\n" : [e] "=&v"(e) : [n] "v"(n) :')[0])
+    # a memory instruction without "memory" among the clobbers
+    load = r'"ds_read_b32 %[e], %[n]\n" "s_waitcnt lgkmcnt(0)\n" : [e] "=&v"(e) : [n] "v"(n) : '
+    assert any('"memory" is not a clobber' in p for p in check_statement(load)[0])
+    assert check_statement(load + '"memory"')[0] == []
