@@ -150,3 +150,28 @@ def test_what_the_hand_scheduled_loops_issue_per_step(tmp_path):
                 seen[family] += 1
     # every kernel that contains a statement has its own copy of the loop
     assert seen["ci_dec_loop"] >= 2 and seen["ci_lin_loop"] >= 4 and seen["ci_lin2_loop"] >= 4, seen
+
+
+@pytest.mark.skipif(not (os.path.exists(OBJDUMP) and os.path.exists(LIB)), reason="needs the built library and llvm-objdump")
+def test_kernels_that_read_staged_bytes_also_stage_them(tmp_path):
+    """The decode step reads its stream bytes from the LDS inside assembly statements; the bytes get there by plain
+    C++ stores that nothing the compiler can see ever reads.  The statements list "memory" so that the stores stay
+    where they are (tests/test_asm_clobbers.py); here the machine code itself is looked at: every kernel with the
+    step's byte reads also stores to the LDS, and the sixteen-wavefront kernels, which stage a window as it lies in
+    memory, sixteen bytes a lane and piece, hold those 16-byte stores."""
+    shutil.copy(LIB, tmp_path / "lib.so")
+    subprocess.run([OBJDUMP, "--offloading", "lib.so"], cwd=tmp_path, check=True, capture_output=True)
+    seen = {}
+    for f in sorted(os.listdir(tmp_path)):
+        if "gfx950" not in f:
+            continue
+        text = subprocess.run([OBJDUMP, "-d", str(tmp_path / f)], check=True, capture_output=True, text=True).stdout
+        for name, body in H.kernels_of(text).items():
+            mn = [i.text.split()[0] for i in body]
+            if "ds_read_u8" in mn:
+                seen[name] = (sum(m.startswith("ds_write") for m in mn), mn.count("ds_write_b128"))
+    assert len(seen) >= 20, sorted(seen)
+    for name, (stores, wide) in seen.items():
+        assert stores >= 9, (name, stores)
+        if "_seg_kernel" in name:
+            assert wide >= 7, (name, wide)  # one per piece of a window, at least
