@@ -161,16 +161,20 @@ def test_kernels_that_read_staged_bytes_also_stage_them(tmp_path):
     memory, sixteen bytes a lane and piece, hold those 16-byte stores."""
     shutil.copy(LIB, tmp_path / "lib.so")
     subprocess.run([OBJDUMP, "--offloading", "lib.so"], cwd=tmp_path, check=True, capture_output=True)
-    seen = {}
+    seen, flat = {}, []
     for f in sorted(os.listdir(tmp_path)):
         if "gfx950" not in f:
             continue
         text = subprocess.run([OBJDUMP, "-d", str(tmp_path / f)], check=True, capture_output=True, text=True).stdout
         for name, body in H.kernels_of(text).items():
             mn = [i.text.split()[0] for i in body]
+            flat += [f"{name}: {m}" for m in mn if m.startswith("flat_")]
             if "ds_read_u8" in mn:
                 seen[name] = (sum(m.startswith("ds_write") for m in mn), mn.count("ds_write_b128"))
     assert len(seen) >= 20, sorted(seen)
+    # (and no kernel holds a flat memory instruction: a flat load counts against the LDS counter too, which every
+    # `s_waitcnt lgkmcnt` of the step would then wait for -- what a `volatile` access compiles to)
+    assert flat == [], flat
     for name, (stores, wide) in seen.items():
         assert stores >= 9, (name, stores)
         if "_seg_kernel" in name:
