@@ -85,9 +85,11 @@ def test_random_cases_with_ordering_checked(family, monkeypatch):
 
 def test_the_gpu_tests_of_the_operators_with_ordering_checked():
     """The tests written for the GPU (tests/test_hostmodel_gpu_suite.py runs them on the plain model), on this build:
-    the operators' files and the four whose kernels have not run on a GPU.  Their tensors are torch's, memory that is
+    the operators' files, the runtime modules, the entry point without allocation and the four files whose kernels have
+    not run on a GPU.  Their tensors are torch's, memory that is
     not the model's, so what is checked here is the LDS side; the arrays are checked in the cases above."""
     files = ["test_gpu_codec.py", "test_gpu_linear.py", "test_gpu_embedding.py", "test_gpu_transposed.py",
+             "test_gpu_runtime.py", "test_zz_no_alloc.py", "test_golden.py",
              "wip_one_stream.py", "wip_transposed_seg.py", "wip_linear_wide.py", "wip_gather_seg.py"]
     env = dict(_env(), OMP_NUM_THREADS="2", PYTHONPATH=ROOT)
     procs = {f: subprocess.Popen([sys.executable, "-m", "pytest", os.path.join("tests", f), "-m", "gpu", "-q", "-p",
